@@ -1,0 +1,458 @@
+// C ABI of libgemmkernels_hip.so: host-side checks, kernel-instance selection and launch.
+// See include/gemmkernels_hip.h for the contract and the reference lines each entry replaces.
+#include "gemmkernels_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "kernels/common.hpp"
+#include "kernels/registry.hpp"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+std::atomic<long long> g_lds_override{0};
+std::atomic<int> g_threads_override{0};
+
+void device_limits(long long* lds, int* threads) {
+  long long l = g_lds_override.load();
+  int t = g_threads_override.load();
+  if (l <= 0 || t <= 0) {
+    int dev = 0, v = 0;
+    long long ql = 160 * 1024;
+    int qt = 1024;
+    if (hipGetDevice(&dev) == hipSuccess) {
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && v > 0) ql = v;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxThreadsPerBlock, dev) == hipSuccess && v > 0) qt = v;
+    } else {
+      (void)hipGetLastError();   // no device: keep the MI355X defaults
+    }
+    if (l <= 0) l = ql;
+    if (t <= 0) t = qt;
+  }
+  *lds = l;
+  *threads = t;
+}
+
+bool is_checked_layout(int kind) { return kind == GK_LAYOUT_COL_MAJOR || kind == GK_LAYOUT_ROW_MAJOR; }
+bool is_row_major(int kind) {
+  return kind == GK_LAYOUT_ROW_MAJOR || kind == GK_LAYOUT_ALIGNED_ROW_MAJOR || kind == GK_LAYOUT_INTERLEAVED_ROW_MAJOR ||
+         kind == GK_LAYOUT_SPLIT_ROW_MAJOR;
+}
+// reference src/config.jl:175-178
+bool require_tile_sized_global(int kind) { return !(kind == GK_LAYOUT_ZERO || is_checked_layout(kind)); }
+
+bool valid_layout_kind(int k) { return k >= GK_LAYOUT_ZERO && k <= GK_LAYOUT_GETT; }
+
+int dtype_size(int dt) {
+  switch (dt) {
+    case GK_F16: case GK_BF16: return 2;
+    case GK_F32: return 4;
+    case GK_F64: return 8;
+    default: return 0;
+  }
+}
+
+bool is_mfma_kind(int k) { return k == GK_OP_MFMA || k == GK_OP_MFMA_COMPLEX || k == GK_OP_MFMA_DUAL; }
+bool is_fpu_kind(int k) { return k == GK_OP_FPU || k == GK_OP_FPU_TROPICAL; }
+
+bool transforms_present(const gk_transforms* t) {
+  if (!t) return false;
+  for (int h = 0; h < 8; ++h)
+    if (t->hook[h].n_ops > 0) return true;
+  return false;
+}
+
+// Builds the run-time key of the kernel instance for a configuration.
+int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key) {
+  memset(key, 0, sizeof(*key));
+  const int ak = c->global_a_layout.kind, bk = c->global_b_layout.kind;
+  const int ck = c->global_c_layout.kind, dk = c->global_d_layout.kind;
+  const bool any_gett = ak == GK_LAYOUT_GETT || bk == GK_LAYOUT_GETT || ck == GK_LAYOUT_GETT || dk == GK_LAYOUT_GETT;
+  const bool any_checked = is_checked_layout(ak) || is_checked_layout(bk) || is_checked_layout(ck) || is_checked_layout(dk);
+  switch (c->op.kind) {
+    case GK_OP_MFMA:
+      if (ak == GK_LAYOUT_DIAGONAL) key->family = gk::FAMILY_DIAGONAL;
+      else if (any_gett) key->family = gk::FAMILY_GETT;
+      else if (any_checked) key->family = gk::FAMILY_MFMA_CHECKED;
+      else key->family = gk::FAMILY_MFMA;
+      break;
+    case GK_OP_FPU:
+    case GK_OP_FPU_TROPICAL:
+      key->family = gk::FAMILY_FPU;
+      key->variant = (c->op.kind == GK_OP_FPU_TROPICAL) ? 1 : 0;
+      break;
+    case GK_OP_MFMA_COMPLEX:
+    case GK_OP_MFMA_DUAL:
+      key->family = gk::FAMILY_COMPLEX;
+      key->variant = (c->op.kind == GK_OP_MFMA_DUAL) ? 1 : 0;
+      break;
+    default:
+      return fail(GK_ERR_INVALID_ARGUMENT, "unknown operator kind %d", c->op.kind);
+  }
+  key->BM = c->block_shape.M;
+  key->BN = c->block_shape.N;
+  key->BK = c->block_shape.K;
+  if (c->compute_warp.M <= 0 || c->compute_warp.N <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "compute_warp must be positive");
+  key->waves_m = c->block_shape.M / c->compute_warp.M;
+  key->waves_n = c->block_shape.N / c->compute_warp.N;
+  key->a_kmajor = is_row_major(ak) ? 1 : 0;    // 'T' A: stored K x M, K contiguous
+  key->b_kmajor = is_row_major(bk) ? 0 : 1;    // 'N' B: stored K x N, K contiguous
+  key->dtype = c->global_a_layout.eltype;
+  key->fused = (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT)) ? 1 : 0;
+  return GK_OK;
+}
+
+void make_args(const gk_config* c, const void* a, const void* b, const void* cc, void* d, const gk_transforms* t,
+               const gk_epilogue* e, gk::GemmArgs* args) {
+  memset(args, 0, sizeof(*args));
+  args->a = a; args->b = b; args->c = cc; args->d = d;
+  args->bias = e ? (const float*)e->bias : nullptr;
+  args->M = c->matmul_shape.M; args->N = c->matmul_shape.N; args->K = c->matmul_shape.K;
+  const bool a_row = is_row_major(c->global_a_layout.kind), b_row = is_row_major(c->global_b_layout.kind);
+  args->lda = c->global_a_layout.ld > 0 ? c->global_a_layout.ld : (a_row ? args->K : args->M);
+  args->ldb = c->global_b_layout.ld > 0 ? c->global_b_layout.ld : (b_row ? args->N : args->K);
+  args->ldc = c->global_c_layout.ld > 0 ? c->global_c_layout.ld : args->M;
+  args->ldd = c->global_d_layout.ld > 0 ? c->global_d_layout.ld : args->M;
+  args->nbm = (args->M + c->block_shape.M - 1) / c->block_shape.M;
+  args->nbn = (args->N + c->block_shape.N - 1) / c->block_shape.N;
+  args->swz_kind = c->cta_swizzle.kind;
+  args->swz_param = c->cta_swizzle.param;
+  args->c_mode = (c->global_c_layout.kind == GK_LAYOUT_ZERO) ? 0 : 1;
+  args->epi_kind = e ? e->kind : 0;
+  args->c_dtype = c->global_c_layout.eltype;
+  args->d_dtype = c->global_d_layout.eltype;
+  args->a_kind = c->global_a_layout.kind;
+  args->b_kind = c->global_b_layout.kind;
+  args->cd_gett = (c->global_d_layout.kind == GK_LAYOUT_GETT) ? 1 : 0;
+  if (t) {
+    for (int h = 0; h < 8; ++h) {
+      const gk_transform& src = t->hook[h];
+      gk::OpList& dst = args->t[h];
+      int n = src.n_ops < 0 ? 0 : (src.n_ops > GK_MAX_OPS ? GK_MAX_OPS : src.n_ops);
+      int out = 0;
+      for (int i = 0; i < n; ++i) {
+        if (src.ops[i].kind == GK_T_IDENTITY) continue;
+        dst.kind[out] = src.ops[i].kind;
+        dst.p0[out] = src.ops[i].p0;
+        dst.p1[out] = src.ops[i].p1;
+        ++out;
+      }
+      dst.n = out;
+    }
+  }
+  auto copy_dim = [](const gk_gett_dim& s, gk::GettDim& d) {
+    d.nmodes = s.nmodes;
+    for (int i = 0; i < GK_MAX_MODES; ++i) {
+      d.extent[i] = s.extent[i];
+      d.stride0[i] = s.stride0[i];
+      d.stride1[i] = s.stride1[i];
+    }
+  };
+  copy_dim(c->gett.m, args->gm);
+  copy_dim(c->gett.n, args->gn);
+  copy_dim(c->gett.k, args->gk);
+}
+
+gk::FamilyFn family_fn(const gk::InstanceKey& key) {
+  switch (key.family) {
+    case gk::FAMILY_MFMA:
+      if (key.a_kmajor) return key.b_kmajor ? gk::family_mfma_tn : gk::family_mfma_tt;
+      return key.b_kmajor ? gk::family_mfma_nn : gk::family_mfma_nt;
+    default:
+      return nullptr;
+  }
+}
+
+int find_instance(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, gk::InstanceInfo* info) {
+  int rc = make_key(c, t, e, key);
+  if (rc != GK_OK) return rc;
+  gk::FamilyFn fn = family_fn(*key);
+  gk::GemmArgs dummy;
+  memset(&dummy, 0, sizeof(dummy));
+  hipError_t err = hipSuccess;
+  if (!fn || !fn(*key, dummy, dim3(1), nullptr, 0, info, &err)) {
+    return fail(GK_ERR_UNSUPPORTED,
+                "no compiled kernel instance for operator %d, block (%d, %d, %d), warps %d x %d, A/B layouts %d/%d, eltype %d",
+                c->op.kind, key->BM, key->BN, key->BK, key->waves_m, key->waves_n, c->global_a_layout.kind,
+                c->global_b_layout.kind, key->dtype);
+  }
+  return GK_OK;
+}
+
+// All checks that need no pointers; reference src/config.jl:203-275 then src/matmul.jl:28-41.
+int validate_config(const gk_config* c, int kernel, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key,
+                    gk::InstanceInfo* info) {
+  if (!c) return fail(GK_ERR_INVALID_ARGUMENT, "config is NULL");
+  const gk_shape& g = c->matmul_shape;
+  const gk_shape& b = c->block_shape;
+  const gk_operator& op = c->op;
+  if (g.M <= 0 || g.N <= 0 || g.K <= 0) return fail(GK_ERR_DIMENSION_MISMATCH, "matmul_shape must be positive, got (%d, %d, %d)", g.M, g.N, g.K);
+  if (b.M <= 0 || b.N <= 0 || b.K <= 0) return fail(GK_ERR_BLOCK_SHAPE, "block_shape must be positive");
+  if (kernel < GK_KERNEL_SINGLESTAGE || kernel > GK_KERNEL_PIPELINED_NG) return fail(GK_ERR_INVALID_ARGUMENT, "unknown kernel kind %d", kernel);
+  const gk_layout* layouts[8] = {&c->global_a_layout, &c->global_b_layout, &c->global_c_layout, &c->global_d_layout,
+                                 &c->shared_a_layout, &c->shared_b_layout, &c->shared_c_layout, &c->shared_d_layout};
+  for (const gk_layout* l : layouts)
+    if (!valid_layout_kind(l->kind)) return fail(GK_ERR_INVALID_ARGUMENT, "unknown layout kind %d", l->kind);
+  if (c->cta_swizzle.kind < GK_SWIZZLE_IDENTITY || c->cta_swizzle.kind > GK_SWIZZLE_XCD)
+    return fail(GK_ERR_INVALID_ARGUMENT, "unknown CTA swizzle kind %d", c->cta_swizzle.kind);
+  if ((c->cta_swizzle.kind == GK_SWIZZLE_HORIZONTALLY_TILED || c->cta_swizzle.kind == GK_SWIZZLE_VERTICALLY_TILED) && c->cta_swizzle.param <= 0)
+    return fail(GK_ERR_INVALID_ARGUMENT, "tiled CTA swizzles need a positive tile size");
+
+  // src/config.jl:203-205
+  if ((long long)b.M * b.K < 128 || (long long)b.K * b.N < 128 || b.K < 8)
+    return fail(GK_ERR_BLOCK_SHAPE,
+                "The block shape is too small. The dimensions of the block shape must adhere to the following constraints: "
+                "BLOCK_M * BLOCK_K >= 128, BLOCK_K * BLOCK_N >= 128, BLOCK_K >= 8.");
+  // src/config.jl:209-212
+  if (b.M < 2 * op.M || b.N < 2 * op.N || b.K < op.K)
+    return fail(GK_ERR_BLOCK_SHAPE,
+                "There is a mismatch between the block shape and the operator shape. Their dimensions must adhere to the "
+                "following constraints: BLOCK_M >= 2 * OPERATOR_M, BLOCK_N >= 2 * OPERATOR_N, BLOCK_K >= OPERATOR_K.");
+  // src/config.jl:136-173, with 64-lane wavefronts
+  if (is_fpu_kind(op.kind)) {
+    if (op.M * op.N < gk::kWaveSize)
+      return fail(GK_ERR_OP_SHAPE, "The operator shape is too small. The dimensions of the operator shape must adhere to the following constraint: OPERATOR_M * OPERATOR_N >= 64.");
+    if (op.mb * op.nb != gk::kWaveSize)
+      return fail(GK_ERR_OP_SHAPE, "The base FPU operator shape should adhere to the following constraint: OPERATOR_M_BASE * OPERATOR_N_BASE = 64.");
+    if (op.kb != 1)
+      return fail(GK_ERR_OP_SHAPE, "The base FPU operator shape should adhere to the following constraint: OPERATOR_K_BASE = 1.");
+    if (op.M % op.mb != 0 || op.N % op.nb != 0 || op.K % op.kb != 0)
+      return fail(GK_ERR_OP_SHAPE, "The operator shape should adhere to the following constraint: OPERATOR_M, OPERATOR_N, OPERATOR_K are multiples of OPERATOR_M_BASE, OPERATOR_N_BASE, OPERATOR_K_BASE, respectively.");
+  } else if (is_mfma_kind(op.kind)) {
+    const bool native = (op.M == 32 && op.N == 32 && op.K == 16);
+    const bool wmma_compat = (op.K == 16) && ((op.M == 16 && op.N == 16) || (op.M == 8 && op.N == 32) || (op.M == 32 && op.N == 8));
+    if (!native && !wmma_compat) return fail(GK_ERR_OP_SHAPE, "Unsupported MFMA Operator shape (M = %d, N = %d, K = %d)!", op.M, op.N, op.K);
+  } else {
+    return fail(GK_ERR_INVALID_ARGUMENT, "unknown operator kind %d", op.kind);
+  }
+  if (c->warps_per_block <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "warps_per_block must be positive");
+  // src/config.jl:263-265
+  const long long w = c->warps_per_block;
+  if ((long long)c->mem_a_warp.M * c->mem_a_warp.K * w > (long long)b.M * b.K)
+    return fail(GK_ERR_MEM_TILE, "mem_a_warp is too big for the selected block shape: need at least one iteration in the memory copy loop!");
+  if ((long long)c->mem_b_warp.K * c->mem_b_warp.N * w > (long long)b.K * b.N)
+    return fail(GK_ERR_MEM_TILE, "mem_b_warp is too big for the selected block shape: need at least one iteration in the memory copy loop!");
+  if ((long long)c->mem_cd_warp.M * c->mem_cd_warp.N * w > (long long)b.M * b.N)
+    return fail(GK_ERR_MEM_TILE, "mem_cd_warp is too big for the selected block shape: need at least one iteration in the memory copy loop!");
+  // src/config.jl:268-275
+  const gk_shape& cw = c->compute_warp;
+  const gk_shape& os = c->compute_op_shape;
+  if (cw.M <= 0 || cw.N <= 0 || cw.K <= 0 || os.M <= 0 || os.N <= 0 || os.K <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "compute_warp and compute_op_shape must be positive");
+  if (b.M % cw.M || b.N % cw.N || b.K % cw.K) return fail(GK_ERR_TILE_MULTIPLE, "block_shape must be a multiple of compute_warp!");
+  if (cw.M % os.M || cw.N % os.N || cw.K % os.K) return fail(GK_ERR_TILE_MULTIPLE, "compute_warp must be a multiple of op_shape!");
+  if (require_tile_sized_global(c->global_a_layout.kind) && (g.M % b.M || g.K % b.K))
+    return fail(GK_ERR_TILE_MULTIPLE, "gemm_shape.MK must be a multiple of block_shape.MK!");
+  if (require_tile_sized_global(c->global_b_layout.kind) && (g.K % b.K || g.N % b.N))
+    return fail(GK_ERR_TILE_MULTIPLE, "gemm_shape.KN must be a multiple of block_shape.KN!");
+  if (require_tile_sized_global(c->global_c_layout.kind) && (g.M % b.M || g.N % b.N))
+    return fail(GK_ERR_TILE_MULTIPLE, "gemm_shape.MN must be a multiple of block_shape.MN!");
+  if (require_tile_sized_global(c->global_d_layout.kind) && (g.M % b.M || g.N % b.N))
+    return fail(GK_ERR_TILE_MULTIPLE, "gemm_shape.MN must be a multiple of block_shape.MN!");
+
+  // the instance that would run; its LDS request is what Kernel.shmem_size returns
+  int rc = find_instance(c, t, e, key, info);
+  if (rc != GK_OK) return rc;
+
+  long long lds_max = 0;
+  int threads_max = 0;
+  device_limits(&lds_max, &threads_max);
+  // src/matmul.jl:28-31
+  if (info->lds_bytes > lds_max)
+    return fail(GK_ERR_LDS, "Requested too much shared memory: The current GPU can use at most %lld bytes, while this configuration required %d bytes",
+                lds_max, info->lds_bytes);
+  // src/matmul.jl:34-36
+  if (kernel != GK_KERNEL_SINGLESTAGE && b.K < 2 * os.K)
+    return fail(GK_ERR_STAGES, "Need at least two stages to use a pipelined kernel, i.e. BLOCK_K >= 2 * OPERATOR_K");
+  // src/matmul.jl:41
+  const long long threads = (long long)c->warps_per_block * gk::kWaveSize;
+  if (threads > threads_max)
+    return fail(GK_ERR_THREADS, "Requested too many threads for this kernel: This kernel can be launched using at most %d threads, while this configuration required %lld",
+                threads_max, threads);
+  if (threads != info->threads)
+    return fail(GK_ERR_UNSUPPORTED, "warps_per_block = %d does not match the %d waves of block_shape / compute_warp", c->warps_per_block,
+                info->threads / gk::kWaveSize);
+  return GK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gk_version(void) { return GK_VERSION; }
+
+size_t gk_last_error(char* buf, size_t n) {
+  if (buf && n > 0) {
+    size_t m = g_last_error.size() < n - 1 ? g_last_error.size() : n - 1;
+    memcpy(buf, g_last_error.data(), m);
+    buf[m] = 0;
+  }
+  return g_last_error.size();
+}
+
+const char* gk_status_string(int status) {
+  switch (status) {
+    case GK_OK: return "GK_OK";
+    case GK_ERR_INVALID_ARGUMENT: return "GK_ERR_INVALID_ARGUMENT";
+    case GK_ERR_LDS: return "GK_ERR_LDS";
+    case GK_ERR_STAGES: return "GK_ERR_STAGES";
+    case GK_ERR_THREADS: return "GK_ERR_THREADS";
+    case GK_ERR_BLOCK_SHAPE: return "GK_ERR_BLOCK_SHAPE";
+    case GK_ERR_OP_SHAPE: return "GK_ERR_OP_SHAPE";
+    case GK_ERR_MEM_TILE: return "GK_ERR_MEM_TILE";
+    case GK_ERR_TILE_MULTIPLE: return "GK_ERR_TILE_MULTIPLE";
+    case GK_ERR_ALIGNMENT: return "GK_ERR_ALIGNMENT";
+    case GK_ERR_UNSUPPORTED: return "GK_ERR_UNSUPPORTED";
+    case GK_ERR_DIMENSION_MISMATCH: return "GK_ERR_DIMENSION_MISMATCH";
+    case GK_ERR_HIP: return "GK_ERR_HIP";
+    default: return "GK_ERR_UNKNOWN";
+  }
+}
+
+int gk_set_device_limits(int64_t lds_bytes, int32_t max_threads) {
+  g_lds_override.store(lds_bytes > 0 ? lds_bytes : 0);
+  g_threads_override.store(max_threads > 0 ? max_threads : 0);
+  return GK_OK;
+}
+
+int gk_validate(const gk_config* conf, int32_t kernel) {
+  gk::InstanceKey key;
+  gk::InstanceInfo info;
+  return validate_config(conf, kernel, nullptr, nullptr, &key, &info);
+}
+
+int gk_number_of_blocks(const gk_config* conf, int32_t* blocks_x, int32_t* blocks_y) {
+  if (!conf || !blocks_x || !blocks_y) return fail(GK_ERR_INVALID_ARGUMENT, "NULL argument");
+  if (conf->block_shape.M <= 0 || conf->block_shape.N <= 0) return fail(GK_ERR_BLOCK_SHAPE, "block_shape must be positive");
+  int gx = 0, gy = 0;
+  gk::number_of_blocks(conf->cta_swizzle.kind, conf->cta_swizzle.param, conf->matmul_shape.M, conf->matmul_shape.N,
+                       conf->block_shape.M, conf->block_shape.N, gx, gy);
+  *blocks_x = gx;
+  *blocks_y = gy;
+  return GK_OK;
+}
+
+int gk_cta_swizzle(const gk_config* conf, int32_t block_x, int32_t block_y, int32_t* block_i, int32_t* block_j) {
+  if (!conf || !block_i || !block_j) return fail(GK_ERR_INVALID_ARGUMENT, "NULL argument");
+  const int nbm = (conf->matmul_shape.M + conf->block_shape.M - 1) / conf->block_shape.M;
+  const int nbn = (conf->matmul_shape.N + conf->block_shape.N - 1) / conf->block_shape.N;
+  int ti = 0, tj = 0;
+  gk::cta_swizzle(conf->cta_swizzle.kind, conf->cta_swizzle.param, block_x, block_y, nbm, nbn, ti, tj);
+  *block_i = ti * conf->block_shape.M;
+  *block_j = tj * conf->block_shape.N;
+  return GK_OK;
+}
+
+int64_t gk_shmem_size(const gk_config* conf, int32_t kernel) {
+  (void)kernel;
+  if (!conf) { fail(GK_ERR_INVALID_ARGUMENT, "config is NULL"); return -1; }
+  gk::InstanceKey key;
+  gk::InstanceInfo info;
+  if (find_instance(conf, nullptr, nullptr, &key, &info) != GK_OK) return -1;
+  return info.lds_bytes;
+}
+
+int32_t gk_threads_per_block(const gk_config* conf) {
+  if (!conf) return -1;
+  return conf->warps_per_block * gk::kWaveSize;
+}
+
+int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const gk_epilogue* epilogue, int32_t kernel,
+                   char* buf, size_t n) {
+  (void)kernel;
+  if (!conf || !buf || n == 0) return fail(GK_ERR_INVALID_ARGUMENT, "NULL argument");
+  gk::InstanceKey key;
+  gk::InstanceInfo info;
+  int rc = find_instance(conf, transforms, epilogue, &key, &info);
+  if (rc != GK_OK) return rc;
+  snprintf(buf, n, "%s", info.name);
+  return GK_OK;
+}
+
+int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
+              const gk_epilogue* epilogue, int32_t kernel, void* stream) {
+  gk::InstanceKey key;
+  gk::InstanceInfo info;
+  int rc = validate_config(conf, kernel, transforms, epilogue, &key, &info);
+  if (rc != GK_OK) return rc;
+
+  const bool a_zero = conf->global_a_layout.kind == GK_LAYOUT_ZERO, b_zero = conf->global_b_layout.kind == GK_LAYOUT_ZERO;
+  if ((!a_zero && !a) || (!b_zero && !b) || !d) return fail(GK_ERR_INVALID_ARGUMENT, "a, b and d must not be NULL");
+  if (conf->global_c_layout.kind != GK_LAYOUT_ZERO && !c) return fail(GK_ERR_INVALID_ARGUMENT, "c must not be NULL unless its layout is Zero");
+  if (epilogue && epilogue->kind != GK_EPILOGUE_DEFAULT && !epilogue->bias) return fail(GK_ERR_INVALID_ARGUMENT, "bias epilogue without a bias pointer");
+
+  gk::GemmArgs args;
+  make_args(conf, a, b, c, d, transforms, epilogue, &args);
+
+  // aligned layouts move 16-byte vectors (reference src/layout.jl:22-34 traps on the device; here it is a host check)
+  auto check_aligned = [&](const gk_layout& l, const void* p, long long ld, const char* what) -> int {
+    if (l.kind != GK_LAYOUT_ALIGNED_COL_MAJOR && l.kind != GK_LAYOUT_ALIGNED_ROW_MAJOR) return GK_OK;
+    const int es = dtype_size(l.eltype);
+    if (es == 0) return fail(GK_ERR_INVALID_ARGUMENT, "unknown element type of %s", what);
+    if (((uintptr_t)p & 15u) != 0) return fail(GK_ERR_ALIGNMENT, "%s is not aligned to 16 bytes", what);
+    if ((ld * es) % 16 != 0) return fail(GK_ERR_ALIGNMENT, "leading dimension of %s (%lld elements) is not a multiple of 16 bytes", what, ld);
+    return GK_OK;
+  };
+  if ((rc = check_aligned(conf->global_a_layout, a, args.lda, "A")) != GK_OK) return rc;
+  if ((rc = check_aligned(conf->global_b_layout, b, args.ldb, "B")) != GK_OK) return rc;
+  if ((rc = check_aligned(conf->global_c_layout, c, args.ldc, "C")) != GK_OK) return rc;
+  if ((rc = check_aligned(conf->global_d_layout, d, args.ldd, "D")) != GK_OK) return rc;
+
+  // leading dimensions must cover the operand
+  {
+    const bool a_row = is_row_major(conf->global_a_layout.kind), b_row = is_row_major(conf->global_b_layout.kind);
+    if (!a_zero && conf->global_a_layout.kind != GK_LAYOUT_DIAGONAL && conf->global_a_layout.kind != GK_LAYOUT_GETT &&
+        args.lda < (a_row ? args.K : args.M))
+      return fail(GK_ERR_DIMENSION_MISMATCH, "lda = %lld is smaller than the leading extent of A", args.lda);
+    if (!b_zero && conf->global_b_layout.kind != GK_LAYOUT_GETT && args.ldb < (b_row ? args.N : args.K))
+      return fail(GK_ERR_DIMENSION_MISMATCH, "ldb = %lld is smaller than the leading extent of B", args.ldb);
+    if (conf->global_d_layout.kind != GK_LAYOUT_GETT && (args.ldd < args.M || (args.c_mode && args.ldc < args.M)))
+      return fail(GK_ERR_DIMENSION_MISMATCH, "ldc/ldd is smaller than M");
+    // the kernels keep per-lane tile offsets in 32 bits
+    const long long span_a = (long long)(a_row ? conf->block_shape.M : conf->block_shape.K) * args.lda * 2;
+    const long long span_b = (long long)(b_row ? conf->block_shape.K : conf->block_shape.N) * args.ldb * 2;
+    if (span_a >= (1ll << 31) || span_b >= (1ll << 31))
+      return fail(GK_ERR_UNSUPPORTED, "leading dimension too large for 32-bit tile offsets");
+  }
+
+  int gx = 0, gy = 0;
+  gk::number_of_blocks(args.swz_kind, args.swz_param, args.M, args.N, conf->block_shape.M, conf->block_shape.N, gx, gy);
+  if (gx <= 0 || gy <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "empty grid");
+
+  gk::FamilyFn fn = family_fn(key);
+  hipError_t err = hipSuccess;
+  if (!fn || !fn(key, args, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream, 1, &info, &err))
+    return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance");
+  if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", info.name, hipGetErrorString(err));
+  return GK_OK;
+}
+
+int32_t gk_sizeof(int32_t which) {
+  switch (which) {
+    case 0: return (int32_t)sizeof(gk_config);
+    case 1: return (int32_t)sizeof(gk_layout);
+    case 2: return (int32_t)sizeof(gk_operator);
+    case 3: return (int32_t)sizeof(gk_transforms);
+    case 4: return (int32_t)sizeof(gk_epilogue);
+    case 5: return (int32_t)sizeof(gk_gett);
+    default: return -1;
+  }
+}
+
+}  // extern "C"

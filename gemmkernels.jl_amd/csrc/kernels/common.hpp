@@ -1,0 +1,233 @@
+// Shared device/host definitions of the gfx950 GEMM kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gk {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef short short4v __attribute__((__vector_size__(4 * sizeof(short))));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int2v __attribute__((ext_vector_type(2)));
+
+#define GK_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+#define GK_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+constexpr int kWaveSize = 64;
+
+// dtype codes (same values as gk_dtype of the C ABI)
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_F32 = 2, DT_F64 = 3 };
+
+// op codes (same values as gk_op_kind of the C ABI)
+enum : int { T_IDENTITY = 0, T_SCALE = 1, T_ADD = 2, T_RELU = 3, T_NEG = 4, T_ABS = 5, T_CLAMP = 6, T_SQUARE = 7 };
+
+// swizzle codes (same values as gk_swizzle_kind)
+enum : int { SWZ_IDENTITY = 0, SWZ_HTILED = 1, SWZ_VTILED = 2, SWZ_LEBESGUE = 3, SWZ_XCD = 4 };
+
+constexpr int kMaxOps = 4;
+constexpr int kMaxModes = 4;
+
+// One transform hook: a short list of elementwise ops.
+struct OpList {
+  int n;
+  int kind[kMaxOps];
+  float p0[kMaxOps];
+  float p1[kMaxOps];
+};
+
+// Hook indices, keyword order of the reference launcher (reference src/matmul.jl:8-15).
+enum : int { H_GL2SH_A = 0, H_GL2SH_B = 1, H_GL2SH_C = 2, H_SH2GL_D = 3, H_SH2RF_A = 4, H_SH2RF_B = 5, H_SH2RF_C = 6, H_RF2SH_D = 7 };
+
+// One GEMM dimension of a tensor contraction (mixed-radix index -> two element offsets).
+struct GettDim {
+  int nmodes;
+  int extent[kMaxModes];
+  long long stride0[kMaxModes];
+  long long stride1[kMaxModes];
+};
+
+__host__ __device__ inline void gett_offsets(const GettDim& d, long long idx, long long& off0, long long& off1) {
+  off0 = 0; off1 = 0;
+  for (int i = 0; i < d.nmodes; ++i) {
+    long long e = d.extent[i];
+    long long digit = idx % e;
+    idx /= e;
+    off0 += digit * d.stride0[i];
+    off1 += digit * d.stride1[i];
+  }
+}
+
+// Arguments common to every GEMM kernel of the library.
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  const void* c;
+  void* d;
+  const float* bias;
+  int M, N, K;
+  long long lda, ldb, ldc, ldd;   // leading dimensions in elements
+  int nbm, nbn;                   // tile grid
+  int swz_kind, swz_param;
+  int c_mode;                     // 0: C is Layout.Zero, 1: C is loaded
+  int epi_kind;                   // 0 default, 1 bias per column, 2 bias per row
+  int c_dtype, d_dtype;
+  int a_kind, b_kind;             // gk_layout_kind of the global A / B layouts (diagonal, GETT ...)
+  int cd_gett;                    // 1: C and D are addressed through gett.m / gett.n stride1
+  OpList t[8];
+  GettDim gm, gn, gk;
+};
+
+// ---------------------------------------------------------------------------------------------
+// CTA swizzle: (blockIdx.x, blockIdx.y) -> tile coordinates.  Identity, HorizontallyTiled,
+// VerticallyTiled and LebesgueCurve follow reference src/cta-swizzle.jl:33-41, 74-82, 109-117,
+// 153-160.  SWZ_XCD is specific to the MI355X: workgroup n of a launch runs on XCD n % 8 and every
+// XCD has a private L2, so consecutive ids are first regrouped per XCD and the tile grid is then
+// walked in panels `param` tiles high, which makes the tiles that share an L2 share rows of A and
+// columns of B.
+// ---------------------------------------------------------------------------------------------
+__host__ __device__ inline unsigned extract_even_bits(unsigned x) {
+  x = x & 0x55555555u;
+  x = (x | (x >> 1)) & 0x33333333u;
+  x = (x | (x >> 2)) & 0x0F0F0F0Fu;
+  x = (x | (x >> 4)) & 0x00FF00FFu;
+  x = (x | (x >> 8)) & 0x0000FFFFu;
+  return x;
+}
+
+__host__ __device__ inline void cta_swizzle(int kind, int param, int bx, int by, int nbm, int nbn, int& ti, int& tj) {
+  switch (kind) {
+    case SWZ_HTILED:
+      ti = bx / param;
+      tj = by * param + bx % param;
+      break;
+    case SWZ_VTILED:
+      ti = bx * param + by % param;
+      tj = by / param;
+      break;
+    case SWZ_LEBESGUE:
+      ti = (int)extract_even_bits((unsigned)bx);
+      tj = (int)extract_even_bits((unsigned)bx >> 1);
+      break;
+    case SWZ_XCD: {
+      const int total = nbm * nbn;
+      int r = bx;
+      if (total % 8 == 0) r = (bx % 8) * (total / 8) + bx / 8;
+      const int g = param > 0 ? param : 1;
+      const int width = g * nbn;
+      const int group = r / width;
+      const int first = group * g;
+      const int gsz = (nbm - first) < g ? (nbm - first) : g;
+      const int in_group = r % width;
+      ti = first + in_group % gsz;
+      tj = in_group / gsz;
+      break;
+    }
+    default:
+      ti = bx;
+      tj = by;
+      break;
+  }
+}
+
+__host__ __device__ inline void number_of_blocks(int kind, int param, int nbm_elems_M, int nbn_elems_N, int BM, int BN, int& gx, int& gy) {
+  // cld() forms of reference src/cta-swizzle.jl:28-31, 69-72, 104-107, 149-151
+  auto cld = [](long long a, long long b) { return (int)((a + b - 1) / b); };
+  switch (kind) {
+    case SWZ_HTILED:
+      gx = cld((long long)nbm_elems_M * param, BM);
+      gy = cld(nbn_elems_N, (long long)BN * param);
+      break;
+    case SWZ_VTILED:
+      gx = cld(nbm_elems_M, (long long)BM * param);
+      gy = cld((long long)nbn_elems_N * param, BN);
+      break;
+    case SWZ_LEBESGUE:
+    case SWZ_XCD:
+      gx = cld(nbm_elems_M, BM) * cld(nbn_elems_N, BN);
+      gy = 1;
+      break;
+    default:
+      gx = cld(nbm_elems_M, BM);
+      gy = cld(nbn_elems_N, BN);
+      break;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Elementwise op lists.  One rounding per op, fp32 arithmetic, no fused multiply-add.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float apply_op(int kind, float p0, float p1, float x) {
+  switch (kind) {
+    case T_SCALE: return x * p0;
+    case T_ADD: return x + p0;
+    case T_RELU: return x > 0.0f ? x : 0.0f;
+    case T_NEG: return -x;
+    case T_ABS: return __builtin_fabsf(x);
+    case T_CLAMP: return x < p0 ? p0 : (x > p1 ? p1 : x);
+    case T_SQUARE: return x * x;
+    default: return x;
+  }
+}
+
+__device__ __forceinline__ float apply_list(const OpList& t, float x) {
+  for (int i = 0; i < t.n; ++i) x = apply_op(t.kind[i], t.p0[i], t.p1[i], x);
+  return x;
+}
+
+// Applies a list to an array of registers with the op switch outside the element loop, so that
+// the (wave-uniform) dispatch is paid once per op and not once per element.
+template <int COUNT>
+__device__ __forceinline__ void apply_list_regs(const OpList& t, float (&x)[COUNT]) {
+  for (int i = 0; i < t.n; ++i) {
+    const float p0 = t.p0[i], p1 = t.p1[i];
+    switch (t.kind[i]) {
+      case T_SCALE:
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = x[e] * p0;
+        break;
+      case T_ADD:
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = x[e] + p0;
+        break;
+      case T_RELU:
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = x[e] > 0.0f ? x[e] : 0.0f;
+        break;
+      case T_NEG:
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = -x[e];
+        break;
+      case T_ABS:
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = __builtin_fabsf(x[e]);
+        break;
+      case T_CLAMP:
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = x[e] < p0 ? p0 : (x[e] > p1 ? p1 : x[e]);
+        break;
+      case T_SQUARE:
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = x[e] * x[e];
+        break;
+      default:
+        break;
+    }
+  }
+}
+
+// waits and barriers placed by hand around the LDS-DMA pipeline
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+}  // namespace gk

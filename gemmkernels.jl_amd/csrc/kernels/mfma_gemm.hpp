@@ -1,0 +1,376 @@
+// Tiled GEMM on the CDNA4 matrix cores: D = epilogue(T_d(sum_k T_a(A) * T_b(B) + T_c(C))).
+//
+// Stands where Kernel.matmul_pipelined stands in the reference (src/kernel.jl:147-350) with
+// Operator.WMMAOp (src/operator.jl:163-245) and the UnsafeAligned{Col,Row}Major layouts
+// (src/layout.jl:192-219, 244-270), re-designed for gfx950:
+//
+//  * one v_mfma_f32_32x32x16 per 32x32x16 product, 64-lane waves, accumulators stay in
+//    registers from the C load to the D store (the reference round-trips them through LDS);
+//  * A and B tiles travel global -> LDS with global_load_lds_dwordx4 (no register staging),
+//    STAGES tiles deep, one s_barrier per K step;
+//  * LDS tiles are XOR-swizzled in 16-byte chunks so that both the DMA writes and the fragment
+//    reads are bank-conflict free (64 banks x 4 B, conflicts are resolved per 32-lane half);
+//  * operands whose K index is contiguous in memory ("K-major": A of a 'T' GEMM, B of an 'N'
+//    GEMM) are read with ds_read_b128, the others ("M-major") with the transposing
+//    ds_read_b64_tr_b16, so all four transposes run at the same speed;
+//  * the MFMA is issued with swapped operands (B fragment first) so that a lane owns 32
+//    consecutive rows m of D and a half-wave writes whole 128-byte lines of column-major D.
+#pragma once
+#include "common.hpp"
+#include <type_traits>
+
+namespace gk {
+
+// ----------------------------------------------------------------------------------------------
+// LDS tile geometry.  A tile holds R rows (m or n) x BK k-values of 16-bit elements.
+//   K-major: LDS row = tile row r, 16-byte chunk c = k / 8
+//   M-major: LDS row = k,          16-byte chunk c = r / 8
+// ----------------------------------------------------------------------------------------------
+template <int R, int BK, bool KMAJOR>
+struct TileGeom {
+  static constexpr int CPR = KMAJOR ? BK / 8 : R / 8;        // chunks per LDS row
+  static constexpr int ROW_BYTES = CPR * 16;
+  static constexpr int BYTES = R * BK * 2;
+  static constexpr int NDMA = BYTES / 1024;                   // wave-wide 16 B/lane DMA instructions per tile
+  static constexpr int RP256 = (256 / ROW_BYTES) > 1 ? (256 / ROW_BYTES) : 1;   // LDS rows per 256 B
+  // K-major: XOR the chunk index with the row (per 256 B) so that 32 consecutive rows at one
+  // chunk index spread evenly over the 16 chunk slots of the 64 banks.
+  __device__ static __forceinline__ int swz_k(int row) { return (row / RP256) & (CPR - 1); }
+  // M-major: XOR the 64-byte group index with k so that 4 consecutive k rows at one group land
+  // in 4 different 64-byte slots of the 256-byte bank period.
+  static constexpr int GROUPS = CPR / 4;
+  static constexpr int GMASK = (GROUPS - 1) < 3 ? (GROUPS - 1) : 3;
+  __device__ static __forceinline__ int swz_m(int k) { return (k / RP256) & GMASK; }
+  static_assert((CPR & (CPR - 1)) == 0, "chunks per row must be a power of two");
+  static_assert(KMAJOR || CPR >= 4, "M-major tiles need at least 32 rows");
+  static_assert(BYTES % 1024 == 0, "tile must be a whole number of DMA instructions");
+};
+
+// Byte offset (from the tile's global origin) that lane `lane` of DMA instruction q fetches, and
+// which lands at LDS chunk position q*64 + lane.
+template <int R, int BK, bool KMAJOR>
+__device__ __forceinline__ unsigned dma_global_offset(int q, int lane, long long ld) {
+  using G = TileGeom<R, BK, KMAJOR>;
+  const int p = q * 64 + lane;
+  const int row = p / G::CPR;
+  const int cs = p % G::CPR;
+  if (KMAJOR) {
+    const int c = cs ^ G::swz_k(row);
+    return (unsigned)(((long long)row * ld + c * 8) * 2);
+  } else {
+    const int g = (cs >> 2) ^ G::swz_m(row);
+    const int c = g * 4 + (cs & 3);
+    return (unsigned)(((long long)row * ld + c * 8) * 2);
+  }
+}
+
+// Fragment of 32 tile rows x 16 k-values: lane l receives the 8 k-values 8*(l/32)..+7 of row
+// row0 + l%32, which is the operand layout of v_mfma_f32_32x32x16.
+//
+// The reads are issued from inline assembly: the compiler would otherwise make every
+// transposing LDS read wait for all outstanding global->LDS DMA (it cannot tell the stages
+// apart), which serialises the pipeline.  Their completion is therefore tracked by hand with
+// wait_lgkmcnt<N>() + pin(), see the main loop.
+template <int R, int BK, bool KMAJOR, int F>
+struct FragReader {
+  typedef TileGeom<R, BK, KMAJOR> G;
+  static constexpr int KSTEPS = BK / 16;
+  static constexpr int NBASE = KMAJOR ? KSTEPS : F;
+  static constexpr int OPS = KMAJOR ? 1 : 2;     // LDS instructions per fragment
+  unsigned base[NBASE];                         // lane-dependent byte offsets inside a tile
+  unsigned cur[NBASE];                          // the same, relative to the current stage
+
+  // row0: first tile row of the wave (multiple of 32)
+  __device__ __forceinline__ void init(int row0, int lane) {
+    if (KMAJOR) {
+      const int row = row0 + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int c = ks * 2 + (lane >> 5);
+        base[ks] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_k(row)));
+      }
+    } else {
+      const int i = lane & 15;
+      const int k = 8 * (lane >> 5) + (i >> 2);
+      const int m = (lane & 16) + 4 * (i & 3);          // offset inside the 32-row fragment
+      const int c = m >> 3;
+      const unsigned lane_part = (unsigned)(k * G::ROW_BYTES + (c & 3) * 16 + (m & 4) * 2);
+#pragma unroll
+      for (int fi = 0; fi < F; ++fi) {
+        const int g = ((row0 >> 5) + fi) ^ G::swz_m(k);
+        base[fi] = lane_part + (unsigned)g * 64u;
+      }
+    }
+  }
+  __device__ __forceinline__ void set_stage(unsigned tile_lds_addr) {
+#pragma unroll
+    for (int i = 0; i < NBASE; ++i) cur[i] = base[i] + tile_lds_addr;
+  }
+  template <int FI, int KS>
+  __device__ __forceinline__ int4v read() const {
+    int4v r;
+    if (KMAJOR) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(cur[KS]), "n"(FI * 32 * G::ROW_BYTES) : "memory");
+    } else {
+      int2v lo, hi;
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(cur[FI]), "n"((KS * 16) * G::ROW_BYTES) : "memory");
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(cur[FI]), "n"((KS * 16 + 4) * G::ROW_BYTES) : "memory");
+      r[0] = lo[0]; r[1] = lo[1]; r[2] = hi[0]; r[3] = hi[1];
+    }
+    return r;
+  }
+  static_assert((KSTEPS * 16 + 4) * G::ROW_BYTES < 65536 || KMAJOR, "LDS immediate offset is 16 bits");
+  static_assert(F * 32 * G::ROW_BYTES <= 65536 || !KMAJOR, "LDS immediate offset is 16 bits");
+};
+
+// Makes every later use of x depend on the point where pin() stands (no instruction is emitted).
+__device__ __forceinline__ void pin(int4v& x) { asm volatile("" : "+v"(x)); }
+
+template <int N>
+__device__ __forceinline__ void wait_lgkmcnt() {
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N < 15 ? N : 15) : "memory");
+}
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+template <int KS, class RA, class RB, int FM, int FN>
+__device__ __forceinline__ void load_frags(const RA& ra, const RB& rb, int4v (&fa)[FM], int4v (&fb)[FN]) {
+  static_for<0, FM>([&](auto fi) { fa[decltype(fi)::value] = ra.template read<decltype(fi)::value, KS>(); });
+  static_for<0, FN>([&](auto fj) { fb[decltype(fj)::value] = rb.template read<decltype(fj)::value, KS>(); });
+}
+
+template <typename T> struct Mfma;
+template <> struct Mfma<_Float16> {
+  __device__ static __forceinline__ float16v run(int4v a, int4v b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<__bf16> {
+  __device__ static __forceinline__ float16v run(int4v a, int4v b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+// fp32 op list on the 8 packed 16-bit values of a fragment, rounded back to T.  gl2sh then
+// sh2rf: the value is rounded to T after each hook like the LDS copy and the fragment of the
+// reference (src/kernel.jl:224-236, 311-319).
+template <typename T>
+__device__ __forceinline__ int4v transform_fragment(int4v f, const OpList& t0, const OpList& t1) {
+  typedef T vec8 __attribute__((ext_vector_type(8)));
+  vec8 v = __builtin_bit_cast(vec8, f);
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
+  if (t0.n > 0) {
+    apply_list_regs<8>(t0, x);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = (float)(T)x[e];
+  }
+  if (t1.n > 0) apply_list_regs<8>(t1, x);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (T)x[e];
+  return __builtin_bit_cast(int4v, v);
+}
+
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, bool A_KMAJOR_, bool B_KMAJOR_, typename T_, bool FUSED_>
+struct MfmaGemmConfig {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, FUSED = FUSED_;
+  typedef T_ T;
+  static constexpr int NWAVES = WAVES_M * WAVES_N;
+  static constexpr int THREADS = NWAVES * kWaveSize;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
+  static constexpr int FM = WTM / 32, FN = WTN / 32;             // 32x32 accumulator blocks per wave
+  static constexpr int KSTEPS = BK / 16;
+  typedef TileGeom<BM, BK, A_KMAJOR> GA;
+  typedef TileGeom<BN, BK, B_KMAJOR> GB;
+  static constexpr int STAGE_BYTES = GA::BYTES + GB::BYTES;
+  static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
+  static constexpr int DMA_A = (GA::NDMA + NWAVES - 1) / NWAVES;   // per wave, per tile
+  static constexpr int DMA_B = (GB::NDMA + NWAVES - 1) / NWAVES;
+  static constexpr int DMA_PER_TILE = DMA_A + DMA_B;
+  static_assert(GA::NDMA % NWAVES == 0 && GB::NDMA % NWAVES == 0, "every wave issues the same number of DMA instructions");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
+  static_assert(STAGES >= 2, "at least two LDS stages");
+  static_assert((STAGES - 2) * DMA_PER_TILE <= 63, "vmcnt is a 6-bit counter");
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs args) {
+  typedef typename Cfg::T T;
+  typedef typename Cfg::GA GA;
+  typedef typename Cfg::GB GB;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, STAGES = Cfg::STAGES;
+  constexpr int FM = Cfg::FM, FN = Cfg::FN, NWAVES = Cfg::NWAVES;
+  constexpr int DMA_A = Cfg::DMA_A, DMA_B = Cfg::DMA_B, DPT = Cfg::DMA_PER_TILE;
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  int ti, tj;
+  cta_swizzle(args.swz_kind, args.swz_param, (int)blockIdx.x, (int)blockIdx.y, args.nbm, args.nbn, ti, tj);
+  if (ti >= args.nbm || tj >= args.nbn) return;   // whole block leaves together
+
+  const int lane = (int)threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
+  const int m0 = ti * BM, n0 = tj * BN;
+
+  // --- global tile origins (bytes) and the per-lane DMA offsets, fixed for the whole K loop ---
+  const char* ga = (const char*)args.a + (Cfg::A_KMAJOR ? (long long)m0 * args.lda : (long long)m0) * 2;
+  const char* gb = (const char*)args.b + (Cfg::B_KMAJOR ? (long long)n0 * args.ldb : (long long)n0) * 2;
+  const long long a_step = (Cfg::A_KMAJOR ? (long long)BK : (long long)BK * args.lda) * 2;
+  const long long b_step = (Cfg::B_KMAJOR ? (long long)BK : (long long)BK * args.ldb) * 2;
+  unsigned offa[DMA_A], offb[DMA_B];
+#pragma unroll
+  for (int i = 0; i < DMA_A; ++i) offa[i] = dma_global_offset<BM, BK, Cfg::A_KMAJOR>(wave + i * NWAVES, lane, args.lda);
+#pragma unroll
+  for (int i = 0; i < DMA_B; ++i) offb[i] = dma_global_offset<BN, BK, Cfg::B_KMAJOR>(wave + i * NWAVES, lane, args.ldb);
+
+  auto issue_tile = [&](int stage) {
+    char* sa = smem + stage * Cfg::STAGE_BYTES;
+    char* sb = sa + GA::BYTES;
+#pragma unroll
+    for (int i = 0; i < DMA_A; ++i)
+      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < DMA_B; ++i)
+      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+    ga += a_step;
+    gb += b_step;
+  };
+
+  const int KT = args.K / BK;
+
+  // --- prologue: start the first STAGES-1 tiles on their way ---
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < KT) issue_tile(s);
+
+  // --- accumulators: C tile (two transforms) or zeros -------------------------------------------
+  // lane l owns rows m = 32*fi + l%32 and columns n = 32*fj + 8*(v/4) + 4*(l/32) + v%4
+  float16v acc[FM][FN];
+  const int mrow = m0 + wm * Cfg::WTM + (lane & 31);
+  const int ncol = n0 + wn * Cfg::WTN + 4 * (lane >> 5);
+  if (args.c_mode != 0) {
+    const float* cp = (const float*)args.c + mrow + (long long)ncol * args.ldc;
+#pragma unroll
+    for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          acc[fi][fj][v] = cp[32 * fi + (long long)(32 * fj + 8 * (v / 4) + (v % 4)) * args.ldc];
+    if (Cfg::FUSED) {
+      if (args.t[H_GL2SH_C].n > 0 || args.t[H_SH2RF_C].n > 0) {
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+          for (int fj = 0; fj < FN; ++fj) {
+            float x[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
+            apply_list_regs<16>(args.t[H_GL2SH_C], x);
+            apply_list_regs<16>(args.t[H_SH2RF_C], x);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[fi][fj][v] = x[v];
+          }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[fi][fj][v] = 0.0f;
+  }
+
+  const bool xf_a = Cfg::FUSED && (args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0);
+  const bool xf_b = Cfg::FUSED && (args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0);
+
+  typedef FragReader<BM, BK, Cfg::A_KMAJOR, FM> RA;
+  typedef FragReader<BN, BK, Cfg::B_KMAJOR, FN> RB;
+  RA ra;
+  RB rb;
+  ra.init(wm * Cfg::WTM, lane);
+  rb.init(wn * Cfg::WTN, lane);
+  const unsigned lds_base = (unsigned)(uintptr_t)GK_LDS_PTR(char, smem);
+
+  // --- main loop ------------------------------------------------------------------------------
+  for (int kt = 0; kt < KT; ++kt) {
+    // tile kt has landed once at most the DMA of the STAGES-2 younger tiles is outstanding
+    if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 2) * DPT>(); else wait_vmcnt<0>();
+    block_barrier();   // every wave's share of tile kt is in LDS; every wave is done with tile kt-1
+    if (kt + STAGES - 1 < KT) issue_tile((kt + STAGES - 1) % STAGES);
+
+    const unsigned stage_addr = lds_base + (unsigned)(kt % STAGES) * Cfg::STAGE_BYTES;
+    ra.set_stage(stage_addr);
+    rb.set_stage(stage_addr + GA::BYTES);
+
+    // fragments are double-buffered: the reads of k-step ks+1 are in flight while the MFMAs of
+    // k-step ks run; LDS reads complete in order, so "at most NEXT outstanding" means that the
+    // current set has arrived.
+    int4v fa[2][FM], fb[2][FN];
+    load_frags<0>(ra, rb, fa[0], fb[0]);
+    static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
+      constexpr int ks = decltype(ks_c)::value;
+      constexpr bool more = (ks + 1 < Cfg::KSTEPS);
+      if constexpr (more) load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+      wait_lgkmcnt<more ? (FM * RA::OPS + FN * RB::OPS) : 0>();
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi) pin(fa[ks & 1][fi]);
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) pin(fb[ks & 1][fj]);
+      if (Cfg::FUSED) {
+        if (xf_a) {
+#pragma unroll
+          for (int fi = 0; fi < FM; ++fi) fa[ks & 1][fi] = transform_fragment<T>(fa[ks & 1][fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
+        }
+        if (xf_b) {
+#pragma unroll
+          for (int fj = 0; fj < FN; ++fj) fb[ks & 1][fj] = transform_fragment<T>(fb[ks & 1][fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
+        }
+      }
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+        for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = Mfma<T>::run(fb[ks & 1][fj], fa[ks & 1][fi], acc[fi][fj]);
+    });
+    // the last wait above was lgkmcnt(0): all LDS reads of this stage are complete before the
+    // next barrier lets a DMA overwrite it
+  }
+
+  // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
+  float* dp = (float*)args.d + mrow + (long long)ncol * args.ldd;
+#pragma unroll
+  for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+    for (int fj = 0; fj < FN; ++fj) {
+      float x[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
+      if (Cfg::FUSED) {
+        apply_list_regs<16>(args.t[H_RF2SH_D], x);
+        if (args.epi_kind == 1) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) x[v] = x[v] + args.bias[ncol + 32 * fj + 8 * (v / 4) + (v % 4)];
+        } else if (args.epi_kind == 2) {
+          const float bv = args.bias[mrow + 32 * fi];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) x[v] = x[v] + bv;
+        }
+        apply_list_regs<16>(args.t[H_SH2GL_D], x);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        dp[32 * fi + (long long)(32 * fj + 8 * (v / 4) + (v % 4)) * args.ldd] = x[v];
+    }
+}
+
+}  // namespace gk

@@ -1,0 +1,59 @@
+// Kernel-instance registry: every translation unit that instantiates kernels exposes one
+// "family" function which, given the run-time key of a launch, either launches (or just
+// describes) the matching compiled instance or reports that it has none.
+#pragma once
+#include "common.hpp"
+
+namespace gk {
+
+struct InstanceKey {
+  int family;        // FAMILY_*
+  int BM, BN, BK;
+  int waves_m, waves_n;
+  int a_kmajor, b_kmajor;   // 1: the K index is contiguous in the operand's memory
+  int dtype;         // element type of A and B
+  int fused;         // 1: transforms / bias present
+  int variant;       // family specific
+};
+
+enum : int { FAMILY_MFMA = 0, FAMILY_MFMA_CHECKED = 1, FAMILY_FPU = 2, FAMILY_COMPLEX = 3, FAMILY_DIAGONAL = 4, FAMILY_GETT = 5 };
+
+struct InstanceInfo {
+  const char* name;
+  int lds_bytes;
+  int threads;
+};
+
+// mode 0: describe only (fills info), mode 1: describe and launch.
+// returns 1 when an instance matched, 0 otherwise; *err receives the launch status.
+typedef int (*FamilyFn)(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode,
+                        InstanceInfo* info, hipError_t* err);
+
+template <class Cfg, class Kernel>
+inline int run_instance(Kernel kernel, const char* name, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode,
+                        InstanceInfo* info, hipError_t* err, int lds_bytes, int threads) {
+  info->name = name;
+  info->lds_bytes = lds_bytes;
+  info->threads = threads;
+  if (mode == 1) {
+    hipError_t e = hipSuccess;
+    if (lds_bytes > 64 * 1024) {
+      // raising the dynamic LDS limit is idempotent and cheap; done on every launch so that the
+      // library stays correct when the caller switches devices
+      e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    }
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(kernel, grid, dim3(threads), lds_bytes, stream, args);
+      e = hipGetLastError();
+    }
+    *err = e;
+  }
+  return 1;
+}
+
+int family_mfma_tn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+int family_mfma_nn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+int family_mfma_nt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+int family_mfma_tt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+
+}  // namespace gk

@@ -1,0 +1,254 @@
+"""Config and get_config (reference src/config.jl), with defaults re-derived for the MI355X:
+64-lane wavefronts, 160 KiB of LDS per workgroup, MFMA 32x32x16 blocks."""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass, fields
+from typing import Optional
+
+from . import _lib
+from . import layout as Layout
+from . import operator as Operator
+from . import cta_swizzle as CTASwizzle
+from .errors import ConfigError
+from .tiling import NT
+
+WARP_SIZE = 64   # lanes per wavefront; the reference's 32 (src/matmul.jl:24) becomes 64 here
+
+
+@dataclass
+class Config:
+    """reference src/config.jl:3-41, field for field."""
+    matmul_shape: NT
+    block_shape: NT
+    warps_per_block: int
+    mem_a_warp: NT
+    mem_a_thread: NT
+    mem_b_warp: NT
+    mem_b_thread: NT
+    mem_cd_warp: NT
+    mem_cd_thread: NT
+    compute_warp: NT
+    compute_op_shape: NT
+    global_a_layout: Layout.LayoutType
+    global_b_layout: Layout.LayoutType
+    global_c_layout: Layout.LayoutType
+    global_d_layout: Layout.LayoutType
+    shared_a_layout: Layout.LayoutType
+    shared_b_layout: Layout.LayoutType
+    shared_c_layout: Layout.LayoutType
+    shared_d_layout: Layout.LayoutType
+    operator: Operator.OperatorType
+    is_a_col_major: bool
+    is_b_col_major: bool
+    cta_swizzle: CTASwizzle.SwizzleType
+
+    def __str__(self):
+        # reference src/config.jl:43-76
+        width = max(len(f.name) for f in fields(self)) + 2
+        return "\n".join(f"{(f.name + ':').ljust(width)}{getattr(self, f.name)}" for f in fields(self)) + "\n"
+
+    def to_c(self, lda: int = 0, ldb: int = 0, ldc: int = 0, ldd: int = 0) -> _lib.gk_config:
+        """Lower to the POD of the C ABI; leading dimensions come from the arrays of the call."""
+        c = _lib.gk_config()
+
+        def shape(dst, src):
+            dst.M, dst.N, dst.K = int(src.get("M", 0)), int(src.get("N", 0)), int(src.get("K", 0))
+
+        shape(c.matmul_shape, self.matmul_shape)
+        shape(c.block_shape, self.block_shape)
+        c.warps_per_block = int(self.warps_per_block)
+        for name in ("mem_a_warp", "mem_a_thread", "mem_b_warp", "mem_b_thread", "mem_cd_warp", "mem_cd_thread",
+                     "compute_warp", "compute_op_shape"):
+            shape(getattr(c, name), getattr(self, name))
+
+        def lay(dst, src: Layout.LayoutType, ld=0):
+            dst.kind, dst.eltype, dst.pad, dst.ld = src.kind, src.T.code, src.pad, int(ld)
+
+        lay(c.global_a_layout, self.global_a_layout, lda)
+        lay(c.global_b_layout, self.global_b_layout, ldb)
+        lay(c.global_c_layout, self.global_c_layout, ldc)
+        lay(c.global_d_layout, self.global_d_layout, ldd)
+        lay(c.shared_a_layout, self.shared_a_layout)
+        lay(c.shared_b_layout, self.shared_b_layout)
+        lay(c.shared_c_layout, self.shared_c_layout)
+        lay(c.shared_d_layout, self.shared_d_layout)
+        op = self.operator
+        c.op.kind, c.op.M, c.op.N, c.op.K = op.kind, op.M, op.N, op.K
+        c.op.mb, c.op.nb, c.op.kb = op.mb, op.nb, op.kb
+        c.op.compute_type, c.op.accum_type = op.CT.code, op.AT.code
+        c.is_a_col_major, c.is_b_col_major = int(self.is_a_col_major), int(self.is_b_col_major)
+        c.cta_swizzle.kind, c.cta_swizzle.param = self.cta_swizzle.kind, self.cta_swizzle.param
+        gmap = None
+        for l in (self.global_a_layout, self.global_b_layout, self.global_c_layout, self.global_d_layout):
+            if l.kind == Layout.GETT_KIND and l.gett is not None:
+                gmap = l.gett
+        if gmap is not None:
+            for dst, src in ((c.gett.m, gmap.m), (c.gett.n, gmap.n), (c.gett.k, gmap.k)):
+                if len(src) > _lib.GK_MAX_MODES:
+                    raise ConfigError(f"at most {_lib.GK_MAX_MODES} tensor modes per GEMM dimension")
+                dst.nmodes = len(src)
+                for i, (e, s0, s1) in enumerate(src):
+                    dst.extent[i], dst.stride0[i], dst.stride1[i] = int(e), int(s0), int(s1)
+        return c
+
+
+def heuristic_block_shape(shared_a_layout, shared_b_layout, shared_c_layout, shared_d_layout) -> NT:
+    """The reference's block-shape heuristic, unchanged (src/config.jl:84-120): grow M and N while
+    a C/D tile fits 64 KiB, then K while the A and B tiles fit 64 KiB together."""
+    def nbytes(layout, a, b):
+        size = Layout.physical_size(layout, (a, b))
+        n = 1
+        for s in size:
+            n *= s
+        return n * layout.T.size
+
+    def num_bytes_cd(M, N, K):
+        return max(nbytes(shared_c_layout, M, N), nbytes(shared_d_layout, M, N))
+
+    def num_bytes_ab(M, N, K):
+        return nbytes(shared_a_layout, M, K) + nbytes(shared_b_layout, K, N)
+
+    def next_mn(M, N, K):
+        return (2 * M, N, K) if M == N else (M, 2 * N, K)
+
+    cur = (1, 1, 1)
+    nxt = next_mn(*cur)
+    while num_bytes_cd(*nxt) <= 64 * 1024:
+        cur, nxt = nxt, next_mn(*nxt)
+    nxt = (cur[0], cur[1], 2 * cur[2])
+    while num_bytes_ab(*nxt) <= 64 * 1024:
+        cur, nxt = nxt, (nxt[0], nxt[1], 2 * nxt[2])
+    return NT(M=cur[0], N=cur[1], K=cur[2])
+
+
+def adjacent_elements(num: int, parent_size: NT, is_col_major: bool) -> NT:
+    """reference src/config.jl:124-134."""
+    p = tuple(parent_size.values())
+    if is_col_major:
+        t = (min(num, p[0]), num // min(num, p[0]))
+    else:
+        t = (num // min(num, p[1]), min(num, p[1]))
+    return NT(zip(parent_size.keys(), t))
+
+
+# MFMA tile table of the library: block shape -> waves (M x N).  The wave tile (compute_warp) is
+# block / waves; every entry is made of 32x32 MFMA blocks.
+_MFMA_TILES = [
+    ((256, 256, 64), (2, 4)),
+    ((256, 128, 64), (2, 2)),
+    ((128, 256, 64), (2, 2)),
+    ((128, 128, 64), (2, 2)),
+    ((64, 64, 64), (2, 2)),
+    ((64, 64, 32), (1, 1)),
+]
+NUM_CUS = 256
+
+
+def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
+    """MI355X block shape: the largest tile of the table that divides the problem and still gives
+    every one of the 256 CUs a workgroup; the smallest dividing tile when none does."""
+    if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
+        return NT(M=64, N=64, K=32)
+    if operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
+        return NT(M=64, N=64, K=32)
+    M, N, K = gemm_shape["M"], gemm_shape["N"], gemm_shape["K"]
+    fitting = [t for t, _ in _MFMA_TILES if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
+    if not fitting:
+        return NT(M=64, N=64, K=32)
+    for t in fitting:
+        if -(-M // t[0]) * -(-N // t[1]) >= NUM_CUS:
+            return NT(M=t[0], N=t[1], K=t[2])
+    return NT(M=fitting[-1][0], N=fitting[-1][1], K=fitting[-1][2])
+
+
+def _default_waves(operator, block_shape):
+    key = (block_shape["M"], block_shape["N"], block_shape["K"])
+    for t, w in _MFMA_TILES:
+        if t == key:
+            return w
+    return None
+
+
+def require_tile_sized_global(layout) -> bool:
+    """reference src/config.jl:175-178."""
+    return layout.kind not in (Layout.ZERO, Layout.COL_MAJOR, Layout.ROW_MAJOR)
+
+
+def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **params) -> Config:
+    """reference src/config.jl:180-316.  Same keywords; defaults for the parameters the caller
+    leaves out are chosen for the MI355X.  All checks of the reference are run (by the library,
+    through gk_validate) and raise ConfigError."""
+    gemm_shape = NT(gemm_shape)
+    global_b_layout = params.get("global_b_layout", global_a_layout)
+    global_d_layout = params.get("global_d_layout", global_c_layout)
+
+    def padded(l):
+        return Layout.Padded[l, 16 // l.T.size] if l.kind not in (Layout.ZERO, Layout.DIAGONAL, Layout.GETT_KIND) else l
+
+    shared_a_layout = params.get("shared_a_layout", padded(global_a_layout))
+    shared_b_layout = params.get("shared_b_layout", padded(global_b_layout))
+    shared_c_layout = params.get("shared_c_layout", global_c_layout)
+    shared_d_layout = params.get("shared_d_layout", global_d_layout)
+
+    tile_sized = any(require_tile_sized_global(l) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
+    block_shape = params.get("block_shape")
+    block_shape = default_block_shape(operator, gemm_shape, tile_sized) if block_shape is None else NT(block_shape)
+    op_shape = Operator.shape(operator)
+
+    is_mfma = operator.kind in (Operator.MFMA, Operator.MFMA_COMPLEX, Operator.MFMA_DUAL)
+    waves = _default_waves(operator, block_shape) if is_mfma else None
+    if waves is not None:
+        warps_default = waves[0] * waves[1]
+        compute_warp_default = NT(M=block_shape.M // waves[0], N=block_shape.N // waves[1], K=op_shape.K)
+    else:
+        # reference src/config.jl:216-229: 8 warps as 4 x 2 unless the block is too small for that
+        warps_default = 8
+        compute_warp_default = NT(M=block_shape.M // 4, N=block_shape.N // 2, K=op_shape.K)
+        if op_shape.M > 0 and op_shape.N > 0 and ((block_shape.M // op_shape.M) < 4 or (block_shape.N // op_shape.N) < 2):
+            compute_warp_default = NT(M=max(op_shape.M, block_shape.M // 4), N=max(op_shape.N, block_shape.N // 2), K=op_shape.K)
+            warps_default = min(block_shape.M // op_shape.M, 4) * min(block_shape.N // op_shape.N, 2)
+    warps_per_block = params.get("warps_per_block", warps_default)
+    compute_warp = NT(params.get("compute_warp", compute_warp_default))
+    if "warps_per_block" in params and "compute_warp" not in params and waves is not None and warps_per_block != warps_default:
+        # keep the reference's 4 x 2 style split for a caller-chosen wave count
+        wm = 4 if warps_per_block % 4 == 0 and warps_per_block >= 8 else (2 if warps_per_block % 2 == 0 else 1)
+        compute_warp = NT(M=block_shape.M // wm, N=block_shape.N // max(1, warps_per_block // wm), K=op_shape.K)
+
+    is_a_col_major = params.get("is_a_col_major", True)
+    is_b_col_major = params.get("is_b_col_major", True)
+    is_cd_col_major = params.get("is_cd_col_major", True)
+
+    # reference src/config.jl:240-260 with 64 lanes: 16 bytes per lane, as few lanes per row as possible
+    lanes = WARP_SIZE * max(1, warps_per_block)
+    n_a = max(1, min(16 // global_a_layout.T.size, (block_shape.M * block_shape.K) // lanes))
+    n_b = max(1, min(16 // global_b_layout.T.size, (block_shape.K * block_shape.N) // lanes))
+    n_c = max(1, min(16 // global_c_layout.T.size, (block_shape.M * block_shape.N) // lanes))
+    mk, kn, mn = NT(M=block_shape.M, K=block_shape.K), NT(K=block_shape.K, N=block_shape.N), NT(M=block_shape.M, N=block_shape.N)
+    mem_a_warp = NT(params.get("mem_a_warp", adjacent_elements(WARP_SIZE * n_a, mk, is_a_col_major)))
+    mem_b_warp = NT(params.get("mem_b_warp", adjacent_elements(WARP_SIZE * n_b, kn, is_b_col_major)))
+    mem_cd_warp = NT(params.get("mem_cd_warp", adjacent_elements(WARP_SIZE * n_c, mn, is_cd_col_major)))
+    mem_a_thread = NT(params.get("mem_a_thread", adjacent_elements(n_a, mk, is_a_col_major)))
+    mem_b_thread = NT(params.get("mem_b_thread", adjacent_elements(n_b, kn, is_b_col_major)))
+    mem_cd_thread = NT(params.get("mem_cd_thread", adjacent_elements(n_c, mn, is_cd_col_major)))
+
+    # src/config.jl:277-279 defaults to Identity; on the MI355X the XCD-aware walk is the default
+    cta_swizzle = params.get("cta_swizzle", CTASwizzle.XCDAware[4])
+
+    conf = Config(gemm_shape, block_shape, warps_per_block, mem_a_warp, mem_a_thread, mem_b_warp, mem_b_thread,
+                  mem_cd_warp, mem_cd_thread, compute_warp, op_shape,
+                  global_a_layout, global_b_layout, global_c_layout, global_d_layout,
+                  shared_a_layout, shared_b_layout, shared_c_layout, shared_d_layout,
+                  operator, is_a_col_major, is_b_col_major, cta_swizzle)
+    check_config(conf, params.get("kernel"))
+    return conf
+
+
+def check_config(conf: Config, kernel=None) -> None:
+    """Every ConfigError of the reference (src/config.jl:203-275, src/matmul.jl:28-41), decided by
+    the library on the host."""
+    c = conf.to_c()
+    code = 0 if kernel is None else kernel.code
+    rc = _lib.lib().gk_validate(ctypes.byref(c), code)
+    if rc != _lib.GK_OK:
+        raise ConfigError(_lib.last_error(), rc)

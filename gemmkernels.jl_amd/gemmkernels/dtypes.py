@@ -1,0 +1,57 @@
+"""Element types, named as in the reference's Julia code."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+
+@dataclass(frozen=True)
+class DType:
+    name: str
+    code: int        # gk_dtype of the C ABI
+    size: int        # bytes
+    is_complex: bool = False
+
+    def __repr__(self):
+        return self.name
+
+
+Float16 = DType("Float16", 0, 2)
+BFloat16 = DType("BFloat16", 1, 2)
+Float32 = DType("Float32", 2, 4)
+Float64 = DType("Float64", 3, 8)
+ComplexF16 = DType("Complex{Float16}", 0, 4, True)
+ComplexF32 = DType("Complex{Float32}", 2, 8, True)
+
+_RANK = {"Float16": 1, "BFloat16": 1, "Float32": 2, "Float64": 3}
+
+
+def promote_type(a: DType, b: DType) -> DType:
+    """Julia's promote_type restricted to the floating types used here."""
+    if a == b:
+        return a
+    if {a.name, b.name} == {"Float16", "BFloat16"}:
+        return Float32
+    return a if _RANK[a.name] >= _RANK[b.name] else b
+
+
+def real_type(t: DType) -> DType:
+    if t == ComplexF16:
+        return Float16
+    if t == ComplexF32:
+        return Float32
+    return t
+
+
+def from_torch(dtype) -> DType:
+    import torch
+    table = {torch.float16: Float16, torch.bfloat16: BFloat16, torch.float32: Float32, torch.float64: Float64,
+             torch.complex64: ComplexF32}
+    if hasattr(torch, "complex32"):
+        table[torch.complex32] = ComplexF16
+    return table[dtype]
+
+
+def to_torch(t: DType):
+    import torch
+    return {"Float16": torch.float16, "BFloat16": torch.bfloat16, "Float32": torch.float32, "Float64": torch.float64,
+            "Complex{Float32}": torch.complex64, "Complex{Float16}": torch.complex32}[t.name]

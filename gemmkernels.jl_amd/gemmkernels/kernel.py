@@ -1,0 +1,33 @@
+"""Kernels (reference src/kernel.jl).  The three names are kept; on gfx950 all of them run the
+LDS-DMA software pipeline for tile-sized aligned layouts, and ``matmul_singlestage`` is the one
+that accepts bounds-checked layouts and honours ``threadblock_condition`` (diagonal A)."""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+from . import _lib
+from .errors import ConfigError
+
+
+@dataclass(frozen=True)
+class KernelKind:
+    code: int
+    name: str
+
+    def __repr__(self):
+        return f"Kernel.{self.name}"
+
+
+matmul_singlestage = KernelKind(0, "matmul_singlestage")     # src/kernel.jl:10-129
+matmul_pipelined = KernelKind(1, "matmul_pipelined")         # src/kernel.jl:147-350
+matmul_pipelined_ng = KernelKind(2, "matmul_pipelined_ng")   # src/kernel.jl:368-574
+
+
+def shmem_size(conf, kernel: KernelKind = matmul_singlestage) -> int:
+    """LDS bytes requested by the kernel instance of ``conf`` (src/kernel.jl:131-145, 352-366, 576-590)."""
+    c = conf.to_c()
+    n = _lib.lib().gk_shmem_size(ctypes.byref(c), kernel.code)
+    if n < 0:
+        raise ConfigError(_lib.last_error(), _lib.GK_ERR_UNSUPPORTED)
+    return int(n)

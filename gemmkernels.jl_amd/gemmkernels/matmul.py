@@ -1,0 +1,240 @@
+"""The launcher ``matmul`` and the BLAS-like ``matmatmul_`` / ``mul_`` (reference src/matmul.jl;
+Julia's ``matmatmul!`` / ``mul!`` lose their ``!`` in Python).
+
+Device arrays are torch CUDA tensors in COLUMN-MAJOR order like Julia's CuArrays: a logical
+(rows, cols) matrix is a tensor with ``stride(0) == 1`` (see ``gemmkernels.colmajor``).  torch is
+only the owner of the memory and of the stream; every flop runs in libgemmkernels_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import numpy as np
+
+from . import _lib
+from . import cta_swizzle as CTASwizzle
+from . import epilogue as Epilogue
+from . import kernel as Kernel
+from . import layout as Layout
+from . import operator as Operator
+from . import transform as Transform
+from .config import Config, default_block_shape, get_config as _get_config
+from .dtypes import BFloat16, DType, Float16, Float32, Float64, from_torch, promote_type
+from .errors import ConfigError, DimensionMismatch
+from .tiling import NT
+
+_HOOKS = ("transform_global_to_shared_a", "transform_global_to_shared_b", "transform_global_to_shared_c",
+          "transform_shared_to_global_d", "transform_shared_to_regs_a", "transform_shared_to_regs_b",
+          "transform_shared_to_regs_c", "transform_regs_to_shared_d")
+
+
+def _ptr(x) -> Optional[int]:
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    return int(x.data_ptr())
+
+
+def _leading_dim(x, layout) -> int:
+    """Leading dimension, in elements, of a column-major device matrix."""
+    if x is None or isinstance(x, int) or layout.kind in (Layout.ZERO, Layout.DIAGONAL, Layout.GETT_KIND):
+        return 0
+    if x.dim() != 2:
+        raise ConfigError("matrix operands must be 2-dimensional")
+    if x.size(0) > 1 and x.stride(0) != 1:
+        raise ConfigError("matrix operands must be column-major (stride(0) == 1); see gemmkernels.colmajor")
+    return int(x.stride(1)) if x.size(1) > 1 else max(int(x.size(0)), 1)
+
+
+def lower_transforms(transforms: dict) -> Optional[_lib.gk_transforms]:
+    if all(t.is_identity for t in transforms.values()):
+        return None
+    out = _lib.gk_transforms()
+    for i, name in enumerate(_HOOKS):
+        ops = transforms[name].ops
+        out.hook[i].n_ops = len(ops)
+        for j, (kind, p0, p1) in enumerate(ops):
+            out.hook[i].ops[j].kind, out.hook[i].ops[j].p0, out.hook[i].ops[j].p1 = kind, p0, p1
+    return out
+
+
+def matmul(conf: Config, a, b, c, d, *,
+           transform_global_to_shared_a=None, transform_global_to_shared_b=None,
+           transform_global_to_shared_c=None, transform_shared_to_global_d=None,
+           transform_shared_to_regs_a=None, transform_shared_to_regs_b=None,
+           transform_shared_to_regs_c=None, transform_regs_to_shared_d=None,
+           epilogue=None, kernel=Kernel.matmul_singlestage, stream=None):
+    """reference src/matmul.jl:7-44: launch geometry, checks (ConfigError) and the asynchronous
+    launch on the current stream.  Same positional and keyword arguments as the reference."""
+    given = dict(transform_global_to_shared_a=transform_global_to_shared_a,
+                 transform_global_to_shared_b=transform_global_to_shared_b,
+                 transform_global_to_shared_c=transform_global_to_shared_c,
+                 transform_shared_to_global_d=transform_shared_to_global_d,
+                 transform_shared_to_regs_a=transform_shared_to_regs_a,
+                 transform_shared_to_regs_b=transform_shared_to_regs_b,
+                 transform_shared_to_regs_c=transform_shared_to_regs_c,
+                 transform_regs_to_shared_d=transform_regs_to_shared_d)
+    transforms = {k: (Transform.Elementwise() if v is None else v) for k, v in given.items()}
+    epilogue = Epilogue.Default() if epilogue is None else epilogue
+
+    cconf = conf.to_c(_leading_dim(a, conf.global_a_layout), _leading_dim(b, conf.global_b_layout),
+                      _leading_dim(c, conf.global_c_layout), _leading_dim(d, conf.global_d_layout))
+    ctrans = lower_transforms(transforms)
+    cepi = None
+    if epilogue.kind != Epilogue.DEFAULT:
+        cepi = _lib.gk_epilogue()
+        cepi.kind = epilogue.kind
+        cepi.bias = _ptr(epilogue.bias)
+    if stream is None:
+        import torch
+        stream = torch.cuda.current_stream().cuda_stream
+    rc = _lib.lib().gk_matmul(ctypes.byref(cconf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                              ctypes.byref(ctrans) if ctrans is not None else None,
+                              ctypes.byref(cepi) if cepi is not None else None,
+                              kernel.code, ctypes.c_void_p(int(stream)))
+    if rc != _lib.GK_OK:
+        msg = _lib.last_error()
+        if rc == _lib.GK_ERR_DIMENSION_MISMATCH:
+            raise DimensionMismatch(msg)
+        raise ConfigError(msg, rc)
+    return d
+
+
+def kernel_name(conf: Config, kernel=Kernel.matmul_singlestage, transforms=None, epilogue=None) -> str:
+    """Name of the compiled kernel instance a launch of ``conf`` runs (for logs and profiles)."""
+    cconf = conf.to_c()
+    buf = ctypes.create_string_buffer(256)
+    ctrans = None
+    if transforms:
+        full = {k: transforms.get(k, Transform.Elementwise()) for k in _HOOKS}
+        ctrans = lower_transforms(full)
+    cepi = None
+    if epilogue is not None and epilogue.kind != Epilogue.DEFAULT:
+        cepi = _lib.gk_epilogue()
+        cepi.kind = epilogue.kind
+    rc = _lib.lib().gk_kernel_name(ctypes.byref(cconf), ctypes.byref(ctrans) if ctrans is not None else None,
+                                   ctypes.byref(cepi) if cepi is not None else None, kernel.code, buf, len(buf))
+    if rc != _lib.GK_OK:
+        raise ConfigError(_lib.last_error(), rc)
+    return buf.value.decode()
+
+
+# ------------------------------------------------------------------------------------------------
+# BLAS-like
+# ------------------------------------------------------------------------------------------------
+
+def _select_kernel(layout_a, layout_b):
+    """reference src/matmul.jl:52-56: the pipelined kernel when both operands are aligned."""
+    if layout_a.is_aligned and layout_b.is_aligned:
+        return Kernel.matmul_pipelined
+    return Kernel.matmul_singlestage
+
+
+_configs = {}
+
+
+def get_config(*args):
+    """Memoised create_config (reference src/matmul.jl:58-65)."""
+    val = _configs.get(args)
+    if val is None:
+        val = _configs[args] = create_config(*args)
+    return val
+
+
+def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stridesB, transB: bool,
+                  C: DType, sizeC, stridesC, alpha: type, zeroAlpha: bool, beta: type, zeroBeta: bool, wmma=None):
+    """reference src/matmul.jl:66-183, with the MI355X operator and block-shape choices."""
+    m = sizeA[1 if transA else 0]
+    k = sizeA[0 if transA else 1]
+    n = sizeB[0 if transB else 1]
+    if m != sizeC[0] or n != sizeC[1] or k != sizeB[1 if transB else 0]:
+        raise DimensionMismatch("Dimensions do not match")
+
+    a_layout_base = Layout.RowMajor if transA else Layout.ColMajor
+    b_layout_base = Layout.RowMajor if transB else Layout.ColMajor
+    a_aligned_layout_base = Layout.UnsafeAlignedRowMajor if transA else Layout.UnsafeAlignedColMajor
+    b_aligned_layout_base = Layout.UnsafeAlignedRowMajor if transB else Layout.UnsafeAlignedColMajor
+
+    # operator: the matrix cores for 16-bit inputs with fp32 accumulation (src/matmul.jl:85-91)
+    mfma_types = [(Float16, Float16, Float32), (BFloat16, BFloat16, Float32), (Float16, Float16, Float16)]
+    compute_type = promote_type(A, B)
+    use_mfma = ((compute_type, compute_type, C) in mfma_types) if wmma is None else bool(wmma)
+
+    shared_a_layout = Layout.Padded[a_aligned_layout_base[compute_type if use_mfma else A], 8]
+    shared_b_layout = Layout.Padded[b_aligned_layout_base[compute_type if use_mfma else B], 8]
+    shared_c_layout = Layout.Zero[C] if zeroBeta else Layout.UnsafeAlignedColMajor[C]
+    shared_d_layout = Layout.UnsafeAlignedColMajor[C]
+
+    if use_mfma:
+        operator = Operator.MFMAOp[32, 32, 16, compute_type, Float32 if C == Float16 else C]
+    else:
+        operator = Operator.FPUOp[8, 8, 1, 8, 8, 1, compute_type, C]
+    block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=True)
+
+    a_aligned = (stridesA[1] * A.size) % 16 == 0
+    b_aligned = (stridesB[1] * B.size) % 16 == 0
+    c_aligned = (stridesC[1] * C.size) % 16 == 0
+    if zeroAlpha:
+        global_a_layout, global_b_layout = Layout.Zero[A], Layout.Zero[B]
+    else:
+        global_a_layout = (a_aligned_layout_base[A] if a_aligned and m % block_shape.M == 0 and k % block_shape.K == 0
+                           else a_layout_base[A])
+        global_b_layout = (b_aligned_layout_base[B] if b_aligned and k % block_shape.K == 0 and n % block_shape.N == 0
+                           else b_layout_base[B])
+    cd_aligned = c_aligned and m % block_shape.M == 0 and n % block_shape.N == 0
+    global_c_layout = Layout.Zero[C] if zeroBeta else (Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C])
+    global_d_layout = Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C]
+
+    conf = _get_config(gemm_shape=NT(M=m, N=n, K=k), block_shape=block_shape, operator=operator,
+                       global_a_layout=global_a_layout, global_b_layout=global_b_layout,
+                       global_c_layout=global_c_layout, global_d_layout=global_d_layout,
+                       shared_a_layout=shared_a_layout, shared_b_layout=shared_b_layout,
+                       shared_c_layout=shared_c_layout, shared_d_layout=shared_d_layout,
+                       is_a_col_major=not transA, is_b_col_major=not transB)
+    return conf, compute_type, _select_kernel(global_a_layout, global_b_layout)
+
+
+def _round_to(dtype: DType, x: float) -> float:
+    if dtype == Float16:
+        return float(np.float16(x))
+    if dtype == BFloat16:
+        import torch
+        return float(torch.tensor(x, dtype=torch.bfloat16))
+    if dtype == Float32:
+        return float(np.float32(x))
+    return float(x)
+
+
+def matmatmul_(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None):
+    """``matmatmul!`` (reference src/matmul.jl:185-204): C = alpha * op(A) * op(B) + beta * C."""
+    tA, tB = transA == 'T', transB == 'T'
+    conf, compute_type, kernel = get_config(
+        from_torch(A.dtype), tuple(A.shape), tuple(A.stride()), tA,
+        from_torch(B.dtype), tuple(B.shape), tuple(B.stride()), tB,
+        from_torch(C.dtype), tuple(C.shape), tuple(C.stride()),
+        type(alpha), alpha == 0, type(beta), beta == 0, wmma)
+    alpha_c = _round_to(compute_type, float(alpha))          # convert(compute_type, alpha), :196
+    beta_c = _round_to(from_torch(C.dtype), float(beta))     # convert(eltype(C), beta), :197
+    ta = Transform.Elementwise(ops=[] if alpha_c == 1.0 else [(Transform.SCALE, alpha_c, 0.0)])
+    tc = Transform.Elementwise(ops=[] if beta_c == 1.0 else [(Transform.SCALE, beta_c, 0.0)])
+    matmul(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)
+    return C
+
+
+class Transpose:
+    """Lazy transpose wrapper, Julia's ``transpose(A)`` / ``A'`` (no conjugation, src/matmul.jl:211-213)."""
+
+    def __init__(self, parent):
+        self.parent = parent
+
+
+Adjoint = Transpose
+
+
+def mul_(C, A, B, alpha=True, beta=False):
+    """``mul!`` (reference src/matmul.jl:207-215): unwraps Transpose/Adjoint and forwards."""
+    tA, tB = isinstance(A, Transpose), isinstance(B, Transpose)
+    return matmatmul_(C, 'T' if tA else 'N', 'T' if tB else 'N', A.parent if tA else A, B.parent if tB else B,
+                      float(alpha), float(beta))
