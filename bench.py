@@ -1,0 +1,139 @@
+#!/usr/bin/env python3
+"""Benchmark of the tiled GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one launch of the headline workload: the FP16 x FP16 -> FP32 GEMM C = A*B + C with
+M = N = K = 4096, column-major, 'N','N' (benchmark config 2), through gemmkernels.matmul -> C ABI ->
+HIP kernel, inputs resident in HBM.  The other three transposes and the other benchmark configs
+are timed after the timed region and reported in extra fields of the same JSON line.
+Prints exactly one JSON line on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "gemmkernels.jl_amd"))
+sys.path.insert(0, ROOT)
+
+METRIC = "TFLOP/s + % FP16 MFMA peak, 4096^3 FP16->FP32 GEMM on 1 MI355X"
+PEAK_FP16_TFLOPS = 2516.6     # MI355X dense FP16/BF16 matrix peak (256 CU x 4 SIMD x 1024 flop/clk x 2.4 GHz)
+PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the headline kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes
+# summarised in profiles/ (None until measured)
+MEASURED_TRAFFIC_BYTES = None
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--no-extras", action="store_true", help="skip the secondary configs and the CPU baseline")
+    return p.parse_args()
+
+
+def time_launches(fn, steps, warmup):
+    """Average duration in microseconds of `steps` back-to-back launches, HIP events on the launch stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) * 1e3 / steps, wall
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import gemmkernels as gk
+    from gemmkernels import configs
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP library has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+
+    # ---------------- headline: config 2, NN ----------------
+    wl = configs.benchmark_config(2, variant="NN")
+    run = wl.prepare()          # uploads the seeded inputs, returns a zero-argument launcher
+    us, wall = time_launches(run, args.steps, args.warmup)
+    tflops = wl.flops / us / 1e6
+    result = {
+        "metric": METRIC,
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us / 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 multiplicands, f32 accumulate",
+        "data": "synthetic (counter-based splitmix64 streams, seeds 2001-2003)",
+        "config": {"workload": wl.description, "kernel": wl.kernel_name},
+        "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_FP16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": wl.kernel_name, "avg_launch_us": round(us, 2), "flop_per_launch": wl.flops},
+    }
+
+    if not args.no_extras:
+        # ---------------- the other transposes and configs (outside the timed region) ----------------
+        extras = {}
+        for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4b", None), (5, None)]:
+            try:
+                w = configs.benchmark_config(cfg, variant=variant)
+                r = w.prepare()
+                u, _ = time_launches(r, 50, 10)
+                entry = {"us": round(u, 2), "kernel": w.kernel_name}
+                if w.bound == "hbm":
+                    entry["GB/s"] = round(w.bytes / u / 1e3, 1)
+                    entry["frac_of_hbm_peak"] = round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)
+                else:
+                    entry["TFLOP/s"] = round(w.flops / u / 1e6, 2)
+                extras[w.name] = entry
+                del r, w
+                torch.cuda.empty_cache()
+            except Exception as e:  # a config that is not built yet must not hide the headline number
+                extras[f"config {cfg}{' ' + variant if variant else ''}"] = {"error": f"{type(e).__name__}: {e}"}
+        result["other_configs"] = extras
+
+        # ---------------- CPU baseline: the reference's own CPU path is BLAS sgemm on host arrays ----------------
+        from oracle import oracle
+        a, b, c = wl.host_inputs()
+        a32, b32 = a.astype(np.float32), b.astype(np.float32)
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            oracle.gemm_blas_f32(a32, b32, c, 1.0, 1.0)
+            times.append(time.perf_counter() - t0)
+        cpu_s = sorted(times)[1]
+        threads = int(os.environ.get("OPENBLAS_NUM_THREADS") or os.environ.get("OMP_NUM_THREADS") or os.cpu_count())
+        result["cpu_baseline"] = {"value": round(wl.flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                                  "sample": "3 full 4096^3 GEMMs on the FP32-converted inputs (numpy -> OpenBLAS sgemm, the "
+                                            "routine behind the reference's LinearAlgebra.mul! oracle), median",
+                                  "seconds": round(cpu_s, 4)}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

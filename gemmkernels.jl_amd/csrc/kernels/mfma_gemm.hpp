@@ -182,6 +182,7 @@ template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, bo
 struct MfmaGemmConfig {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, FUSED = FUSED_;
+  static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / 16) % 2 == 0);   // cross-step fragment prefetch
   typedef T_ T;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int THREADS = NWAVES * kWaveSize;
@@ -199,6 +200,7 @@ struct MfmaGemmConfig {
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
   static_assert(STAGES >= 2, "at least two LDS stages");
   static_assert((STAGES - 2) * DMA_PER_TILE <= 63, "vmcnt is a 6-bit counter");
+  static_assert(FM * FN > 0, "empty wave tile");
 };
 
 template <class Cfg>
@@ -211,6 +213,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr int DMA_A = Cfg::DMA_A, DMA_B = Cfg::DMA_B, DPT = Cfg::DMA_PER_TILE;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+#ifdef GK_PHASE_TRACE
+  // development aid (never defined in the library build): per-block phase timestamps
+  long long trace_t[5];
+  trace_t[0] = clock64();
+  const long long trace_w0 = wall_clock64();
+#endif
 
   int ti, tj;
   cta_swizzle(args.swz_kind, args.swz_param, (int)blockIdx.x, (int)blockIdx.y, args.nbm, args.nbn, ti, tj);
@@ -233,6 +241,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   for (int i = 0; i < DMA_B; ++i) offb[i] = dma_global_offset<BN, BK, Cfg::B_KMAJOR>(wave + i * NWAVES, lane, args.ldb);
 
   auto issue_tile = [&](int stage) {
+#ifdef GK_ABLATE_DMA
+    (void)stage; return;
+#endif
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
 #pragma unroll
@@ -302,50 +313,109 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   rb.init(wn * Cfg::WTN, lane);
   const unsigned lds_base = (unsigned)(uintptr_t)GK_LDS_PTR(char, smem);
 
+#ifdef GK_PHASE_TRACE
+  trace_t[1] = clock64();
+#endif
   // --- main loop ------------------------------------------------------------------------------
-  for (int kt = 0; kt < KT; ++kt) {
-    // tile kt has landed once at most the DMA of the STAGES-2 younger tiles is outstanding
-    if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 2) * DPT>(); else wait_vmcnt<0>();
-    block_barrier();   // every wave's share of tile kt is in LDS; every wave is done with tile kt-1
-    if (kt + STAGES - 1 < KT) issue_tile((kt + STAGES - 1) % STAGES);
+  // Fragments are double-buffered: the LDS reads of the next k-step are in flight while the MFMAs
+  // of the current one run.  LDS reads complete in order, so "at most NEXT outstanding" means that
+  // the current set has arrived.
+  int4v fa[2][FM], fb[2][FN];
+  constexpr int FRAG_OPS = FM * RA::OPS + FN * RB::OPS;
 
-    const unsigned stage_addr = lds_base + (unsigned)(kt % STAGES) * Cfg::STAGE_BYTES;
-    ra.set_stage(stage_addr);
-    rb.set_stage(stage_addr + GA::BYTES);
-
-    // fragments are double-buffered: the reads of k-step ks+1 are in flight while the MFMAs of
-    // k-step ks run; LDS reads complete in order, so "at most NEXT outstanding" means that the
-    // current set has arrived.
-    int4v fa[2][FM], fb[2][FN];
-    load_frags<0>(ra, rb, fa[0], fb[0]);
-    static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
-      constexpr int ks = decltype(ks_c)::value;
-      constexpr bool more = (ks + 1 < Cfg::KSTEPS);
-      if constexpr (more) load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-      wait_lgkmcnt<more ? (FM * RA::OPS + FN * RB::OPS) : 0>();
+  auto compute = [&](auto ks_c) {
+    constexpr int ks = decltype(ks_c)::value;
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi) pin(fa[ks & 1][fi]);
+    for (int fi = 0; fi < FM; ++fi) pin(fa[ks & 1][fi]);
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) pin(fb[ks & 1][fj]);
-      if (Cfg::FUSED) {
-        if (xf_a) {
+    for (int fj = 0; fj < FN; ++fj) pin(fb[ks & 1][fj]);
+    if (Cfg::FUSED) {
+      if (xf_a) {
 #pragma unroll
-          for (int fi = 0; fi < FM; ++fi) fa[ks & 1][fi] = transform_fragment<T>(fa[ks & 1][fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
-        }
-        if (xf_b) {
-#pragma unroll
-          for (int fj = 0; fj < FN; ++fj) fb[ks & 1][fj] = transform_fragment<T>(fb[ks & 1][fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
-        }
+        for (int fi = 0; fi < FM; ++fi) fa[ks & 1][fi] = transform_fragment<T>(fa[ks & 1][fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
       }
+      if (xf_b) {
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi)
+        for (int fj = 0; fj < FN; ++fj) fb[ks & 1][fj] = transform_fragment<T>(fb[ks & 1][fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
+      }
+    }
 #pragma unroll
-        for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = Mfma<T>::run(fb[ks & 1][fj], fa[ks & 1][fi], acc[fi][fj]);
-    });
-    // the last wait above was lgkmcnt(0): all LDS reads of this stage are complete before the
-    // next barrier lets a DMA overwrite it
+    for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) {
+#ifdef GK_ABLATE_MFMA
+        acc[fi][fj][0] += __builtin_bit_cast(float, fb[ks & 1][fj][0] ^ fa[ks & 1][fi][0]);
+#else
+        acc[fi][fj] = Mfma<T>::run(fb[ks & 1][fj], fa[ks & 1][fi], acc[fi][fj]);
+#endif
+      }
+  };
+
+  if constexpr (!Cfg::PREFETCH) {
+    // Two LDS stages: the DMA of tile kt+1 runs while tile kt is consumed; the first fragments of a
+    // tile are read after the barrier that publishes it.
+    for (int kt = 0; kt < KT; ++kt) {
+      // tile kt has landed once at most the DMA of the STAGES-2 younger tiles is outstanding
+      if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 2) * DPT>(); else wait_vmcnt<0>();
+      block_barrier();   // every wave's share of tile kt is in LDS; every wave is done with tile kt-1
+      const unsigned stage_addr = lds_base + (unsigned)(kt % STAGES) * Cfg::STAGE_BYTES;
+      ra.set_stage(stage_addr);
+      rb.set_stage(stage_addr + GA::BYTES);
+      load_frags<0>(ra, rb, fa[0], fb[0]);
+      if (kt + STAGES - 1 < KT) issue_tile((kt + STAGES - 1) % STAGES);
+      static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
+        constexpr int ks = decltype(ks_c)::value;
+        constexpr bool more = (ks + 1 < Cfg::KSTEPS);
+        if constexpr (more) load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+        wait_lgkmcnt<more ? FRAG_OPS : 0>();
+        compute(ks_c);
+      });
+      // the last wait above was lgkmcnt(0): all LDS reads of this stage are complete before the
+      // next barrier lets a DMA overwrite it
+    }
+  } else {
+    // Three or more LDS stages: the barrier of step kt publishes tile kt+1, so the first fragments
+    // of tile kt+1 are read at the end of step kt and the MFMAs of a step start right after its
+    // barrier, with neither the LDS latency nor the DMA issue in the way.
+    static_assert(!Cfg::PREFETCH || (Cfg::KSTEPS % 2 == 0), "fragment buffers alternate per k-step");
+    if (STAGES - 1 <= KT) wait_vmcnt<(STAGES - 2) * DPT>(); else wait_vmcnt<0>();
+    block_barrier();
+    ra.set_stage(lds_base);
+    rb.set_stage(lds_base + GA::BYTES);
+    load_frags<0>(ra, rb, fa[0], fb[0]);
+    for (int kt = 0; kt < KT; ++kt) {
+      // tiles <= kt+1 have landed once at most the STAGES-3 younger tiles are outstanding
+      if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 3) * DPT>(); else wait_vmcnt<0>();
+      block_barrier();   // tile kt+1 is visible; every wave is done reading tile kt-1
+      const bool issue = (kt + STAGES - 1 < KT);
+      const bool last = (kt + 1 >= KT);
+      static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
+        constexpr int ks = decltype(ks_c)::value;
+        if constexpr (ks + 1 < Cfg::KSTEPS) {
+          load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+          wait_lgkmcnt<FRAG_OPS>();
+          if constexpr (ks == 0) {
+            if (issue) issue_tile((kt + STAGES - 1) % STAGES);
+          }
+        } else {
+          if (!last) {
+            const unsigned stage_addr = lds_base + (unsigned)((kt + 1) % STAGES) * Cfg::STAGE_BYTES;
+            ra.set_stage(stage_addr);
+            rb.set_stage(stage_addr + GA::BYTES);
+            load_frags<0>(ra, rb, fa[0], fb[0]);
+            wait_lgkmcnt<FRAG_OPS>();
+          } else {
+            wait_lgkmcnt<0>();
+          }
+        }
+        compute(ks_c);
+      });
+    }
   }
 
+#ifdef GK_PHASE_TRACE
+  trace_t[2] = clock64();
+#endif
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   float* dp = (float*)args.d + mrow + (long long)ncol * args.ldd;
 #pragma unroll
@@ -371,6 +441,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int v = 0; v < 16; ++v)
         dp[32 * fi + (long long)(32 * fj + 8 * (v / 4) + (v % 4)) * args.ldd] = x[v];
     }
+#ifdef GK_PHASE_TRACE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  trace_t[3] = clock64();
+  if (threadIdx.x == 0) {
+    long long* out = (long long*)args.bias + (size_t)blockIdx.x * 8;
+    out[0] = trace_t[0]; out[1] = trace_t[1]; out[2] = trace_t[2]; out[3] = trace_t[3];
+    out[4] = trace_w0; out[5] = wall_clock64();
+  }
+#endif
 }
 
 }  // namespace gk

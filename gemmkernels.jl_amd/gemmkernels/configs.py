@@ -1,0 +1,148 @@
+"""The configurations used by tests and benchmarks (the role of reference configs/configs.jl:
+``Configuration`` :31-47, ``generate_inputs`` :77-96, ``run_gemm`` :99-110 and the ``@get_*_config``
+macros :161-490), plus the five benchmark workloads with their seeded synthetic inputs.
+
+Seeds: workload n uses 1000n + {1: A, 2: B, 3: C, 4: bias / diagonal}.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Optional
+
+import numpy as np
+
+from . import cta_swizzle as CTASwizzle
+from . import epilogue as Epilogue
+from . import kernel as Kernel
+from . import layout as Layout
+from . import operator as Operator
+from . import rng
+from . import transform as Transform
+from .arrays import colmajor, colmajor_empty
+from .config import get_config
+from .dtypes import Float16, Float32
+from .matmul import kernel_name, matmul
+from .tiling import NT
+
+
+@dataclass
+class Workload:
+    name: str
+    description: str
+    flops: int
+    bytes: int
+    bound: str                      # "mfma", "hbm" or "latency"
+    make_host: Callable[[], dict]   # seeded numpy inputs
+    make_launch: Callable[[dict], Callable[[], None]]
+    kernel_name: str = ""
+    _host: Optional[dict] = field(default=None, repr=False)
+
+    def host(self) -> dict:
+        if self._host is None:
+            self._host = self.make_host()
+        return self._host
+
+    def host_inputs(self):
+        h = self.host()
+        return h.get("a"), h.get("b"), h.get("c")
+
+    def prepare(self):
+        """Upload the inputs and return a zero-argument function that enqueues one launch.  The
+        device tensors are reachable as attributes of the returned function (``.d`` is the output)."""
+        return self.make_launch(self.host())
+
+
+def _aligned(T, transposed):
+    return Layout.UnsafeAlignedRowMajor[T] if transposed else Layout.UnsafeAlignedColMajor[T]
+
+
+def mfma_config(M, N, K, ta=False, tb=False, zero_c=False, block_shape=None, **kw):
+    """An MFMA configuration with aligned layouts in the spirit of @get_wmma_config
+    (reference configs/configs.jl:246-289)."""
+    params = dict(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+                  global_a_layout=_aligned(Float16, ta), global_b_layout=_aligned(Float16, tb),
+                  global_c_layout=Layout.Zero[Float32] if zero_c else Layout.UnsafeAlignedColMajor[Float32],
+                  global_d_layout=Layout.UnsafeAlignedColMajor[Float32],
+                  is_a_col_major=not ta, is_b_col_major=not tb)
+    if block_shape is not None:
+        params["block_shape"] = NT(M=block_shape[0], N=block_shape[1], K=block_shape[2])
+    params.update(kw)
+    return get_config(**params)
+
+
+def _attach(fn, **tensors):
+    for k, v in tensors.items():
+        setattr(fn, k, v)
+    return fn
+
+
+def _config2(variant: str) -> Workload:
+    ta, tb = variant[0] == "T", variant[1] == "T"
+    M = N = K = 4096
+    conf = mfma_config(M, N, K, ta, tb)
+
+    def host():
+        return dict(a=rng.matrix("upm1_f16", 2001, (K, M) if ta else (M, K)),
+                    b=rng.matrix("upm1_f16", 2002, (N, K) if tb else (K, N)),
+                    c=rng.matrix("upm1_f32", 2003, (M, N)))
+
+    def launch(h):
+        import torch
+        a, b, c = colmajor(h["a"]), colmajor(h["b"]), colmajor(h["c"])
+        d = colmajor_empty((M, N), torch.float32)
+
+        def run():
+            matmul(conf, a, b, c, d, kernel=Kernel.matmul_pipelined)
+        return _attach(run, a=a, b=b, c=c, d=d, conf=conf)
+
+    return Workload(
+        name=f"config 2 {variant}",
+        description=f"config 2: C = A*B + C, FP16 A/B ~ U[-1,1), FP32 C ~ U[-1,1) read and accumulated, M=N=K=4096, "
+                    f"column-major '{variant[0]}','{variant[1]}', alpha=beta=1",
+        flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + 2 * M * N * 4, bound="mfma",
+        make_host=host, make_launch=launch, kernel_name=kernel_name(conf, Kernel.matmul_pipelined))
+
+
+def _config3() -> Workload:
+    M, N, K = 4096, 4096, 2048
+    conf = mfma_config(M, N, K, zero_c=True)
+    transforms = dict(transform_global_to_shared_a=Transform.Elementwise(lambda x: x * 0.5),
+                      transform_shared_to_global_d=Transform.Elementwise(Transform.relu))
+
+    def host():
+        return dict(a=rng.matrix("upm1_f16", 3001, (M, K)), b=rng.matrix("upm1_f16", 3002, (K, N)),
+                    bias=rng.normal_f32(3004, N))
+
+    def launch(h):
+        import torch
+        a, b = colmajor(h["a"]), colmajor(h["b"])
+        bias = torch.from_numpy(h["bias"]).cuda()
+        d = colmajor_empty((M, N), torch.float32)
+        epi = Epilogue.Bias(bias)
+
+        def run():
+            matmul(conf, a, b, None, d, epilogue=epi, kernel=Kernel.matmul_pipelined, **transforms)
+        return _attach(run, a=a, b=b, bias=bias, d=d, conf=conf)
+
+    return Workload(
+        name="config 3",
+        description="config 3: D = relu((0.5*A)*B + bias[j]), FP16 A/B ~ U[-1,1), FP32 D, M=N=4096, K=2048, bias ~ N(0,1) per "
+                    "column (Epilogue.Bias), scale on the global->shared load of A, ReLU on the shared->global store of D",
+        flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + N * 4 + M * N * 4, bound="mfma",
+        make_host=host, make_launch=launch,
+        kernel_name=kernel_name(conf, Kernel.matmul_pipelined, transforms, Epilogue.Bias(0)))
+
+
+def benchmark_config(n, variant: Optional[str] = None) -> Workload:
+    """The benchmark workloads 1, 2 (variant NN/NT/TN/TT), 3, "4a", "4b", 5."""
+    if n == 2:
+        return _config2(variant or "NN")
+    if n == 3:
+        return _config3()
+    builders = _LATE_BUILDERS
+    if n in builders:
+        return builders[n]()
+    raise NotImplementedError(f"benchmark config {n}")
+
+
+_LATE_BUILDERS = {}

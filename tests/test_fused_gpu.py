@@ -1,0 +1,97 @@
+"""GPU parity of the fused transforms and epilogues (benchmark config 3 and the eight hooks of the
+launcher) against the CPU oracle, which restates the reference's order of operations."""
+import numpy as np
+import pytest
+
+import gemmkernels as gk
+from gemmkernels import Epilogue, Kernel, Transform, configs, rng
+import helpers
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+E = Transform.Elementwise
+
+
+def small_inputs(M, N, K, seed):
+    return (rng.matrix("upm1_f16", seed + 1, (M, K)), rng.matrix("upm1_f16", seed + 2, (K, N)),
+            rng.matrix("upm1_f32", seed + 3, (M, N)))
+
+
+def test_config3_reduced(gpu):
+    M, N, K = 256, 384, 128
+    conf = configs.mfma_config(M, N, K, zero_c=True, block_shape=(128, 128, 64))
+    a, b, _ = small_inputs(M, N, K, 3000)
+    bias = rng.normal_f32(3004, N)
+    tr = dict(transform_global_to_shared_a=E(lambda x: x * 0.5), transform_shared_to_global_d=E(Transform.relu))
+    d = helpers.run_gpu(conf, a, b, None, (M, N), transforms=tr, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
+    ref = helpers.run_oracle(conf, a, b, None, (M, N), transforms=tr, epilogue=Epilogue.Bias(0), bias=bias)
+    assert oracle.rel_frobenius(d, ref) <= TOL
+    # textbook form in float64
+    ref64 = np.maximum(0.5 * a.astype(np.float64) @ b.astype(np.float64) + bias[None, :].astype(np.float64), 0.0)
+    assert oracle.rel_frobenius(d, ref64) <= TOL
+    assert (d >= 0).all()
+
+
+def test_bias_only_closed_form(gpu):
+    """A = 0  =>  D[i, j] = relu(bias[j]) exactly (per-column bias, reference src/epilogue.jl:44-52)."""
+    M, N, K = 256, 256, 64
+    conf = configs.mfma_config(M, N, K, zero_c=True, block_shape=(128, 128, 64))
+    a = np.zeros((M, K), dtype=np.float16, order="F")
+    b = rng.matrix("upm1_f16", 5, (K, N))
+    bias = rng.normal_f32(6, N)
+    tr = dict(transform_shared_to_global_d=E(Transform.relu))
+    d = helpers.run_gpu(conf, a, b, None, (M, N), transforms=tr, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d, np.broadcast_to(np.maximum(bias, 0)[None, :], (M, N)))
+    # per-row variant
+    bias_m = rng.normal_f32(7, M)
+    d = helpers.run_gpu(conf, a, b, None, (M, N), transforms=tr, epilogue_cls=Epilogue.BiasRow, bias=bias_m, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d, np.broadcast_to(np.maximum(bias_m, 0)[:, None], (M, N)))
+
+
+def test_exact_scaling_and_relu_idempotence(gpu):
+    M, N, K = 256, 256, 128
+    a, b, _ = small_inputs(M, N, K, 40)
+    conf = configs.mfma_config(M, N, K, zero_c=True, block_shape=(128, 128, 64))
+    d1 = helpers.run_gpu(conf, a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
+    d2 = helpers.run_gpu(conf, a, b, None, (M, N), transforms=dict(transform_global_to_shared_a=E(lambda x: x * 0.5)), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d2, 0.5 * d1)           # a power-of-two scale commutes with every rounding
+    r1 = helpers.run_gpu(conf, a, b, None, (M, N), transforms=dict(transform_shared_to_global_d=E(Transform.relu)), kernel=Kernel.matmul_pipelined)
+    r2 = helpers.run_gpu(conf, a, b, None, (M, N), transforms=dict(transform_regs_to_shared_d=E(Transform.relu), transform_shared_to_global_d=E(Transform.relu)), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(r1, np.maximum(d1, 0)) and np.array_equal(r1, r2)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_all_eight_hooks(gpu, ta, tb):
+    """Every hook carries a different op list; the oracle applies them at the same points with the
+    same rounding (alpha on A in FP16, beta on C in FP32 as matmatmul! does, src/matmul.jl:196-201)."""
+    M, N, K = 256, 256, 192
+    conf = configs.mfma_config(M, N, K, ta, tb, block_shape=(128, 128, 64))
+    a = rng.matrix("upm1_f16", 51, (K, M) if ta else (M, K))
+    b = rng.matrix("upm1_f16", 52, (N, K) if tb else (K, N))
+    c = rng.matrix("upm1_f32", 53, (M, N))
+    bias = rng.normal_f32(54, N)
+    tr = dict(transform_global_to_shared_a=E(lambda x: x * 0.75),
+              transform_global_to_shared_b=E(lambda x: abs(x)),
+              transform_global_to_shared_c=E(lambda x: x + 0.125),
+              transform_shared_to_regs_a=E(lambda x: x * 2.0 - 0.25),
+              transform_shared_to_regs_b=E(lambda x: -x),
+              transform_shared_to_regs_c=E(lambda x: x * 3.0),
+              transform_regs_to_shared_d=E(lambda x: Transform.clamp(x, -20.0, 25.0)),
+              transform_shared_to_global_d=E(lambda x: Transform.square(x) * 0.01))
+    d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=tr, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
+    ref = helpers.run_oracle(conf, a, b, c, (M, N), transforms=tr, epilogue=Epilogue.Bias(0), bias=bias)
+    assert oracle.rel_frobenius(d, ref) <= TOL
+
+
+def test_config3_full_size(gpu):
+    w = configs.benchmark_config(3)
+    run = w.prepare()
+    run()
+    import torch
+    torch.cuda.synchronize()
+    d = gk.to_numpy(run.d)
+    h = w.host()
+    ref = np.maximum(0.5 * oracle.gemm_blas_f32(h["a"], h["b"], None) + h["bias"][None, :], 0.0)
+    assert oracle.rel_frobenius(d, ref) <= TOL
+    assert (d >= 0).all()
