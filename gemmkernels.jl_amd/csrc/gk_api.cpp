@@ -266,6 +266,11 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   if (require_tile_sized_global(c->global_d_layout.kind) && (g.M % b.M || g.N % b.N))
     return fail(GK_ERR_TILE_MULTIPLE, "gemm_shape.MN must be a multiple of block_shape.MN!");
 
+  // src/matmul.jl:34-36 (decidable from the configuration alone, so it is checked before the
+  // instance lookup)
+  if (kernel != GK_KERNEL_SINGLESTAGE && b.K < 2 * os.K)
+    return fail(GK_ERR_STAGES, "Need at least two stages to use a pipelined kernel, i.e. BLOCK_K >= 2 * OPERATOR_K");
+
   // the instance that would run; its LDS request is what Kernel.shmem_size returns
   int rc = find_instance(c, t, e, key, info);
   if (rc != GK_OK) return rc;
@@ -277,9 +282,6 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   if (info->lds_bytes > lds_max)
     return fail(GK_ERR_LDS, "Requested too much shared memory: The current GPU can use at most %lld bytes, while this configuration required %d bytes",
                 lds_max, info->lds_bytes);
-  // src/matmul.jl:34-36
-  if (kernel != GK_KERNEL_SINGLESTAGE && b.K < 2 * os.K)
-    return fail(GK_ERR_STAGES, "Need at least two stages to use a pipelined kernel, i.e. BLOCK_K >= 2 * OPERATOR_K");
   // src/matmul.jl:41
   const long long threads = (long long)c->warps_per_block * gk::kWaveSize;
   if (threads > threads_max)

@@ -1,0 +1,46 @@
+"""The C-ABI library loads without a GPU and exports every symbol the header declares."""
+import ctypes
+import os
+import re
+
+from gemmkernels import _lib
+
+HEADER = os.path.join(os.path.dirname(__file__), "..", "include", "gemmkernels_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gk_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = declared_functions()
+    assert len(names) >= 12
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in names:
+        assert hasattr(handle, name), f"{name} is declared in the header but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == names, "the Python binding must cover exactly the header"
+
+
+def test_struct_sizes_match_the_library():
+    lib = _lib.lib()     # lib() itself raises on any mismatch
+    for which, struct in enumerate((_lib.gk_config, _lib.gk_layout, _lib.gk_operator, _lib.gk_transforms, _lib.gk_epilogue, _lib.gk_gett)):
+        assert lib.gk_sizeof(which) == ctypes.sizeof(struct)
+    assert lib.gk_sizeof(99) == -1
+
+
+def test_version_and_status_strings():
+    lib = _lib.lib()
+    assert lib.gk_version() == 100
+    assert _lib.status_string(0) == "GK_OK"
+    assert _lib.status_string(_lib.GK_ERR_LDS) == "GK_ERR_LDS"
+    assert _lib.status_string(12345) == "GK_ERR_UNKNOWN"
+
+
+def test_null_config_is_an_error_not_a_crash():
+    lib = _lib.lib()
+    assert lib.gk_validate(None, 0) == _lib.GK_ERR_INVALID_ARGUMENT
+    assert "NULL" in _lib.last_error()
+    assert lib.gk_shmem_size(None, 0) == -1
+    assert lib.gk_matmul(None, None, None, None, None, None, None, 0, None) == _lib.GK_ERR_INVALID_ARGUMENT

@@ -1,0 +1,165 @@
+"""Config, get_config and every launch-time error, decided on the host (no GPU).
+Known answers are hand-evaluated from the reference source lines cited at each test."""
+import ctypes
+
+import pytest
+
+import gemmkernels as gk
+from gemmkernels import CTASwizzle, Kernel, Layout, Operator, NT, Float16, Float32, ConfigError, DimensionMismatch, _lib
+from gemmkernels import config as cfgmod
+from gemmkernels.matmul import create_config
+
+F16, F32 = Float16, Float32
+ACM, ARM = Layout.UnsafeAlignedColMajor, Layout.UnsafeAlignedRowMajor
+
+
+def test_heuristic_block_shape_reference_answers():
+    # reference src/config.jl:84-120 with Padded{.,8} FP16 A/B: C/D FP32 128x128x4 = 64 KiB, then
+    # K = 64: 136*64*2 + 72*128*2 = 35840 B fits, K = 128: 69632 B does not
+    pa, pb = Layout.Padded[ACM[F16], 8], Layout.Padded[ACM[F16], 8]
+    assert gk.heuristic_block_shape(pa, pb, ACM[F32], ACM[F32]) == NT(M=128, N=128, K=64)
+    # FP16 C/D: 256 x 128 x 2 = 64 KiB
+    assert gk.heuristic_block_shape(pa, pb, ACM[F16], ACM[F16]) == NT(M=256, N=128, K=64)
+    # row-major A pads the K extent instead (src/layout.jl:246)
+    assert gk.heuristic_block_shape(Layout.Padded[ARM[F16], 8], pb, ACM[F32], ACM[F32]) == NT(M=128, N=128, K=64)
+
+
+def test_physical_size():
+    # src/layout.jl:113, :194 / :152, :246 / :342-345 / :381-383
+    assert Layout.physical_size(Layout.Padded[ACM[F16], 8], NT(M=128, K=64)) == (136, 64)
+    assert Layout.physical_size(Layout.Padded[ARM[F16], 8], NT(M=128, K=64)) == (72, 128)
+    assert Layout.physical_size(ACM[F32], NT(M=128, N=128)) == (128, 128)
+    assert Layout.physical_size(Layout.SplitColMajor[F32], NT(M=64, N=64)) == (64, 64, 2)
+    assert Layout.physical_size(Layout.Padded[Layout.SplitRowMajor[F16], 8], NT(M=64, K=32)) == (40, 64, 2)
+    assert Layout.physical_size(Layout.Padded[Layout.SplitColMajor[F16], 8], NT(M=64, K=32)) == (72, 32, 2)
+
+
+def test_adjacent_elements_reference_answers():
+    # src/config.jl:124-134; the mem tiles of the reference's default 128x128x64 config with 32 lanes
+    assert gk.adjacent_elements(256, NT(M=128, K=64), True) == NT(M=128, K=2)
+    assert gk.adjacent_elements(256, NT(M=128, K=64), False) == NT(M=4, K=64)
+    assert gk.adjacent_elements(8, NT(M=128, K=64), True) == NT(M=8, K=1)
+    assert gk.adjacent_elements(8, NT(M=128, K=64), False) == NT(M=1, K=8)
+    assert gk.adjacent_elements(256, NT(K=64, N=128), True) == NT(K=64, N=4)
+    assert gk.adjacent_elements(128, NT(M=128, N=128), True) == NT(M=128, N=1)
+    assert gk.adjacent_elements(4, NT(M=128, N=128), True) == NT(M=4, N=1)
+
+
+def base_kwargs(M=4096, N=4096, K=4096, **kw):
+    d = dict(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAOp[32, 32, 16, F16, F32],
+             global_a_layout=ACM[F16], global_c_layout=ACM[F32])
+    d.update(kw)
+    return d
+
+
+def test_get_config_defaults_for_the_headline_problem():
+    conf = gk.get_config(**base_kwargs())
+    assert conf.block_shape == NT(M=256, N=256, K=64)
+    assert conf.warps_per_block == 8 and conf.compute_warp == NT(M=128, N=64, K=16)
+    assert conf.compute_op_shape == NT(M=32, N=32, K=16)
+    # 64-lane waves, 16 bytes per lane (src/config.jl:240-260 with 64 lanes)
+    assert conf.mem_a_warp == NT(M=256, K=2) and conf.mem_a_thread == NT(M=8, K=1)
+    assert conf.mem_b_warp == NT(K=64, N=8) and conf.mem_b_thread == NT(K=8, N=1)
+    assert conf.mem_cd_warp == NT(M=256, N=1) and conf.mem_cd_thread == NT(M=4, N=1)
+    assert conf.global_b_layout == conf.global_a_layout and conf.global_d_layout == conf.global_c_layout
+    assert conf.shared_a_layout == Layout.Padded[ACM[F16], 8]           # src/config.jl:191-194
+    assert conf.cta_swizzle == CTASwizzle.XCDAware[4]
+    assert Kernel.shmem_size(conf, Kernel.matmul_pipelined) == 2 * (256 * 64 * 2 + 256 * 64 * 2)
+    assert "block_shape:" in str(conf) and "(M = 256, N = 256, K = 64)" in str(conf)
+
+
+def test_default_block_shape_shrinks_to_fill_the_chip():
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=4096, N=4096, K=4096)) == NT(M=256, N=256, K=64)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=2048, N=2048, K=2048)) == NT(M=128, N=128, K=64)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=256, N=256, K=256)) == NT(M=64, N=64, K=32)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=4096, N=4096, K=2048 + 32)) == NT(M=64, N=64, K=32)
+
+
+ERROR_CASES = [
+    # (name, kwargs overrides, expected status)
+    ("block too small (src/config.jl:203-205)", dict(block_shape=NT(M=64, N=64, K=4), compute_warp=NT(M=32, N=32, K=16)), _lib.GK_ERR_BLOCK_SHAPE),
+    ("block < 2 x operator (src/config.jl:209-212)", dict(block_shape=NT(M=32, N=128, K=64), compute_warp=NT(M=32, N=32, K=16), warps_per_block=4), _lib.GK_ERR_BLOCK_SHAPE),
+    ("unsupported matrix-core shape (src/config.jl:159-169)", dict(operator=Operator.MFMAOp[16, 16, 4, F16, F32]), _lib.GK_ERR_OP_SHAPE),
+    ("FPU base shape is not one wave (src/config.jl:147-149)", dict(operator=Operator.FPUOp[8, 8, 1, 4, 8, 1, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
+    ("FPU kb != 1 (src/config.jl:151-153)", dict(operator=Operator.FPUOp[8, 8, 2, 8, 8, 2, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
+    ("FPU operator smaller than a wave (src/config.jl:142-145)", dict(operator=Operator.FPUOp[4, 8, 1, 4, 8, 1, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
+    ("FPU shape not a multiple of its base (src/config.jl:155-157)", dict(operator=Operator.FPUOp[12, 8, 1, 8, 8, 1, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
+    ("mem_a_warp too big (src/config.jl:263)", dict(block_shape=NT(M=128, N=128, K=64), mem_a_warp=NT(M=128, K=64)), _lib.GK_ERR_MEM_TILE),
+    ("mem_b_warp too big (src/config.jl:264)", dict(block_shape=NT(M=128, N=128, K=64), mem_b_warp=NT(K=64, N=128)), _lib.GK_ERR_MEM_TILE),
+    ("mem_cd_warp too big (src/config.jl:265)", dict(block_shape=NT(M=128, N=128, K=64), mem_cd_warp=NT(M=128, N=128)), _lib.GK_ERR_MEM_TILE),
+    ("block not a multiple of compute_warp (src/config.jl:270)", dict(block_shape=NT(M=128, N=128, K=64), compute_warp=NT(M=96, N=64, K=16)), _lib.GK_ERR_TILE_MULTIPLE),
+    ("compute_warp not a multiple of the operator (src/config.jl:271)", dict(block_shape=NT(M=128, N=128, K=64), compute_warp=NT(M=64, N=16, K=16), warps_per_block=16), _lib.GK_ERR_TILE_MULTIPLE),
+    ("gemm not a multiple of the block, aligned layouts (src/config.jl:272-275)", dict(gemm_shape=NT(M=1000, N=1024, K=1024), block_shape=NT(M=128, N=128, K=64)), _lib.GK_ERR_TILE_MULTIPLE),
+    ("no compiled instance", dict(block_shape=NT(M=192, N=192, K=64), compute_warp=NT(M=96, N=96, K=16), warps_per_block=4, gemm_shape=NT(M=384, N=384, K=128)), _lib.GK_ERR_UNSUPPORTED),
+    ("warps_per_block disagrees with block / compute_warp", dict(block_shape=NT(M=128, N=128, K=64), compute_warp=NT(M=64, N=64, K=16), warps_per_block=8), _lib.GK_ERR_UNSUPPORTED),
+]
+
+
+@pytest.mark.parametrize("name,over,status", ERROR_CASES, ids=[c[0] for c in ERROR_CASES])
+def test_config_errors(name, over, status):
+    with pytest.raises(ConfigError) as ei:
+        gk.get_config(**base_kwargs(**over))
+    assert ei.value.status == status, ei.value.message
+    assert len(ei.value.message) > 10
+
+
+def test_checked_layouts_lift_the_divisibility_rule():
+    # src/config.jl:175-178: Zero / ColMajor / RowMajor do not need tile-sized operands
+    with pytest.raises(ConfigError) as ei:
+        gk.get_config(**base_kwargs(M=1000, N=1000, K=1000, block_shape=NT(M=64, N=64, K=32),
+                                    global_a_layout=Layout.ColMajor[F16], global_b_layout=Layout.ColMajor[F16],
+                                    global_c_layout=Layout.ColMajor[F32], global_d_layout=ACM[F32]))
+    assert ei.value.status == _lib.GK_ERR_TILE_MULTIPLE      # D is still an aligned layout
+
+
+def test_lds_stage_and_thread_limits():
+    conf = gk.get_config(**base_kwargs())
+    try:
+        _lib.lib().gk_set_device_limits(64 * 1024, 0)          # src/matmul.jl:28-31
+        with pytest.raises(ConfigError) as ei:
+            gk.check_config(conf, Kernel.matmul_pipelined)
+        assert ei.value.status == _lib.GK_ERR_LDS and "shared memory" in ei.value.message
+        _lib.lib().gk_set_device_limits(0, 256)                # src/matmul.jl:41
+        with pytest.raises(ConfigError) as ei:
+            gk.check_config(conf, Kernel.matmul_pipelined)
+        assert ei.value.status == _lib.GK_ERR_THREADS
+    finally:
+        _lib.lib().gk_set_device_limits(0, 0)
+    gk.check_config(conf, Kernel.matmul_pipelined)
+    # src/matmul.jl:34-36: pipelined kernels need BLOCK_K >= 2 * OPERATOR_K; single-stage does not
+    kw = base_kwargs(block_shape=NT(M=64, N=64, K=16), compute_warp=NT(M=32, N=32, K=16), warps_per_block=4, kernel=Kernel.matmul_pipelined)
+    with pytest.raises(ConfigError) as ei:
+        gk.get_config(**kw)
+    assert ei.value.status == _lib.GK_ERR_STAGES
+
+
+def test_alignment_and_null_pointer_checks_happen_before_any_launch():
+    conf = gk.get_config(**base_kwargs(M=256, N=256, K=256, block_shape=NT(M=128, N=128, K=64)))
+    c = conf.to_c(256, 256, 256, 256)
+    lib = _lib.lib()
+    call = lambda a, b, cc, d: lib.gk_matmul(ctypes.byref(c), a, b, cc, d, None, None, Kernel.matmul_pipelined.code, None)
+    assert call(0x1008, 0x2000, 0x3000, 0x4000) == _lib.GK_ERR_ALIGNMENT and "A is not aligned" in _lib.last_error()
+    assert call(0x1000, 0x2000, 0x3000, 0x4004) == _lib.GK_ERR_ALIGNMENT
+    assert call(None, 0x2000, 0x3000, 0x4000) == _lib.GK_ERR_INVALID_ARGUMENT
+    assert call(0x1000, 0x2000, None, 0x4000) == _lib.GK_ERR_INVALID_ARGUMENT      # C is not Zero
+    c_bad = conf.to_c(260, 256, 256, 256)                                            # lda * 2 B not a multiple of 16
+    assert lib.gk_matmul(ctypes.byref(c_bad), 0x1000, 0x2000, 0x3000, 0x4000, None, None, 1, None) == _lib.GK_ERR_ALIGNMENT
+    c_small = conf.to_c(128, 256, 256, 256)                                          # lda < M
+    assert lib.gk_matmul(ctypes.byref(c_small), 0x1000, 0x2000, 0x3000, 0x4000, None, None, 1, None) == _lib.GK_ERR_DIMENSION_MISMATCH
+
+
+def test_create_config_choices():
+    # reference src/matmul.jl:66-183
+    args = (F16, (4096, 4096), (1, 4096), False, F16, (4096, 4096), (1, 4096), False, F32, (4096, 4096), (1, 4096), float, False, float, False, None)
+    conf, compute_type, kernel = create_config(*args)
+    assert compute_type == F16 and kernel == Kernel.matmul_pipelined
+    assert conf.operator.kind == Operator.MFMA and conf.block_shape == NT(M=256, N=256, K=64)
+    assert conf.global_a_layout == ACM[F16] and conf.global_c_layout == ACM[F32]
+    # transposed operands pick the row-major family and flip is_*_col_major (:79-83, :160-161)
+    conf, _, _ = create_config(F16, (4096, 4096), (1, 4096), True, F16, (4096, 4096), (1, 4096), True, F32, (4096, 4096), (1, 4096), float, False, float, False, None)
+    assert conf.global_a_layout == ARM[F16] and conf.global_b_layout == ARM[F16] and not conf.is_a_col_major
+    # beta == 0 elides the C load (:139-145)
+    conf, _, _ = create_config(F16, (4096, 4096), (1, 4096), False, F16, (4096, 4096), (1, 4096), False, F32, (4096, 4096), (1, 4096), float, False, float, True, None)
+    assert conf.global_c_layout == Layout.Zero[F32] and conf.shared_c_layout == Layout.Zero[F32]
+    with pytest.raises(DimensionMismatch):                                           # :75-77
+        create_config(F16, (128, 64), (1, 128), False, F16, (128, 128), (1, 128), False, F32, (128, 128), (1, 128), float, False, float, False, None)

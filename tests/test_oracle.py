@@ -1,0 +1,221 @@
+"""Pins the CPU oracle (the C restatement in oracle/gk_oracle.c) before it is trusted as the
+checker: conversions against numpy, GEMM against float64 matmul and pure-Python brute force,
+closed forms, layouts with index-distinct values, transform and epilogue order."""
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import oracle
+from oracle.oracle import F16, BF16, F32, F64, Layout, Problem
+
+
+def test_half_conversions_match_numpy_exhaustively():
+    lib = oracle.lib()
+    bits = np.arange(65536, dtype=np.uint16)
+    ref = bits.view(np.float16).astype(np.float32)
+    got = np.array([lib.gko_half_to_float(int(b)) for b in bits], dtype=np.float32)
+    finite = np.isfinite(ref)
+    assert np.array_equal(got[finite], ref[finite]) and np.isnan(got[~finite & np.isnan(ref)]).all()
+    rs = np.random.RandomState(0)
+    xs = np.concatenate([rs.standard_normal(20000), rs.standard_normal(5000) * 1e-6, rs.standard_normal(5000) * 7e4,
+                         np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 2.0 ** -24, 2.0 ** -25, 3 * 2.0 ** -25, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11])])
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).view(np.uint16)
+    have = np.array([lib.gko_double_to_half(float(x)) for x in xs], dtype=np.uint16)
+    assert np.array_equal(have, want)
+
+
+def plain(M, N, K, ta=False, tb=False, dt=F16, cd=F32, zero_c=False, **kw):
+    a = Layout(oracle.L_ROW if ta else oracle.L_COL, dt, K if ta else M)
+    b = Layout(oracle.L_ROW if tb else oracle.L_COL, dt, N if tb else K)
+    c = Layout(oracle.L_ZERO, cd) if zero_c else Layout(oracle.L_COL, cd, M)
+    return Problem(M, N, K, a, b, c, Layout(oracle.L_COL, cd, M), compute_dtype=dt, accum_dtype=cd, **kw)
+
+
+def rand(shape, dtype, seed):
+    rs = np.random.RandomState(seed)
+    return np.asfortranarray((rs.randint(-1024, 1024, size=shape) / 1024.0).astype(dtype))
+
+
+@pytest.mark.parametrize("ta,tb", list(itertools.product([False, True], repeat=2)))
+def test_gemm_against_float64_and_brute_force(ta, tb):
+    M, N, K = 7, 5, 9
+    a = rand((K, M) if ta else (M, K), np.float16, 1)
+    b = rand((N, K) if tb else (K, N), np.float16, 2)
+    c = rand((M, N), np.float32, 3)
+    d = np.zeros((M, N), np.float32, order="F")
+    oracle.matmul(plain(M, N, K, ta, tb), a, b, c, d)
+    # pure-Python triple loop, float64 (products and partial sums of these dyadic inputs are exact)
+    A = a.T if ta else a
+    B = b.T if tb else b
+    want = np.zeros((M, N))
+    for i in range(M):
+        for j in range(N):
+            s = float(c[i, j])
+            for k in range(K):
+                s += float(A[i, k]) * float(B[k, j])
+            want[i, j] = s
+    assert np.array_equal(d.astype(np.float64), want)          # exact: sums of multiples of 2^-20 below 2^24
+    assert np.array_equal(want, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb))
+
+
+def test_gemm_medium_against_float64_both_accumulators():
+    M, N, K = 96, 80, 200
+    a, b, c = rand((M, K), np.float16, 4), rand((K, N), np.float16, 5), rand((M, N), np.float32, 6)
+    d = np.zeros((M, N), np.float32, order="F")
+    oracle.matmul(plain(M, N, K), a, b, c, d)
+    ref = oracle.gemm_f64(a, b, c, 1.0, 1.0)
+    assert oracle.rel_frobenius(d, ref) < 1e-6
+    oracle.matmul(plain(M, N, K), a, b, c, d, wide_accum=True)
+    assert np.array_equal(d, ref.astype(np.float32))
+
+
+def test_closed_forms():
+    n = 16
+    eye = np.asfortranarray(np.eye(n, dtype=np.float16))
+    b, c = rand((n, n), np.float16, 7), rand((n, n), np.float32, 8)
+    d = np.zeros((n, n), np.float32, order="F")
+    oracle.matmul(plain(n, n, n), eye, b, c, d)
+    assert np.array_equal(d, b.astype(np.float32) + c)                       # A = I
+    ones = np.asfortranarray(np.ones((n, n), np.float16))
+    oracle.matmul(plain(n, n, n, zero_c=True), ones, ones, None, d)
+    assert np.array_equal(d, np.full((n, n), float(n), np.float32))          # all ones => K
+    a1 = np.zeros((n, n), np.float16, order="F"); a1[3, 5] = 2.0
+    b1 = np.zeros((n, n), np.float16, order="F"); b1[5, 11] = 0.25
+    oracle.matmul(plain(n, n, n, zero_c=True), a1, b1, None, d)
+    want = np.zeros((n, n), np.float32); want[3, 11] = 0.5
+    assert np.array_equal(d, want)                                           # single non-zero
+
+
+def test_layout_index_maps_with_distinct_values():
+    """Each element carries a distinct value, so a swapped index or a wrong leading dimension moves
+    a known number to a wrong place."""
+    M, K = 3, 4
+    vals = np.arange(1, 1 + 5 * 6, dtype=np.float32)
+    buf = np.asfortranarray(vals.reshape((5, 6), order="F"))                 # ld = 5 > M
+    one = np.asfortranarray(np.eye(K, dtype=np.float32))
+    d = np.zeros((M, K), np.float32, order="F")
+    p = Problem(M, K, K, Layout(oracle.L_COL, F32, 5), Layout(oracle.L_COL, F32, K), Layout(oracle.L_ZERO, F32),
+                Layout(oracle.L_COL, F32, M), compute_dtype=F32, accum_dtype=F32)
+    oracle.matmul(p, buf, one, None, d)
+    assert np.array_equal(d, buf[:M, :K])                                    # (r, c) at p[r + c*ld]
+    p.a = Layout(oracle.L_ROW, F32, 5)
+    oracle.matmul(p, buf, one, None, d)
+    assert np.array_equal(d, buf[:K, :M].T)                                  # (r, c) at p[c + r*ld]
+    diag = np.array([2, 3, 5, 7], np.float32)
+    p2 = Problem(K, K, K, Layout(oracle.L_DIAG, F32), Layout(oracle.L_COL, F32, K), Layout(oracle.L_ZERO, F32),
+                 Layout(oracle.L_COL, F32, K), compute_dtype=F32, accum_dtype=F32)
+    bb = np.asfortranarray(np.arange(1, 17, dtype=np.float32).reshape((4, 4), order="F"))
+    d2 = np.zeros((K, K), np.float32, order="F")
+    oracle.matmul(p2, diag, bb, None, d2)
+    assert np.array_equal(d2, np.diag(diag) @ bb)                            # reference src/layout.jl:225-236
+
+
+def test_gett_index_map_against_einsum_with_primes():
+    """D[a,b,c,d] = sum_{e,f} A[a,e,b,f] * B[d,f,c,e] with distinct extents and prime values."""
+    ea, eb, ec, ed, ee, ef = 2, 3, 2, 2, 3, 2
+    rs = np.random.RandomState(9)
+    primes = np.array([2, 3, 5, 7, 11, 13, 17, 19, 23, 29, 31], np.float32)
+    A = np.asfortranarray(rs.choice(primes, size=(ea, ee, eb, ef)).astype(np.float32))
+    B = np.asfortranarray(rs.choice(primes, size=(ed, ef, ec, ee)).astype(np.float32))
+    sA, sB = [s // 4 for s in A.strides], [s // 4 for s in B.strides]
+    M, N, K = ea * eb, ec * ed, ee * ef
+    D = np.zeros((ea, eb, ec, ed), np.float32, order="F")
+    sD = [s // 4 for s in D.strides]
+    la = Layout(oracle.L_GETT, F32, 0, [(ea, sA[0]), (eb, sA[2])], [(ee, sA[1]), (ef, sA[3])])     # rows m=(a,b), cols k=(e,f)
+    lb = Layout(oracle.L_GETT, F32, 0, [(ee, sB[3]), (ef, sB[1])], [(ec, sB[2]), (ed, sB[0])])     # rows k=(e,f), cols n=(c,d)
+    ld = Layout(oracle.L_GETT, F32, 0, [(ea, sD[0]), (eb, sD[1])], [(ec, sD[2]), (ed, sD[3])])
+    p = Problem(M, N, K, la, lb, Layout(oracle.L_ZERO, F32), ld, compute_dtype=F32, accum_dtype=F32)
+    oracle.matmul(p, A, B, None, D)
+    want = np.einsum("aebf,dfce->abcd", A.astype(np.float64), B.astype(np.float64))
+    assert np.array_equal(D.astype(np.float64), want)
+
+
+def test_transform_order_rounding_points_and_bias():
+    """gl2sh result is rounded to the shared type, sh2rf to the compute type, the bias is added
+    before the last transform (reference src/epilogue.jl:67-70)."""
+    M = N = K = 4
+    a = np.asfortranarray(np.full((M, K), 1.0 + 2.0 ** -10, np.float16))     # 1 + ulp
+    b = np.asfortranarray(np.eye(K, dtype=np.float16))
+    d = np.zeros((M, N), np.float32, order="F")
+    p = plain(M, N, K, zero_c=True, transforms={"global_to_shared_a": [(oracle.T_SCALE, 0.75, 0.0)],
+                                                "shared_to_regs_a": [(oracle.T_SCALE, 4.0, 0.0)]})
+    oracle.matmul(p, a, b, None, d)
+    step1 = np.float16(np.float32(a[0, 0]) * np.float32(0.75))              # rounded to FP16 in LDS
+    assert d[0, 0] == np.float32(np.float16(np.float32(step1) * np.float32(4.0)))
+    assert d[0, 0] != np.float32(np.float32(a[0, 0]) * np.float32(3.0))      # a fused 3x would differ
+    bias = np.array([1.0, -2.0, 3.0, -4.0], np.float32)
+    p = plain(M, N, K, zero_c=True, transforms={"shared_to_global_d": [(oracle.T_RELU, 0.0, 0.0)]}, epilogue=oracle.EPI_BIAS_COL, bias=bias)
+    zero = np.zeros((M, K), np.float16, order="F")
+    oracle.matmul(p, zero, b, None, d)
+    assert np.array_equal(d, np.broadcast_to(np.maximum(bias, 0)[None, :], (M, N)))
+    p.epilogue = oracle.EPI_BIAS_ROW
+    oracle.matmul(p, zero, b, None, d)
+    assert np.array_equal(d, np.broadcast_to(np.maximum(bias, 0)[:, None], (M, N)))
+    # relu before the bias (regs_to_shared_d) is a different function: relu(0) + bias = bias
+    p = plain(M, N, K, zero_c=True, transforms={"regs_to_shared_d": [(oracle.T_RELU, 0.0, 0.0)]}, epilogue=oracle.EPI_BIAS_COL, bias=bias)
+    oracle.matmul(p, zero, b, None, d)
+    assert np.array_equal(d, np.broadcast_to(bias[None, :], (M, N)))
+
+
+def test_alpha_beta_linearity_and_c_alias():
+    M, N, K = 12, 10, 14
+    a, b, c = rand((M, K), np.float16, 10), rand((K, N), np.float16, 11), rand((M, N), np.float32, 12)
+    tr = {"shared_to_regs_a": [(oracle.T_SCALE, 2.0, 0.0)], "shared_to_regs_c": [(oracle.T_SCALE, 3.0, 0.0)]}
+    cc = c.copy(order="F")
+    oracle.matmul(plain(M, N, K, transforms=tr), a, b, cc, cc)               # d aliases c
+    assert np.array_equal(cc.astype(np.float64), oracle.gemm_f64(a, b, c, 2.0, 3.0))
+
+
+def test_fp32_fma_chain_is_sequential_in_k():
+    """FPUOp.mma is a scalar fma chain in ascending k (reference src/operator.jl:139-153)."""
+    K = 64
+    rs = np.random.RandomState(13)
+    a = np.asfortranarray(rs.standard_normal((1, K)).astype(np.float32))
+    b = np.asfortranarray(rs.standard_normal((K, 1)).astype(np.float32))
+    d = np.zeros((1, 1), np.float32, order="F")
+    oracle.matmul(plain(1, 1, K, dt=F32, zero_c=True), a, b, None, d)
+    acc = np.float64(0.0)
+    for k in range(K):   # fma in float32 == round(float64 exact product + acc) for float32 inputs (product exact in f64)
+        acc = np.float64(np.float32(np.float64(a[0, k]) * np.float64(b[k, 0]) + acc))
+    assert d[0, 0] == np.float32(acc)
+
+
+def test_complex_against_numpy_and_identities():
+    M, N, K = 6, 5, 8
+    rs = np.random.RandomState(14)
+    def cplx(shape):
+        return np.asfortranarray((rs.randint(-512, 512, size=shape + (2,)) / 512.0).astype(np.float16))
+    a, b = cplx((M, K)), cplx((K, N))
+    az = a[..., 0].astype(np.float64) + 1j * a[..., 1].astype(np.float64)
+    bz = b[..., 0].astype(np.float64) + 1j * b[..., 1].astype(np.float64)
+    def inter(x):   # (rows, cols, 2) logical -> interleaved col-major buffer
+        return np.ascontiguousarray(np.transpose(x, (1, 0, 2)))          # memory: col, row, (re, im)
+    p = Problem(M, N, K, Layout(oracle.L_ICOL, F16, M), Layout(oracle.L_ICOL, F16, K), Layout(oracle.L_ZERO, F32),
+                Layout(oracle.L_ICOL, F32, M), compute_dtype=F16, accum_dtype=F32, op_kind=oracle.OP_COMPLEX)
+    d = np.zeros((N, M, 2), np.float32)
+    oracle.matmul(p, inter(a), inter(b), None, d)
+    got = (d[..., 0] + 1j * d[..., 1]).T
+    assert np.allclose(got, az @ bz, rtol=0, atol=1e-5)
+    # real inputs => imaginary part exactly zero
+    a0 = a.copy(); a0[..., 1] = 0
+    b0 = b.copy(); b0[..., 1] = 0
+    oracle.matmul(p, inter(a0), inter(b0), None, d)
+    assert np.all(d[..., 1] == 0)
+    # B = i * I  =>  A * B = (-im(A), re(A))
+    bi = np.zeros((K, K, 2), np.float16); bi[np.arange(K), np.arange(K), 1] = 1
+    p2 = Problem(M, K, K, Layout(oracle.L_ICOL, F16, M), Layout(oracle.L_ICOL, F16, K), Layout(oracle.L_ZERO, F32),
+                 Layout(oracle.L_ICOL, F32, M), compute_dtype=F16, accum_dtype=F32, op_kind=oracle.OP_COMPLEX)
+    d2 = np.zeros((K, M, 2), np.float32)
+    oracle.matmul(p2, inter(a), inter(bi), None, d2)
+    assert np.array_equal(d2[..., 0].T, -a[..., 1].astype(np.float32)) and np.array_equal(d2[..., 1].T, a[..., 0].astype(np.float32))
+
+
+def test_tropical_and_dual():
+    M, N, K = 5, 4, 6
+    a, b, c = rand((M, K), np.float32, 15), rand((K, N), np.float32, 16), rand((M, N), np.float32, 17)
+    d = np.zeros((M, N), np.float32, order="F")
+    oracle.matmul(plain(M, N, K, dt=F32, op_kind=oracle.OP_TROPICAL), a, b, c, d)
+    want = np.maximum(c, (a[:, :, None] + b[None, :, :]).max(axis=1))      # max-plus product (reference configs/configs.jl:226)
+    assert np.array_equal(d, want)
