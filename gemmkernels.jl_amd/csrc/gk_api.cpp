@@ -96,7 +96,7 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
     case GK_OP_FPU:
     case GK_OP_FPU_TROPICAL:
       key->family = gk::FAMILY_FPU;
-      key->variant = (c->op.kind == GK_OP_FPU_TROPICAL) ? 1 : 0;
+      key->variant = ((c->op.kind == GK_OP_FPU_TROPICAL) ? 1 : 0) + (any_checked ? 2 : 0);
       break;
     case GK_OP_MFMA_COMPLEX:
     case GK_OP_MFMA_DUAL:
@@ -175,6 +175,10 @@ gk::FamilyFn family_fn(const gk::InstanceKey& key) {
     case gk::FAMILY_MFMA:
       if (key.a_kmajor) return key.b_kmajor ? gk::family_mfma_tn : gk::family_mfma_tt;
       return key.b_kmajor ? gk::family_mfma_nn : gk::family_mfma_nt;
+    case gk::FAMILY_FPU:
+      return gk::family_fpu;
+    case gk::FAMILY_MFMA_CHECKED:
+      return gk::family_mfma_checked;
     default:
       return nullptr;
   }

@@ -162,9 +162,20 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
     return NT(M=fitting[-1][0], N=fitting[-1][1], K=fitting[-1][2])
 
 
-def _default_waves(operator, block_shape):
+# tiles of the vector-ALU kernel and of the bounds-checked MFMA kernel
+_FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2))]
+_CHECKED_TILES = [((64, 64, 32), (2, 2))]
+
+
+def _default_waves(operator, block_shape, checked=False):
     key = (block_shape["M"], block_shape["N"], block_shape["K"])
-    for t, w in _MFMA_TILES:
+    if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
+        table = _FPU_TILES
+    elif operator.kind == Operator.MFMA and checked:
+        table = _CHECKED_TILES
+    else:
+        table = _MFMA_TILES
+    for t, w in table:
         if t == key:
             return w
     return None
@@ -196,8 +207,8 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
     block_shape = default_block_shape(operator, gemm_shape, tile_sized) if block_shape is None else NT(block_shape)
     op_shape = Operator.shape(operator)
 
-    is_mfma = operator.kind in (Operator.MFMA, Operator.MFMA_COMPLEX, Operator.MFMA_DUAL)
-    waves = _default_waves(operator, block_shape) if is_mfma else None
+    checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
+    waves = _default_waves(operator, block_shape, checked)
     if waves is not None:
         warps_default = waves[0] * waves[1]
         compute_warp_default = NT(M=block_shape.M // waves[0], N=block_shape.N // waves[1], K=op_shape.K)

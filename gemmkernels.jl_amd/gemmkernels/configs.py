@@ -133,6 +133,35 @@ def _config3() -> Workload:
         kernel_name=kernel_name(conf, Kernel.matmul_pipelined, transforms, Epilogue.Bias(0)))
 
 
+def _config1() -> Workload:
+    M = N = K = 256
+    from .matmul import create_config
+    from .dtypes import Float32 as F32
+
+    def host():
+        return dict(a=rng.matrix("u01_f32", 1001, (M, K)), b=rng.matrix("u01_f32", 1002, (K, N)), c=None)
+
+    conf, _, kern = create_config(F32, (M, K), (1, M), False, F32, (K, N), (1, K), False, F32, (M, N), (1, M),
+                                  bool, False, bool, True, None)
+
+    def launch(h):
+        import torch
+        from .matmul import mul_
+        a, b = colmajor(h["a"]), colmajor(h["b"])
+        d = colmajor_empty((M, N), torch.float32)
+        d.zero_()
+
+        def run():
+            mul_(d, a, b)             # mul!(C, A, B): alpha = 1, beta = 0  =>  FPUOp, C as Layout.Zero
+        return _attach(run, a=a, b=b, d=d, conf=conf)
+
+    return Workload(
+        name="config 1",
+        description="config 1: C = A*B through mul!, FP32, M=N=K=256, column-major NN, A,B ~ U[0,1), beta = 0 (FPUOp on the vector ALUs)",
+        flops=2 * M * N * K, bytes=3 * M * N * 4, bound="latency", make_host=host, make_launch=launch,
+        kernel_name=kernel_name(conf, kern))
+
+
 def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     """The benchmark workloads 1, 2 (variant NN/NT/TN/TT), 3, "4a", "4b", 5."""
     if n == 2:
@@ -145,4 +174,4 @@ def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     raise NotImplementedError(f"benchmark config {n}")
 
 
-_LATE_BUILDERS = {}
+_LATE_BUILDERS = {1: _config1}

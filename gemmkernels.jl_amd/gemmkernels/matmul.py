@@ -171,21 +171,30 @@ def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stri
         operator = Operator.MFMAOp[32, 32, 16, compute_type, Float32 if C == Float16 else C]
     else:
         operator = Operator.FPUOp[8, 8, 1, 8, 8, 1, compute_type, C]
-    block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=True)
-
     a_aligned = (stridesA[1] * A.size) % 16 == 0
     b_aligned = (stridesB[1] * B.size) % 16 == 0
     c_aligned = (stridesC[1] * C.size) % 16 == 0
-    if zeroAlpha:
-        global_a_layout, global_b_layout = Layout.Zero[A], Layout.Zero[B]
-    else:
-        global_a_layout = (a_aligned_layout_base[A] if a_aligned and m % block_shape.M == 0 and k % block_shape.K == 0
-                           else a_layout_base[A])
-        global_b_layout = (b_aligned_layout_base[B] if b_aligned and k % block_shape.K == 0 and n % block_shape.N == 0
-                           else b_layout_base[B])
-    cd_aligned = c_aligned and m % block_shape.M == 0 and n % block_shape.N == 0
-    global_c_layout = Layout.Zero[C] if zeroBeta else (Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C])
-    global_d_layout = Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C]
+
+    def layouts_for(block_shape):
+        # src/matmul.jl:121-156: vector loads and stores need 16-byte aligned columns and whole tiles
+        if zeroAlpha:
+            ga, gb = Layout.Zero[A], Layout.Zero[B]
+        else:
+            ga = (a_aligned_layout_base[A] if a_aligned and m % block_shape.M == 0 and k % block_shape.K == 0
+                  else a_layout_base[A])
+            gb = (b_aligned_layout_base[B] if b_aligned and k % block_shape.K == 0 and n % block_shape.N == 0
+                  else b_layout_base[B])
+        cd_aligned = c_aligned and m % block_shape.M == 0 and n % block_shape.N == 0
+        gc = Layout.Zero[C] if zeroBeta else (Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C])
+        gd = Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C]
+        return ga, gb, gc, gd
+
+    block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=True)
+    global_a_layout, global_b_layout, global_c_layout, global_d_layout = layouts_for(block_shape)
+    if any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout)):
+        # some operand needs bounds checks: the bounds-checked kernels have one tile shape
+        block_shape = NT(M=64, N=64, K=32)
+        global_a_layout, global_b_layout, global_c_layout, global_d_layout = layouts_for(block_shape)
 
     conf = _get_config(gemm_shape=NT(M=m, N=n, K=k), block_shape=block_shape, operator=operator,
                        global_a_layout=global_a_layout, global_b_layout=global_b_layout,

@@ -1,0 +1,96 @@
+"""GPU parity of the BLAS-like entry points (matmatmul_ / mul_), in the manner of the reference's
+test/blas.jl:11-68: sizes that are not multiples of any tile (10, 1000) next to 128 / 256, all four
+transposes, random alpha and beta, the matrix cores for FP16 inputs and the vector ALUs for FP32."""
+import numpy as np
+import pytest
+import torch
+
+import gemmkernels as gk
+from gemmkernels import Transpose, configs, rng
+from gemmkernels.matmul import create_config
+from gemmkernels.dtypes import Float16, Float32
+import helpers
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def operands(M, N, K, ta, tb, dtype, seed):
+    kind = "upm1_f16" if dtype == np.float16 else "upm1_f32"
+    a = rng.matrix(kind, seed + 1, (K, M) if ta else (M, K)).astype(dtype)
+    b = rng.matrix(kind, seed + 2, (N, K) if tb else (K, N)).astype(dtype)
+    c = rng.matrix("upm1_f32", seed + 3, (M, N))
+    return a, b, c
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims", [(10, 10, 10), (128, 128, 128), (256, 256, 256), (1000, 1000, 1000), (10, 1000, 256), (130, 70, 33)])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_matmatmul(gpu, dims, ta, tb, dtype):
+    M, N, K = dims
+    a, b, c = operands(M, N, K, ta == "T", tb == "T", dtype, 100)
+    rs = np.random.RandomState(M + N)
+    alpha, beta = float(np.float16(rs.rand())), float(np.float32(rs.rand()))      # reference test/blas.jl:22-23
+    A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
+    print("case", dims, ta, tb, dtype.__name__, flush=True)
+    gk.matmatmul_(C, ta, tb, A, B, alpha, beta)
+    torch.cuda.synchronize()
+    ref = oracle.gemm_f64(a, b, c, alpha, beta, ta == "T", tb == "T")
+    err = oracle.rel_frobenius(gk.to_numpy(C), ref)
+    # FP16: alpha is applied to A in FP16 like the reference does (src/matmul.jl:196-199), which
+    # rounds every scaled element: 2^-11 relative per element, averaged down by the sum
+    assert err <= (1e-3 if dtype == np.float16 else 1e-5), err
+
+
+def test_fp32_is_bit_exact_against_the_sequential_fma_chain(gpu):
+    """FPUOp semantics: one fp32 fma per k in ascending order (reference src/operator.jl:139-153);
+    the oracle's C restatement is that loop, so the results must be identical."""
+    for (M, N, K, ta, tb) in [(256, 256, 256, False, False), (64, 192, 96, True, False), (100, 36, 50, False, True), (77, 65, 129, True, True)]:
+        a, b, c = operands(M, N, K, ta, tb, np.float32, 7)
+        sa, sb = a.shape, b.shape
+        conf, _, kern = create_config(Float32, sa, (1, sa[0]), ta, Float32, sb, (1, sb[0]), tb, Float32, (M, N), (1, M),
+                                      float, False, float, False, None)
+        d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=kern)
+        ref = helpers.run_oracle(conf, a, b, c, (M, N))
+        assert np.array_equal(d, ref), (M, N, K, ta, tb)
+
+
+def test_mul_wrappers_and_zero_alpha(gpu):
+    M, N, K = 128, 64, 96
+    a, b, c = operands(M, N, K, True, False, np.float16, 9)
+    A, B = gk.colmajor(a), gk.colmajor(b)
+    C = gk.colmajor(np.asfortranarray(np.full((M, N), np.nan, np.float32)))
+    gk.mul_(C, Transpose(A), B)                           # alpha = true, beta = false: C is never read
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(gk.to_numpy(C), oracle.gemm_f64(a, b, None, 1.0, 0.0, True, False)) <= 1e-3
+    C = gk.colmajor(c)
+    gk.matmatmul_(C, "T", "N", A, B, 0.0, 2.0)            # alpha = 0: A and B are Layout.Zero, C = 2 C exactly
+    torch.cuda.synchronize()
+    assert np.array_equal(gk.to_numpy(C), 2.0 * c)
+    with pytest.raises(gk.DimensionMismatch):
+        gk.matmatmul_(C, "N", "N", A, B, 1.0, 0.0)
+
+
+def test_tropical(gpu):
+    """max-plus product on the vector ALUs (reference src/operator.jl:134-137, configs/configs.jl:209-244)."""
+    from gemmkernels import Layout, Operator, Kernel, NT
+    M, N, K = 128, 128, 64
+    a, b, c = operands(M, N, K, False, False, np.float32, 11)
+    conf = gk.get_config(gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=64, N=64, K=32),
+                         operator=Operator.TropicalFPUOp[8, 8, 1, 8, 8, 1, Float32, Float32],
+                         global_a_layout=Layout.UnsafeAlignedColMajor[Float32], global_c_layout=Layout.UnsafeAlignedColMajor[Float32])
+    d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    want = np.maximum(c, (a[:, :, None] + b[None, :, :]).max(axis=1))
+    assert np.array_equal(d, want)
+
+
+def test_config1_benchmark_workload(gpu):
+    w = configs.benchmark_config(1)
+    run = w.prepare()
+    run()
+    torch.cuda.synchronize()
+    h = w.host()
+    d = gk.to_numpy(run.d)
+    assert oracle.rel_frobenius(d, oracle.gemm_f64(h["a"], h["b"], None)) <= 1e-5
+    conf = run.conf
+    assert np.array_equal(d, helpers.run_oracle(conf, h["a"], h["b"], None, (256, 256)))
