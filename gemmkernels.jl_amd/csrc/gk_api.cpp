@@ -114,6 +114,12 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   key->waves_n = c->block_shape.N / c->compute_warp.N;
   key->a_kmajor = is_row_major(ak) ? 1 : 0;    // 'T' A: stored K x M, K contiguous
   key->b_kmajor = is_row_major(bk) ? 0 : 1;    // 'N' B: stored K x N, K contiguous
+  if (key->family == gk::FAMILY_GETT) {
+    // the contiguous tensor mode decides which LDS tile layout an operand gets
+    key->a_kmajor = (c->gett.k.stride0[0] == 1) ? 1 : 0;
+    key->b_kmajor = (c->gett.k.stride1[0] == 1) ? 1 : 0;
+    key->variant = 1;
+  }
   key->dtype = c->global_a_layout.eltype;
   key->fused = (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT)) ? 1 : 0;
   return GK_OK;
@@ -173,6 +179,7 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
 gk::FamilyFn family_fn(const gk::InstanceKey& key) {
   switch (key.family) {
     case gk::FAMILY_MFMA:
+    case gk::FAMILY_GETT:
       if (key.a_kmajor) return key.b_kmajor ? gk::family_mfma_tn : gk::family_mfma_tt;
       return key.b_kmajor ? gk::family_mfma_nn : gk::family_mfma_nt;
     case gk::FAMILY_FPU:
@@ -197,6 +204,47 @@ int find_instance(const gk_config* c, const gk_transforms* t, const gk_epilogue*
                 c->op.kind, key->BM, key->BN, key->BK, key->waves_m, key->waves_n, c->global_a_layout.kind,
                 c->global_b_layout.kind, key->dtype);
   }
+  return GK_OK;
+}
+
+// Tensor-contraction index maps: what the GETT loader assumes about the mode tables.
+int validate_gett(const gk_config* c) {
+  const gk_gett& g = c->gett;
+  if (c->op.kind != GK_OP_MFMA) return fail(GK_ERR_UNSUPPORTED, "tensor-contraction layouts need the MFMA operator");
+  if (c->global_a_layout.kind != GK_LAYOUT_GETT || c->global_b_layout.kind != GK_LAYOUT_GETT ||
+      c->global_d_layout.kind != GK_LAYOUT_GETT ||
+      (c->global_c_layout.kind != GK_LAYOUT_GETT && c->global_c_layout.kind != GK_LAYOUT_ZERO))
+    return fail(GK_ERR_UNSUPPORTED, "a tensor contraction needs GETT layouts for A, B and D (C: GETT or Zero)");
+  const gk_gett_dim* dims[3] = {&g.m, &g.n, &g.k};
+  const int want[3] = {c->matmul_shape.M, c->matmul_shape.N, c->matmul_shape.K};
+  const char* names[3] = {"M", "N", "K"};
+  long long span[3] = {0, 0, 0};   // largest element offset in A, B, D
+  for (int d = 0; d < 3; ++d) {
+    if (dims[d]->nmodes < 1 || dims[d]->nmodes > GK_MAX_MODES) return fail(GK_ERR_INVALID_ARGUMENT, "%s needs 1..%d tensor modes", names[d], GK_MAX_MODES);
+    long long prod = 1;
+    for (int i = 0; i < dims[d]->nmodes; ++i) {
+      if (dims[d]->extent[i] <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "mode extents must be positive");
+      prod *= dims[d]->extent[i];
+      const long long e1 = dims[d]->extent[i] - 1;
+      if (d == 0) { span[0] += e1 * dims[d]->stride0[i]; span[2] += e1 * dims[d]->stride1[i]; }
+      if (d == 1) { span[1] += e1 * dims[d]->stride0[i]; span[2] += e1 * dims[d]->stride1[i]; }
+      if (d == 2) { span[0] += e1 * dims[d]->stride0[i]; span[1] += e1 * dims[d]->stride1[i]; }
+    }
+    if (prod != want[d]) return fail(GK_ERR_DIMENSION_MISMATCH, "the extents of the %s modes multiply to %lld, matmul_shape.%s is %d", names[d], prod, names[d], want[d]);
+  }
+  if (span[0] * 2 >= (1ll << 31) || span[1] * 2 >= (1ll << 31)) return fail(GK_ERR_UNSUPPORTED, "tensor too large for 32-bit tile offsets");
+  if (g.k.extent[0] % c->block_shape.K != 0)
+    return fail(GK_ERR_TILE_MULTIPLE, "BLOCK_K = %d must divide the extent %d of the first K mode", c->block_shape.K, g.k.extent[0]);
+  if (g.m.extent[0] % 32 != 0 || g.n.extent[0] % 32 != 0)
+    return fail(GK_ERR_TILE_MULTIPLE, "the first M mode and the first N mode must have extents that are multiples of 32");
+  // 16-byte vectors: one mode of each operand is contiguous and every other stride keeps the alignment
+  const bool a_k = g.k.stride0[0] == 1, b_k = g.k.stride1[0] == 1;
+  if (!a_k && g.m.stride0[0] != 1) return fail(GK_ERR_ALIGNMENT, "A must be contiguous along its first M mode or its first K mode");
+  if (!b_k && g.n.stride0[0] != 1) return fail(GK_ERR_ALIGNMENT, "B must be contiguous along its first N mode or its first K mode");
+  for (int i = 0; i < g.m.nmodes; ++i) if (!(i == 0 && !a_k) && g.m.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of M mode %d of A is not a multiple of 16 bytes", i);
+  for (int i = 0; i < g.k.nmodes; ++i) if (!(i == 0 && a_k) && g.k.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of K mode %d of A is not a multiple of 16 bytes", i);
+  for (int i = 0; i < g.n.nmodes; ++i) if (!(i == 0 && !b_k) && g.n.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of N mode %d of B is not a multiple of 16 bytes", i);
+  for (int i = 0; i < g.k.nmodes; ++i) if (!(i == 0 && b_k) && g.k.stride1[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of K mode %d of B is not a multiple of 16 bytes", i);
   return GK_OK;
 }
 
@@ -269,6 +317,12 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
     return fail(GK_ERR_TILE_MULTIPLE, "gemm_shape.MN must be a multiple of block_shape.MN!");
   if (require_tile_sized_global(c->global_d_layout.kind) && (g.M % b.M || g.N % b.N))
     return fail(GK_ERR_TILE_MULTIPLE, "gemm_shape.MN must be a multiple of block_shape.MN!");
+
+  if (c->global_a_layout.kind == GK_LAYOUT_GETT || c->global_b_layout.kind == GK_LAYOUT_GETT ||
+      c->global_c_layout.kind == GK_LAYOUT_GETT || c->global_d_layout.kind == GK_LAYOUT_GETT) {
+    int rc_g = validate_gett(c);
+    if (rc_g != GK_OK) return rc_g;
+  }
 
   // src/matmul.jl:34-36 (decidable from the configuration alone, so it is checked before the
   // instance lookup)
@@ -419,6 +473,9 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   if ((rc = check_aligned(conf->global_b_layout, b, args.ldb, "B")) != GK_OK) return rc;
   if ((rc = check_aligned(conf->global_c_layout, c, args.ldc, "C")) != GK_OK) return rc;
   if ((rc = check_aligned(conf->global_d_layout, d, args.ldd, "D")) != GK_OK) return rc;
+
+  if (key.family == gk::FAMILY_GETT && ((((uintptr_t)a | (uintptr_t)b) & 15u) != 0))
+    return fail(GK_ERR_ALIGNMENT, "tensor operands must be aligned to 16 bytes");
 
   // leading dimensions must cover the operand
   {

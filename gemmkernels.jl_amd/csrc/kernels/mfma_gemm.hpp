@@ -46,23 +46,60 @@ struct TileGeom {
   static_assert(BYTES % 1024 == 0, "tile must be a whole number of DMA instructions");
 };
 
-// Byte offset (from the tile's global origin) that lane `lane` of DMA instruction q fetches, and
-// which lands at LDS chunk position q*64 + lane.
+// Tile-local coordinates (row r, first k) of the 8 elements that lane `lane` of DMA instruction q
+// fetches; they land at LDS chunk position q*64 + lane.
 template <int R, int BK, bool KMAJOR>
-__device__ __forceinline__ unsigned dma_global_offset(int q, int lane, long long ld) {
+__device__ __forceinline__ void dma_lane_coords(int q, int lane, int& r, int& k) {
   using G = TileGeom<R, BK, KMAJOR>;
   const int p = q * 64 + lane;
   const int row = p / G::CPR;
   const int cs = p % G::CPR;
   if (KMAJOR) {
-    const int c = cs ^ G::swz_k(row);
-    return (unsigned)(((long long)row * ld + c * 8) * 2);
+    r = row;
+    k = (cs ^ G::swz_k(row)) * 8;
   } else {
     const int g = (cs >> 2) ^ G::swz_m(row);
-    const int c = g * 4 + (cs & 3);
-    return (unsigned)(((long long)row * ld + c * 8) * 2);
+    r = (g * 4 + (cs & 3)) * 8;
+    k = row;
   }
 }
+
+// Byte offset of those elements from the tile's global origin for a plain matrix with leading
+// dimension ld.
+template <int R, int BK, bool KMAJOR>
+__device__ __forceinline__ unsigned dma_global_offset(int q, int lane, long long ld) {
+  int r, k;
+  dma_lane_coords<R, BK, KMAJOR>(q, lane, r, k);
+  return (unsigned)((KMAJOR ? (long long)r * ld + k : (long long)k * ld + r) * 2);
+}
+
+// Tensor-contraction index maps: walks the K index of a contraction tile by tile.  The first K
+// mode is consumed BK at a time (BK divides its extent), the others are the digits of a counter.
+struct KWalker {
+  int kf, d1, d2, d3;
+  __device__ __forceinline__ void reset() { kf = d1 = d2 = d3 = 0; }
+  __device__ __forceinline__ void advance(const GettDim& gk, int bk) {
+    kf += bk;
+    if (kf >= gk.extent[0]) {
+      kf = 0;
+      if (gk.nmodes > 1 && ++d1 >= gk.extent[1]) {
+        d1 = 0;
+        if (gk.nmodes > 2 && ++d2 >= gk.extent[2]) {
+          d2 = 0;
+          if (gk.nmodes > 3) ++d3;
+        }
+      }
+    }
+  }
+  // element offset of the tile's first k in the tensor whose K strides are `stride`
+  __device__ __forceinline__ long long offset(const GettDim& gk, const long long* stride) const {
+    long long o = (long long)kf * stride[0];
+    if (gk.nmodes > 1) o += (long long)d1 * stride[1];
+    if (gk.nmodes > 2) o += (long long)d2 * stride[2];
+    if (gk.nmodes > 3) o += (long long)d3 * stride[3];
+    return o;
+  }
+};
 
 // Fragment of 32 tile rows x 16 k-values: lane l receives the 8 k-values 8*(l/32)..+7 of row
 // row0 + l%32, which is the operand layout of v_mfma_f32_32x32x16.
@@ -178,10 +215,11 @@ __device__ __forceinline__ int4v transform_fragment(int4v f, const OpList& t0, c
   return __builtin_bit_cast(int4v, v);
 }
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, bool A_KMAJOR_, bool B_KMAJOR_, typename T_, bool FUSED_>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, bool A_KMAJOR_, bool B_KMAJOR_, typename T_, bool FUSED_, bool GETT_ = false>
 struct MfmaGemmConfig {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, FUSED = FUSED_;
+  static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
   static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / 16) % 2 == 0);   // cross-step fragment prefetch
   typedef T_ T;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -230,15 +268,43 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const int m0 = ti * BM, n0 = tj * BN;
 
   // --- global tile origins (bytes) and the per-lane DMA offsets, fixed for the whole K loop ---
-  const char* ga = (const char*)args.a + (Cfg::A_KMAJOR ? (long long)m0 * args.lda : (long long)m0) * 2;
-  const char* gb = (const char*)args.b + (Cfg::B_KMAJOR ? (long long)n0 * args.ldb : (long long)n0) * 2;
-  const long long a_step = (Cfg::A_KMAJOR ? (long long)BK : (long long)BK * args.lda) * 2;
-  const long long b_step = (Cfg::B_KMAJOR ? (long long)BK : (long long)BK * args.ldb) * 2;
+  const char* ga;
+  const char* gb;
+  long long a_step = 0, b_step = 0;
   unsigned offa[DMA_A], offb[DMA_B];
+  KWalker walk;
+  walk.reset();
+  if constexpr (!Cfg::GETT) {
+    ga = (const char*)args.a + (Cfg::A_KMAJOR ? (long long)m0 * args.lda : (long long)m0) * 2;
+    gb = (const char*)args.b + (Cfg::B_KMAJOR ? (long long)n0 * args.ldb : (long long)n0) * 2;
+    a_step = (Cfg::A_KMAJOR ? (long long)BK : (long long)BK * args.lda) * 2;
+    b_step = (Cfg::B_KMAJOR ? (long long)BK : (long long)BK * args.ldb) * 2;
 #pragma unroll
-  for (int i = 0; i < DMA_A; ++i) offa[i] = dma_global_offset<BM, BK, Cfg::A_KMAJOR>(wave + i * NWAVES, lane, args.lda);
+    for (int i = 0; i < DMA_A; ++i) offa[i] = dma_global_offset<BM, BK, Cfg::A_KMAJOR>(wave + i * NWAVES, lane, args.lda);
 #pragma unroll
-  for (int i = 0; i < DMA_B; ++i) offb[i] = dma_global_offset<BN, BK, Cfg::B_KMAJOR>(wave + i * NWAVES, lane, args.ldb);
+    for (int i = 0; i < DMA_B; ++i) offb[i] = dma_global_offset<BN, BK, Cfg::B_KMAJOR>(wave + i * NWAVES, lane, args.ldb);
+  } else {
+    // element (m, k) of A lives at offM(m) + offK(k): the row part is a mixed-radix walk over the M
+    // modes (done once per lane), the k part inside a tile is linear in the first K mode
+    ga = (const char*)args.a;
+    gb = (const char*)args.b;
+#pragma unroll
+    for (int i = 0; i < DMA_A; ++i) {
+      int r, k;
+      dma_lane_coords<BM, BK, Cfg::A_KMAJOR>(wave + i * NWAVES, lane, r, k);
+      long long o0, o1;
+      gett_offsets(args.gm, m0 + r, o0, o1);
+      offa[i] = (unsigned)((o0 + (long long)k * args.gk.stride0[0]) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < DMA_B; ++i) {
+      int r, k;
+      dma_lane_coords<BN, BK, Cfg::B_KMAJOR>(wave + i * NWAVES, lane, r, k);
+      long long o0, o1;
+      gett_offsets(args.gn, n0 + r, o0, o1);
+      offb[i] = (unsigned)((o0 + (long long)k * args.gk.stride1[0]) * 2);
+    }
+  }
 
   auto issue_tile = [&](int stage) {
 #ifdef GK_ABLATE_DMA
@@ -246,14 +312,23 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #endif
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
+    const char* pa = ga;
+    const char* pb = gb;
+    if constexpr (Cfg::GETT) {
+      pa = ga + walk.offset(args.gk, args.gk.stride0) * 2;
+      pb = gb + walk.offset(args.gk, args.gk.stride1) * 2;
+      walk.advance(args.gk, BK);
+    }
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i)
-      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i)
-      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
-    ga += a_step;
-    gb += b_step;
+      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+    if constexpr (!Cfg::GETT) {
+      ga += a_step;
+      gb += b_step;
+    }
   };
 
   const int KT = args.K / BK;
@@ -268,15 +343,31 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   float16v acc[FM][FN];
   const int mrow = m0 + wm * Cfg::WTM + (lane & 31);
   const int ncol = n0 + wn * Cfg::WTN + 4 * (lane >> 5);
+  // element offset of the lane's first element of accumulator block (fi, fj) in C / D, and the
+  // stride between its consecutive columns.  With a tensor-contraction map the first M mode and
+  // the first N mode cover whole 32-wide blocks, so only the block origin needs the digit walk.
+  auto cd_offset = [&](int fi, int fj, long long ld) -> long long {
+    if constexpr (!Cfg::GETT) {
+      return (long long)(mrow + 32 * fi) + (long long)(ncol + 32 * fj) * ld;
+    } else {
+      long long t0, om, on;
+      gett_offsets(args.gm, m0 + wm * Cfg::WTM + 32 * fi, t0, om);
+      gett_offsets(args.gn, n0 + wn * Cfg::WTN + 32 * fj, t0, on);
+      return om + (long long)(lane & 31) * args.gm.stride1[0] + on + (long long)(4 * (lane >> 5)) * args.gn.stride1[0];
+    }
+  };
+  auto cd_nstride = [&](long long ld) -> long long {
+    if constexpr (!Cfg::GETT) return ld; else return args.gn.stride1[0];
+  };
   if (args.c_mode != 0) {
-    const float* cp = (const float*)args.c + mrow + (long long)ncol * args.ldc;
 #pragma unroll
     for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < FN; ++fj) {
+        const float* cp = (const float*)args.c + cd_offset(fi, fj, args.ldc);
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          acc[fi][fj][v] = cp[32 * fi + (long long)(32 * fj + 8 * (v / 4) + (v % 4)) * args.ldc];
+        for (int v = 0; v < 16; ++v) acc[fi][fj][v] = cp[(long long)(8 * (v / 4) + (v % 4)) * cd_nstride(args.ldc)];
+      }
     if (Cfg::FUSED) {
       if (args.t[H_GL2SH_C].n > 0 || args.t[H_SH2RF_C].n > 0) {
 #pragma unroll
@@ -417,11 +508,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   trace_t[2] = clock64();
 #endif
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
-  float* dp = (float*)args.d + mrow + (long long)ncol * args.ldd;
 #pragma unroll
   for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
     for (int fj = 0; fj < FN; ++fj) {
+      float* dp = (float*)args.d + cd_offset(fi, fj, args.ldd);
       float x[16];
 #pragma unroll
       for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
@@ -439,7 +530,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       }
 #pragma unroll
       for (int v = 0; v < 16; ++v)
-        dp[32 * fi + (long long)(32 * fj + 8 * (v / 4) + (v % 4)) * args.ldd] = x[v];
+        dp[(long long)(8 * (v / 4) + (v % 4)) * cd_nstride(args.ldd)] = x[v];
     }
 #ifdef GK_PHASE_TRACE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -162,6 +162,49 @@ def _config1() -> Workload:
         kernel_name=kernel_name(conf, kern))
 
 
+def gett_config(a_modes, b_modes, d_modes, extents, block_shape=None, zero_c=True, **kw):
+    """A tensor-contraction configuration: the index arithmetic of the contraction lives in the
+    Layout loaders (the pattern of reference benchmarks/tensor-contractions/run.jl:22-85)."""
+    gmap = Layout.gett_map(a_modes, b_modes, d_modes, extents)
+    M, N, K = gmap.extent("m"), gmap.extent("n"), gmap.extent("k")
+    params = dict(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+                  global_a_layout=Layout.GETT[Float16, gmap], global_b_layout=Layout.GETT[Float16, gmap],
+                  global_c_layout=Layout.Zero[Float32] if zero_c else Layout.GETT[Float32, gmap],
+                  global_d_layout=Layout.GETT[Float32, gmap],
+                  shared_a_layout=Layout.UnsafeAlignedColMajor[Float16], shared_b_layout=Layout.UnsafeAlignedColMajor[Float16],
+                  shared_c_layout=Layout.Zero[Float32] if zero_c else Layout.UnsafeAlignedColMajor[Float32],
+                  shared_d_layout=Layout.UnsafeAlignedColMajor[Float32])
+    if block_shape is not None:
+        params["block_shape"] = NT(M=block_shape[0], N=block_shape[1], K=block_shape[2])
+    params.update(kw)
+    return get_config(**params), gmap
+
+
+def _config5() -> Workload:
+    ext = dict(a=64, b=64, c=64, d=64, e=64, f=64)
+    conf, gmap = gett_config("aebf", "dfce", "abcd", ext)
+    M = N = K = 4096
+
+    def host():
+        return dict(a=rng.matrix("upm1_f16", 5001, (64, 64, 64, 64)), b=rng.matrix("upm1_f16", 5002, (64, 64, 64, 64)), c=None)
+
+    def launch(h):
+        import torch
+        a, b = colmajor(h["a"]), colmajor(h["b"])
+        d = colmajor_empty((64, 64, 64, 64), torch.float32)
+
+        def run():
+            matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+        return _attach(run, a=a, b=b, d=d, conf=conf)
+
+    return Workload(
+        name="config 5",
+        description="config 5: GETT D[a,b,c,d] = sum_{e,f} A[a,e,b,f] * B[d,f,c,e], all extents 64 (M=N=K=4096), FP16 in ~ U[-1,1), "
+                    "FP32 out, dense column-major tensors, contraction index map in the Layout loader",
+        flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + M * N * 4, bound="mfma", make_host=host, make_launch=launch,
+        kernel_name=kernel_name(conf, Kernel.matmul_pipelined))
+
+
 def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     """The benchmark workloads 1, 2 (variant NN/NT/TN/TT), 3, "4a", "4b", 5."""
     if n == 2:
@@ -174,4 +217,4 @@ def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     raise NotImplementedError(f"benchmark config {n}")
 
 
-_LATE_BUILDERS = {1: _config1}
+_LATE_BUILDERS = {1: _config1, 5: _config5}

@@ -125,3 +125,32 @@ def physical_size(layout: LayoutType, logical_size) -> tuple:
     if layout.kind == SPLIT_COL_MAJOR:
         return (t[0] + layout.pad, *t[1:], 2)
     return (t[0] + layout.pad, *t[1:])
+
+
+def gett_map(a_modes: str, b_modes: str, d_modes: str, extents: dict) -> GETTMap:
+    """Index map of the contraction ``D[d_modes] = sum A[a_modes] * B[b_modes]`` over dense
+    column-major tensors (first index fastest), einsum-style mode letters.
+
+    M modes are those shared by A and D, N modes by B and D, K modes by A and B.  Within each GEMM
+    dimension the mode that is contiguous in A (for M, K) or B (for N, K) goes first, so that the
+    loader can move 16-byte vectors; the others follow by increasing stride."""
+    def strides(modes):
+        out, s = {}, 1
+        for ch in modes:
+            out[ch] = s
+            s *= extents[ch]
+        return out
+
+    sa, sb, sd = strides(a_modes), strides(b_modes), strides(d_modes)
+    m_modes = [ch for ch in a_modes if ch in d_modes]
+    n_modes = [ch for ch in b_modes if ch in d_modes]
+    k_modes = [ch for ch in a_modes if ch in b_modes]
+    if set(m_modes) | set(n_modes) != set(d_modes) or set(m_modes) & set(n_modes):
+        raise ValueError("every mode of D must come from exactly one of A and B")
+    m_modes.sort(key=lambda ch: sa[ch])
+    n_modes.sort(key=lambda ch: sb[ch])
+    # K: a mode that is contiguous in A or in B must lead
+    k_modes.sort(key=lambda ch: min(sa[ch], sb[ch]))
+    return GETTMap(m=tuple((extents[ch], sa[ch], sd[ch]) for ch in m_modes),
+                   n=tuple((extents[ch], sb[ch], sd[ch]) for ch in n_modes),
+                   k=tuple((extents[ch], sa[ch], sb[ch]) for ch in k_modes))

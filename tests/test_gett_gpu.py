@@ -1,0 +1,112 @@
+"""GPU parity of the tensor-contraction (GETT) layouts: D[a,b,c,d] = sum_{e,f} A[a,e,b,f] * B[d,f,c,e]
+(benchmark config 5) and other mode permutations, against numpy einsum, the CPU oracle's own index
+map, and -- bit for bit -- the plain GEMM kernel run on explicitly materialised matrices."""
+import numpy as np
+import pytest
+import torch
+
+import gemmkernels as gk
+from gemmkernels import Kernel, Layout, configs, rng
+import helpers
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gett(conf, A, B, d_shape):
+    a, b = gk.colmajor(A), gk.colmajor(B)
+    d = gk.colmajor_empty(d_shape, torch.float32)
+    d.fill_(float("nan"))
+    gk.matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    return gk.to_numpy(d)
+
+
+def small_ints(shape, seed):
+    rs = np.random.RandomState(seed)
+    return np.asfortranarray(rs.randint(-4, 5, size=shape).astype(np.float16))
+
+
+def test_small_contraction_is_exact_against_einsum(gpu):
+    ext = dict(a=32, b=2, c=2, d=32, e=32, f=2)
+    conf, gmap = configs.gett_config("aebf", "dfce", "abcd", ext, block_shape=(64, 64, 32))
+    assert gk.kernel_name(conf, Kernel.matmul_pipelined).endswith("_gett")
+    A = small_ints((32, 32, 2, 2), 1)     # A[a,e,b,f]
+    B = small_ints((32, 2, 2, 32), 2)     # B[d,f,c,e]
+    D = run_gett(conf, A, B, (32, 2, 2, 32))
+    want = np.einsum("aebf,dfce->abcd", A.astype(np.float64), B.astype(np.float64))
+    assert np.array_equal(D.astype(np.float64), want)          # small integers: every sum is exact
+    # the CPU oracle walks the same mode tables
+    ref = np.zeros((32, 2, 2, 32), np.float32, order="F")
+    p = helpers.oracle_problem(conf, (0, 0, 0, 0))
+    oracle.matmul(p, A, B, None, ref)
+    assert np.array_equal(ref, D)
+
+
+def test_distinct_extents_and_k_major_operands(gpu):
+    """TCCG-style D[a,b,c] = sum_d A[b,d,a] * B[d,c] (the contraction of the reference benchmark
+    script, benchmarks/tensor-contractions/run.jl:10-20): here A is contiguous along an M mode and B
+    along the K mode."""
+    ext = dict(a=3, b=64, c=128, d=64)
+    conf, gmap = configs.gett_config("bda", "dc", "abc", ext, block_shape=(64, 64, 32))
+    A = small_ints((64, 64, 3), 3)        # A[b,d,a]
+    B = small_ints((64, 128), 4)          # B[d,c]
+    D = run_gett(conf, A, B, (3, 64, 128))
+    want = np.einsum("bda,dc->abc", A.astype(np.float64), B.astype(np.float64))
+    assert np.array_equal(D.astype(np.float64), want)
+
+
+def materialise(A, B, ext, gmap):
+    """A_mat[m, k] and B_mat[n, k] with the kernel's own index orders (modes fastest first)."""
+    a_modes, b_modes = "aebf", "dfce"
+    def order(tensor_modes, dims):     # letters of the modes in `dims`, fastest first, identified by stride
+        strides, s = {}, 1
+        for ch in tensor_modes:
+            strides[s] = ch
+            s *= ext[ch]
+        return strides
+    sa, sb = order(a_modes, None), order(b_modes, None)
+    m_letters = [sa[s0] for _, s0, _ in gmap.m]
+    n_letters = [sb[s0] for _, s0, _ in gmap.n]
+    k_letters = [sa[s0] for _, s0, _ in gmap.k]
+    M, N, K = gmap.extent("m"), gmap.extent("n"), gmap.extent("k")
+    # einsum to (m modes..., k modes...) then Fortran-reshape (first listed = fastest)
+    A_mat = np.einsum(f"{a_modes}->{''.join(m_letters + k_letters)}", A).reshape((M, K), order="F")
+    B_mat = np.einsum(f"{b_modes}->{''.join(n_letters + k_letters)}", B).reshape((N, K), order="F")
+    return np.asfortranarray(A_mat), np.asfortranarray(B_mat), m_letters, n_letters
+
+
+@pytest.mark.parametrize("extent,block", [(16, None), (64, None)])
+def test_bit_exact_against_the_plain_kernel_on_materialised_matrices(gpu, extent, block):
+    """Same kernel, same tile shape, same K order => the same MFMA sequence => identical bits."""
+    if extent == 16:
+        ext = dict(a=32, b=4, c=4, d=32, e=64, f=2)      # M = N = 128, K = 128
+        block = (128, 128, 64)
+    else:
+        ext = dict(a=64, b=64, c=64, d=64, e=64, f=64)   # benchmark config 5
+        block = (256, 256, 64)
+    conf, gmap = configs.gett_config("aebf", "dfce", "abcd", ext, block_shape=block)
+    shape_a = tuple(ext[ch] for ch in "aebf")
+    shape_b = tuple(ext[ch] for ch in "dfce")
+    A = rng.matrix("upm1_f16", 5001, shape_a)
+    B = rng.matrix("upm1_f16", 5002, shape_b)
+    D = run_gett(conf, A, B, tuple(ext[ch] for ch in "abcd"))
+    A_mat, B_mat, m_letters, n_letters = materialise(A, B, ext, gmap)
+    M, N, K = A_mat.shape[0], B_mat.shape[0], A_mat.shape[1]
+    plain = configs.mfma_config(M, N, K, ta=False, tb=True, zero_c=True, block_shape=block)
+    D_mat = helpers.run_gpu(plain, A_mat, B_mat, None, (M, N), kernel=Kernel.matmul_pipelined)
+    # D_mat[m, n'] with m = (m_letters), n' = (n_letters), fastest first -> back to D[a,b,c,d]
+    D_back = np.einsum(f"{''.join(m_letters + n_letters)}->abcd",
+                       D_mat.reshape(tuple(ext[ch] for ch in m_letters + n_letters), order="F"))
+    assert np.array_equal(D, D_back)
+    # and the value itself, against BLAS on the materialised matrices
+    ref = oracle.gemm_blas_f32(A_mat, B_mat, None, 1.0, 0.0, False, True)
+    assert oracle.rel_frobenius(D_mat, ref) <= 1e-3
+
+
+def test_gett_config_errors():
+    from gemmkernels import ConfigError
+    with pytest.raises(ConfigError):      # BLOCK_K must divide the first K mode
+        configs.gett_config("aebf", "dfce", "abcd", dict(a=32, b=2, c=2, d=32, e=16, f=4), block_shape=(64, 64, 32))
+    with pytest.raises(ConfigError):      # first M mode not a multiple of 32
+        configs.gett_config("aebf", "dfce", "abcd", dict(a=16, b=4, c=2, d=32, e=32, f=2), block_shape=(64, 64, 32))
