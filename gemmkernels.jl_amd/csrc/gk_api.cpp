@@ -184,6 +184,8 @@ gk::FamilyFn family_fn(const gk::InstanceKey& key) {
       return key.b_kmajor ? gk::family_mfma_nn : gk::family_mfma_nt;
     case gk::FAMILY_FPU:
       return gk::family_fpu;
+    case gk::FAMILY_DIAGONAL:
+      return gk::family_diagonal;
     case gk::FAMILY_MFMA_CHECKED:
       return gk::family_mfma_checked;
     default:
@@ -322,6 +324,25 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
       c->global_c_layout.kind == GK_LAYOUT_GETT || c->global_d_layout.kind == GK_LAYOUT_GETT) {
     int rc_g = validate_gett(c);
     if (rc_g != GK_OK) return rc_g;
+  }
+
+  if (c->global_a_layout.kind == GK_LAYOUT_DIAGONAL) {
+    if (g.M != g.K) return fail(GK_ERR_DIMENSION_MISMATCH, "Diagonal only supports a square A matrix (M == K)");
+    const int bkind = c->global_b_layout.kind;
+    if ((bkind != GK_LAYOUT_ALIGNED_COL_MAJOR && bkind != GK_LAYOUT_ALIGNED_ROW_MAJOR) ||
+        c->global_d_layout.kind != GK_LAYOUT_ALIGNED_COL_MAJOR ||
+        (c->global_c_layout.kind != GK_LAYOUT_ALIGNED_COL_MAJOR && c->global_c_layout.kind != GK_LAYOUT_ZERO))
+      return fail(GK_ERR_UNSUPPORTED, "a diagonal A needs aligned layouts for B, C and D");
+    if (t) {
+      // off-diagonal zeros of A are never materialised: the A hooks must map 0 to 0
+      const int hooks[2] = {GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A};
+      for (int h : hooks)
+        for (int i = 0; i < t->hook[h].n_ops && i < GK_MAX_OPS; ++i) {
+          const gk_op& o = t->hook[h].ops[i];
+          if (o.kind == GK_T_ADD && o.p0 != 0.0f) return fail(GK_ERR_UNSUPPORTED, "a transform of a diagonal A must keep zero at zero");
+          if (o.kind == GK_T_CLAMP && (o.p0 > 0.0f || o.p1 < 0.0f)) return fail(GK_ERR_UNSUPPORTED, "a transform of a diagonal A must keep zero at zero");
+        }
+    }
   }
 
   // src/matmul.jl:34-36 (decidable from the configuration alone, so it is checked before the
@@ -474,6 +495,8 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   if ((rc = check_aligned(conf->global_c_layout, c, args.ldc, "C")) != GK_OK) return rc;
   if ((rc = check_aligned(conf->global_d_layout, d, args.ldd, "D")) != GK_OK) return rc;
 
+  if (key.family == gk::FAMILY_DIAGONAL && (((uintptr_t)a & 15u) != 0))
+    return fail(GK_ERR_ALIGNMENT, "the diagonal of A must be aligned to 16 bytes");
   if (key.family == gk::FAMILY_GETT && ((((uintptr_t)a | (uintptr_t)b) & 15u) != 0))
     return fail(GK_ERR_ALIGNMENT, "tensor operands must be aligned to 16 bytes");
 

@@ -1,0 +1,119 @@
+// D = diag(a) * B (+ C): the GEMM whose A operand is Layout.Diagonal (reference
+// src/layout.jl:225-236, run by matmul_singlestage with threadblock_condition, src/kernel.jl:60).
+//
+// The reference builds the dense tile of A in shared memory and skips the K blocks that hold no
+// diagonal element.  Taken to its end that skip leaves exactly one product per output element,
+// D[i,j] = fma(a[i], B[i,j], C[i,j]), which is what this kernel computes: every other term of the
+// sum is an exact zero, so the result is bit-identical to the full product.  The work is pure
+// streaming (read B, read C, write D), bound by HBM bandwidth: each lane moves 16-byte vectors and
+// a workgroup covers its block_shape.M x block_shape.N tile of D in one pass.
+#pragma once
+#include "common.hpp"
+
+namespace gk {
+
+// B_ROWMAJOR: B is the 'T' operand, stored N x K with K = M contiguous along j ... i.e. element
+// (i, j) lives at b[j + i*ldb]; otherwise at b[i + j*ldb].
+template <bool B_ROWMAJOR, typename T>
+__global__ void __launch_bounds__(1024) diagonal_gemm_kernel(const GemmArgs args, int BM, int BN) {
+  typedef T vec8 __attribute__((ext_vector_type(8)));
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int ti, tj;
+  cta_swizzle(args.swz_kind, args.swz_param, (int)blockIdx.x, (int)blockIdx.y, args.nbm, args.nbn, ti, tj);
+  if (ti >= args.nbm || tj >= args.nbn) return;
+  const int m0 = ti * BM, n0 = tj * BN;
+  const T* A = (const T*)args.a;
+  const T* B = (const T*)args.b;
+  const float* C = (const float*)args.c;
+  float* D = (float*)args.d;
+  const bool xf_a = args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0;
+  const bool xf_b = args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0;
+  const bool xf_c = args.t[H_GL2SH_C].n > 0 || args.t[H_SH2RF_C].n > 0;
+  const bool xf_d = args.t[H_RF2SH_D].n > 0 || args.t[H_SH2GL_D].n > 0 || args.epi_kind != 0;
+
+  auto finish = [&](int i, int j, const float (&av)[8], const float (&bv)[8]) {
+    float c[8];
+    if (args.c_mode != 0) {
+      const float4v c0 = *(const float4v*)&C[i + (long long)j * args.ldc];
+      const float4v c1 = *(const float4v*)&C[i + 4 + (long long)j * args.ldc];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { c[e] = c0[e]; c[4 + e] = c1[e]; }
+      if (xf_c) { apply_list_regs<8>(args.t[H_GL2SH_C], c); apply_list_regs<8>(args.t[H_SH2RF_C], c); }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) c[e] = 0.0f;
+    }
+    float x[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __builtin_fmaf(av[e], bv[e], c[e]);
+    if (xf_d) {
+      apply_list_regs<8>(args.t[H_RF2SH_D], x);
+      if (args.epi_kind == 1) {
+        const float bj = args.bias[j];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = x[e] + bj;
+      } else if (args.epi_kind == 2) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = x[e] + args.bias[i + e];
+      }
+      apply_list_regs<8>(args.t[H_SH2GL_D], x);
+    }
+    *(float4v*)&D[i + (long long)j * args.ldd] = (float4v){x[0], x[1], x[2], x[3]};
+    *(float4v*)&D[i + 4 + (long long)j * args.ldd] = (float4v){x[4], x[5], x[6], x[7]};
+  };
+  auto prep = [&](vec8 v, bool xf, const OpList& t0, const OpList& t1, float (&out)[8]) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = (float)v[e];
+    if (xf) {
+      if (t0.n > 0) {
+        apply_list_regs<8>(t0, out);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (float)(T)out[e];
+      }
+      if (t1.n > 0) {
+        apply_list_regs<8>(t1, out);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (float)(T)out[e];
+      }
+    }
+  };
+
+  if (!B_ROWMAJOR) {
+    // chunk = 8 consecutive rows i of one column j
+    const int chunks_m = BM / 8, total = chunks_m * BN;
+    for (int q = (int)threadIdx.x; q < total; q += (int)blockDim.x) {
+      const int i = m0 + (q % chunks_m) * 8, j = n0 + q / chunks_m;
+      float av[8], bv[8];
+      prep(*(const vec8*)&A[i], xf_a, args.t[H_GL2SH_A], args.t[H_SH2RF_A], av);
+      prep(*(const vec8*)&B[i + (long long)j * args.ldb], xf_b, args.t[H_GL2SH_B], args.t[H_SH2RF_B], bv);
+      finish(i, j, av, bv);
+    }
+  } else {
+    // transpose 64 (i) x 64 (j) sub-tiles of B through LDS so that both the loads (along j) and the
+    // stores (along i) are 16-byte vectors
+    T* tile = (T*)smem;                   // [64 i][64 + 8 j]
+    constexpr int PITCH = 72;
+    for (int sm = 0; sm < BM; sm += 64)
+      for (int sn = 0; sn < BN; sn += 64) {
+        __syncthreads();
+        for (int q = (int)threadIdx.x; q < 64 * 8; q += (int)blockDim.x) {
+          const int il = q / 8, jl = (q % 8) * 8;
+          *(vec8*)&tile[il * PITCH + jl] = *(const vec8*)&B[(n0 + sn + jl) + (long long)(m0 + sm + il) * args.ldb];
+        }
+        __syncthreads();
+        for (int q = (int)threadIdx.x; q < 8 * 64; q += (int)blockDim.x) {
+          const int il = (q % 8) * 8, jl = q / 8;
+          vec8 bvec;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) bvec[e] = tile[(il + e) * PITCH + jl];
+          const int i = m0 + sm + il, j = n0 + sn + jl;
+          float av[8], bv[8];
+          prep(*(const vec8*)&A[i], xf_a, args.t[H_GL2SH_A], args.t[H_SH2RF_A], av);
+          prep(bvec, xf_b, args.t[H_GL2SH_B], args.t[H_SH2RF_B], bv);
+          finish(i, j, av, bv);
+        }
+      }
+  }
+}
+
+}  // namespace gk

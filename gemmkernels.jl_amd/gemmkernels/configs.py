@@ -180,6 +180,44 @@ def gett_config(a_modes, b_modes, d_modes, extents, block_shape=None, zero_c=Tru
     return get_config(**params), gmap
 
 
+def diagonal_config(M, N, tb=False, zero_c=False, **kw):
+    """@get_wmma_diagonal_config of the reference (configs/configs.jl:331-383): A is given by its
+    diagonal, the kernel is matmul_singlestage."""
+    params = dict(gemm_shape=NT(M=M, N=N, K=M), operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+                  global_a_layout=Layout.Diagonal[Float16], global_b_layout=_aligned(Float16, tb),
+                  global_c_layout=Layout.Zero[Float32] if zero_c else Layout.UnsafeAlignedColMajor[Float32],
+                  global_d_layout=Layout.UnsafeAlignedColMajor[Float32],
+                  shared_a_layout=Layout.Padded[Layout.UnsafeAlignedColMajor[Float16], 8],
+                  is_a_col_major=True, is_b_col_major=not tb)
+    params.update(kw)
+    return get_config(**params)
+
+
+def _config4b() -> Workload:
+    M = N = 4096
+    conf = diagonal_config(M, N, zero_c=True)
+
+    def host():
+        return dict(a=rng.uniform_pm1_f16(4004, M), b=rng.matrix("upm1_f16", 4002, (M, N)), c=None)
+
+    def launch(h):
+        import torch
+        a = torch.from_numpy(h["a"]).cuda()
+        b = colmajor(h["b"])
+        d = colmajor_empty((M, N), torch.float32)
+
+        def run():
+            matmul(conf, a, b, None, d, kernel=Kernel.matmul_singlestage)
+        return _attach(run, a=a, b=b, d=d, conf=conf)
+
+    return Workload(
+        name="config 4b",
+        description="config 4b: D = diag(a) * B, a 4096 FP16 ~ U[-1,1), B 4096x4096 FP16 ~ U[-1,1), D FP32, no C "
+                    "(Layout.Diagonal, single-stage kernel); bandwidth bound",
+        flops=M * N, bytes=M * 2 + M * N * 2 + M * N * 4, bound="hbm", make_host=host, make_launch=launch,
+        kernel_name=kernel_name(conf, Kernel.matmul_singlestage))
+
+
 def _config5() -> Workload:
     ext = dict(a=64, b=64, c=64, d=64, e=64, f=64)
     conf, gmap = gett_config("aebf", "dfce", "abcd", ext)
@@ -217,4 +255,4 @@ def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     raise NotImplementedError(f"benchmark config {n}")
 
 
-_LATE_BUILDERS = {1: _config1, 5: _config5}
+_LATE_BUILDERS = {1: _config1, "4b": _config4b, 5: _config5}
