@@ -138,6 +138,12 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
   args->ldd = c->global_d_layout.ld > 0 ? c->global_d_layout.ld : args->M;
   args->nbm = (args->M + c->block_shape.M - 1) / c->block_shape.M;
   args->nbn = (args->N + c->block_shape.N - 1) / c->block_shape.N;
+  if (c->op.kind == GK_OP_MFMA_COMPLEX || c->op.kind == GK_OP_MFMA_DUAL) {
+    // interleaved complex operands seen as real matrices: M and K double, and so does every
+    // leading dimension (counted in real elements)
+    args->M *= 2; args->K *= 2;
+    args->lda *= 2; args->ldb *= 2; args->ldc *= 2; args->ldd *= 2;
+  }
   args->swz_kind = c->cta_swizzle.kind;
   args->swz_param = c->cta_swizzle.param;
   args->c_mode = (c->global_c_layout.kind == GK_LAYOUT_ZERO) ? 0 : 1;
@@ -186,6 +192,8 @@ gk::FamilyFn family_fn(const gk::InstanceKey& key) {
       return gk::family_fpu;
     case gk::FAMILY_DIAGONAL:
       return gk::family_diagonal;
+    case gk::FAMILY_COMPLEX:
+      return gk::family_complex;
     case gk::FAMILY_MFMA_CHECKED:
       return gk::family_mfma_checked;
     default:
@@ -326,6 +334,14 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
     if (rc_g != GK_OK) return rc_g;
   }
 
+  if (op.kind == GK_OP_MFMA_COMPLEX || op.kind == GK_OP_MFMA_DUAL) {
+    auto inter = [](int k) { return k == GK_LAYOUT_INTERLEAVED_COL_MAJOR || k == GK_LAYOUT_INTERLEAVED_ROW_MAJOR; };
+    if (!inter(c->global_a_layout.kind) || !inter(c->global_b_layout.kind) || c->global_d_layout.kind != GK_LAYOUT_INTERLEAVED_COL_MAJOR ||
+        (c->global_c_layout.kind != GK_LAYOUT_INTERLEAVED_COL_MAJOR && c->global_c_layout.kind != GK_LAYOUT_ZERO))
+      return fail(GK_ERR_UNSUPPORTED, "complex and dual operators need Interleaved layouts for A and B and InterleavedColMajor for C and D");
+    if (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT))
+      return fail(GK_ERR_UNSUPPORTED, "transforms and bias are not available with the complex and dual operators");
+  }
   if (c->global_a_layout.kind == GK_LAYOUT_DIAGONAL) {
     if (g.M != g.K) return fail(GK_ERR_DIMENSION_MISMATCH, "Diagonal only supports a square A matrix (M == K)");
     const int bkind = c->global_b_layout.kind;
@@ -483,8 +499,9 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
 
   // aligned layouts move 16-byte vectors (reference src/layout.jl:22-34 traps on the device; here it is a host check)
   auto check_aligned = [&](const gk_layout& l, const void* p, long long ld, const char* what) -> int {
-    if (l.kind != GK_LAYOUT_ALIGNED_COL_MAJOR && l.kind != GK_LAYOUT_ALIGNED_ROW_MAJOR) return GK_OK;
-    const int es = dtype_size(l.eltype);
+    const bool interleaved = l.kind == GK_LAYOUT_INTERLEAVED_COL_MAJOR || l.kind == GK_LAYOUT_INTERLEAVED_ROW_MAJOR;
+    if (l.kind != GK_LAYOUT_ALIGNED_COL_MAJOR && l.kind != GK_LAYOUT_ALIGNED_ROW_MAJOR && !interleaved) return GK_OK;
+    const int es = dtype_size(l.eltype);   // ld already counts real elements for interleaved data
     if (es == 0) return fail(GK_ERR_INVALID_ARGUMENT, "unknown element type of %s", what);
     if (((uintptr_t)p & 15u) != 0) return fail(GK_ERR_ALIGNMENT, "%s is not aligned to 16 bytes", what);
     if ((ld * es) % 16 != 0) return fail(GK_ERR_ALIGNMENT, "leading dimension of %s (%lld elements) is not a multiple of 16 bytes", what, ld);
@@ -518,7 +535,8 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   }
 
   int gx = 0, gy = 0;
-  gk::number_of_blocks(args.swz_kind, args.swz_param, args.M, args.N, conf->block_shape.M, conf->block_shape.N, gx, gy);
+  gk::number_of_blocks(args.swz_kind, args.swz_param, conf->matmul_shape.M, conf->matmul_shape.N, conf->block_shape.M,
+                       conf->block_shape.N, gx, gy);
   if (gx <= 0 || gy <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "empty grid");
 
   gk::FamilyFn fn = family_fn(key);

@@ -16,8 +16,8 @@ struct MfmaCheckedConfig {
   typedef T_ T;
   static constexpr int NWAVES = WAVES_M * WAVES_N, THREADS = NWAVES * kWaveSize;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, FM = WTM / 32, FN = WTN / 32, KSTEPS = BK / 16;
-  typedef TileGeom<BM, BK, true> GA;     // both LDS tiles are K-major whatever the memory order
-  typedef TileGeom<BN, BK, true> GB;
+  typedef OperandGeom<BM, BK, OPK_KMAJOR, false> GA;     // both LDS tiles are K-major whatever the memory order
+  typedef OperandGeom<BN, BK, OPK_KMAJOR, false> GB;
   static constexpr int LDS_BYTES = GA::BYTES + GB::BYTES;
   static constexpr int A_PER_THREAD = BM * BK / THREADS, B_PER_THREAD = BN * BK / THREADS;
   static_assert((BM * BK) % THREADS == 0 && (BN * BK) % THREADS == 0, "tile loads divide evenly over the threads");
@@ -85,13 +85,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
       }
       constexpr int CPR = BK / 8;
       const int c = k >> 3;
-      const int swz = (r / TileGeom<64, BK, true>::RP256) & (CPR - 1);
+      const int swz = (r / OperandGeom<64, BK, OPK_KMAJOR, false>::RP256) & (CPR - 1);
       *(T*)(dst + 16 * (r * CPR + (c ^ swz)) + (k & 7) * 2) = x;
     }
   };
 
-  typedef FragReader<BM, BK, true, FM> RA;
-  typedef FragReader<BN, BK, true, FN> RB;
+  typedef FragReader<BM, BK, OPK_KMAJOR, false, FM> RA;
+  typedef FragReader<BN, BK, OPK_KMAJOR, false, FN> RB;
   RA ra;
   RB rb;
   ra.init(wm * Cfg::WTM, lane);
@@ -107,17 +107,19 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
     __syncthreads();
     static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
       constexpr int ks = decltype(ks_c)::value;
-      int4v fa[FM], fb[FN];
+      typename RA::Raw fa[FM];
+      typename RB::Raw fb[FN];
       load_frags<ks>(ra, rb, fa, fb);
       wait_lgkmcnt<0>();
+      int4v va[FM], vb[FN];
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi) pin(fa[fi]);
+      for (int fi = 0; fi < FM; ++fi) { RA::pin_raw(fa[fi]); va[fi] = RA::finish(fa[fi]); }
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) pin(fb[fj]);
+      for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[fj]); vb[fj] = RB::finish(fb[fj]); }
 #pragma unroll
       for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
-        for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = Mfma<T>::run(fb[fj], fa[fi], acc[fi][fj]);
+        for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = Mfma<T>::run(vb[fj], va[fi], acc[fi][fj]);
     });
     __syncthreads();
   }

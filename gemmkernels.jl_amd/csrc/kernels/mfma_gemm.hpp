@@ -22,55 +22,51 @@
 namespace gk {
 
 // ----------------------------------------------------------------------------------------------
-// LDS tile geometry.  A tile holds R rows (m or n) x BK k-values of 16-bit elements.
-//   K-major: LDS row = tile row r, 16-byte chunk c = k / 8
-//   M-major: LDS row = k,          16-byte chunk c = r / 8
+// Operand tiles in LDS.  R is the number of MFMA rows of the block tile in the operand's own
+// dimension (m or n), BK the number of 16-bit k-values per K step.
+//   OPK_KMAJOR: LDS row = tile row, 16-byte chunk c = k / 8            (memory contiguous along k)
+//   OPK_MMAJOR: LDS row = k,        16-byte chunk c = row / 8          (memory contiguous along m / n)
+//   OPK_CROWK : interleaved complex data contiguous along m / n: LDS row = complex k, one 32-bit
+//               (re, im) element per complex row index
+// EXPAND marks the A operand of a complex (or dual-number) product: one complex row feeds two MFMA
+// rows, so the tile holds R/2 complex rows.
 // ----------------------------------------------------------------------------------------------
-template <int R, int BK, bool KMAJOR>
-struct TileGeom {
-  static constexpr int CPR = KMAJOR ? BK / 8 : R / 8;        // chunks per LDS row
-  static constexpr int ROW_BYTES = CPR * 16;
-  static constexpr int BYTES = R * BK * 2;
-  static constexpr int NDMA = BYTES / 1024;                   // wave-wide 16 B/lane DMA instructions per tile
+enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_CROWK = 2 };
+enum : int { FIX_NONE = 0, FIX_COMPLEX = 1, FIX_DUAL = 2 };
+
+template <int R, int BK, int KIND, bool EXPAND>
+struct OperandGeom {
+  static constexpr int LDS_ROWS = KIND == OPK_KMAJOR ? (EXPAND ? R / 2 : R) : (KIND == OPK_MMAJOR ? BK : BK / 2);
+  static constexpr int ROW_BYTES = KIND == OPK_KMAJOR ? BK * 2 : (KIND == OPK_MMAJOR ? R * 2 : (EXPAND ? R * 2 : R * 4));
+  static constexpr int CPR = ROW_BYTES / 16;                   // 16-byte chunks per LDS row
+  static constexpr int BYTES = LDS_ROWS * ROW_BYTES;
+  static constexpr int NDMA = BYTES / 1024;                    // wave-wide 16 B/lane DMA instructions per tile
   static constexpr int RP256 = (256 / ROW_BYTES) > 1 ? (256 / ROW_BYTES) : 1;   // LDS rows per 256 B
-  // K-major: XOR the chunk index with the row (per 256 B) so that 32 consecutive rows at one
-  // chunk index spread evenly over the 16 chunk slots of the 64 banks.
+  // K-major: XOR the chunk index with the row (per 256 B) so that 32 consecutive rows at one chunk
+  // index spread evenly over the 16 chunk slots of the 64 banks.
   __device__ static __forceinline__ int swz_k(int row) { return (row / RP256) & (CPR - 1); }
-  // M-major: XOR the 64-byte group index with k so that 4 consecutive k rows at one group land
-  // in 4 different 64-byte slots of the 256-byte bank period.
+  // M-major: XOR the 64-byte group index with k so that 4 consecutive k rows at one group land in
+  // 4 different 64-byte slots of the 256-byte bank period.
   static constexpr int GROUPS = CPR / 4;
   static constexpr int GMASK = (GROUPS - 1) < 3 ? (GROUPS - 1) : 3;
   __device__ static __forceinline__ int swz_m(int k) { return (k / RP256) & GMASK; }
   static_assert((CPR & (CPR - 1)) == 0, "chunks per row must be a power of two");
-  static_assert(KMAJOR || CPR >= 4, "M-major tiles need at least 32 rows");
+  static_assert(KIND != OPK_MMAJOR || CPR >= 4, "M-major tiles need at least 32 rows");
   static_assert(BYTES % 1024 == 0, "tile must be a whole number of DMA instructions");
+  static_assert(!EXPAND || KIND != OPK_MMAJOR, "complex operands are K-major or complex-row tiles");
 };
 
-// Tile-local coordinates (row r, first k) of the 8 elements that lane `lane` of DMA instruction q
-// fetches; they land at LDS chunk position q*64 + lane.
-template <int R, int BK, bool KMAJOR>
-__device__ __forceinline__ void dma_lane_coords(int q, int lane, int& r, int& k) {
-  using G = TileGeom<R, BK, KMAJOR>;
+// Where lane `lane` of DMA instruction q reads: LDS row `row` of the tile and the first of its 8
+// consecutive 16-bit elements `col` inside that row's span of memory (swizzle undone).  The data
+// lands at LDS chunk position q*64 + lane.
+template <class G, int KIND>
+__device__ __forceinline__ void dma_lane_coords(int q, int lane, int& row, int& col) {
   const int p = q * 64 + lane;
-  const int row = p / G::CPR;
+  row = p / G::CPR;
   const int cs = p % G::CPR;
-  if (KMAJOR) {
-    r = row;
-    k = (cs ^ G::swz_k(row)) * 8;
-  } else {
-    const int g = (cs >> 2) ^ G::swz_m(row);
-    r = (g * 4 + (cs & 3)) * 8;
-    k = row;
-  }
-}
-
-// Byte offset of those elements from the tile's global origin for a plain matrix with leading
-// dimension ld.
-template <int R, int BK, bool KMAJOR>
-__device__ __forceinline__ unsigned dma_global_offset(int q, int lane, long long ld) {
-  int r, k;
-  dma_lane_coords<R, BK, KMAJOR>(q, lane, r, k);
-  return (unsigned)((KMAJOR ? (long long)r * ld + k : (long long)k * ld + r) * 2);
+  if (KIND == OPK_KMAJOR) col = (cs ^ G::swz_k(row)) * 8;
+  else if (KIND == OPK_MMAJOR) col = (((cs >> 2) ^ G::swz_m(row)) * 4 + (cs & 3)) * 8;
+  else col = cs * 8;
 }
 
 // Tensor-contraction index maps: walks the K index of a contraction tile by tile.  The first K
@@ -101,32 +97,49 @@ struct KWalker {
   }
 };
 
-// Fragment of 32 tile rows x 16 k-values: lane l receives the 8 k-values 8*(l/32)..+7 of row
+// Makes every later use of x depend on the point where pin() stands (no instruction is emitted).
+__device__ __forceinline__ void pin(int4v& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin(int2v& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin(int& x) { asm volatile("" : "+v"(x)); }
+
+template <int N>
+__device__ __forceinline__ void wait_lgkmcnt() {
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N < 15 ? N : 15) : "memory");
+}
+
+// Fragment of 32 MFMA rows x 16 k-values: lane l receives the 8 k-values 8*(l/32)..+7 of row
 // row0 + l%32, which is the operand layout of v_mfma_f32_32x32x16.
 //
 // The reads are issued from inline assembly: the compiler would otherwise make every
 // transposing LDS read wait for all outstanding global->LDS DMA (it cannot tell the stages
-// apart), which serialises the pipeline.  Their completion is therefore tracked by hand with
-// wait_lgkmcnt<N>() + pin(), see the main loop.
-template <int R, int BK, bool KMAJOR, int F>
+// apart), which serialises the pipeline.  Their completion is therefore tracked by hand:
+// read() only issues, the registers it names (Raw) must not be looked at before
+// wait_lgkmcnt<N>() + pin_raw(), and finish() turns them into the MFMA operand afterwards.
+template <int R, int BK, int KIND, bool EXPAND, int F>
 struct FragReader {
-  typedef TileGeom<R, BK, KMAJOR> G;
+  typedef OperandGeom<R, BK, KIND, EXPAND> G;
   static constexpr int KSTEPS = BK / 16;
-  static constexpr int NBASE = KMAJOR ? KSTEPS : F;
-  static constexpr int OPS = KMAJOR ? 1 : 2;     // LDS instructions per fragment
+  static constexpr int NBASE = KIND == OPK_KMAJOR ? KSTEPS : (KIND == OPK_MMAJOR ? F : 1);
+  static constexpr int OPS = KIND == OPK_KMAJOR ? 1 : (KIND == OPK_MMAJOR ? 2 : 4);   // LDS instructions per fragment
+  static constexpr int FRAG_ROWS = EXPAND ? 16 : 32;           // tile rows (complex rows when EXPAND) per fragment
+  struct Raw {
+    int4v q;          // OPK_KMAJOR
+    int2v lo, hi;     // OPK_MMAJOR
+    int x0, x1, x2, x3;   // OPK_CROWK
+  };
   unsigned base[NBASE];                         // lane-dependent byte offsets inside a tile
   unsigned cur[NBASE];                          // the same, relative to the current stage
 
-  // row0: first tile row of the wave (multiple of 32)
+  // row0: first MFMA row of the wave inside the block tile (multiple of 32)
   __device__ __forceinline__ void init(int row0, int lane) {
-    if (KMAJOR) {
-      const int row = row0 + (lane & 31);
+    if (KIND == OPK_KMAJOR) {
+      const int row = EXPAND ? ((row0 + (lane & 31)) >> 1) : (row0 + (lane & 31));
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
         const int c = ks * 2 + (lane >> 5);
-        base[ks] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_k(row)));
+        base[ks < NBASE ? ks : 0] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_k(row)));
       }
-    } else {
+    } else if (KIND == OPK_MMAJOR) {
       const int i = lane & 15;
       const int k = 8 * (lane >> 5) + (i >> 2);
       const int m = (lane & 16) + 4 * (i & 3);          // offset inside the 32-row fragment
@@ -135,8 +148,11 @@ struct FragReader {
 #pragma unroll
       for (int fi = 0; fi < F; ++fi) {
         const int g = ((row0 >> 5) + fi) ^ G::swz_m(k);
-        base[fi] = lane_part + (unsigned)g * 64u;
+        base[fi < NBASE ? fi : 0] = lane_part + (unsigned)g * 64u;
       }
+    } else {
+      const int elem = EXPAND ? ((row0 + (lane & 31)) >> 1) : (row0 + (lane & 31));
+      base[0] = (unsigned)(4 * (lane >> 5) * G::ROW_BYTES + elem * 4);
     }
   }
   __device__ __forceinline__ void set_stage(unsigned tile_lds_addr) {
@@ -144,28 +160,54 @@ struct FragReader {
     for (int i = 0; i < NBASE; ++i) cur[i] = base[i] + tile_lds_addr;
   }
   template <int FI, int KS>
-  __device__ __forceinline__ int4v read() const {
-    int4v r;
-    if (KMAJOR) {
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(cur[KS]), "n"(FI * 32 * G::ROW_BYTES) : "memory");
+  __device__ __forceinline__ void read(Raw& r) const {
+    if (KIND == OPK_KMAJOR) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
+    } else if (KIND == OPK_MMAJOR) {
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.lo) : "v"(cur[FI < NBASE ? FI : 0]), "n"((KS * 16) * G::ROW_BYTES) : "memory");
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.hi) : "v"(cur[FI < NBASE ? FI : 0]), "n"((KS * 16 + 4) * G::ROW_BYTES) : "memory");
     } else {
-      int2v lo, hi;
-      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(cur[FI]), "n"((KS * 16) * G::ROW_BYTES) : "memory");
-      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(cur[FI]), "n"((KS * 16 + 4) * G::ROW_BYTES) : "memory");
-      r[0] = lo[0]; r[1] = lo[1]; r[2] = hi[0]; r[3] = hi[1];
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x0) : "v"(cur[0]), "n"((KS * 8 + 0) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x1) : "v"(cur[0]), "n"((KS * 8 + 1) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x2) : "v"(cur[0]), "n"((KS * 8 + 2) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x3) : "v"(cur[0]), "n"((KS * 8 + 3) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
     }
-    return r;
   }
-  static_assert((KSTEPS * 16 + 4) * G::ROW_BYTES < 65536 || KMAJOR, "LDS immediate offset is 16 bits");
-  static_assert(F * 32 * G::ROW_BYTES <= 65536 || !KMAJOR, "LDS immediate offset is 16 bits");
+  __device__ static __forceinline__ void pin_raw(Raw& r) {
+    if (KIND == OPK_KMAJOR) pin(r.q);
+    else if (KIND == OPK_MMAJOR) { pin(r.lo); pin(r.hi); }
+    else { pin(r.x0); pin(r.x1); pin(r.x2); pin(r.x3); }
+  }
+  __device__ static __forceinline__ int4v finish(const Raw& r) {
+    if (KIND == OPK_KMAJOR) return r.q;
+    int4v v;
+    if (KIND == OPK_MMAJOR) { v[0] = r.lo[0]; v[1] = r.lo[1]; v[2] = r.hi[0]; v[3] = r.hi[1]; }
+    else { v[0] = r.x0; v[1] = r.x1; v[2] = r.x2; v[3] = r.x3; }
+    return v;
+  }
+  static_assert(KIND != OPK_MMAJOR || (KSTEPS * 16 + 4) * G::ROW_BYTES < 65536, "LDS immediate offset is 16 bits");
+  static_assert(KIND != OPK_KMAJOR || F * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
+  static_assert(KIND != OPK_CROWK || (KSTEPS * 8) * G::ROW_BYTES + F * FRAG_ROWS * 4 <= 65536, "LDS immediate offset is 16 bits");
 };
 
-// Makes every later use of x depend on the point where pin() stands (no instruction is emitted).
-__device__ __forceinline__ void pin(int4v& x) { asm volatile("" : "+v"(x)); }
-
-template <int N>
-__device__ __forceinline__ void wait_lgkmcnt() {
-  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N < 15 ? N : 15) : "memory");
+// The A operand of a complex product D = A * B computed as the real product of the expanded
+// matrix [re -im; im re] with the interleaved B: every register of the fragment holds one complex
+// value (re in the low half, im in the high half); the even MFMA row of a pair needs (re, -im),
+// the odd one (im, re).  Dual numbers (re, du) need (re, 0) and (du, re)
+// (reference src/operator.jl:307-311 and :366-369).
+template <int FIX>
+__device__ __forceinline__ int4v expand_fixup(int4v x, int lane) {
+  if (FIX == FIX_NONE) return x;
+  const bool odd = (lane & 1) != 0;
+  const unsigned sel = odd ? 0x01000302u : 0x03020100u;                       // swap halves on odd rows
+  const unsigned flip = (FIX == FIX_COMPLEX && !odd) ? 0x80000000u : 0u;       // negate the imaginary half
+  const unsigned keep = (FIX == FIX_DUAL && !odd) ? 0x0000FFFFu : 0xFFFFFFFFu; // drop the dual half
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    unsigned v = __builtin_amdgcn_perm((unsigned)x[i], (unsigned)x[i], sel);
+    x[i] = (int)((v ^ flip) & keep);
+  }
+  return x;
 }
 
 template <int I, int N, class F>
@@ -177,9 +219,9 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 template <int KS, class RA, class RB, int FM, int FN>
-__device__ __forceinline__ void load_frags(const RA& ra, const RB& rb, int4v (&fa)[FM], int4v (&fb)[FN]) {
-  static_for<0, FM>([&](auto fi) { fa[decltype(fi)::value] = ra.template read<decltype(fi)::value, KS>(); });
-  static_for<0, FN>([&](auto fj) { fb[decltype(fj)::value] = rb.template read<decltype(fj)::value, KS>(); });
+__device__ __forceinline__ void load_frags(const RA& ra, const RB& rb, typename RA::Raw (&fa)[FM], typename RB::Raw (&fb)[FN]) {
+  static_for<0, FM>([&](auto fi) { ra.template read<decltype(fi)::value, KS>(fa[decltype(fi)::value]); });
+  static_for<0, FN>([&](auto fj) { rb.template read<decltype(fj)::value, KS>(fb[decltype(fj)::value]); });
 }
 
 template <typename T> struct Mfma;
@@ -215,10 +257,13 @@ __device__ __forceinline__ int4v transform_fragment(int4v f, const OpList& t0, c
   return __builtin_bit_cast(int4v, v);
 }
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, bool A_KMAJOR_, bool B_KMAJOR_, typename T_, bool FUSED_, bool GETT_ = false>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int A_KIND_, int B_KIND_, typename T_, bool FUSED_,
+          bool GETT_ = false, int FIX_ = FIX_NONE>
 struct MfmaGemmConfig {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
-  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, FUSED = FUSED_;
+  static constexpr int A_KIND = A_KIND_, B_KIND = B_KIND_, FIX = FIX_;
+  static constexpr bool FUSED = FUSED_;
+  static constexpr bool EXPAND_A = (FIX_ != FIX_NONE);   // complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
   static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / 16) % 2 == 0);   // cross-step fragment prefetch
   typedef T_ T;
@@ -227,8 +272,8 @@ struct MfmaGemmConfig {
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
   static constexpr int FM = WTM / 32, FN = WTN / 32;             // 32x32 accumulator blocks per wave
   static constexpr int KSTEPS = BK / 16;
-  typedef TileGeom<BM, BK, A_KMAJOR> GA;
-  typedef TileGeom<BN, BK, B_KMAJOR> GB;
+  typedef OperandGeom<BM, BK, A_KIND, EXPAND_A> GA;
+  typedef OperandGeom<BN, BK, B_KIND, false> GB;
   static constexpr int STAGE_BYTES = GA::BYTES + GB::BYTES;
   static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
   static constexpr int DMA_A = (GA::NDMA + NWAVES - 1) / NWAVES;   // per wave, per tile
@@ -239,6 +284,7 @@ struct MfmaGemmConfig {
   static_assert(STAGES >= 2, "at least two LDS stages");
   static_assert((STAGES - 2) * DMA_PER_TILE <= 63, "vmcnt is a 6-bit counter");
   static_assert(FM * FN > 0, "empty wave tile");
+  static_assert(!GETT || (A_KIND != OPK_CROWK && B_KIND != OPK_CROWK && FIX == FIX_NONE), "contractions are real");
 };
 
 template <class Cfg>
@@ -275,14 +321,26 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   KWalker walk;
   walk.reset();
   if constexpr (!Cfg::GETT) {
-    ga = (const char*)args.a + (Cfg::A_KMAJOR ? (long long)m0 * args.lda : (long long)m0) * 2;
-    gb = (const char*)args.b + (Cfg::B_KMAJOR ? (long long)n0 * args.ldb : (long long)n0) * 2;
-    a_step = (Cfg::A_KMAJOR ? (long long)BK : (long long)BK * args.lda) * 2;
-    b_step = (Cfg::B_KMAJOR ? (long long)BK : (long long)BK * args.ldb) * 2;
+    // tile origin and K step in 16-bit elements (lda / ldb are in 16-bit elements as well; an
+    // interleaved complex matrix counts two per complex number)
+    const long long a_org = Cfg::A_KIND == OPK_KMAJOR ? (long long)(Cfg::EXPAND_A ? m0 / 2 : m0) * args.lda : (long long)m0;
+    const long long b_org = Cfg::B_KIND == OPK_KMAJOR ? (long long)n0 * args.ldb : (Cfg::B_KIND == OPK_MMAJOR ? (long long)n0 : 2ll * n0);
+    ga = (const char*)args.a + a_org * 2;
+    gb = (const char*)args.b + b_org * 2;
+    a_step = (Cfg::A_KIND == OPK_KMAJOR ? (long long)BK : (long long)GA::LDS_ROWS * args.lda) * 2;
+    b_step = (Cfg::B_KIND == OPK_KMAJOR ? (long long)BK : (long long)GB::LDS_ROWS * args.ldb) * 2;
 #pragma unroll
-    for (int i = 0; i < DMA_A; ++i) offa[i] = dma_global_offset<BM, BK, Cfg::A_KMAJOR>(wave + i * NWAVES, lane, args.lda);
+    for (int i = 0; i < DMA_A; ++i) {
+      int row, col;
+      dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
+      offa[i] = (unsigned)(((long long)row * args.lda + col) * 2);
+    }
 #pragma unroll
-    for (int i = 0; i < DMA_B; ++i) offb[i] = dma_global_offset<BN, BK, Cfg::B_KMAJOR>(wave + i * NWAVES, lane, args.ldb);
+    for (int i = 0; i < DMA_B; ++i) {
+      int row, col;
+      dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
+      offb[i] = (unsigned)(((long long)row * args.ldb + col) * 2);
+    }
   } else {
     // element (m, k) of A lives at offM(m) + offK(k): the row part is a mixed-radix walk over the M
     // modes (done once per lane), the k part inside a tile is linear in the first K mode
@@ -290,16 +348,18 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     gb = (const char*)args.b;
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i) {
-      int r, k;
-      dma_lane_coords<BM, BK, Cfg::A_KMAJOR>(wave + i * NWAVES, lane, r, k);
+      int row, col;
+      dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
+      const int r = Cfg::A_KIND == OPK_KMAJOR ? row : col, k = Cfg::A_KIND == OPK_KMAJOR ? col : row;
       long long o0, o1;
       gett_offsets(args.gm, m0 + r, o0, o1);
       offa[i] = (unsigned)((o0 + (long long)k * args.gk.stride0[0]) * 2);
     }
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i) {
-      int r, k;
-      dma_lane_coords<BN, BK, Cfg::B_KMAJOR>(wave + i * NWAVES, lane, r, k);
+      int row, col;
+      dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
+      const int r = Cfg::B_KIND == OPK_KMAJOR ? row : col, k = Cfg::B_KIND == OPK_KMAJOR ? col : row;
       long long o0, o1;
       gett_offsets(args.gn, n0 + r, o0, o1);
       offb[i] = (unsigned)((o0 + (long long)k * args.gk.stride1[0]) * 2);
@@ -396,8 +456,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const bool xf_a = Cfg::FUSED && (args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0);
   const bool xf_b = Cfg::FUSED && (args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0);
 
-  typedef FragReader<BM, BK, Cfg::A_KMAJOR, FM> RA;
-  typedef FragReader<BN, BK, Cfg::B_KMAJOR, FN> RB;
+  typedef FragReader<BM, BK, Cfg::A_KIND, Cfg::EXPAND_A, FM> RA;
+  typedef FragReader<BN, BK, Cfg::B_KIND, false, FN> RB;
   RA ra;
   RB rb;
   ra.init(wm * Cfg::WTM, lane);
@@ -411,23 +471,32 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // Fragments are double-buffered: the LDS reads of the next k-step are in flight while the MFMAs
   // of the current one run.  LDS reads complete in order, so "at most NEXT outstanding" means that
   // the current set has arrived.
-  int4v fa[2][FM], fb[2][FN];
+  typename RA::Raw fa[2][FM];
+  typename RB::Raw fb[2][FN];
   constexpr int FRAG_OPS = FM * RA::OPS + FN * RB::OPS;
 
+  // runs after the wait that covers the reads of buffer ks & 1
   auto compute = [&](auto ks_c) {
     constexpr int ks = decltype(ks_c)::value;
+    int4v va[FM], vb[FN];
 #pragma unroll
-    for (int fi = 0; fi < FM; ++fi) pin(fa[ks & 1][fi]);
+    for (int fi = 0; fi < FM; ++fi) {
+      RA::pin_raw(fa[ks & 1][fi]);
+      va[fi] = expand_fixup<Cfg::FIX>(RA::finish(fa[ks & 1][fi]), lane);
+    }
 #pragma unroll
-    for (int fj = 0; fj < FN; ++fj) pin(fb[ks & 1][fj]);
+    for (int fj = 0; fj < FN; ++fj) {
+      RB::pin_raw(fb[ks & 1][fj]);
+      vb[fj] = RB::finish(fb[ks & 1][fj]);
+    }
     if (Cfg::FUSED) {
       if (xf_a) {
 #pragma unroll
-        for (int fi = 0; fi < FM; ++fi) fa[ks & 1][fi] = transform_fragment<T>(fa[ks & 1][fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
+        for (int fi = 0; fi < FM; ++fi) va[fi] = transform_fragment<T>(va[fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
       }
       if (xf_b) {
 #pragma unroll
-        for (int fj = 0; fj < FN; ++fj) fb[ks & 1][fj] = transform_fragment<T>(fb[ks & 1][fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
+        for (int fj = 0; fj < FN; ++fj) vb[fj] = transform_fragment<T>(vb[fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
       }
     }
 #pragma unroll
@@ -435,9 +504,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj) {
 #ifdef GK_ABLATE_MFMA
-        acc[fi][fj][0] += __builtin_bit_cast(float, fb[ks & 1][fj][0] ^ fa[ks & 1][fi][0]);
+        acc[fi][fj][0] += __builtin_bit_cast(float, vb[fj][0] ^ va[fi][0]);
 #else
-        acc[fi][fj] = Mfma<T>::run(fb[ks & 1][fj], fa[ks & 1][fi], acc[fi][fj]);
+        acc[fi][fj] = Mfma<T>::run(vb[fj], va[fi], acc[fi][fj]);
 #endif
       }
   };

@@ -150,9 +150,17 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
     every one of the 256 CUs a workgroup; the smallest dividing tile when none does."""
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         return NT(M=64, N=64, K=32)
-    if operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
-        return NT(M=64, N=64, K=32)
     M, N, K = gemm_shape["M"], gemm_shape["N"], gemm_shape["K"]
+    if operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
+        # complex tiles, in complex elements; every MFMA row pair is one complex row
+        fitting = [t for t, _ in _COMPLEX_TILES if M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0]
+        if operator.kind == Operator.MFMA_DUAL:
+            fitting = [t for t in fitting if t in ((64, 128, 32), (64, 64, 32))]
+        for t in fitting:
+            if (M // t[0]) * (N // t[1]) >= NUM_CUS:
+                return NT(M=t[0], N=t[1], K=t[2])
+        t = fitting[-1] if fitting else (64, 64, 32)
+        return NT(M=t[0], N=t[1], K=t[2])
     fitting = [t for t, _ in _MFMA_TILES if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
     if not fitting:
         return NT(M=64, N=64, K=32)
@@ -161,6 +169,9 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
             return NT(M=t[0], N=t[1], K=t[2])
     return NT(M=fitting[-1][0], N=fitting[-1][1], K=fitting[-1][2])
 
+
+# complex / dual tiles (complex elements) -> waves
+_COMPLEX_TILES = [((128, 256, 32), (2, 4)), ((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 
 # tiles of the vector-ALU kernel and of the bounds-checked MFMA kernel
 _FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2))]
@@ -173,6 +184,8 @@ def _default_waves(operator, block_shape, checked=False):
         table = _FPU_TILES
     elif operator.kind == Operator.MFMA and checked:
         table = _CHECKED_TILES
+    elif operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
+        table = _COMPLEX_TILES
     else:
         table = _MFMA_TILES
     for t, w in table:

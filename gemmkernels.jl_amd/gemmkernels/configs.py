@@ -218,6 +218,54 @@ def _config4b() -> Workload:
         kernel_name=kernel_name(conf, Kernel.matmul_singlestage))
 
 
+def complex_config(M, N, K, ta=False, tb=False, zero_c=True, dual=False, **kw):
+    """@get_wmma_complex_config / @get_wmma_dual_config of the reference (configs/configs.jl:385-490):
+    interleaved Complex{Float16} in global memory, planar in shared memory, Complex{Float32} out."""
+    il = lambda t: Layout.InterleavedRowMajor[Float16] if t else Layout.InterleavedColMajor[Float16]
+    sp = lambda t: Layout.Padded[Layout.SplitRowMajor[Float16], 8] if t else Layout.Padded[Layout.SplitColMajor[Float16], 8]
+    op = (Operator.MFMADualOp if dual else Operator.MFMAComplexOp)[16, 16, 16, Float16, Float32]
+    params = dict(gemm_shape=NT(M=M, N=N, K=K), operator=op,
+                  global_a_layout=il(ta), global_b_layout=il(tb),
+                  global_c_layout=Layout.Zero[Float32] if zero_c else Layout.InterleavedColMajor[Float32],
+                  global_d_layout=Layout.InterleavedColMajor[Float32],
+                  shared_a_layout=sp(ta), shared_b_layout=sp(tb),
+                  shared_c_layout=Layout.Zero[Float32] if zero_c else Layout.SplitColMajor[Float32],
+                  shared_d_layout=Layout.SplitColMajor[Float32],
+                  is_a_col_major=not ta, is_b_col_major=not tb)
+    params.update(kw)
+    return get_config(**params)
+
+
+def complex_matrix(seed, rows, cols):
+    """Interleaved Complex{Float16} matrix as a real array of shape (2, rows, cols), column-major:
+    re and im ~ U[-1,1) from one stream in storage order."""
+    return rng.matrix("upm1_f16", seed, (2, rows, cols))
+
+
+def _config4a() -> Workload:
+    M = N = K = 2048
+    conf = complex_config(M, N, K)
+
+    def host():
+        return dict(a=complex_matrix(4001, M, K), b=complex_matrix(4002, K, N), c=None)
+
+    def launch(h):
+        import torch
+        a, b = colmajor(h["a"]), colmajor(h["b"])
+        d = colmajor_empty((2, M, N), torch.float32)
+
+        def run():
+            matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+        return _attach(run, a=a, b=b, d=d, conf=conf)
+
+    return Workload(
+        name="config 4a",
+        description="config 4a: complex D = A*B, Complex{Float16} in (interleaved, re/im ~ U[-1,1)), Complex{Float32} out, "
+                    "M=N=K=2048, column-major NN; 8*N^3 real flop",
+        flops=8 * M * N * K, bytes=M * K * 4 + K * N * 4 + M * N * 8, bound="mfma", make_host=host, make_launch=launch,
+        kernel_name=kernel_name(conf, Kernel.matmul_pipelined))
+
+
 def _config5() -> Workload:
     ext = dict(a=64, b=64, c=64, d=64, e=64, f=64)
     conf, gmap = gett_config("aebf", "dfce", "abcd", ext)
@@ -255,4 +303,4 @@ def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     raise NotImplementedError(f"benchmark config {n}")
 
 
-_LATE_BUILDERS = {1: _config1, "4b": _config4b, 5: _config5}
+_LATE_BUILDERS = {1: _config1, "4a": _config4a, "4b": _config4b, 5: _config5}

@@ -41,6 +41,16 @@ def _leading_dim(x, layout) -> int:
     """Leading dimension, in elements, of a column-major device matrix."""
     if x is None or isinstance(x, int) or layout.kind in (Layout.ZERO, Layout.DIAGONAL, Layout.GETT_KIND):
         return 0
+    if layout.kind in (Layout.INTERLEAVED_COL_MAJOR, Layout.INTERLEAVED_ROW_MAJOR):
+        # interleaved complex data: a real tensor of logical shape (2, rows, cols), column-major,
+        # or a complex tensor of shape (rows, cols); the leading dimension counts complex elements
+        if x.is_complex():
+            if x.dim() != 2 or (x.size(0) > 1 and x.stride(0) != 1):
+                raise ConfigError("complex operands must be column-major matrices")
+            return int(x.stride(1)) if x.size(1) > 1 else max(int(x.size(0)), 1)
+        if x.dim() != 3 or x.size(0) != 2 or x.stride(0) != 1 or (x.size(1) > 1 and x.stride(1) != 2):
+            raise ConfigError("interleaved complex operands must have shape (2, rows, cols) in column-major order")
+        return int(x.stride(2)) // 2 if x.size(2) > 1 else max(int(x.size(1)), 1)
     if x.dim() != 2:
         raise ConfigError("matrix operands must be 2-dimensional")
     if x.size(0) > 1 and x.stride(0) != 1:

@@ -1,0 +1,92 @@
+"""GPU parity of the complex and dual-number GEMM (benchmark config 4a; reference
+configs/configs.jl:385-490, test sweep :656-695) against numpy complex128 and the CPU oracle.
+Tolerance: relative Frobenius error <= 1e-3 (FP16 in, FP32 accumulate)."""
+import numpy as np
+import pytest
+import torch
+
+import gemmkernels as gk
+from gemmkernels import Kernel, configs, rng
+import helpers
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def to_c128(x):            # (2, rows, cols) -> complex (rows, cols)
+    return x[0].astype(np.float64) + 1j * x[1].astype(np.float64)
+
+
+def run(conf, a, b, c, M, N):
+    ta, tb = gk.colmajor(a), gk.colmajor(b)
+    tc = None if c is None else gk.colmajor(c)
+    td = gk.colmajor_empty((2, M, N), torch.float32)
+    td.fill_(float("nan"))
+    gk.matmul(conf, ta, tb, tc, td, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    return gk.to_numpy(td)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("dims,block", [((128, 128, 64), (32, 64, 32)), ((128, 128, 128), (64, 64, 32)), ((128, 256, 96), (64, 128, 32)),
+                                        ((256, 512, 64), (128, 256, 32))])
+def test_complex_all_transposes(gpu, dims, block, ta, tb):
+    M, N, K = dims
+    conf = configs.complex_config(M, N, K, ta, tb, block_shape=gk.NT(M=block[0], N=block[1], K=block[2]))
+    a = configs.complex_matrix(61, K if ta else M, M if ta else K)
+    b = configs.complex_matrix(62, N if tb else K, K if tb else N)
+    print("case", dims, block, ta, tb, gk.kernel_name(conf, Kernel.matmul_pipelined), flush=True)
+    d = run(conf, a, b, None, M, N)
+    A = to_c128(a).T if ta else to_c128(a)          # 'T' is a plain transpose, no conjugation (src/matmul.jl:211-213)
+    B = to_c128(b).T if tb else to_c128(b)
+    assert oracle.rel_frobenius(to_c128(d), A @ B) <= TOL
+    # the CPU oracle restates WMMAComplexOp.mma (src/operator.jl:307-311)
+    ref = np.zeros((2, M, N), np.float32, order="F")
+    p = helpers.oracle_problem(conf, (a.shape[1], b.shape[1], M, M))
+    oracle.matmul(p, a, b, None, ref)
+    assert oracle.rel_frobenius(to_c128(d), to_c128(ref)) <= TOL
+
+
+def test_complex_identities_and_c(gpu):
+    M = N = K = 128
+    conf = configs.complex_config(M, N, K, block_shape=gk.NT(M=64, N=64, K=32))
+    a = configs.complex_matrix(71, M, K)
+    b = configs.complex_matrix(72, K, N)
+    a_real, b_real = a.copy(order="F"), b.copy(order="F")
+    a_real[1] = 0
+    b_real[1] = 0
+    d = run(conf, a_real, b_real, None, M, N)
+    assert np.all(d[1] == 0)                                   # real inputs => imaginary part exactly zero
+    bi = np.zeros((2, K, N), np.float16, order="F")
+    bi[1, np.arange(K), np.arange(K)] = 1                      # B = i * I  =>  A * B = (-im A, re A)
+    d = run(conf, a, bi, None, M, N)
+    assert np.array_equal(d[0], -a[1].astype(np.float32)) and np.array_equal(d[1], a[0].astype(np.float32))
+    conf_c = configs.complex_config(M, N, K, zero_c=False, block_shape=gk.NT(M=64, N=64, K=32))
+    c = rng.matrix("upm1_f32", 73, (2, M, N))
+    d = run(conf_c, a, b, c, M, N)
+    assert oracle.rel_frobenius(to_c128(d), to_c128(a) @ to_c128(b) + to_c128(c)) <= TOL
+
+
+@pytest.mark.parametrize("block", [(64, 64, 32), (64, 128, 32)])
+def test_dual_numbers(gpu, block):
+    """(re, du): re = a_re b_re, du = a_re b_du + a_du b_re (reference src/operator.jl:366-369)."""
+    M, N, K = 128, 256, 64
+    conf = configs.complex_config(M, N, K, dual=True, block_shape=gk.NT(M=block[0], N=block[1], K=block[2]))
+    a = configs.complex_matrix(81, M, K)
+    b = configs.complex_matrix(82, K, N)
+    d = run(conf, a, b, None, M, N)
+    a0, a1, b0, b1 = (x.astype(np.float64) for x in (a[0], a[1], b[0], b[1]))
+    assert oracle.rel_frobenius(d[0], a0 @ b0) <= TOL
+    assert oracle.rel_frobenius(d[1], a0 @ b1 + a1 @ b0) <= TOL
+
+
+def test_config4a_full_size(gpu):
+    w = configs.benchmark_config("4a")
+    r = w.prepare()
+    r()
+    torch.cuda.synchronize()
+    h = w.host()
+    d = to_c128(gk.to_numpy(r.d))
+    ref = (to_c128(h["a"]).astype(np.complex64) @ to_c128(h["b"]).astype(np.complex64))
+    assert oracle.rel_frobenius(d, ref) <= TOL
