@@ -26,7 +26,7 @@ PEAK_FP16_TFLOPS = 2516.6     # MI355X dense FP16/BF16 matrix peak (256 CU x 4 S
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the headline kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # summarised in profiles/ (None until measured)
-MEASURED_TRAFFIC_BYTES = None
+MEASURED_TRAFFIC_BYTES = 335_686_000   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131141.3 * 2.0 + 65536.0) KiB
 
 
 def parse_args():
@@ -35,6 +35,9 @@ def parse_args():
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--no-extras", action="store_true", help="skip the secondary configs and the CPU baseline")
+    p.add_argument("--copy-calibration", action="store_true",
+                   help="instead of the benchmark, run a plain 256 MiB device-to-device copy 10 times: the reference "
+                        "reading for the FETCH_SIZE / WRITE_SIZE counters of rocprofv3")
     return p.parse_args()
 
 
@@ -70,6 +73,15 @@ def main():
         print("bench.py: no GPU visible; the HIP library has no CPU fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
+
+    if args.copy_calibration:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")     # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 10}}))
+        return
 
     # ---------------- headline: config 2, NN ----------------
     wl = configs.benchmark_config(2, variant="NN")

@@ -122,6 +122,26 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   }
   key->dtype = c->global_a_layout.eltype;
   key->fused = (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT)) ? 1 : 0;
+  if (key->fused && t && (key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT)) {
+    // level 1 covers A / B hooks that are one exact 16-bit scale (or nothing); anything else needs
+    // the generic per-element path of level 2
+    auto simple = [&](int h0, int h1) {
+      const gk_transform& a0 = t->hook[h0];
+      const gk_transform& a1 = t->hook[h1];
+      int n = 0;
+      const gk_op* one = nullptr;
+      for (int i = 0; i < a0.n_ops && i < GK_MAX_OPS; ++i) if (a0.ops[i].kind != GK_T_IDENTITY) { ++n; one = &a0.ops[i]; }
+      for (int i = 0; i < a1.n_ops && i < GK_MAX_OPS; ++i) if (a1.ops[i].kind != GK_T_IDENTITY) { ++n; one = &a1.ops[i]; }
+      if (n == 0) return true;
+      if (n != 1 || one->kind != GK_T_SCALE || c->global_a_layout.eltype != GK_F16) return false;
+      return (float)(_Float16)one->p0 == one->p0;
+    };
+    if (!simple(GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A) || !simple(GK_HOOK_GLOBAL_TO_SHARED_B, GK_HOOK_SHARED_TO_REGS_B))
+      key->fused = 2;
+    if (c->global_a_layout.eltype != GK_F16) key->fused = 2;   // level 1 is compiled for FP16 only
+  }
+  if (key->fused && !t && c->global_a_layout.eltype != GK_F16 && (key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT))
+    key->fused = 2;
   return GK_OK;
 }
 
@@ -169,6 +189,22 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
       dst.n = out;
     }
   }
+  // one exact FP16 scale over the two load hooks of an operand -> packed multiply in the kernel
+  auto single_scale = [&](int h0, int h1, int* fast, float* scale) {
+    const gk::OpList& a0 = args->t[h0];
+    const gk::OpList& a1 = args->t[h1];
+    *fast = 0;
+    *scale = 1.0f;
+    if (a0.n + a1.n != 1) return;
+    const gk::OpList& one = a0.n ? a0 : a1;
+    if (one.kind[0] != GK_T_SCALE) return;
+    const float v = one.p0[0];
+    if ((float)(_Float16)v != v) return;
+    *fast = 1;
+    *scale = v;
+  };
+  single_scale(GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A, &args->fast_scale_a, &args->scale_a);
+  single_scale(GK_HOOK_GLOBAL_TO_SHARED_B, GK_HOOK_SHARED_TO_REGS_B, &args->fast_scale_b, &args->scale_b);
   auto copy_dim = [](const gk_gett_dim& s, gk::GettDim& d) {
     d.nmodes = s.nmodes;
     for (int i = 0; i < GK_MAX_MODES; ++i) {

@@ -81,6 +81,10 @@ struct GemmArgs {
   int a_kind, b_kind;             // gk_layout_kind of the global A / B layouts (diagonal, GETT ...)
   int cd_gett;                    // 1: C and D are addressed through gett.m / gett.n stride1
   OpList t[8];
+  // set by the host when the two load hooks of A (resp. B) amount to one multiplication by a
+  // constant that is exact in the operand's 16-bit type: done as a packed 16-bit multiply
+  int fast_scale_a, fast_scale_b;
+  float scale_a, scale_b;
   GettDim gm, gn, gk;
 };
 

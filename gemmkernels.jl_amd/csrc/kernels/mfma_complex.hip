@@ -18,7 +18,7 @@ int family_complex(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipS
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
       key.a_kmajor == akm_ && key.b_kmajor == bkm_ && key.variant == dual_) {                                             \
     typedef MfmaGemmConfig<2 * bm_, bn_, 2 * bk_, wm_, wn_, st_, (akm_ ? OPK_KMAJOR : OPK_CROWK),                          \
-                           (bkm_ ? OPK_KMAJOR : OPK_CROWK), _Float16, false, false, (dual_ ? FIX_DUAL : FIX_COMPLEX)> Cfg; \
+                           (bkm_ ? OPK_KMAJOR : OPK_CROWK), _Float16, 0, false, (dual_ ? FIX_DUAL : FIX_COMPLEX)> Cfg; \
     return run_instance<Cfg>(mfma_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
 #define GK_CPLX_T(bm_, bn_, bk_, wm_, wn_, st_, dual_, TAG)                                     \

@@ -257,12 +257,27 @@ __device__ __forceinline__ int4v transform_fragment(int4v f, const OpList& t0, c
   return __builtin_bit_cast(int4v, v);
 }
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int A_KIND_, int B_KIND_, typename T_, bool FUSED_,
+// One multiplication by a constant that is exact in FP16: the FP16 product rounded to nearest even
+// is the fp32 product (exact, 22 significant bits) rounded to FP16, so the packed FP16 multiply
+// gives the same bits as the generic path at a quarter of the instructions.
+__device__ __forceinline__ int4v scale_fragment_f16(int4v f, float scale) {
+  half8 v = __builtin_bit_cast(half8, f);
+  const _Float16 s = (_Float16)scale;
+  v = v * s;
+  return __builtin_bit_cast(int4v, v);
+}
+
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int A_KIND_, int B_KIND_, typename T_, int FUSE_,
           bool GETT_ = false, int FIX_ = FIX_NONE>
 struct MfmaGemmConfig {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr int A_KIND = A_KIND_, B_KIND = B_KIND_, FIX = FIX_;
-  static constexpr bool FUSED = FUSED_;
+  // 0: no transform and no bias; 1: C / D hooks, bias and at most one exact 16-bit scale on A and on B
+  // (a packed multiply per fragment); 2: arbitrary op lists on A and B as well (evaluated in fp32 per
+  // element inside the K loop: complete, and markedly slower)
+  static constexpr int FUSE = FUSE_;
+  static constexpr bool FUSED = FUSE_ != 0;
+  static constexpr bool FUSED_AB_GENERIC = FUSE_ == 2;
   static constexpr bool EXPAND_A = (FIX_ != FIX_NONE);   // complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
   static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / 16) % 2 == 0);   // cross-step fragment prefetch
@@ -455,6 +470,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 
   const bool xf_a = Cfg::FUSED && (args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0);
   const bool xf_b = Cfg::FUSED && (args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0);
+  // kept in registers for the whole K loop: a scalar load inside the loop would make the compiler
+  // wait for lgkmcnt(0), which also drains the LDS reads that are meant to stay in flight
+  const bool fast_a = std::is_same<T, _Float16>::value && args.fast_scale_a != 0;
+  const bool fast_b = std::is_same<T, _Float16>::value && args.fast_scale_b != 0;
+  const float scale_a = args.scale_a, scale_b = args.scale_b;
 
   typedef FragReader<BM, BK, Cfg::A_KIND, Cfg::EXPAND_A, FM> RA;
   typedef FragReader<BN, BK, Cfg::B_KIND, false, FN> RB;
@@ -491,12 +511,22 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     }
     if (Cfg::FUSED) {
       if (xf_a) {
+        if (fast_a) {
 #pragma unroll
-        for (int fi = 0; fi < FM; ++fi) va[fi] = transform_fragment<T>(va[fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
+          for (int fi = 0; fi < FM; ++fi) va[fi] = scale_fragment_f16(va[fi], scale_a);
+        } else if constexpr (Cfg::FUSED_AB_GENERIC) {
+#pragma unroll
+          for (int fi = 0; fi < FM; ++fi) va[fi] = transform_fragment<T>(va[fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
+        }
       }
       if (xf_b) {
+        if (fast_b) {
 #pragma unroll
-        for (int fj = 0; fj < FN; ++fj) vb[fj] = transform_fragment<T>(vb[fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
+          for (int fj = 0; fj < FN; ++fj) vb[fj] = scale_fragment_f16(vb[fj], scale_b);
+        } else if constexpr (Cfg::FUSED_AB_GENERIC) {
+#pragma unroll
+          for (int fj = 0; fj < FN; ++fj) vb[fj] = transform_fragment<T>(vb[fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
+        }
       }
     }
 #pragma unroll

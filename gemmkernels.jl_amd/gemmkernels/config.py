@@ -49,8 +49,15 @@ class Config:
         return "\n".join(f"{(f.name + ':').ljust(width)}{getattr(self, f.name)}" for f in fields(self)) + "\n"
 
     def to_c(self, lda: int = 0, ldb: int = 0, ldc: int = 0, ldd: int = 0) -> _lib.gk_config:
-        """Lower to the POD of the C ABI; leading dimensions come from the arrays of the call."""
+        """Lower to the POD of the C ABI; leading dimensions come from the arrays of the call.
+        The result is cached per set of leading dimensions (a Config is immutable once built)."""
+        cache = self.__dict__.setdefault("_c_cache", {})
+        key = (lda, ldb, ldc, ldd)
+        hit = cache.get(key)
+        if hit is not None:
+            return hit
         c = _lib.gk_config()
+        cache[key] = c
 
         def shape(dst, src):
             dst.M, dst.N, dst.K = int(src.get("M", 0)), int(src.get("N", 0)), int(src.get("K", 0))

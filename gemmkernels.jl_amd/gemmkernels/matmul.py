@@ -58,10 +58,19 @@ def _leading_dim(x, layout) -> int:
     return int(x.stride(1)) if x.size(1) > 1 else max(int(x.size(0)), 1)
 
 
+_IDENTITY = Transform.Elementwise()
+_DEFAULT_EPILOGUE = Epilogue.Default()
+_lowered = {}
+
+
 def lower_transforms(transforms: dict) -> Optional[_lib.gk_transforms]:
     if all(t.is_identity for t in transforms.values()):
         return None
-    out = _lib.gk_transforms()
+    key = tuple(transforms[name].ops for name in _HOOKS)
+    hit = _lowered.get(key)
+    if hit is not None:
+        return hit
+    out = _lowered[key] = _lib.gk_transforms()
     for i, name in enumerate(_HOOKS):
         ops = transforms[name].ops
         out.hook[i].n_ops = len(ops)
@@ -86,8 +95,8 @@ def matmul(conf: Config, a, b, c, d, *,
                  transform_shared_to_regs_b=transform_shared_to_regs_b,
                  transform_shared_to_regs_c=transform_shared_to_regs_c,
                  transform_regs_to_shared_d=transform_regs_to_shared_d)
-    transforms = {k: (Transform.Elementwise() if v is None else v) for k, v in given.items()}
-    epilogue = Epilogue.Default() if epilogue is None else epilogue
+    transforms = {k: (_IDENTITY if v is None else v) for k, v in given.items()}
+    epilogue = _DEFAULT_EPILOGUE if epilogue is None else epilogue
 
     cconf = conf.to_c(_leading_dim(a, conf.global_a_layout), _leading_dim(b, conf.global_b_layout),
                       _leading_dim(c, conf.global_c_layout), _leading_dim(d, conf.global_d_layout))
