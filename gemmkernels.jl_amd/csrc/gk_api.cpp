@@ -397,6 +397,18 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
     }
   }
 
+  // element types of C and D: fp32 everywhere; the real MFMA kernels also read and write 16-bit
+  // matrices (fp32 accumulation, one rounding at the store; the reference's F16 -> F16 WMMA
+  // configuration, configs/configs.jl:574)
+  {
+    const bool cd16_ok = op.kind == GK_OP_MFMA && c->global_a_layout.kind != GK_LAYOUT_DIAGONAL;
+    auto cd_ok = [&](int dt) { return dt == GK_F32 || (cd16_ok && (dt == GK_F16 || dt == GK_BF16)); };
+    if (!cd_ok(c->global_d_layout.eltype))
+      return fail(GK_ERR_UNSUPPORTED, "element type %d of D is not available with this operator", c->global_d_layout.eltype);
+    if (c->global_c_layout.kind != GK_LAYOUT_ZERO && !cd_ok(c->global_c_layout.eltype))
+      return fail(GK_ERR_UNSUPPORTED, "element type %d of C is not available with this operator", c->global_c_layout.eltype);
+  }
+
   // src/matmul.jl:34-36 (decidable from the configuration alone, so it is checked before the
   // instance lookup)
   if (kernel != GK_KERNEL_SINGLESTAGE && b.K < 2 * os.K)

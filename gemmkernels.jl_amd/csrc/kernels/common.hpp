@@ -226,6 +226,19 @@ __device__ __forceinline__ void apply_list_regs(const OpList& t, float (&x)[COUN
   }
 }
 
+// One element of C / D in the element type the layout names (accumulators are fp32; a 16-bit D gets
+// one rounding, at the store).
+__device__ __forceinline__ float load_cd(const void* base, int dtype, long long idx) {
+  if (dtype == DT_F32) return ((const float*)base)[idx];
+  if (dtype == DT_F16) return (float)((const _Float16*)base)[idx];
+  return (float)((const __bf16*)base)[idx];
+}
+__device__ __forceinline__ void store_cd(void* base, int dtype, long long idx, float x) {
+  if (dtype == DT_F32) ((float*)base)[idx] = x;
+  else if (dtype == DT_F16) ((_Float16*)base)[idx] = (_Float16)x;
+  else ((__bf16*)base)[idx] = (__bf16)x;
+}
+
 // waits and barriers placed by hand around the LDS-DMA pipeline
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

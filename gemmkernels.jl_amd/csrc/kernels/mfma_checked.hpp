@@ -58,7 +58,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
         float c = 0.0f;
         const int r = mrow + 32 * fi, cc = ncol + 32 * fj + 8 * (v / 4) + (v % 4);
         if (args.c_mode != 0) {
-          if (r < args.M && cc < args.N) c = ((const float*)args.c)[r + (long long)cc * args.ldc];
+          if (r < args.M && cc < args.N) c = load_cd(args.c, args.c_dtype, r + (long long)cc * args.ldc);
           c = apply_list(args.t[H_GL2SH_C], c);
           c = apply_list(args.t[H_SH2RF_C], c);
         }
@@ -124,7 +124,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
     __syncthreads();
   }
 
-  float* D = (float*)args.d;
 #pragma unroll
   for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
@@ -136,7 +135,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
         if (args.epi_kind == 1) x = x + args.bias[cc < args.N ? cc : 0];
         else if (args.epi_kind == 2) x = x + args.bias[r < args.M ? r : 0];
         x = apply_list(args.t[H_SH2GL_D], x);
-        if (r < args.M && cc < args.N) D[r + (long long)cc * args.ldd] = x;
+        if (r < args.M && cc < args.N) store_cd(args.d, args.d_dtype, r + (long long)cc * args.ldd, x);
       }
 }
 

@@ -439,9 +439,21 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj) {
-        const float* cp = (const float*)args.c + cd_offset(fi, fj, args.ldc);
+        const long long off = cd_offset(fi, fj, args.ldc);
+        const long long ns = cd_nstride(args.ldc);
+        if (args.c_dtype == DT_F32) {
+          const float* cp = (const float*)args.c + off;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[fi][fj][v] = cp[(long long)(8 * (v / 4) + (v % 4)) * cd_nstride(args.ldc)];
+          for (int v = 0; v < 16; ++v) acc[fi][fj][v] = cp[(long long)(8 * (v / 4) + (v % 4)) * ns];
+        } else if (args.c_dtype == DT_F16) {
+          const _Float16* cp = (const _Float16*)args.c + off;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[fi][fj][v] = (float)cp[(long long)(8 * (v / 4) + (v % 4)) * ns];
+        } else {
+          const __bf16* cp = (const __bf16*)args.c + off;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[fi][fj][v] = (float)cp[(long long)(8 * (v / 4) + (v % 4)) * ns];
+        }
       }
     if (Cfg::FUSED) {
       if (args.t[H_GL2SH_C].n > 0 || args.t[H_SH2RF_C].n > 0) {
@@ -611,7 +623,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
     for (int fj = 0; fj < FN; ++fj) {
-      float* dp = (float*)args.d + cd_offset(fi, fj, args.ldd);
+      const long long off = cd_offset(fi, fj, args.ldd);
+      const long long ns = cd_nstride(args.ldd);
       float x[16];
 #pragma unroll
       for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
@@ -627,9 +640,20 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
         apply_list_regs<16>(args.t[H_SH2GL_D], x);
       }
+      // the accumulator is rounded once, to the element type of D
+      if (args.d_dtype == DT_F32) {
+        float* dp = (float*)args.d + off;
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        dp[(long long)(8 * (v / 4) + (v % 4)) * cd_nstride(args.ldd)] = x[v];
+        for (int v = 0; v < 16; ++v) dp[(long long)(8 * (v / 4) + (v % 4)) * ns] = x[v];
+      } else if (args.d_dtype == DT_F16) {
+        _Float16* dp = (_Float16*)args.d + off;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dp[(long long)(8 * (v / 4) + (v % 4)) * ns] = (_Float16)x[v];
+      } else {
+        __bf16* dp = (__bf16*)args.d + off;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dp[(long long)(8 * (v / 4) + (v % 4)) * ns] = (__bf16)x[v];
+      }
     }
 #ifdef GK_PHASE_TRACE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -79,9 +79,11 @@ def run_gpu(conf, a, b, c, d_shape, d_dtype=None, transforms=None, epilogue_cls=
     """Same inputs through the product: gemmkernels.matmul -> C ABI -> HIP kernel."""
     import torch
     from gemmkernels import Kernel
-    ta = None if a is None else gk.colmajor(a)
-    tb = None if b is None else gk.colmajor(b)
-    tc = None if c is None else gk.colmajor(c)
+    def up(x, layout):     # uint16 arrays are bfloat16 bit patterns
+        if x is None:
+            return None
+        return gk.colmajor(x, torch.bfloat16 if (x.dtype == np.uint16 and layout.T.name == "BFloat16") else None)
+    ta, tb, tc = up(a, conf.global_a_layout), up(b, conf.global_b_layout), up(c, conf.global_c_layout)
     td = tc if alias_cd else gk.colmajor_empty(d_shape, d_dtype or torch.float32)
     if not alias_cd:
         td.fill_(float("nan"))

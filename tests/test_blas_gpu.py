@@ -42,6 +42,21 @@ def test_matmatmul(gpu, dims, ta, tb, dtype):
     assert err <= (1e-3 if dtype == np.float16 else 1e-5), err
 
 
+@pytest.mark.parametrize("dims", [(256, 256, 256), (1000, 200, 72)])
+def test_matmatmul_f16_output(gpu, dims):
+    """FP16 A, B and C (reference test/blas.jl:15, the (Float16, Float16, Float16) row): FP32
+    accumulation on the matrix cores, beta in FP16, one rounding at the store."""
+    M, N, K = dims
+    a, b, c = operands(M, N, K, False, True, np.float16, 300)
+    c = c.astype(np.float16)
+    A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
+    gk.matmatmul_(C, "N", "T", A, B, 0.5, 0.25)
+    torch.cuda.synchronize()
+    out = gk.to_numpy(C)
+    assert out.dtype == np.float16
+    assert oracle.rel_frobenius(out, oracle.gemm_f64(a, b, c, 0.5, 0.25, False, True)) <= 1e-3
+
+
 def test_fp32_is_bit_exact_against_the_sequential_fma_chain(gpu):
     """FPUOp semantics: one fp32 fma per k in ascending order (reference src/operator.jl:139-153);
     the oracle's C restatement is that loop, so the results must be identical."""

@@ -90,6 +90,9 @@ ERROR_CASES = [
     ("block not a multiple of compute_warp (src/config.jl:270)", dict(block_shape=NT(M=128, N=128, K=64), compute_warp=NT(M=96, N=64, K=16)), _lib.GK_ERR_TILE_MULTIPLE),
     ("compute_warp not a multiple of the operator (src/config.jl:271)", dict(block_shape=NT(M=128, N=128, K=64), compute_warp=NT(M=64, N=16, K=16), warps_per_block=16), _lib.GK_ERR_TILE_MULTIPLE),
     ("gemm not a multiple of the block, aligned layouts (src/config.jl:272-275)", dict(gemm_shape=NT(M=1000, N=1024, K=1024), block_shape=NT(M=128, N=128, K=64)), _lib.GK_ERR_TILE_MULTIPLE),
+    ("FP64 D with the matrix cores", dict(global_d_layout=ACM[gk.Float64]), _lib.GK_ERR_UNSUPPORTED),
+    ("FP16 D on the vector ALUs", dict(operator=Operator.FPUOp[8, 8, 1, 8, 8, 1, F32, F32], block_shape=NT(M=64, N=64, K=32),
+                                       global_a_layout=ACM[F32], global_b_layout=ACM[F32], global_d_layout=ACM[F16]), _lib.GK_ERR_UNSUPPORTED),
     ("no compiled instance", dict(block_shape=NT(M=192, N=192, K=64), compute_warp=NT(M=96, N=96, K=16), warps_per_block=4, gemm_shape=NT(M=384, N=384, K=128)), _lib.GK_ERR_UNSUPPORTED),
     ("warps_per_block disagrees with block / compute_warp", dict(block_shape=NT(M=128, N=128, K=64), compute_warp=NT(M=64, N=64, K=16), warps_per_block=8), _lib.GK_ERR_UNSUPPORTED),
 ]

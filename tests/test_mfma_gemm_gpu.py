@@ -149,3 +149,62 @@ def test_full_size_4096(gpu, ta, tb):
     conf0 = make_config(M, N, K, ta, tb, (256, 256, 64), (2, 4), zero_c=True)
     d0 = helpers.run_gpu(conf0, a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
     assert oracle.rel_frobenius(d - d0, c) <= 1e-4
+
+
+@pytest.mark.parametrize("block,waves", [((256, 256, 64), (2, 4)), ((128, 128, 64), (2, 2)), ((64, 64, 32), (1, 1))])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+def test_f16_c_and_d(gpu, block, waves, ta, tb):
+    """FP16 C and D with FP32 accumulation (the reference's F16 -> F16 WMMA configuration,
+    configs/configs.jl:574, accumulates in FP16; one rounding at the store is at least as accurate)."""
+    import torch
+    BM, BN, BK = block
+    M, N, K = 2 * BM, BN, 4 * BK
+    la = Layout.UnsafeAlignedRowMajor[Float16] if ta else Layout.UnsafeAlignedColMajor[Float16]
+    lb = Layout.UnsafeAlignedRowMajor[Float16] if tb else Layout.UnsafeAlignedColMajor[Float16]
+    conf = gk.get_config(
+        gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=BM, N=BN, K=BK), warps_per_block=waves[0] * waves[1],
+        compute_warp=NT(M=BM // waves[0], N=BN // waves[1], K=16), operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+        global_a_layout=la, global_b_layout=lb, global_c_layout=Layout.UnsafeAlignedColMajor[Float16],
+        global_d_layout=Layout.UnsafeAlignedColMajor[Float16], is_a_col_major=not ta, is_b_col_major=not tb)
+    a, b, _ = inputs(M, N, K, ta, tb, 2300)
+    c = rng.matrix("upm1_f16", 2304, (M, N))
+    d = helpers.run_gpu(conf, a, b, c, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
+    assert d.dtype == np.float16
+    ref = helpers.run_oracle(conf, a, b, c, (M, N), d_dtype=np.float16)
+    assert oracle.rel_frobenius(d, ref) <= TOL
+    # a different summation order moves a result across an FP16 rounding boundary only rarely, and then by one ulp
+    differ = d != ref
+    assert differ.mean() < 0.02
+    assert np.all(np.abs(d.astype(np.float64) - ref.astype(np.float64))[differ] <= np.spacing(np.abs(ref).astype(np.float16))[differ])
+    assert oracle.rel_frobenius(d, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= TOL
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("d16", [False, True])
+def test_bf16(gpu, ta, tb, d16):
+    """BFloat16 multiplicands (v_mfma_f32_32x32x16_bf16), FP32 or BFloat16 C / D."""
+    import torch
+    from gemmkernels import BFloat16
+    M, N, K = 256, 384, 320
+    block, waves = (128, 128, 64), (2, 2)
+    a = gk.bf16_bits(rng.matrix("upm1_f32", 2401, (K, M) if ta else (M, K)))
+    b = gk.bf16_bits(rng.matrix("upm1_f32", 2402, (N, K) if tb else (K, N)))
+    c32 = rng.matrix("upm1_f32", 2403, (M, N))
+    c = gk.bf16_bits(c32) if d16 else c32
+    CD = BFloat16 if d16 else Float32
+    la = Layout.UnsafeAlignedRowMajor[BFloat16] if ta else Layout.UnsafeAlignedColMajor[BFloat16]
+    lb = Layout.UnsafeAlignedRowMajor[BFloat16] if tb else Layout.UnsafeAlignedColMajor[BFloat16]
+    conf = gk.get_config(
+        gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=block[0], N=block[1], K=block[2]), warps_per_block=4,
+        compute_warp=NT(M=64, N=64, K=16), operator=Operator.MFMAOp[32, 32, 16, BFloat16, Float32],
+        global_a_layout=la, global_b_layout=lb, global_c_layout=Layout.UnsafeAlignedColMajor[CD],
+        global_d_layout=Layout.UnsafeAlignedColMajor[CD], is_a_col_major=not ta, is_b_col_major=not tb)
+    d = helpers.run_gpu(conf, a, b, c, (M, N), d_dtype=torch.bfloat16 if d16 else torch.float32, kernel=Kernel.matmul_pipelined)
+    ref = helpers.run_oracle(conf, a, b, c, (M, N), d_dtype=np.uint16 if d16 else np.float32)
+    if d16:
+        ref = gk.bf16_values(ref)
+    tol = 4e-3 if d16 else TOL        # a BFloat16 result carries 2^-9 relative rounding per element
+    assert oracle.rel_frobenius(d, ref) <= tol
+    A, B = gk.bf16_values(a), gk.bf16_values(b)
+    C = gk.bf16_values(c) if d16 else c
+    assert oracle.rel_frobenius(d, oracle.gemm_f64(A, B, C, 1.0, 1.0, ta, tb)) <= tol
