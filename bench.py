@@ -58,6 +58,21 @@ def time_launches(fn, steps, warmup):
     return start.elapsed_time(stop) * 1e3 / steps, wall
 
 
+def launch_distribution(fn, launches=40):
+    """Min and median duration in microseconds of single launches, each bracketed by its own pair of events."""
+    import torch
+    times = []
+    for _ in range(launches):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        stop.record()
+        stop.synchronize()
+        times.append(start.elapsed_time(stop) * 1e3)
+    times.sort()
+    return times[0], times[len(times) // 2]
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -109,6 +124,12 @@ def main():
     }
 
     if not args.no_extras:
+        lo, med = launch_distribution(run)
+        result["single_launch_us"] = {"min": round(lo, 2), "median": round(med, 2), "launches": 40}
+        try:
+            result["shader_clock_mhz_after_run"] = int(torch.cuda.clock_rate())
+        except Exception:       # needs the amdsmi python module
+            pass
         # ---------------- the other transposes and configs (outside the timed region) ----------------
         extras = {}
         for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4b", None), (5, None)]:
@@ -127,6 +148,34 @@ def main():
                 torch.cuda.empty_cache()
             except Exception as e:  # a config that is not built yet must not hide the headline number
                 extras[f"config {cfg}{' ' + variant if variant else ''}"] = {"error": f"{type(e).__name__}: {e}"}
+        # config 4b is bandwidth bound: a second figure with four buffer sets (384 MiB, more than the
+        # 256 MiB of last-level cache) used in rotation, so that no launch finds its operands cached
+        try:
+            w = configs.benchmark_config("4b")
+            runs = [w.prepare() for _ in range(4)]
+            state = {"i": 0}
+
+            def rotate():
+                runs[state["i"] & 3]()
+                state["i"] += 1
+            u, _ = time_launches(rotate, 48, 8)
+            extras["config 4b"]["rotating_buffers"] = {"us": round(u, 2), "GB/s": round(w.bytes / u / 1e3, 1),
+                                                       "frac_of_hbm_peak": round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)}
+            del runs
+            torch.cuda.empty_cache()
+        except Exception as e:
+            extras.setdefault("config 4b", {})["rotating_buffers"] = {"error": f"{type(e).__name__}: {e}"}
+        # the vendor library on the headline shape, for orientation only: FP16 in, FP16 out, no C read
+        # (torch.mm -> hipBLASLt), so it moves 96 MiB less per launch than config 2 does
+        try:
+            x = torch.randn(4096, 4096, device="cuda").to(torch.float16)
+            y = torch.randn(4096, 4096, device="cuda").to(torch.float16)
+            out = torch.empty(4096, 4096, device="cuda", dtype=torch.float16)
+            u, _ = time_launches(lambda: torch.mm(x, y, out=out), 50, 10)
+            extras["vendor_library_fp16_out_no_c"] = {"us": round(u, 2), "TFLOP/s": round(wl.flops / u / 1e6, 2)}
+            del x, y, out
+        except Exception as e:
+            extras["vendor_library_fp16_out_no_c"] = {"error": f"{type(e).__name__}: {e}"}
         result["other_configs"] = extras
 
         # ---------------- CPU baseline: the reference's own CPU path is BLAS sgemm on host arrays ----------------

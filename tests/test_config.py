@@ -166,3 +166,20 @@ def test_create_config_choices():
     assert conf.global_c_layout == Layout.Zero[F32] and conf.shared_c_layout == Layout.Zero[F32]
     with pytest.raises(DimensionMismatch):                                           # :75-77
         create_config(F16, (128, 64), (1, 128), False, F16, (128, 128), (1, 128), False, F32, (128, 128), (1, 128), float, False, float, False, None)
+
+
+def test_every_tile_of_the_python_tables_has_a_compiled_instance():
+    """The tile tables the defaults are drawn from and the instances compiled into the library
+    must not drift apart: every entry resolves to a kernel name."""
+    from gemmkernels import config as cfg, configs
+    for (bm, bn, bk), (wm, wn) in cfg._MFMA_TILES:
+        conf = configs.mfma_config(2 * bm, 2 * bn, 4 * bk, block_shape=(bm, bn, bk), warps_per_block=wm * wn,
+                                   compute_warp=NT(M=bm // wm, N=bn // wn, K=16))
+        assert f"{bm}x{bn}x{bk}_w{wm}x{wn}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    for (bm, bn, bk), (wm, wn) in cfg._FPU_TILES:
+        conf = gk.get_config(gemm_shape=NT(M=2 * bm, N=2 * bn, K=2 * bk), block_shape=NT(M=bm, N=bn, K=bk),
+                             operator=Operator.FPUOp[8, 8, 1, 8, 8, 1, F32, F32], global_a_layout=ACM[F32], global_c_layout=ACM[F32])
+        assert f"{bm}x{bn}x{bk}_w{wm}x{wn}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    for (bm, bn, bk), (wm, wn) in cfg._COMPLEX_TILES:
+        conf = configs.complex_config(2 * bm, 2 * bn, 4 * bk, block_shape=NT(M=bm, N=bn, K=bk))
+        assert f"{bm}x{bn}x{bk}_w{wm}x{wn}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
