@@ -530,6 +530,36 @@ int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const
   return GK_OK;
 }
 
+int gk_heuristic_block_shape(const gk_layout* sa, const gk_layout* sb, const gk_layout* sc, const gk_layout* sd, gk_shape* out) {
+  if (!sa || !sb || !sc || !sd || !out) return fail(GK_ERR_INVALID_ARGUMENT, "NULL argument");
+  const gk_layout* ls[4] = {sa, sb, sc, sd};
+  for (const gk_layout* l : ls)
+    if (!valid_layout_kind(l->kind) || dtype_size(l->eltype) == 0) return fail(GK_ERR_INVALID_ARGUMENT, "unknown layout kind or element type");
+  // bytes of a rows x cols tile in a shared layout: Layout.physical_size (src/layout.jl:76, 113, 152,
+  // 194, 246, 342-345, 381-383): padding goes to the leading physical dimension, planar complex
+  // layouts hold two planes, interleaved ones two reals per element
+  auto nbytes = [](const gk_layout* l, long long rows, long long cols) -> long long {
+    const bool row = is_row_major(l->kind) || l->kind == GK_LAYOUT_SPLIT_ROW_MAJOR;
+    long long lead = row ? cols : rows, other = row ? rows : cols;
+    long long n = (lead + l->pad) * other;
+    if (l->kind == GK_LAYOUT_SPLIT_COL_MAJOR || l->kind == GK_LAYOUT_SPLIT_ROW_MAJOR ||
+        l->kind == GK_LAYOUT_INTERLEAVED_COL_MAJOR || l->kind == GK_LAYOUT_INTERLEAVED_ROW_MAJOR)
+      n *= 2;
+    return n * dtype_size(l->eltype);
+  };
+  const long long limit = 64 * 1024;
+  long long M = 1, N = 1, K = 1;
+  for (;;) {     // src/config.jl:104-110
+    const long long m2 = (M == N) ? 2 * M : M, n2 = (M == N) ? N : 2 * N;
+    const long long cd = std::max(nbytes(sc, m2, n2), nbytes(sd, m2, n2));
+    if (cd > limit) break;
+    M = m2; N = n2;
+  }
+  while (nbytes(sa, M, 2 * K) + nbytes(sb, 2 * K, N) <= limit) K *= 2;   // src/config.jl:112-117
+  out->M = (int32_t)M; out->N = (int32_t)N; out->K = (int32_t)K;
+  return GK_OK;
+}
+
 int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
               const gk_epilogue* epilogue, int32_t kernel, void* stream) {
   gk::InstanceKey key;

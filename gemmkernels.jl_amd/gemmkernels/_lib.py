@@ -100,6 +100,8 @@ _SIGNATURES = {
                                       ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]),
     "gk_shmem_size": (ctypes.c_int64, [ctypes.POINTER(gk_config), ctypes.c_int32]),
     "gk_threads_per_block": (ctypes.c_int32, [ctypes.POINTER(gk_config)]),
+    "gk_heuristic_block_shape": (ctypes.c_int, [ctypes.POINTER(gk_layout), ctypes.POINTER(gk_layout), ctypes.POINTER(gk_layout),
+                                                ctypes.POINTER(gk_layout), ctypes.POINTER(gk_shape)]),
     "gk_kernel_name": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.POINTER(gk_transforms), ctypes.POINTER(gk_epilogue),
                                       ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]),
     "gk_matmul": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

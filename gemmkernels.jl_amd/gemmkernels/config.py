@@ -224,6 +224,12 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
 
     tile_sized = any(require_tile_sized_global(l) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
     block_shape = params.get("block_shape")
+    if block_shape is None and global_a_layout.kind == Layout.DIAGONAL and gemm_shape.M % 64 == 0 and gemm_shape.N % 64 == 0:
+        # a diagonal A makes the product a streaming pass over B and D: many small workgroups keep more
+        # memory requests in flight than a few large ones (measured against HBM with rotating buffers)
+        block_shape = NT(M=64, N=64, K=32 if gemm_shape.K % 32 == 0 else gemm_shape.K)
+        params.setdefault("warps_per_block", 4)
+        params.setdefault("compute_warp", NT(M=32, N=32, K=16))
     block_shape = default_block_shape(operator, gemm_shape, tile_sized) if block_shape is None else NT(block_shape)
     op_shape = Operator.shape(operator)
 

@@ -111,6 +111,16 @@ function validate(conf::GkConfig, kernel::Symbol = :matmul_singlestage)
     nothing
 end
 
+"`heuristic_block_shape` of the reference (src/config.jl:84-120), answered by the library."
+function heuristic_block_shape(shared_a::Type, shared_b::Type, shared_c::Type, shared_d::Type)
+    out = Ref(GkShape(0, 0, 0))
+    rc = ccall((:gk_heuristic_block_shape, libgk[]), Cint,
+               (Ref{GkLayout}, Ref{GkLayout}, Ref{GkLayout}, Ref{GkLayout}, Ref{GkShape}),
+               Ref(lower_layout(shared_a)), Ref(lower_layout(shared_b)), Ref(lower_layout(shared_c)), Ref(lower_layout(shared_d)), out)
+    rc == 0 || throw(ConfigError(last_error(), rc))
+    (M = Int(out[].M), N = Int(out[].N), K = Int(out[].K))
+end
+
 function __init__()
     sizes = (sizeof(GkConfig), sizeof(GkLayout), sizeof(GkOperator), sizeof(GkTransforms), sizeof(GkEpilogue), sizeof(GkGett))
     isfile(libgk[]) || return

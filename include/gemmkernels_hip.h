@@ -228,6 +228,13 @@ int64_t gk_shmem_size(const gk_config* conf, int32_t kernel);
 /* Threads per block of the launch (src/matmul.jl:24, with 64-lane wavefronts). */
 int32_t gk_threads_per_block(const gk_config* conf);
 
+/* heuristic_block_shape (src/config.jl:84-120), the reference's own rule, unchanged: M and N double
+ * in turn while a C / D tile in its shared layout fits 64 KiB, then K doubles while the A and B tiles
+ * fit 64 KiB together.  Only kind, eltype and pad of the four shared layouts are read.  This is the
+ * reference-compatible answer; gk_matmul itself runs the tiles compiled for the MI355X. */
+int gk_heuristic_block_shape(const gk_layout* shared_a, const gk_layout* shared_b, const gk_layout* shared_c,
+                             const gk_layout* shared_d, gk_shape* block_shape);
+
 /* Name of the kernel instance gk_matmul would launch, for logs and profiles. */
 int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const gk_epilogue* epilogue,
                    int32_t kernel, char* buf, size_t n);

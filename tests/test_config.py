@@ -24,6 +24,35 @@ def test_heuristic_block_shape_reference_answers():
     assert gk.heuristic_block_shape(Layout.Padded[ARM[F16], 8], pb, ACM[F32], ACM[F32]) == NT(M=128, N=128, K=64)
 
 
+def test_heuristic_block_shape_of_the_library_matches_the_python_mirror():
+    """gk_heuristic_block_shape (what a Julia binding would call) against gk.heuristic_block_shape."""
+    import ctypes
+    from gemmkernels import ComplexF16, ComplexF32
+
+    def c_layout(l):
+        out = _lib.gk_layout()
+        out.kind, out.eltype, out.pad, out.ld = l.kind, l.T.code, l.pad, 0
+        return out
+
+    SCM, SRM = Layout.SplitColMajor, Layout.SplitRowMajor
+    cases = [
+        (Layout.Padded[ACM[F16], 8], Layout.Padded[ACM[F16], 8], ACM[F32], ACM[F32]),
+        (Layout.Padded[ACM[F16], 8], Layout.Padded[ACM[F16], 8], ACM[F16], ACM[F16]),
+        (Layout.Padded[ARM[F16], 8], Layout.Padded[ARM[F16], 8], ACM[F32], ACM[F32]),
+        (ACM[F32], ACM[F32], ACM[F32], ACM[F32]),
+        (ACM[gk.Float64], ARM[gk.Float64], ACM[gk.Float64], ACM[gk.Float64]),
+        (Layout.Padded[SCM[F16], 8], Layout.Padded[SCM[F16], 8], SCM[F32], SCM[F32]),     # configs/configs.jl:397-401
+        (Layout.Padded[SRM[F16], 8], Layout.Padded[SCM[F16], 8], SCM[F32], SCM[F32]),
+    ]
+    for layouts in cases:
+        want = gk.heuristic_block_shape(*layouts)
+        cl = [c_layout(l) for l in layouts]
+        got = _lib.gk_shape()
+        rc = _lib.lib().gk_heuristic_block_shape(*(ctypes.byref(x) for x in cl), ctypes.byref(got))
+        assert rc == _lib.GK_OK
+        assert (got.M, got.N, got.K) == (want.M, want.N, want.K), layouts
+
+
 def test_physical_size():
     # src/layout.jl:113, :194 / :152, :246 / :342-345 / :381-383
     assert Layout.physical_size(Layout.Padded[ACM[F16], 8], NT(M=128, K=64)) == (136, 64)
