@@ -62,9 +62,9 @@ bool valid_layout_kind(int k) { return k >= GK_LAYOUT_ZERO && k <= GK_LAYOUT_GET
 
 int dtype_size(int dt) {
   switch (dt) {
-    case GK_F16: case GK_BF16: return 2;
-    case GK_F32: return 4;
-    case GK_F64: return 8;
+    case GK_F16: case GK_BF16: case GK_I16: return 2;
+    case GK_F32: case GK_I32: return 4;
+    case GK_F64: case GK_I64: return 8;
     default: return 0;
   }
 }
@@ -121,6 +121,7 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
     key->variant = 1;
   }
   key->dtype = c->global_a_layout.eltype;
+  key->acc_dtype = c->global_d_layout.eltype;
   key->fused = (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT)) ? 1 : 0;
   if (key->fused && t && (key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT)) {
     // level 1 covers A / B hooks that are one exact 16-bit scale (or nothing); anything else needs
@@ -400,7 +401,20 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   // element types of C and D: fp32 everywhere; the real MFMA kernels also read and write 16-bit
   // matrices (fp32 accumulation, one rounding at the store; the reference's F16 -> F16 WMMA
   // configuration, configs/configs.jl:574)
-  {
+  if (is_fpu_kind(op.kind)) {
+    // the vector-ALU kernels accumulate in the element type of C and D; the pairs (A and B, C and D)
+    // are those the reference runs FPUOp with (configs/configs.jl:489-497)
+    const int ab = c->global_a_layout.eltype, cd = c->global_d_layout.eltype;
+    if (c->global_b_layout.eltype != ab) return fail(GK_ERR_UNSUPPORTED, "A and B must have the same element type");
+    const bool pair_ok = (ab == GK_F16 && cd == GK_F32) || (ab == GK_F32 && (cd == GK_F32 || cd == GK_F64)) ||
+                         (ab == GK_F64 && cd == GK_F64) || (ab == GK_I16 && cd == GK_I16) || (ab == GK_I32 && cd == GK_I32) ||
+                         (ab == GK_I64 && cd == GK_I64);
+    if (!pair_ok) return fail(GK_ERR_UNSUPPORTED, "element types %d (A, B) and %d (D) are not a pair the vector-ALU operator is compiled for", ab, cd);
+    if (c->global_c_layout.kind != GK_LAYOUT_ZERO && c->global_c_layout.eltype != cd)
+      return fail(GK_ERR_UNSUPPORTED, "C and D must have the same element type");
+    if (op.kind == GK_OP_FPU_TROPICAL && cd != GK_F32) return fail(GK_ERR_UNSUPPORTED, "the max-plus operator is compiled for fp32");
+    if (e && e->kind != GK_EPILOGUE_DEFAULT && cd != GK_F32) return fail(GK_ERR_UNSUPPORTED, "the bias epilogue is fp32 (src/epilogue.jl:44-52)");
+  } else {
     const bool cd16_ok = op.kind == GK_OP_MFMA && c->global_a_layout.kind != GK_LAYOUT_DIAGONAL;
     auto cd_ok = [&](int dt) { return dt == GK_F32 || (cd16_ok && (dt == GK_F16 || dt == GK_BF16)); };
     if (!cd_ok(c->global_d_layout.eltype))

@@ -23,7 +23,7 @@ typedef int int2v __attribute__((ext_vector_type(2)));
 constexpr int kWaveSize = 64;
 
 // dtype codes (same values as gk_dtype of the C ABI)
-enum : int { DT_F16 = 0, DT_BF16 = 1, DT_F32 = 2, DT_F64 = 3 };
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_F32 = 2, DT_F64 = 3, DT_I16 = 4, DT_I32 = 5, DT_I64 = 6 };
 
 // op codes (same values as gk_op_kind of the C ABI)
 enum : int { T_IDENTITY = 0, T_SCALE = 1, T_ADD = 2, T_RELU = 3, T_NEG = 4, T_ABS = 5, T_CLAMP = 6, T_SQUARE = 7 };

@@ -2,55 +2,117 @@
 // reference (src/operator.jl:35-153) together with the kernels that drive them
 // (src/kernel.jl:10-129, 147-350).
 //
-// Every output element is one fp32 accumulator updated by a scalar fused multiply-add per k, in
+// Every output element is one accumulator updated by a scalar fused multiply-add per k, in
 // ascending k, exactly like FPUOp.mma (src/operator.jl:139-153), so results are bit-identical to
-// a sequential fmaf loop on the host.  A wave is an 8 x 8 grid of lanes (the reference's base
-// shape mb x nb = 32 lanes becomes 64 here); a lane owns TM x TN outputs in 4-wide chunks so that
-// LDS reads and D stores are 16-byte accesses.  Tiles go global -> registers -> LDS with the next
-// tile's global loads in flight during the FMAs of the current one.  With CHECKED the loads and
-// stores are per element and bounds-checked (reference Layout.ColMajor / RowMajor,
-// src/layout.jl:117-184: out-of-range loads give 0, out-of-range stores are dropped), so any
-// problem size and any leading dimension works.
+// a sequential fma loop on the host.  The accumulator type TACC is the element type of C and D and
+// the multiplicands are converted to it before the fma, which is what Julia's promotion makes of
+// fma(a::CT, b::CT, c::AT) for the type triples the reference runs (configs/configs.jl:489-497):
+// Float16 -> Float32, Float32 -> Float32, Float32 -> Float64, Float64 -> Float64 and Int16 / Int32 /
+// Int64 with wrap-around.  A wave is an 8 x 8 grid of lanes (the reference's base shape mb x nb =
+// 32 lanes becomes 64 here); a lane owns TM x TN outputs in 4-wide chunks so that LDS reads and D
+// stores are vector accesses.  Tiles go global -> registers -> LDS with the next tile's global
+// loads in flight during the fmas of the current one.  With CHECKED the loads and stores are per
+// element and bounds-checked (reference Layout.ColMajor / RowMajor, src/layout.jl:117-184:
+// out-of-range loads give 0, out-of-range stores are dropped), so any problem size and any leading
+// dimension works.
 #pragma once
 #include "common.hpp"
+#include <type_traits>
 
 namespace gk {
 
-template <typename T> struct FpuIn;
-template <> struct FpuIn<float> {
-  static constexpr int DT = DT_F32;
-  __device__ static __forceinline__ float to_float(float x) { return x; }
-  __device__ static __forceinline__ float round(float x) { return x; }
-};
-template <> struct FpuIn<_Float16> {
-  static constexpr int DT = DT_F16;
-  __device__ static __forceinline__ float to_float(_Float16 x) { return (float)x; }
-  __device__ static __forceinline__ float round(float x) { return (float)(_Float16)x; }
-};
+// dtype code of an element type
+template <typename T> struct DtypeOf;
+template <> struct DtypeOf<_Float16> { static constexpr int DT = DT_F16; };
+template <> struct DtypeOf<float> { static constexpr int DT = DT_F32; };
+template <> struct DtypeOf<double> { static constexpr int DT = DT_F64; };
+template <> struct DtypeOf<short> { static constexpr int DT = DT_I16; };
+template <> struct DtypeOf<int> { static constexpr int DT = DT_I32; };
+template <> struct DtypeOf<long long> { static constexpr int DT = DT_I64; };
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, typename TIN_, bool A_KMAJOR_, bool B_KMAJOR_, bool CHECKED_, bool TROPICAL_>
+// The type a transform of a T-typed value is evaluated in (one rounding per op): fp32 for the
+// 16- and 32-bit floats, fp64 for fp64, the integer type itself for integers.
+template <typename T> struct ArithOf { typedef T type; };
+template <> struct ArithOf<_Float16> { typedef float type; };
+
+// One elementwise op in arithmetic type X.  The fp32 forms are those of apply_op; integers wrap.
+template <typename X>
+__device__ __forceinline__ X apply_op_t(int kind, float p0, float p1, X x) {
+  if constexpr (std::is_same<X, float>::value) {
+    return apply_op(kind, p0, p1, x);
+  } else if constexpr (std::is_floating_point<X>::value) {
+    const X q0 = (X)p0, q1 = (X)p1;
+    switch (kind) {
+      case T_SCALE: return x * q0;
+      case T_ADD: return x + q0;
+      case T_RELU: return x > (X)0 ? x : (X)0;
+      case T_NEG: return -x;
+      case T_ABS: return x < (X)0 ? -x : x;
+      case T_CLAMP: return x < q0 ? q0 : (x > q1 ? q1 : x);
+      case T_SQUARE: return x * x;
+      default: return x;
+    }
+  } else {
+    typedef typename std::make_unsigned<X>::type U;
+    const X q0 = (X)p0, q1 = (X)p1;
+    switch (kind) {
+      case T_SCALE: return (X)((U)x * (U)q0);
+      case T_ADD: return (X)((U)x + (U)q0);
+      case T_RELU: return x > 0 ? x : (X)0;
+      case T_NEG: return (X)((U)0 - (U)x);
+      case T_ABS: return x < 0 ? (X)((U)0 - (U)x) : x;
+      case T_CLAMP: return x < q0 ? q0 : (x > q1 ? q1 : x);
+      case T_SQUARE: return (X)((U)x * (U)x);
+      default: return x;
+    }
+  }
+}
+
+template <typename X>
+__device__ __forceinline__ X apply_list_t(const OpList& t, X x) {
+  for (int i = 0; i < t.n; ++i) x = apply_op_t<X>(t.kind[i], t.p0[i], t.p1[i], x);
+  return x;
+}
+
+// acc <- a * b + acc with one rounding (floats) or wrap-around (integers): operator_fma of FPUOp
+template <typename TACC>
+__device__ __forceinline__ TACC fpu_fma(TACC a, TACC b, TACC c) {
+  if constexpr (std::is_same<TACC, float>::value) return __builtin_fmaf(a, b, c);
+  else if constexpr (std::is_same<TACC, double>::value) return __builtin_fma(a, b, c);
+  else {
+    typedef typename std::make_unsigned<TACC>::type U;
+    return (TACC)((U)a * (U)b + (U)c);
+  }
+}
+
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, typename TIN_, bool A_KMAJOR_, bool B_KMAJOR_, bool CHECKED_,
+          bool TROPICAL_, typename TACC_ = float>
 struct FpuGemmConfig {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, CHECKED = CHECKED_, TROPICAL = TROPICAL_;
   typedef TIN_ TIN;
+  typedef TACC_ TACC;
   static constexpr int THREADS = WAVES_M * WAVES_N * kWaveSize;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   static constexpr int TM = WTM / 8, TN = WTN / 8;          // outputs per lane
   static constexpr int CM = TM / 4, CN = TN / 4;            // 4-wide chunks per lane
   static constexpr int PAD = 4;
-  static constexpr int LDA_S = BM + PAD, LDB_S = BN + PAD;  // LDS row pitch (floats), rows are k
-  static constexpr int LDS_BYTES = (BK * LDA_S + BK * LDB_S) * 4;
+  static constexpr int LDA_S = BM + PAD, LDB_S = BN + PAD;  // LDS row pitch (elements of TACC), rows are k
+  static constexpr int LDS_BYTES = (BK * LDA_S + BK * LDB_S) * (int)sizeof(TACC);
   static constexpr int A_CHUNKS = BM * BK / 4, B_CHUNKS = BN * BK / 4;
   static constexpr int A_PER_THREAD = A_CHUNKS / THREADS, B_PER_THREAD = B_CHUNKS / THREADS;
   static_assert(TM % 4 == 0 && TN % 4 == 0, "a lane owns whole 4-wide chunks");
   static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "tile loads divide evenly over the threads");
+  static_assert(!TROPICAL || std::is_same<TACC, float>::value, "the max-plus product is compiled for fp32");
 };
 
 // Loads the 4 elements of chunk `chunk` of an R x BK operand tile: rows r0.. of the operand,
-// k from k0.  MAJOR_K: memory is contiguous along k.  Out-of-range elements read as 0.
+// k from k0.  MAJOR_K: memory is contiguous along k.  Out-of-range elements read as 0.  The values
+// stay in the operand's own type until the load hooks have run.
 template <class Cfg, int R, bool KMAJOR>
 __device__ __forceinline__ void load_chunk(const typename Cfg::TIN* __restrict__ base, long long ld, int r0, int k0, int chunk,
-                                           int r_limit, int k_limit, bool zero, float (&out)[4], int& r_local, int& k_local) {
+                                           int r_limit, int k_limit, bool zero, typename Cfg::TIN (&out)[4], bool (&pad_k)[4],
+                                           int& r_local, int& k_local) {
   typedef typename Cfg::TIN TIN;
   if (KMAJOR) {
     constexpr int CPR = Cfg::BK / 4;          // chunks per row
@@ -62,22 +124,24 @@ __device__ __forceinline__ void load_chunk(const typename Cfg::TIN* __restrict__
     r_local = (chunk % CPK) * 4;
   }
   const int r = r0 + r_local, k = k0 + k_local;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) pad_k[e] = false;
   if (zero) {          // Layout.Zero: nothing is read (alpha == 0, reference src/matmul.jl:127-130)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) out[e] = 0.0f;
+    for (int e = 0; e < 4; ++e) out[e] = (TIN)0;
   } else if (!Cfg::CHECKED) {
     const TIN* p = base + (KMAJOR ? (long long)r * ld + k : (long long)k * ld + r);
     typedef TIN vec4 __attribute__((ext_vector_type(4)));
     const vec4 v = *(const vec4*)p;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) out[e] = FpuIn<TIN>::to_float(v[e]);
+    for (int e = 0; e < 4; ++e) out[e] = v[e];
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int rr = KMAJOR ? r : r + e, kk = KMAJOR ? k + e : k;
-      // padding: 0 for the ordinary product; -inf along k for the tropical one so that max() ignores it
-      float x = (Cfg::TROPICAL && kk >= k_limit) ? -__builtin_inff() : 0.0f;
-      if (rr < r_limit && kk < k_limit) x = FpuIn<TIN>::to_float(base[KMAJOR ? (long long)rr * ld + kk : (long long)kk * ld + rr]);
+      TIN x = (TIN)0;
+      pad_k[e] = kk >= k_limit;     // the tropical product pads k with -inf so that max() ignores it
+      if (rr < r_limit && kk < k_limit) x = base[KMAJOR ? (long long)rr * ld + kk : (long long)kk * ld + rr];
       out[e] = x;
     }
   }
@@ -86,10 +150,13 @@ __device__ __forceinline__ void load_chunk(const typename Cfg::TIN* __restrict__
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs args) {
   typedef typename Cfg::TIN TIN;
+  typedef typename Cfg::TACC TACC;
+  typedef typename ArithOf<TIN>::type TAR;       // arithmetic type of the A / B hooks
+  typedef TACC acc4 __attribute__((ext_vector_type(4)));
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, TM = Cfg::TM, TN = Cfg::TN;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  float* As = (float*)smem;                       // [BK][LDA_S], rows are k
-  float* Bs = As + BK * Cfg::LDA_S;               // [BK][LDB_S]
+  TACC* As = (TACC*)smem;                         // [BK][LDA_S], rows are k
+  TACC* Bs = As + BK * Cfg::LDA_S;                // [BK][LDB_S]
 
   int ti, tj;
   cta_swizzle(args.swz_kind, args.swz_param, (int)blockIdx.x, (int)blockIdx.y, args.nbm, args.nbn, ti, tj);
@@ -100,70 +167,81 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
   const int m0 = ti * BM, n0 = tj * BN;
   const TIN* A = (const TIN*)args.a;
   const TIN* B = (const TIN*)args.b;
+  const TACC* C = (const TACC*)args.c;
   const bool zero_ab = (args.a_kind == 0 /* Layout.Zero */);
   const bool xf_a = args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0;
   const bool xf_b = args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0;
 
   // accumulators: acc[i][j] is row wm*WTM + (i/4)*32 + 4*ly + i%4, column wn*WTN + (j/4)*32 + 4*lx + j%4
-  float acc[TM][TN];
+  TACC acc[TM][TN];
   auto row_of = [&](int i) { return m0 + wm * Cfg::WTM + (i / 4) * 32 + 4 * ly + (i % 4); };
   auto col_of = [&](int j) { return n0 + wn * Cfg::WTN + (j / 4) * 32 + 4 * lx + (j % 4); };
 #pragma unroll
   for (int j = 0; j < TN; ++j)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      float c = 0.0f;
+      TACC c = (TACC)0;
       if (args.c_mode != 0) {
         const int r = row_of(i), cc = col_of(j);
-        if (!Cfg::CHECKED || (r < args.M && cc < args.N)) c = ((const float*)args.c)[r + (long long)cc * args.ldc];
-        c = apply_list(args.t[H_GL2SH_C], c);
-        c = apply_list(args.t[H_SH2RF_C], c);
+        if (!Cfg::CHECKED || (r < args.M && cc < args.N)) c = C[r + (long long)cc * args.ldc];
+        c = apply_list_t<TACC>(args.t[H_GL2SH_C], c);
+        c = apply_list_t<TACC>(args.t[H_SH2RF_C], c);
       }
       acc[i][j] = c;
     }
 
-  float ra[Cfg::A_PER_THREAD][4], rb[Cfg::B_PER_THREAD][4];
+  TIN ra[Cfg::A_PER_THREAD][4], rb[Cfg::B_PER_THREAD][4];
+  bool pa[Cfg::A_PER_THREAD][4], pb[Cfg::B_PER_THREAD][4];
   int ar[Cfg::A_PER_THREAD], ak[Cfg::A_PER_THREAD], br[Cfg::B_PER_THREAD], bk[Cfg::B_PER_THREAD];
 
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < Cfg::A_PER_THREAD; ++i) {
-      load_chunk<Cfg, BM, Cfg::A_KMAJOR>(A, args.lda, m0, k0, tid + i * Cfg::THREADS, args.M, args.K, zero_ab, ra[i], ar[i], ak[i]);
+      load_chunk<Cfg, BM, Cfg::A_KMAJOR>(A, args.lda, m0, k0, tid + i * Cfg::THREADS, args.M, args.K, zero_ab, ra[i], pa[i], ar[i], ak[i]);
     }
 #pragma unroll
     for (int i = 0; i < Cfg::B_PER_THREAD; ++i) {
-      load_chunk<Cfg, BN, Cfg::B_KMAJOR>(B, args.ldb, n0, k0, tid + i * Cfg::THREADS, args.N, args.K, zero_ab, rb[i], br[i], bk[i]);
+      load_chunk<Cfg, BN, Cfg::B_KMAJOR>(B, args.ldb, n0, k0, tid + i * Cfg::THREADS, args.N, args.K, zero_ab, rb[i], pb[i], br[i], bk[i]);
     }
   };
-  // transforms of the two load hooks, each rounded to the element type of its destination
-  auto xform = [&](float (&v)[4], const OpList& t0, const OpList& t1) {
+  // the two load hooks, each rounded to the element type of its destination (the operand's own
+  // type), then the conversion to the accumulator type for the fma
+  auto prepare = [&](const TIN (&v)[4], const bool (&pad)[4], bool xf, const OpList& t0, const OpList& t1, TACC (&out)[4]) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      float x = v[e];
-      if (t0.n > 0) x = FpuIn<TIN>::round(apply_list(t0, x));
-      if (t1.n > 0) x = FpuIn<TIN>::round(apply_list(t1, x));
-      v[e] = x;
+      TIN x = v[e];
+      if (xf) {
+        if (t0.n > 0) x = (TIN)apply_list_t<TAR>(t0, (TAR)x);
+        if (t1.n > 0) x = (TIN)apply_list_t<TAR>(t1, (TAR)x);
+      }
+      TACC y = (TACC)x;
+      if constexpr (Cfg::TROPICAL && Cfg::CHECKED) {
+        if (pad[e]) y = -__builtin_inff();
+      }
+      out[e] = y;
     }
   };
   auto stash = [&]() {
 #pragma unroll
     for (int i = 0; i < Cfg::A_PER_THREAD; ++i) {
-      if (xf_a) xform(ra[i], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
+      TACC v[4];
+      prepare(ra[i], pa[i], xf_a, args.t[H_GL2SH_A], args.t[H_SH2RF_A], v);
       if (Cfg::A_KMAJOR) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) As[(ak[i] + e) * Cfg::LDA_S + ar[i]] = ra[i][e];
+        for (int e = 0; e < 4; ++e) As[(ak[i] + e) * Cfg::LDA_S + ar[i]] = v[e];
       } else {
-        *(float4v*)&As[ak[i] * Cfg::LDA_S + ar[i]] = (float4v){ra[i][0], ra[i][1], ra[i][2], ra[i][3]};
+        *(acc4*)&As[ak[i] * Cfg::LDA_S + ar[i]] = (acc4){v[0], v[1], v[2], v[3]};
       }
     }
 #pragma unroll
     for (int i = 0; i < Cfg::B_PER_THREAD; ++i) {
-      if (xf_b) xform(rb[i], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
+      TACC v[4];
+      prepare(rb[i], pb[i], xf_b, args.t[H_GL2SH_B], args.t[H_SH2RF_B], v);
       if (Cfg::B_KMAJOR) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) Bs[(bk[i] + e) * Cfg::LDB_S + br[i]] = rb[i][e];
+        for (int e = 0; e < 4; ++e) Bs[(bk[i] + e) * Cfg::LDB_S + br[i]] = v[e];
       } else {
-        *(float4v*)&Bs[bk[i] * Cfg::LDB_S + br[i]] = (float4v){rb[i][0], rb[i][1], rb[i][2], rb[i][3]};
+        *(acc4*)&Bs[bk[i] * Cfg::LDB_S + br[i]] = (acc4){v[0], v[1], v[2], v[3]};
       }
     }
   };
@@ -175,53 +253,56 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
     stash();
     __syncthreads();
     if (kt + 1 < KT) fetch((kt + 1) * BK);
-    const float* ap = As + wm * Cfg::WTM + 4 * ly;
-    const float* bp = Bs + wn * Cfg::WTN + 4 * lx;
+    const TACC* ap = As + wm * Cfg::WTM + 4 * ly;
+    const TACC* bp = Bs + wn * Cfg::WTN + 4 * lx;
 #pragma unroll 4
     for (int k = 0; k < BK; ++k) {
-      float a[TM], b[TN];
+      TACC a[TM], b[TN];
 #pragma unroll
       for (int c = 0; c < Cfg::CM; ++c) {
-        const float4v v = *(const float4v*)&ap[k * Cfg::LDA_S + c * 32];
+        const acc4 v = *(const acc4*)&ap[k * Cfg::LDA_S + c * 32];
         a[4 * c] = v[0]; a[4 * c + 1] = v[1]; a[4 * c + 2] = v[2]; a[4 * c + 3] = v[3];
       }
 #pragma unroll
       for (int c = 0; c < Cfg::CN; ++c) {
-        const float4v v = *(const float4v*)&bp[k * Cfg::LDB_S + c * 32];
+        const acc4 v = *(const acc4*)&bp[k * Cfg::LDB_S + c * 32];
         b[4 * c] = v[0]; b[4 * c + 1] = v[1]; b[4 * c + 2] = v[2]; b[4 * c + 3] = v[3];
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-          if (Cfg::TROPICAL) {
-            const float s = a[i] + b[j];
+          if constexpr (Cfg::TROPICAL) {
+            const TACC s = a[i] + b[j];
             acc[i][j] = s > acc[i][j] ? s : acc[i][j];
           } else {
-            acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
+            acc[i][j] = fpu_fma<TACC>(a[i], b[j], acc[i][j]);
           }
         }
     }
   }
 
-  // epilogue: transform, bias, transform, store (4 consecutive rows per 16-byte store)
-  float* D = (float*)args.d;
+  // epilogue: transform, bias, transform, store (4 consecutive rows per vector store); the bias of
+  // Epilogue.Bias is fp32 (reference src/epilogue.jl:44-52) and only offered with fp32 accumulators
+  TACC* D = (TACC*)args.d;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int cc = col_of(j);
 #pragma unroll
     for (int c = 0; c < Cfg::CM; ++c) {
-      float x[4];
+      TACC x[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float v = apply_list(args.t[H_RF2SH_D], acc[4 * c + e][j]);
-        if (args.epi_kind == 1) v = v + args.bias[Cfg::CHECKED ? (cc < args.N ? cc : 0) : cc];
-        else if (args.epi_kind == 2) { const int r = row_of(4 * c + e); v = v + args.bias[Cfg::CHECKED ? (r < args.M ? r : 0) : r]; }
-        x[e] = apply_list(args.t[H_SH2GL_D], v);
+        TACC v = apply_list_t<TACC>(args.t[H_RF2SH_D], acc[4 * c + e][j]);
+        if constexpr (std::is_same<TACC, float>::value) {
+          if (args.epi_kind == 1) v = v + args.bias[Cfg::CHECKED ? (cc < args.N ? cc : 0) : cc];
+          else if (args.epi_kind == 2) { const int r = row_of(4 * c + e); v = v + args.bias[Cfg::CHECKED ? (r < args.M ? r : 0) : r]; }
+        }
+        x[e] = apply_list_t<TACC>(args.t[H_SH2GL_D], v);
       }
       const int r = row_of(4 * c);
       if (!Cfg::CHECKED) {
-        *(float4v*)&D[r + (long long)cc * args.ldd] = (float4v){x[0], x[1], x[2], x[3]};
+        *(acc4*)&D[r + (long long)cc * args.ldd] = (acc4){x[0], x[1], x[2], x[3]};
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)

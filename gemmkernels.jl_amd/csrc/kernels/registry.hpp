@@ -13,6 +13,7 @@ struct InstanceKey {
   int waves_m, waves_n;
   int a_kmajor, b_kmajor;   // 1: the K index is contiguous in the operand's memory
   int dtype;         // element type of A and B
+  int acc_dtype;     // element type of C / D and of the accumulators (vector-ALU kernels)
   int fused;         // 1: transforms / bias present
   int variant;       // family specific
 };
@@ -64,6 +65,7 @@ int family_mfma_nn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, 
 int family_mfma_nt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_tt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_fpu(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+int family_fpu_types(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_complex(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_diagonal(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_checked(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);

@@ -10,7 +10,7 @@ int family_fpu(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStrea
   // key.variant: bit 0 tropical, bit 1 bounds-checked
 #define GK_FPU(bm_, bn_, bk_, wm_, wn_, TYPE, akm_, bkm_, chk_, trop_, NAME)                                               \
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
-      key.dtype == FpuIn<TYPE>::DT && key.a_kmajor == akm_ && key.b_kmajor == bkm_ && key.variant == (trop_ + 2 * chk_)) { \
+      key.dtype == DtypeOf<TYPE>::DT && key.acc_dtype == DT_F32 && key.a_kmajor == akm_ && key.b_kmajor == bkm_ && key.variant == (trop_ + 2 * chk_)) { \
     typedef FpuGemmConfig<bm_, bn_, bk_, wm_, wn_, TYPE, (akm_ != 0), (bkm_ != 0), (chk_ != 0), (trop_ != 0)> Cfg;          \
     return run_instance<Cfg>(fpu_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
@@ -28,8 +28,8 @@ int family_fpu(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStrea
   GK_FPU_T(64, 64, 32, 2, 2, float, 1, 1, "64x64x32_w2x2_f32_tropical_checked")
 #undef GK_FPU_T
 #undef GK_FPU
-  (void)args; (void)grid; (void)stream; (void)mode; (void)info; (void)err;
-  return 0;
+  // the other element types of FPUOp
+  return family_fpu_types(key, args, grid, stream, mode, info, err);
 }
 
 int family_mfma_checked(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode,

@@ -54,7 +54,7 @@ typedef enum gk_status {
   GK_ERR_HIP = 12                /* HIP runtime error at launch */
 } gk_status;
 
-typedef enum gk_dtype { GK_F16 = 0, GK_BF16 = 1, GK_F32 = 2, GK_F64 = 3 } gk_dtype;
+typedef enum gk_dtype { GK_F16 = 0, GK_BF16 = 1, GK_F32 = 2, GK_F64 = 3, GK_I16 = 4, GK_I32 = 5, GK_I64 = 6 } gk_dtype;
 
 /* Operators (reference src/operator.jl).  GK_OP_MFMA stands where WMMAOp stands in the reference
  * (:163-245) and runs v_mfma_f32_32x32x16_{f16,bf16}; GK_OP_MFMA_COMPLEX is WMMAComplexOp

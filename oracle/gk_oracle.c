@@ -35,7 +35,7 @@
 #endif
 
 /* ---- dtypes ---- */
-enum { GKO_F16 = 0, GKO_BF16 = 1, GKO_F32 = 2, GKO_F64 = 3 };
+enum { GKO_F16 = 0, GKO_BF16 = 1, GKO_F32 = 2, GKO_F64 = 3, GKO_I16 = 4, GKO_I32 = 5, GKO_I64 = 6 };
 
 /* ---- layout kinds ---- */
 enum {
@@ -245,11 +245,99 @@ static int64_t layout_store_index(const gko_layout* L, int64_t r, int64_t c) {
 /* ---------------- the GEMM ---------------- */
 static int is_complex_layout(const gko_layout* L) { return L->kind == GKO_L_ICOL || L->kind == GKO_L_IROW; }
 
+/* ---------------- integer element types ---------------- */
+/* FPUOp with Int16 / Int32 / Int64 (reference configs/configs.jl:495-497): Julia's fma on integers
+ * is a*b + c with wrap-around, and so is every elementwise op.  Values are carried in uint64 and
+ * wrapped to the element width after each operation, which is the same residue class. */
+static int64_t wrap_int(int dtype, uint64_t x) {
+  switch (dtype) {
+    case GKO_I16: return (int64_t)(int16_t)(uint16_t)x;
+    case GKO_I32: return (int64_t)(int32_t)(uint32_t)x;
+    default: return (int64_t)x;
+  }
+}
+
+static int64_t load_int(int dtype, const void* p, int64_t idx) {
+  switch (dtype) {
+    case GKO_I16: return ((const int16_t*)p)[idx];
+    case GKO_I32: return ((const int32_t*)p)[idx];
+    default: return ((const int64_t*)p)[idx];
+  }
+}
+
+static void store_int(int dtype, void* p, int64_t idx, int64_t v) {
+  switch (dtype) {
+    case GKO_I16: ((int16_t*)p)[idx] = (int16_t)v; break;
+    case GKO_I32: ((int32_t*)p)[idx] = (int32_t)v; break;
+    default: ((int64_t*)p)[idx] = v; break;
+  }
+}
+
+static int64_t apply_transform_int(const gko_transform* t, int dtype, int64_t x) {
+  for (int i = 0; i < t->n; ++i) {
+    const gko_op* o = &t->ops[i];
+    const int64_t q0 = wrap_int(dtype, (uint64_t)(int64_t)o->p0), q1 = wrap_int(dtype, (uint64_t)(int64_t)o->p1);
+    switch (o->kind) {
+      case GKO_T_SCALE: x = wrap_int(dtype, (uint64_t)x * (uint64_t)q0); break;
+      case GKO_T_ADD: x = wrap_int(dtype, (uint64_t)x + (uint64_t)q0); break;
+      case GKO_T_RELU: x = x > 0 ? x : 0; break;
+      case GKO_T_NEG: x = wrap_int(dtype, (uint64_t)0 - (uint64_t)x); break;
+      case GKO_T_ABS: x = x < 0 ? wrap_int(dtype, (uint64_t)0 - (uint64_t)x) : x; break;
+      case GKO_T_CLAMP: x = x < q0 ? q0 : (x > q1 ? q1 : x); break;
+      case GKO_T_SQUARE: x = wrap_int(dtype, (uint64_t)x * (uint64_t)x); break;
+      default: break;
+    }
+  }
+  return x;
+}
+
+static int64_t layout_load_int(const gko_layout* L, const void* p, int64_t r, int64_t c) {
+  switch (L->kind) {
+    case GKO_L_COL: return load_int(L->dtype, p, r + c * L->ld);
+    case GKO_L_ROW: return load_int(L->dtype, p, c + r * L->ld);
+    default: return 0;     /* Layout.Zero */
+  }
+}
+
+static int gko_matmul_int(const gko_problem* P, const void* a, const void* b, const void* c, void* d) {
+  const int64_t M = P->M, N = P->N, K = P->K;
+  const int dt = P->accum_dtype;
+  if (P->op_kind != GKO_OP_FMA || P->epilogue != 0) return 1;
+  const gko_layout* Ls[4] = {&P->a, &P->b, &P->c, &P->d};
+  for (int i = 0; i < 4; ++i)
+    if (Ls[i]->kind != GKO_L_ZERO && Ls[i]->kind != GKO_L_COL && Ls[i]->kind != GKO_L_ROW) return 1;
+  int64_t* out = (int64_t*)malloc(sizeof(int64_t) * (size_t)M * (size_t)N);
+  if (!out) return 2;
+  for (int64_t j = 0; j < N; ++j)
+    for (int64_t i = 0; i < M; ++i) {
+      int64_t acc = 0;
+      if (P->c.kind != GKO_L_ZERO) {
+        acc = apply_transform_int(&P->t[2], dt, layout_load_int(&P->c, c, i, j));
+        acc = apply_transform_int(&P->t[6], dt, acc);
+      }
+      for (int64_t k = 0; k < K; ++k) {      /* ascending k, one wrapped a*b + c per step (src/operator.jl:139-153) */
+        int64_t x = apply_transform_int(&P->t[4], P->a.dtype, apply_transform_int(&P->t[0], P->a.dtype, layout_load_int(&P->a, a, i, k)));
+        int64_t y = apply_transform_int(&P->t[5], P->b.dtype, apply_transform_int(&P->t[1], P->b.dtype, layout_load_int(&P->b, b, k, j)));
+        acc = wrap_int(dt, (uint64_t)x * (uint64_t)y + (uint64_t)acc);
+      }
+      acc = apply_transform_int(&P->t[7], dt, acc);
+      out[(size_t)j * M + i] = apply_transform_int(&P->t[3], dt, acc);
+    }
+  for (int64_t j = 0; j < N; ++j)
+    for (int64_t i = 0; i < M; ++i) {
+      int64_t idx = layout_store_index(&P->d, i, j);
+      if (idx >= 0) store_int(P->d.dtype, d, idx, out[(size_t)j * M + i]);
+    }
+  free(out);
+  return 0;
+}
+
 /*
  * D = epilogue(T_d(sum_k T_a(A) * T_b(B) + T_c(C))).  Returns 0 on success.
  * a, b, c, d are host pointers in the layouts of the problem; d may alias c.
  */
 int gko_matmul(const gko_problem* P, const void* a, const void* b, const void* c, void* d) {
+  if (P->accum_dtype >= GKO_I16) return gko_matmul_int(P, a, b, c, d);
   const int64_t M = P->M, N = P->N, K = P->K;
   const int two = (P->op_kind == GKO_OP_COMPLEX || P->op_kind == GKO_OP_DUAL) ? 2 : 1;
   const int wide_t = (P->compute_dtype == GKO_F64);   /* transforms of A/B in fp64 only for fp64 data */

@@ -18,7 +18,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libgk_oracle.so")
 
-F16, BF16, F32, F64 = 0, 1, 2, 3
+F16, BF16, F32, F64, I16, I32, I64 = 0, 1, 2, 3, 4, 5, 6
 L_ZERO, L_COL, L_ROW, L_DIAG, L_ICOL, L_IROW, L_GETT = range(7)
 OP_FMA, OP_TROPICAL, OP_COMPLEX, OP_DUAL = range(4)
 T_IDENTITY, T_SCALE, T_ADD, T_RELU, T_NEG, T_ABS, T_CLAMP, T_SQUARE = range(8)

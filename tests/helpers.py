@@ -7,7 +7,8 @@ import gemmkernels as gk
 from gemmkernels import Layout, Operator, Epilogue, Transform
 from oracle import oracle
 
-_DT = {"Float16": oracle.F16, "BFloat16": oracle.BF16, "Float32": oracle.F32, "Float64": oracle.F64}
+_DT = {"Float16": oracle.F16, "BFloat16": oracle.BF16, "Float32": oracle.F32, "Float64": oracle.F64,
+       "Int16": oracle.I16, "Int32": oracle.I32, "Int64": oracle.I64}
 HOOK_KW = {"transform_global_to_shared_a": "global_to_shared_a", "transform_global_to_shared_b": "global_to_shared_b",
            "transform_global_to_shared_c": "global_to_shared_c", "transform_shared_to_global_d": "shared_to_global_d",
            "transform_shared_to_regs_a": "shared_to_regs_a", "transform_shared_to_regs_b": "shared_to_regs_b",
@@ -86,7 +87,7 @@ def run_gpu(conf, a, b, c, d_shape, d_dtype=None, transforms=None, epilogue_cls=
     ta, tb, tc = up(a, conf.global_a_layout), up(b, conf.global_b_layout), up(c, conf.global_c_layout)
     td = tc if alias_cd else gk.colmajor_empty(d_shape, d_dtype or torch.float32)
     if not alias_cd:
-        td.fill_(float("nan"))
+        td.fill_(float("nan") if td.is_floating_point() else -12345)    # poison: every element must be written
     epi = None
     keep = None
     if epilogue_cls is not None:

@@ -219,3 +219,57 @@ def test_tropical_and_dual():
     oracle.matmul(plain(M, N, K, dt=F32, op_kind=oracle.OP_TROPICAL), a, b, c, d)
     want = np.maximum(c, (a[:, :, None] + b[None, :, :]).max(axis=1))      # max-plus product (reference configs/configs.jl:226)
     assert np.array_equal(d, want)
+
+
+@pytest.mark.parametrize("code,np_t,bits", [(oracle.I16, np.int16, 16), (oracle.I32, np.int32, 32), (oracle.I64, np.int64, 64)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+def test_integer_gemm_wraps_like_julia(code, np_t, bits, ta, tb):
+    """Int16 / Int32 / Int64 FPUOp (reference configs/configs.jl:495-497): alpha * A * B + beta * C
+    with wrap-around, against exact Python integers reduced modulo 2^bits.  The magnitudes are
+    chosen so that Int16 and Int32 really overflow."""
+    M, N, K = 7, 5, 9
+    rs = np.random.RandomState(bits)
+    hi = {16: 300, 32: 70000, 64: 2 ** 40}[bits]
+    a = np.asfortranarray(rs.randint(-hi, hi, size=(K, M) if ta else (M, K)).astype(np_t))
+    b = np.asfortranarray(rs.randint(-hi, hi, size=(N, K) if tb else (K, N)).astype(np_t))
+    c = np.asfortranarray(rs.randint(-hi, hi, size=(M, N)).astype(np_t))
+    p = plain(M, N, K, ta, tb, dt=code, cd=code)
+    p.transforms = {"shared_to_regs_a": [(oracle.T_SCALE, 2.0, 0.0)], "shared_to_regs_c": [(oracle.T_SCALE, 3.0, 0.0)]}
+    d = np.zeros((M, N), np_t, order="F")
+    oracle.matmul(p, a, b, c, d)
+    A = [[int(x) for x in row] for row in (a.T if ta else a)]
+    B = [[int(x) for x in row] for row in (b.T if tb else b)]
+    mod, half = 1 << bits, 1 << (bits - 1)
+    for i in range(M):
+        for j in range(N):
+            exact = 3 * int(c[i, j]) + sum(2 * A[i][k] * B[k][j] for k in range(K))
+            want = (exact + half) % mod - half
+            assert int(d[i, j]) == want, (i, j)
+    if bits < 64:
+        assert np.any(np.abs(np.array([[3 * int(c[i, j]) + sum(2 * A[i][k] * B[k][j] for k in range(K)) for j in range(N)] for i in range(M)], dtype=object)) >= half)
+
+
+def test_float64_accumulation_of_float32_inputs():
+    """(Float32, Float32, Float64) and (Float64, Float64, Float64) of the reference's FPUOp list
+    (configs/configs.jl:491-492): products of two float32 values are exact in float64, so a short sum
+    equals numpy's float64 matmul bit for bit when no rounding can occur, and agrees to a few ulps otherwise."""
+    M, N, K = 6, 4, 8
+    a, b = rand((M, K), np.float32, 1), rand((K, N), np.float32, 2)
+    c = rand((M, N), np.float64, 3)
+    p = plain(M, N, K, dt=F32, cd=F64)
+    d = np.zeros((M, N), np.float64, order="F")
+    oracle.matmul(p, a, b, c, d)
+    assert np.array_equal(d, a.astype(np.float64) @ b.astype(np.float64) + c)      # 11-bit inputs: every partial sum is exact
+    a64, b64 = np.asfortranarray(np.random.RandomState(4).standard_normal((M, K))), np.asfortranarray(np.random.RandomState(5).standard_normal((K, N)))
+    p = plain(M, N, K, dt=F64, cd=F64, zero_c=True)
+    oracle.matmul(p, a64, b64, None, d)
+    assert np.allclose(d, a64 @ b64, rtol=1e-14, atol=1e-15)
+    # sequential fma chain in ascending k
+    import math
+    acc = 0.0
+    for k in range(K):
+        acc = math.fma(a64[2, k], b64[k, 1], acc) if hasattr(math, "fma") else None
+        if acc is None:
+            break
+    if acc is not None:
+        assert d[2, 1] == acc
