@@ -639,6 +639,38 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   return GK_OK;
 }
 
+int gk_dev_alloc(size_t bytes, void** ptr) {
+  if (!ptr) return fail(GK_ERR_INVALID_ARGUMENT, "ptr is NULL");
+  *ptr = nullptr;
+  hipError_t e = hipMalloc(ptr, bytes ? bytes : 1);
+  if (e != hipSuccess) return fail(GK_ERR_HIP, "hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+  return GK_OK;
+}
+
+int gk_dev_free(void* ptr) {
+  hipError_t e = hipFree(ptr);
+  if (e != hipSuccess) return fail(GK_ERR_HIP, "hipFree failed: %s", hipGetErrorString(e));
+  return GK_OK;
+}
+
+int gk_copy_to_device(void* dst, const void* src, size_t bytes) {
+  hipError_t e = hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice);
+  if (e != hipSuccess) return fail(GK_ERR_HIP, "host to device copy of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+  return GK_OK;
+}
+
+int gk_copy_to_host(void* dst, const void* src, size_t bytes) {
+  hipError_t e = hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost);
+  if (e != hipSuccess) return fail(GK_ERR_HIP, "device to host copy of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+  return GK_OK;
+}
+
+int gk_synchronize(void) {
+  hipError_t e = hipDeviceSynchronize();
+  if (e != hipSuccess) return fail(GK_ERR_HIP, "hipDeviceSynchronize failed: %s", hipGetErrorString(e));
+  return GK_OK;
+}
+
 int32_t gk_sizeof(int32_t which) {
   switch (which) {
     case 0: return (int32_t)sizeof(gk_config);

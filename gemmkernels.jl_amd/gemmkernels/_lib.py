@@ -106,6 +106,11 @@ _SIGNATURES = {
                                       ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]),
     "gk_matmul": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                  ctypes.POINTER(gk_transforms), ctypes.POINTER(gk_epilogue), ctypes.c_int32, ctypes.c_void_p]),
+    "gk_dev_alloc": (ctypes.c_int, [ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]),
+    "gk_dev_free": (ctypes.c_int, [ctypes.c_void_p]),
+    "gk_copy_to_device": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+    "gk_copy_to_host": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+    "gk_synchronize": (ctypes.c_int, []),
     "gk_sizeof": (ctypes.c_int32, [ctypes.c_int32]),
 }
 

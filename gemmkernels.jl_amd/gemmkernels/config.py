@@ -151,6 +151,10 @@ _MFMA_TILES = [
 ]
 NUM_CUS = 256
 
+# measured winners by problem (filled by gemmkernels.tuning.install / load, or from the JSON file
+# named by the environment variable GEMMKERNELS_TUNING_TABLE)
+TUNED = {}
+
 
 def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
     """MI355X block shape: the largest tile of the table that divides the problem and still gives
@@ -224,6 +228,20 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
 
     tile_sized = any(require_tile_sized_global(l) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
     block_shape = params.get("block_shape")
+    if block_shape is None and operator.kind == Operator.MFMA and TUNED:
+        # a measured winner for exactly this problem (gemmkernels.tuning), unless the caller chose otherwise
+        key = (f"mfma/{global_a_layout.T.name}/{'N' if params.get('is_a_col_major', True) else 'T'}"
+               f"{'N' if params.get('is_b_col_major', True) else 'T'}/{gemm_shape.M}x{gemm_shape.N}x{gemm_shape.K}")
+        hit = TUNED.get(key)
+        aligned = all(l.kind in (Layout.ALIGNED_COL_MAJOR, Layout.ALIGNED_ROW_MAJOR, Layout.ZERO)
+                      for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
+        if hit is not None and aligned:
+            bm, bn, bk = hit["block"]
+            wm, wn = hit["waves"]
+            block_shape = NT(M=bm, N=bn, K=bk)
+            params.setdefault("warps_per_block", wm * wn)
+            params.setdefault("compute_warp", NT(M=bm // wm, N=bn // wn, K=16))
+            params.setdefault("cta_swizzle", CTASwizzle.XCDAware[int(hit.get("panel", 4))])
     if block_shape is None and global_a_layout.kind == Layout.DIAGONAL and gemm_shape.M % 64 == 0 and gemm_shape.N % 64 == 0:
         # a diagonal A makes the product a streaming pass over B and D: many small workgroups keep more
         # memory requests in flight than a few large ones (measured against HBM with rotating buffers)
@@ -289,3 +307,15 @@ def check_config(conf: Config, kernel=None) -> None:
     rc = _lib.lib().gk_validate(ctypes.byref(c), code)
     if rc != _lib.GK_OK:
         raise ConfigError(_lib.last_error(), rc)
+
+
+def _load_tuning_table_from_environment() -> None:
+    import json
+    import os
+    path = os.environ.get("GEMMKERNELS_TUNING_TABLE")
+    if path and os.path.exists(path):
+        with open(path) as f:
+            TUNED.update(json.load(f))
+
+
+_load_tuning_table_from_environment()

@@ -316,6 +316,11 @@ def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None)
         type(alpha), alpha == 0, type(beta), beta == 0, wmma)
     alpha_c = _round_to(compute_type, float(alpha))          # convert(compute_type, alpha), :196
     beta_c = _round_to(from_torch(C.dtype), float(beta))     # convert(eltype(C), beta), :197
+    for name, value in (("alpha", alpha_c), ("beta", beta_c)):
+        if float(np.float32(value)) != value:
+            # transform parameters travel as binary32; Float64 (or large integer) factors that do not
+            # fit would silently change the result
+            raise ConfigError(f"{name} = {value!r} is not representable in binary32, the parameter type of the transform hooks")
     ta = Transform.Elementwise(ops=[] if alpha_c == 1.0 else [(Transform.SCALE, alpha_c, 0.0)])
     tc = Transform.Elementwise(ops=[] if beta_c == 1.0 else [(Transform.SCALE, beta_c, 0.0)])
     return plan(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)

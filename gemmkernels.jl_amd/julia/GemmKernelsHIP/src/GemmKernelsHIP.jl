@@ -121,6 +121,25 @@ function heuristic_block_shape(shared_a::Type, shared_b::Type, shared_c::Type, s
     (M = Int(out[].M), N = Int(out[].N), K = Int(out[].K))
 end
 
+# Device memory without AMDGPU.jl: the library's own thin wrappers over hipMalloc / hipMemcpy.
+check(rc) = rc == 0 ? nothing : throw(ConfigError(last_error(), rc))
+function dev_alloc(bytes::Integer)
+    p = Ref{Ptr{Cvoid}}(C_NULL)
+    check(ccall((:gk_dev_alloc, libgk[]), Cint, (Csize_t, Ref{Ptr{Cvoid}}), bytes, p))
+    p[]
+end
+dev_free(p::Ptr{Cvoid}) = check(ccall((:gk_dev_free, libgk[]), Cint, (Ptr{Cvoid},), p))
+function to_device(x::Array)
+    p = dev_alloc(sizeof(x))
+    check(ccall((:gk_copy_to_device, libgk[]), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t), p, x, sizeof(x)))
+    p
+end
+function to_host!(x::Array, p::Ptr{Cvoid})
+    check(ccall((:gk_copy_to_host, libgk[]), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t), x, p, sizeof(x)))
+    x
+end
+synchronize() = check(ccall((:gk_synchronize, libgk[]), Cint, ()))
+
 function __init__()
     sizes = (sizeof(GkConfig), sizeof(GkLayout), sizeof(GkOperator), sizeof(GkTransforms), sizeof(GkEpilogue), sizeof(GkGett))
     isfile(libgk[]) || return

@@ -244,6 +244,16 @@ int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const
 int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
               const gk_transforms* transforms, const gk_epilogue* epilogue, int32_t kernel, void* stream);
 
+/* Device memory for callers that have no GPU array package of their own (a Julia session without
+ * AMDGPU.jl, a C test): thin wrappers over hipMalloc / hipFree / hipMemcpy / hipDeviceSynchronize on
+ * the current device.  The reference relies on CUDA.jl's CuArray for this (src/matmul.jl:185-215,
+ * configs/configs.jl:96-103); gk_matmul itself never allocates. */
+int gk_dev_alloc(size_t bytes, void** ptr);
+int gk_dev_free(void* ptr);
+int gk_copy_to_device(void* dst_device, const void* src_host, size_t bytes);
+int gk_copy_to_host(void* dst_host, const void* src_device, size_t bytes);
+int gk_synchronize(void);
+
 /* sizeof() of the ABI structs as compiled, so that a binding can check its own mirror:
  * 0 gk_config, 1 gk_layout, 2 gk_operator, 3 gk_transforms, 4 gk_epilogue, 5 gk_gett. */
 int32_t gk_sizeof(int32_t which);
