@@ -10,15 +10,18 @@
 #include <cstring>
 #include <string>
 
+#include "gk_internal.hpp"
 #include "kernels/common.hpp"
 #include "kernels/registry.hpp"
 
 namespace {
-
 thread_local std::string g_last_error;
+}
+
+namespace gk_internal {
 
 int fail(int code, const char* fmt, ...) {
-  char buf[512];
+  char buf[2048];
   va_list ap;
   va_start(ap, fmt);
   vsnprintf(buf, sizeof(buf), fmt, ap);
@@ -26,6 +29,12 @@ int fail(int code, const char* fmt, ...) {
   g_last_error = buf;
   return code;
 }
+
+}  // namespace gk_internal
+
+namespace {
+
+using gk_internal::fail;
 
 std::atomic<long long> g_lds_override{0};
 std::atomic<int> g_threads_override{0};
@@ -297,7 +306,7 @@ int validate_gett(const gk_config* c) {
 
 // All checks that need no pointers; reference src/config.jl:203-275 then src/matmul.jl:28-41.
 int validate_config(const gk_config* c, int kernel, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key,
-                    gk::InstanceInfo* info) {
+                    gk::InstanceInfo* info, const gk::InstanceInfo* custom = nullptr) {
   if (!c) return fail(GK_ERR_INVALID_ARGUMENT, "config is NULL");
   const gk_shape& g = c->matmul_shape;
   const gk_shape& b = c->block_shape;
@@ -429,7 +438,13 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
     return fail(GK_ERR_STAGES, "Need at least two stages to use a pipelined kernel, i.e. BLOCK_K >= 2 * OPERATOR_K");
 
   // the instance that would run; its LDS request is what Kernel.shmem_size returns
-  int rc = find_instance(c, t, e, key, info);
+  int rc = GK_OK;
+  if (custom) {      // a kernel specialised at run time: its resources are known to the caller
+    rc = make_key(c, t, e, key);
+    *info = *custom;
+  } else {
+    rc = find_instance(c, t, e, key, info);
+  }
   if (rc != GK_OK) return rc;
 
   long long lds_max = 0;
@@ -574,11 +589,17 @@ int gk_heuristic_block_shape(const gk_layout* sa, const gk_layout* sb, const gk_
   return GK_OK;
 }
 
-int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
-              const gk_epilogue* epilogue, int32_t kernel, void* stream) {
-  gk::InstanceKey key;
-  gk::InstanceInfo info;
-  int rc = validate_config(conf, kernel, transforms, epilogue, &key, &info);
+}  // extern "C"
+
+namespace gk_internal {
+
+// Everything gk_matmul does before the launch: configuration checks, operand checks, kernel
+// arguments and grid.  `custom` replaces the lookup of a compiled instance (run-time compiled kernels).
+int prepare_launch(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
+                   const gk_epilogue* epilogue, int32_t kernel, const gk::InstanceInfo* custom, Launch* out) {
+  gk::InstanceKey& key = out->key;
+  gk::InstanceInfo& info = out->info;
+  int rc = validate_config(conf, kernel, transforms, epilogue, &key, &info, custom);
   if (rc != GK_OK) return rc;
 
   const bool a_zero = conf->global_a_layout.kind == GK_LAYOUT_ZERO, b_zero = conf->global_b_layout.kind == GK_LAYOUT_ZERO;
@@ -586,7 +607,7 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   if (conf->global_c_layout.kind != GK_LAYOUT_ZERO && !c) return fail(GK_ERR_INVALID_ARGUMENT, "c must not be NULL unless its layout is Zero");
   if (epilogue && epilogue->kind != GK_EPILOGUE_DEFAULT && !epilogue->bias) return fail(GK_ERR_INVALID_ARGUMENT, "bias epilogue without a bias pointer");
 
-  gk::GemmArgs args;
+  gk::GemmArgs& args = out->args;
   make_args(conf, a, b, c, d, transforms, epilogue, &args);
 
   // aligned layouts move 16-byte vectors (reference src/layout.jl:22-34 traps on the device; here it is a host check)
@@ -631,11 +652,25 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
                        conf->block_shape.N, gx, gy);
   if (gx <= 0 || gy <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "empty grid");
 
-  gk::FamilyFn fn = family_fn(key);
+  out->gx = gx;
+  out->gy = gy;
+  return GK_OK;
+}
+
+}  // namespace gk_internal
+
+extern "C" {
+
+int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
+              const gk_epilogue* epilogue, int32_t kernel, void* stream) {
+  gk_internal::Launch L;
+  int rc = gk_internal::prepare_launch(conf, a, b, c, d, transforms, epilogue, kernel, nullptr, &L);
+  if (rc != GK_OK) return rc;
+  gk::FamilyFn fn = family_fn(L.key);
   hipError_t err = hipSuccess;
-  if (!fn || !fn(key, args, dim3((unsigned)gx, (unsigned)gy), (hipStream_t)stream, 1, &info, &err))
+  if (!fn || !fn(L.key, L.args, dim3((unsigned)L.gx, (unsigned)L.gy), (hipStream_t)stream, 1, &L.info, &err))
     return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance");
-  if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", info.name, hipGetErrorString(err));
+  if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", L.info.name, hipGetErrorString(err));
   return GK_OK;
 }
 

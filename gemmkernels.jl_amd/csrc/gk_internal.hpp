@@ -1,0 +1,24 @@
+// Shared between the translation units of the host layer (not part of the C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "gemmkernels_hip.h"
+#include "kernels/common.hpp"
+#include "kernels/registry.hpp"
+
+namespace gk_internal {
+
+// Records the thread-local error message and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+struct Launch {
+  gk::InstanceKey key;
+  gk::InstanceInfo info;
+  gk::GemmArgs args;
+  int gx, gy;
+};
+
+int prepare_launch(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
+                   const gk_epilogue* epilogue, int32_t kernel, const gk::InstanceInfo* custom, Launch* out);
+
+}  // namespace gk_internal

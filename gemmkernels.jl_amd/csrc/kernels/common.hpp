@@ -226,6 +226,38 @@ __device__ __forceinline__ void apply_list_regs(const OpList& t, float (&x)[COUN
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Transform hooks.  The kernels compiled into the library interpret the op lists of the launch
+// arguments.  A translation unit that defines GK_USER_HOOKS before including this header supplies
+//   struct gk::UserHooks { static constexpr bool present[8];
+//                          template <int H> static __device__ float apply(float x); };
+// and every hook becomes inline code of the caller's choosing: that is how kernels specialised
+// at run time carry arbitrary elementwise functions, like the functors the reference inlines
+// through its JIT (src/transform.jl:20-30).
+// ---------------------------------------------------------------------------------------------
+template <int H>
+__device__ __forceinline__ bool hook_present(const GemmArgs& args) {
+#ifdef GK_USER_HOOKS
+  (void)args;
+  return UserHooks::present[H];
+#else
+  return args.t[H].n > 0;
+#endif
+}
+
+template <int H, int COUNT>
+__device__ __forceinline__ void hook_regs(const GemmArgs& args, float (&x)[COUNT]) {
+#ifdef GK_USER_HOOKS
+  (void)args;
+  if constexpr (UserHooks::present[H]) {
+#pragma unroll
+    for (int e = 0; e < COUNT; ++e) x[e] = UserHooks::template apply<H>(x[e]);
+  }
+#else
+  apply_list_regs<COUNT>(args.t[H], x);
+#endif
+}
+
 // One element of C / D in the element type the layout names (accumulators are fp32; a 16-bit D gets
 // one rounding, at the store).
 __device__ __forceinline__ float load_cd(const void* base, int dtype, long long idx) {

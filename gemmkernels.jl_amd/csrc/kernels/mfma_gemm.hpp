@@ -239,19 +239,19 @@ template <> struct Mfma<__bf16> {
 // fp32 op list on the 8 packed 16-bit values of a fragment, rounded back to T.  gl2sh then
 // sh2rf: the value is rounded to T after each hook like the LDS copy and the fragment of the
 // reference (src/kernel.jl:224-236, 311-319).
-template <typename T>
-__device__ __forceinline__ int4v transform_fragment(int4v f, const OpList& t0, const OpList& t1) {
+template <typename T, int H0, int H1>
+__device__ __forceinline__ int4v transform_fragment(int4v f, const GemmArgs& args) {
   typedef T vec8 __attribute__((ext_vector_type(8)));
   vec8 v = __builtin_bit_cast(vec8, f);
   float x[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = (float)v[e];
-  if (t0.n > 0) {
-    apply_list_regs<8>(t0, x);
+  if (hook_present<H0>(args)) {
+    hook_regs<H0, 8>(args, x);
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = (float)(T)x[e];
   }
-  if (t1.n > 0) apply_list_regs<8>(t1, x);
+  if (hook_present<H1>(args)) hook_regs<H1, 8>(args, x);
 #pragma unroll
   for (int e = 0; e < 8; ++e) v[e] = (T)x[e];
   return __builtin_bit_cast(int4v, v);
@@ -456,7 +456,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
       }
     if (Cfg::FUSED) {
-      if (args.t[H_GL2SH_C].n > 0 || args.t[H_SH2RF_C].n > 0) {
+      if (hook_present<H_GL2SH_C>(args) || hook_present<H_SH2RF_C>(args)) {
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
@@ -464,8 +464,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             float x[16];
 #pragma unroll
             for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
-            apply_list_regs<16>(args.t[H_GL2SH_C], x);
-            apply_list_regs<16>(args.t[H_SH2RF_C], x);
+            hook_regs<H_GL2SH_C, 16>(args, x);
+            hook_regs<H_SH2RF_C, 16>(args, x);
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[fi][fj][v] = x[v];
           }
@@ -480,8 +480,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         for (int v = 0; v < 16; ++v) acc[fi][fj][v] = 0.0f;
   }
 
-  const bool xf_a = Cfg::FUSED && (args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0);
-  const bool xf_b = Cfg::FUSED && (args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0);
+  const bool xf_a = Cfg::FUSED && (hook_present<H_GL2SH_A>(args) || hook_present<H_SH2RF_A>(args));
+  const bool xf_b = Cfg::FUSED && (hook_present<H_GL2SH_B>(args) || hook_present<H_SH2RF_B>(args));
   // kept in registers for the whole K loop: a scalar load inside the loop would make the compiler
   // wait for lgkmcnt(0), which also drains the LDS reads that are meant to stay in flight
   const bool fast_a = std::is_same<T, _Float16>::value && args.fast_scale_a != 0;
@@ -528,7 +528,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           for (int fi = 0; fi < FM; ++fi) va[fi] = scale_fragment_f16(va[fi], scale_a);
         } else if constexpr (Cfg::FUSED_AB_GENERIC) {
 #pragma unroll
-          for (int fi = 0; fi < FM; ++fi) va[fi] = transform_fragment<T>(va[fi], args.t[H_GL2SH_A], args.t[H_SH2RF_A]);
+          for (int fi = 0; fi < FM; ++fi) va[fi] = transform_fragment<T, H_GL2SH_A, H_SH2RF_A>(va[fi], args);
         }
       }
       if (xf_b) {
@@ -537,7 +537,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           for (int fj = 0; fj < FN; ++fj) vb[fj] = scale_fragment_f16(vb[fj], scale_b);
         } else if constexpr (Cfg::FUSED_AB_GENERIC) {
 #pragma unroll
-          for (int fj = 0; fj < FN; ++fj) vb[fj] = transform_fragment<T>(vb[fj], args.t[H_GL2SH_B], args.t[H_SH2RF_B]);
+          for (int fj = 0; fj < FN; ++fj) vb[fj] = transform_fragment<T, H_GL2SH_B, H_SH2RF_B>(vb[fj], args);
         }
       }
     }
@@ -629,7 +629,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
       for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
       if (Cfg::FUSED) {
-        apply_list_regs<16>(args.t[H_RF2SH_D], x);
+        hook_regs<H_RF2SH_D, 16>(args, x);
         if (args.epi_kind == 1) {
 #pragma unroll
           for (int v = 0; v < 16; ++v) x[v] = x[v] + args.bias[ncol + 32 * fj + 8 * (v / 4) + (v % 4)];
@@ -638,7 +638,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
           for (int v = 0; v < 16; ++v) x[v] = x[v] + bv;
         }
-        apply_list_regs<16>(args.t[H_SH2GL_D], x);
+        hook_regs<H_SH2GL_D, 16>(args, x);
       }
       // the accumulator is rounded once, to the element type of D
       if (args.d_dtype == DT_F32) {

@@ -106,6 +106,11 @@ _SIGNATURES = {
                                       ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]),
     "gk_matmul": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                  ctypes.POINTER(gk_transforms), ctypes.POINTER(gk_epilogue), ctypes.c_int32, ctypes.c_void_p]),
+    "gk_rtc_compile": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.POINTER(ctypes.c_char_p), ctypes.c_int32,
+                                      ctypes.POINTER(ctypes.c_void_p)]),
+    "gk_rtc_matmul": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(gk_config), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                     ctypes.c_void_p, ctypes.POINTER(gk_epilogue), ctypes.c_void_p]),
+    "gk_rtc_kernel_name": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
     "gk_dev_alloc": (ctypes.c_int, [ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]),
     "gk_dev_free": (ctypes.c_int, [ctypes.c_void_p]),
     "gk_copy_to_device": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
@@ -127,6 +132,13 @@ def lib() -> ctypes.CDLL:
             raise RuntimeError(
                 f"{LIB_PATH} is missing: build the HIP library first (make -C gemmkernels.jl_amd/csrc, "
                 "or __graft_entry__.build()). There is no CPU fallback.")
+        try:
+            # torch carries its own copy of the HIP runtime; a process must hold exactly one, so when
+            # torch is installed it is loaded first and this library binds to that copy.  (Loading the
+            # library first would make a later `import torch` find a runtime it was not built with.)
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         handle = ctypes.CDLL(LIB_PATH)
         for name, (restype, argtypes) in _SIGNATURES.items():
             fn = getattr(handle, name)

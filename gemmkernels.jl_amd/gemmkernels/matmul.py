@@ -81,6 +81,8 @@ _lowered = {}
 def lower_transforms(transforms: dict) -> Optional[_lib.gk_transforms]:
     if all(t.is_identity for t in transforms.values()):
         return None
+    if any(t.expr is not None for t in transforms.values()):
+        raise ConfigError("expression transforms need a specialised kernel (gemmkernels.specialize)")
     key = tuple(transforms[name].ops for name in _HOOKS)
     hit = _lowered.get(key)
     if hit is not None:
@@ -101,6 +103,54 @@ def _raise(rc: int):
     raise ConfigError(msg, rc)
 
 
+class SpecializedKernel:
+    """A kernel compiled at run time (hipRTC) for one configuration with its transform hooks inlined:
+    arbitrary C expressions in x, and block shapes outside the table compiled into the library.  The
+    counterpart of the reference's one-JIT-compiled-kernel-per-Config with inlined functors
+    (src/matmul.jl:38, src/transform.jl:26-30).  The first construction for a given configuration and
+    set of expressions compiles (seconds); later ones are served from the library's cache."""
+
+    def __init__(self, conf: Config, transforms: dict):
+        self.conf = conf
+        exprs = (ctypes.c_char_p * 8)()
+        self.expressions = []
+        for i, name in enumerate(_HOOKS):
+            t = transforms.get(name) or _IDENTITY
+            e = t.c_expression()
+            self.expressions.append(e)
+            exprs[i] = e.encode() if e is not None else None
+        handle = ctypes.c_void_p()
+        cconf = conf.to_c()
+        rc = _lib.lib().gk_rtc_compile(ctypes.byref(cconf), exprs, Kernel.matmul_pipelined.code, ctypes.byref(handle))
+        if rc != _lib.GK_OK:
+            _raise(rc)
+        self._handle = handle
+        buf = ctypes.create_string_buffer(200)
+        _lib.lib().gk_rtc_kernel_name(handle, buf, len(buf))
+        self.name = buf.value.decode()
+
+    def plan(self, a, b, c, d, epilogue=None) -> "Plan":
+        return Plan(self.conf, a, b, c, d, {}, _DEFAULT_EPILOGUE if epilogue is None else epilogue, Kernel.matmul_pipelined,
+                    specialized=self)
+
+    def __call__(self, a, b, c, d, epilogue=None, stream=None):
+        return self.plan(a, b, c, d, epilogue)(stream)
+
+
+def specialize(conf: Config, *,
+               transform_global_to_shared_a=None, transform_global_to_shared_b=None,
+               transform_global_to_shared_c=None, transform_shared_to_global_d=None,
+               transform_shared_to_regs_a=None, transform_shared_to_regs_b=None,
+               transform_shared_to_regs_c=None, transform_regs_to_shared_d=None) -> SpecializedKernel:
+    """Compile (or fetch from the cache) the kernel of ``conf`` with these hooks inlined.  A hook is a
+    ``Transform.Elementwise`` (op list or ``expr="..."``) or directly a C expression string in x."""
+    given = dict(transform_global_to_shared_a=transform_global_to_shared_a, transform_global_to_shared_b=transform_global_to_shared_b,
+                 transform_global_to_shared_c=transform_global_to_shared_c, transform_shared_to_global_d=transform_shared_to_global_d,
+                 transform_shared_to_regs_a=transform_shared_to_regs_a, transform_shared_to_regs_b=transform_shared_to_regs_b,
+                 transform_shared_to_regs_c=transform_shared_to_regs_c, transform_regs_to_shared_d=transform_regs_to_shared_d)
+    return SpecializedKernel(conf, {k: (Transform.Elementwise(expr=v) if isinstance(v, str) else v) for k, v in given.items()})
+
+
 class Plan:
     """One launch with everything but the stream lowered ahead of time: the descriptors of the
     configuration, the transforms and the epilogue, and the operand addresses.  Calling the plan is
@@ -111,21 +161,27 @@ class Plan:
 
     __slots__ = ("_fn", "_conf", "_trans", "_epi", "_args", "_keep", "d")
 
-    def __init__(self, conf: Config, a, b, c, d, transforms: dict, epilogue, kernel):
+    def __init__(self, conf: Config, a, b, c, d, transforms: dict, epilogue, kernel, specialized=None):
+        if specialized is None and any(t.expr is not None for t in transforms.values()):
+            specialized = SpecializedKernel(conf, transforms)       # expression hooks: a run-time compiled kernel
         cconf = conf.to_c(_leading_dim(a, conf.global_a_layout), _leading_dim(b, conf.global_b_layout),
                           _leading_dim(c, conf.global_c_layout), _leading_dim(d, conf.global_d_layout))
         self._conf = _lib.gk_config.from_buffer_copy(cconf)        # to_c hands out a cached, shared descriptor
-        self._trans = lower_transforms(transforms)
+        self._trans = None if specialized is not None else lower_transforms(transforms)
         self._epi = None
         if epilogue.kind != Epilogue.DEFAULT:
             self._epi = _lib.gk_epilogue()
             self._epi.kind = epilogue.kind
             self._epi.bias = _ptr(epilogue.bias)
-        self._fn = _lib.lib().gk_matmul
-        self._args = (ctypes.byref(self._conf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
-                      ctypes.byref(self._trans) if self._trans is not None else None,
-                      ctypes.byref(self._epi) if self._epi is not None else None, kernel.code)
-        self._keep = (a, b, c, d, epilogue)
+        epi_ref = ctypes.byref(self._epi) if self._epi is not None else None
+        if specialized is not None:
+            self._fn = _lib.lib().gk_rtc_matmul
+            self._args = (specialized._handle, ctypes.byref(self._conf), _ptr(a), _ptr(b), _ptr(c), _ptr(d), epi_ref)
+        else:
+            self._fn = _lib.lib().gk_matmul
+            self._args = (ctypes.byref(self._conf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                          ctypes.byref(self._trans) if self._trans is not None else None, epi_ref, kernel.code)
+        self._keep = (a, b, c, d, epilogue, specialized)
         self.d = d
 
     def __call__(self, stream=None):
@@ -170,11 +226,14 @@ def matmul(conf: Config, a, b, c, d, *,
             transform_global_to_shared_c is None and transform_shared_to_global_d is None and
             transform_shared_to_regs_a is None and transform_shared_to_regs_b is None and
             transform_shared_to_regs_c is None and transform_regs_to_shared_d is None):
-        ctrans = lower_transforms(_collect(dict(
+        collected = _collect(dict(
             transform_global_to_shared_a=transform_global_to_shared_a, transform_global_to_shared_b=transform_global_to_shared_b,
             transform_global_to_shared_c=transform_global_to_shared_c, transform_shared_to_global_d=transform_shared_to_global_d,
             transform_shared_to_regs_a=transform_shared_to_regs_a, transform_shared_to_regs_b=transform_shared_to_regs_b,
-            transform_shared_to_regs_c=transform_shared_to_regs_c, transform_regs_to_shared_d=transform_regs_to_shared_d)))
+            transform_shared_to_regs_c=transform_shared_to_regs_c, transform_regs_to_shared_d=transform_regs_to_shared_d))
+        if any(t.expr is not None for t in collected.values()):
+            return Plan(conf, a, b, c, d, collected, _DEFAULT_EPILOGUE if epilogue is None else epilogue, kernel)(stream)
+        ctrans = lower_transforms(collected)
 
     cconf = conf.to_c(_leading_dim(a, conf.global_a_layout), _leading_dim(b, conf.global_b_layout),
                       _leading_dim(c, conf.global_c_layout), _leading_dim(d, conf.global_d_layout))

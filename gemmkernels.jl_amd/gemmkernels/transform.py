@@ -100,8 +100,18 @@ def identity(x):
 class Elementwise:
     """``Transform.Elementwise(f)``; ``Elementwise()`` is the identity (src/transform.jl:24)."""
 
-    def __init__(self, func: Optional[Callable] = None, ops: Optional[List[Tuple[int, float, float]]] = None):
+    def __init__(self, func: Optional[Callable] = None, ops: Optional[List[Tuple[int, float, float]]] = None,
+                 expr: Optional[str] = None):
         self.func = identity if func is None else func
+        self.expr = expr
+        if expr is not None:
+            # a C expression in the fp32 variable x, outside the closed vocabulary: the launch compiles
+            # a kernel specialised for it at run time (the counterpart of the reference inlining an
+            # arbitrary Julia functor, src/transform.jl:26-30)
+            if "x" not in expr:
+                raise ConfigError("unsupported transform: the expression does not depend on x")
+            self.ops = ()
+            return
         if ops is not None:
             self.ops = tuple((int(k), float(p0), float(p1)) for k, p0, p1 in ops)
         else:
@@ -114,11 +124,41 @@ class Elementwise:
 
     @property
     def is_identity(self) -> bool:
-        return len(self.ops) == 0
+        return len(self.ops) == 0 and self.expr is None
+
+    def c_expression(self) -> Optional[str]:
+        """The hook as a C expression in x (None for the identity): the given expression, or the op
+        list spelled with the helper functions every specialised kernel is compiled with."""
+        if self.expr is not None:
+            return self.expr
+        if not self.ops:
+            return None
+
+        def lit(v: float) -> str:
+            import numpy as np
+            return float(np.float32(v)).hex() + "f"          # exact binary32 literal
+
+        e = "x"
+        for kind, p0, p1 in self.ops:
+            if kind == SCALE:
+                e = f"({e} * {lit(p0)})"
+            elif kind == ADD:
+                e = f"({e} + {lit(p0)})"
+            elif kind == RELU:
+                e = f"gk_relu({e})"
+            elif kind == NEG:
+                e = f"(-{e})"
+            elif kind == ABS:
+                e = f"gk_abs({e})"
+            elif kind == CLAMP:
+                e = f"gk_clamp({e}, {lit(p0)}, {lit(p1)})"
+            elif kind == SQUARE:
+                e = f"gk_square({e})"
+        return e
 
     def __call__(self, x, tile=None):
         """Host evaluation (src/transform.jl:26)."""
         return self.func(x)
 
     def __repr__(self):
-        return f"Transform.Elementwise({list(self.ops)})"
+        return f"Transform.Elementwise(expr={self.expr!r})" if self.expr is not None else f"Transform.Elementwise({list(self.ops)})"

@@ -244,6 +244,22 @@ int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const
 int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
               const gk_transforms* transforms, const gk_epilogue* epilogue, int32_t kernel, void* stream);
 
+/* Kernels specialised at run time (hipRTC).  The reference compiles one kernel per Config type and
+ * inlines arbitrary Julia functors at the eight transform hooks (src/matmul.jl:38,
+ * src/transform.jl:20-30); gk_matmul offers a closed op vocabulary and a table of tiles instead.
+ * gk_rtc_compile closes that gap for the real MFMA operator with aligned layouts: hooks[h] is NULL
+ * (identity) or a C expression in the fp32 variable x, e.g. "x > 0.0f ? x : 0.01f * x", for hook h
+ * in the order of gk_hook; block_shape / compute_warp may be any tile the kernel template accepts
+ * (32x32 accumulator blocks, BLOCK_K of 32, 64 or 128, at most 160 KiB of LDS).  Expressions are
+ * evaluated in fp32 without contraction and the result is rounded to the hook's destination type,
+ * like the op lists of gk_matmul.  Compiled kernels are cached by configuration, expressions and
+ * device and live until the process ends.  gk_rtc_matmul runs the same checks as gk_matmul. */
+typedef struct gk_rtc_kernel gk_rtc_kernel;
+int gk_rtc_compile(const gk_config* conf, const char* const hooks[8], int32_t kernel, gk_rtc_kernel** out);
+int gk_rtc_matmul(gk_rtc_kernel* kernel, const gk_config* conf, const void* a, const void* b, const void* c, void* d,
+                  const gk_epilogue* epilogue, void* stream);
+int gk_rtc_kernel_name(const gk_rtc_kernel* kernel, char* buf, size_t n);
+
 /* Device memory for callers that have no GPU array package of their own (a Julia session without
  * AMDGPU.jl, a C test): thin wrappers over hipMalloc / hipFree / hipMemcpy / hipDeviceSynchronize on
  * the current device.  The reference relies on CUDA.jl's CuArray for this (src/matmul.jl:185-215,
