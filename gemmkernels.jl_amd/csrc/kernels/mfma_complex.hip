@@ -27,6 +27,7 @@ int family_complex(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipS
   GK_CPLX(bm_, bn_, bk_, wm_, wn_, st_, 1, 1, dual_, "mfma_" TAG "_tn_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_CPLX(bm_, bn_, bk_, wm_, wn_, st_, 1, 0, dual_, "mfma_" TAG "_tt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)
   GK_CPLX_T(128, 256, 32, 2, 4, 3, 0, "complex")
+  GK_CPLX_T(128, 128, 32, 2, 2, 4, 0, "complex")
   GK_CPLX_T(64, 128, 32, 2, 2, 3, 0, "complex")
   GK_CPLX_T(64, 64, 32, 4, 2, 2, 0, "complex")
   GK_CPLX_T(32, 64, 32, 2, 2, 2, 0, "complex")

@@ -182,7 +182,7 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
 
 
 # complex / dual tiles (complex elements) -> waves
-_COMPLEX_TILES = [((128, 256, 32), (2, 4)), ((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
+_COMPLEX_TILES = [((128, 256, 32), (2, 4)), ((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 
 # tiles of the vector-ALU kernel and of the bounds-checked MFMA kernel
 _FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2))]

@@ -30,6 +30,7 @@ def run(conf, a, b, c, M, N):
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("dims,block", [((128, 128, 64), (32, 64, 32)), ((128, 128, 128), (64, 64, 32)), ((128, 256, 96), (64, 128, 32)),
+                                        ((256, 256, 160), (128, 128, 32)),
                                         ((256, 512, 64), (128, 256, 32))])
 def test_complex_all_transposes(gpu, dims, block, ta, tb):
     M, N, K = dims
