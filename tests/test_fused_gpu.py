@@ -84,6 +84,39 @@ def test_all_eight_hooks(gpu, ta, tb):
     assert oracle.rel_frobenius(d, ref) <= TOL
 
 
+ALL_TILES = [((256, 256, 64), (2, 4)), ((256, 256, 64), (2, 2)), ((256, 256, 32), (2, 4)), ((256, 256, 32), (4, 2)), ((256, 256, 32), (2, 2)),
+             ((256, 128, 64), (2, 2)), ((128, 256, 64), (2, 2)), ((128, 128, 64), (2, 2)), ((128, 128, 64), (4, 2)), ((128, 128, 32), (2, 2)),
+             ((64, 64, 64), (2, 2)), ((64, 64, 32), (1, 1))]
+
+
+@pytest.mark.parametrize("block,waves", ALL_TILES)
+@pytest.mark.parametrize("level", [1, 2])
+def test_every_tile_at_both_fuse_levels(gpu, block, waves, level):
+    """Level 1: C / D hooks, bias and one exact FP16 scale on A; level 2: arbitrary op lists on A and B
+    evaluated per element inside the K loop (the large-code kernels).  'T','N' puts both operands on
+    the direct-read path, 'N','T' on the transposing reads."""
+    from gemmkernels import NT
+    BM, BN, BK = block
+    M, N, K = 2 * BM, BN, 3 * BK
+    for ta, tb in ((True, False), (False, True)):
+        conf = configs.mfma_config(M, N, K, ta, tb, block_shape=block, warps_per_block=waves[0] * waves[1],
+                                   compute_warp=NT(M=BM // waves[0], N=BN // waves[1], K=16))
+        a = rng.matrix("upm1_f16", 61, (K, M) if ta else (M, K))
+        b = rng.matrix("upm1_f16", 62, (N, K) if tb else (K, N))
+        c = rng.matrix("upm1_f32", 63, (M, N))
+        bias = rng.normal_f32(64, N)
+        tr = dict(transform_global_to_shared_a=E(lambda x: x * 0.5), transform_shared_to_global_d=E(Transform.relu),
+                  transform_shared_to_regs_c=E(lambda x: x * 3.0))
+        if level == 2:
+            tr["transform_shared_to_regs_a"] = E(lambda x: Transform.square(x) - 0.25)
+            tr["transform_global_to_shared_b"] = E(lambda x: abs(x) * 1.5)
+        name = gk.kernel_name(conf, Kernel.matmul_pipelined, tr, Epilogue.Bias(0))
+        print("case", block, waves, level, ta, tb, name, flush=True)
+        d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=tr, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
+        ref = helpers.run_oracle(conf, a, b, c, (M, N), transforms=tr, epilogue=Epilogue.Bias(0), bias=bias)
+        assert oracle.rel_frobenius(d, ref) <= TOL, (ta, tb)
+
+
 def test_config3_full_size(gpu):
     w = configs.benchmark_config(3)
     run = w.prepare()
