@@ -23,7 +23,10 @@
  *
  * Parity pinning: the real/complex/tropical/dual GEMM functions are pinned in tests/ against
  * numpy float64 matmul, closed forms (identity, all-ones, single non-zero, diagonal product),
- * brute force on tiny shapes and linearity; layouts against index-distinct prime fixtures.
+ * brute force on tiny shapes and linearity; layouts against index-distinct prime fixtures; the
+ * integer element types (Int16 / Int32 / Int64, configs/configs.jl:495-497) against exact Python
+ * integers reduced modulo 2^bits with magnitudes that overflow; Float32 -> Float64 and Float64
+ * against numpy float64 matmul on dyadic inputs (bit-exact) and a math.fma chain.
  */
 #include <math.h>
 #include <stdint.h>
