@@ -323,6 +323,17 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   if ((c->cta_swizzle.kind == GK_SWIZZLE_HORIZONTALLY_TILED || c->cta_swizzle.kind == GK_SWIZZLE_VERTICALLY_TILED) && c->cta_swizzle.param <= 0)
     return fail(GK_ERR_INVALID_ARGUMENT, "tiled CTA swizzles need a positive tile size");
 
+  if (t) {
+    for (int h = 0; h < 8; ++h) {
+      if (t->hook[h].n_ops < 0 || t->hook[h].n_ops > GK_MAX_OPS)
+        return fail(GK_ERR_INVALID_ARGUMENT, "hook %d carries %d ops, a hook holds 0..%d", h, t->hook[h].n_ops, GK_MAX_OPS);
+      for (int i = 0; i < t->hook[h].n_ops; ++i)
+        if (t->hook[h].ops[i].kind < GK_T_IDENTITY || t->hook[h].ops[i].kind > GK_T_SQUARE)
+          return fail(GK_ERR_INVALID_ARGUMENT, "unknown elementwise op %d in hook %d", t->hook[h].ops[i].kind, h);
+    }
+  }
+  if (e && (e->kind < GK_EPILOGUE_DEFAULT || e->kind > GK_EPILOGUE_BIAS_ROW)) return fail(GK_ERR_INVALID_ARGUMENT, "unknown epilogue kind %d", e->kind);
+
   // src/config.jl:203-205
   if ((long long)b.M * b.K < 128 || (long long)b.K * b.N < 128 || b.K < 8)
     return fail(GK_ERR_BLOCK_SHAPE,
@@ -549,11 +560,10 @@ int32_t gk_threads_per_block(const gk_config* conf) {
 
 int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const gk_epilogue* epilogue, int32_t kernel,
                    char* buf, size_t n) {
-  (void)kernel;
   if (!conf || !buf || n == 0) return fail(GK_ERR_INVALID_ARGUMENT, "NULL argument");
   gk::InstanceKey key;
   gk::InstanceInfo info;
-  int rc = find_instance(conf, transforms, epilogue, &key, &info);
+  int rc = validate_config(conf, kernel, transforms, epilogue, &key, &info);      // a name only for a launch that would pass
   if (rc != GK_OK) return rc;
   snprintf(buf, n, "%s", info.name);
   return GK_OK;

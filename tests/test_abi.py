@@ -44,3 +44,21 @@ def test_null_config_is_an_error_not_a_crash():
     assert "NULL" in _lib.last_error()
     assert lib.gk_shmem_size(None, 0) == -1
     assert lib.gk_matmul(None, None, None, None, None, None, None, 0, None) == _lib.GK_ERR_INVALID_ARGUMENT
+
+
+def test_malformed_transforms_and_epilogues_are_refused():
+    import gemmkernels as gk
+    from gemmkernels import configs, Kernel
+    conf = configs.mfma_config(256, 256, 128).to_c()
+    lib = _lib.lib()
+    t = _lib.gk_transforms()
+    t.hook[2].n_ops = 5                                    # more than a hook holds
+    buf = ctypes.create_string_buffer(64)
+    assert lib.gk_kernel_name(ctypes.byref(conf), ctypes.byref(t), None, Kernel.matmul_pipelined.code, buf, 64) == _lib.GK_ERR_INVALID_ARGUMENT
+    t.hook[2].n_ops = 1
+    t.hook[2].ops[0].kind = 42                              # not an op of the vocabulary
+    assert lib.gk_kernel_name(ctypes.byref(conf), ctypes.byref(t), None, Kernel.matmul_pipelined.code, buf, 64) == _lib.GK_ERR_INVALID_ARGUMENT
+    e = _lib.gk_epilogue()
+    e.kind = 7
+    assert lib.gk_kernel_name(ctypes.byref(conf), None, ctypes.byref(e), Kernel.matmul_pipelined.code, buf, 64) == _lib.GK_ERR_INVALID_ARGUMENT
+    assert "epilogue" in _lib.last_error()
