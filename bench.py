@@ -126,10 +126,6 @@ def main():
     if not args.no_extras:
         lo, med = launch_distribution(run)
         result["single_launch_us"] = {"min": round(lo, 2), "median": round(med, 2), "launches": 40}
-        try:
-            result["shader_clock_mhz_after_run"] = int(torch.cuda.clock_rate())
-        except Exception:       # needs the amdsmi python module
-            pass
         # ---------------- the other transposes and configs (outside the timed region) ----------------
         extras = {}
         for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4b", None), (5, None)]:
