@@ -62,3 +62,33 @@ def test_malformed_transforms_and_epilogues_are_refused():
     e.kind = 7
     assert lib.gk_kernel_name(ctypes.byref(conf), None, ctypes.byref(e), Kernel.matmul_pipelined.code, buf, 64) == _lib.GK_ERR_INVALID_ARGUMENT
     assert "epilogue" in _lib.last_error()
+
+
+def test_error_messages_are_per_thread():
+    """gk_last_error is thread-local: concurrent callers never read each other's message."""
+    import threading
+    import gemmkernels as gk
+    from gemmkernels import configs, Kernel, NT
+    good = configs.mfma_config(256, 256, 128).to_c()
+    lds_hungry = configs.mfma_config(512, 512, 128, block_shape=(256, 256, 64)).to_c()
+    bad_block = _lib.gk_config.from_buffer_copy(good)
+    bad_block.block_shape.K = 4
+    lib = _lib.lib()
+    failures = []
+
+    def worker(conf, want_status, needle):
+        for _ in range(300):
+            rc = lib.gk_validate(ctypes.byref(conf), Kernel.matmul_pipelined.code)
+            msg = _lib.last_error() if rc != _lib.GK_OK else ""
+            if rc != want_status or needle not in msg:
+                failures.append((rc, msg))
+                return
+
+    threads = [threading.Thread(target=worker, args=(good, _lib.GK_OK, "")),
+               threading.Thread(target=worker, args=(bad_block, _lib.GK_ERR_BLOCK_SHAPE, "block shape")),
+               threading.Thread(target=worker, args=(lds_hungry, _lib.GK_OK, ""))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures[:2]

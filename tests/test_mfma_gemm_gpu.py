@@ -208,3 +208,35 @@ def test_bf16(gpu, ta, tb, d16):
     A, B = gk.bf16_values(a), gk.bf16_values(b)
     C = gk.bf16_values(c) if d16 else c
     assert oracle.rel_frobenius(d, oracle.gemm_f64(A, B, C, 1.0, 1.0, ta, tb)) <= tol
+
+
+def test_concurrent_launches_from_two_host_threads_on_two_streams(gpu):
+    """The launcher is re-entrant: two host threads enqueue different GEMMs on their own streams."""
+    import threading
+    import torch
+    results, errors = {}, []
+
+    def worker(tag, M, N, K, ta, tb, seed):
+        try:
+            conf = make_config(M, N, K, ta, tb, (128, 128, 64), (2, 2))
+            a, b, c = inputs(M, N, K, ta, tb, seed)
+            A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
+            D = gk.colmajor_empty((M, N), torch.float32)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    gk.matmul(conf, A, B, C, D, kernel=Kernel.matmul_pipelined)
+            stream.synchronize()
+            results[tag] = (gk.to_numpy(D), oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb))
+        except Exception as e:      # surfaced by the assertion below
+            errors.append((tag, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=("x", 512, 256, 320, False, False, 3100)),
+               threading.Thread(target=worker, args=("y", 256, 384, 192, True, True, 3200))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for tag, (d, ref) in results.items():
+        assert oracle.rel_frobenius(d, ref) <= TOL, tag
