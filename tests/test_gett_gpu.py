@@ -56,6 +56,30 @@ def test_distinct_extents_and_k_major_operands(gpu):
     assert np.array_equal(D.astype(np.float64), want)
 
 
+def test_tccg_benchmark_at_the_reference_sizes_with_fp16_output(gpu):
+    """The contraction the reference benchmarks (benchmarks/tensor-contractions/run.jl:10-21, 86-88):
+    D_abc = A_bda * B_dc with a = 64, b = 32, c = d = 2048, Float16 A, B and D.  D is stored with `a`
+    fastest while the GEMM's M index runs over (b, a), so the D stores are strided; accumulation is
+    FP32 with one rounding at the store."""
+    from gemmkernels import Layout, Float16, rng
+    ext = dict(a=64, b=32, c=2048, d=2048)
+    gmap = Layout.gett_map("bda", "dc", "abc", ext)
+    conf, _ = configs.gett_config("bda", "dc", "abc", ext, global_d_layout=Layout.GETT[Float16, gmap],
+                                  shared_d_layout=Layout.UnsafeAlignedColMajor[Float16])
+    A = rng.matrix("upm1_f16", 5101, (32 * 2048, 64)).reshape((32, 2048, 64), order="F")      # A[b,d,a]
+    B = rng.matrix("upm1_f16", 5102, (2048, 2048))                                              # B[d,c]
+    a, b = gk.colmajor(A), gk.colmajor(B)
+    d = gk.colmajor_empty((64, 32, 2048), torch.float16)
+    d.fill_(float("nan"))
+    print("case", gk.kernel_name(conf, Kernel.matmul_pipelined), flush=True)
+    gk.matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    D = gk.to_numpy(d)
+    assert D.dtype == np.float16 and np.isfinite(D).all()
+    want = np.einsum("bda,dc->abc", A.astype(np.float32), B.astype(np.float32))
+    assert oracle.rel_frobenius(D, want) <= 1e-3
+
+
 def materialise(A, B, ext, gmap):
     """A_mat[m, k] and B_mat[n, k] with the kernel's own index orders (modes fastest first)."""
     a_modes, b_modes = "aebf", "dfce"
