@@ -35,6 +35,10 @@ def parse_args():
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--no-extras", action="store_true", help="skip the secondary configs and the CPU baseline")
+    p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4b", "5"],
+                   help="benchmark config to time as the step (default: 2, the headline; the others are for profiling one "
+                        "kernel at a time and imply --no-extras)")
+    p.add_argument("--variant", default="NN", choices=["NN", "NT", "TN", "TT"], help="transposes of config 2")
     p.add_argument("--copy-calibration", action="store_true",
                    help="instead of the benchmark, run a plain 256 MiB device-to-device copy 10 times: the reference "
                         "reading for the FETCH_SIZE / WRITE_SIZE counters of rocprofv3")
@@ -96,6 +100,25 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 10}}))
+        return
+
+    if args.workload != "2" or args.variant != "NN":
+        # one of the other workloads as the step: same JSON shape, for profiling a single kernel
+        key = int(args.workload) if args.workload.isdigit() else args.workload
+        wl = configs.benchmark_config(key, variant=args.variant if key == 2 else None)
+        run = wl.prepare()
+        us, _ = time_launches(run, args.steps, args.warmup)
+        hbm = wl.bound == "hbm"
+        achieved = wl.bytes / us / 1e3 if hbm else wl.flops / us / 1e6
+        peak = PEAK_HBM_GBS if hbm else PEAK_FP16_TFLOPS
+        print(json.dumps({
+            "metric": "GB/s" if hbm else "TFLOP/s", "value": round(achieved, 2), "unit": "GB/s" if hbm else "TFLOP/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16 multiplicands, f32 accumulate" if key != 1 else "f32", "data": "synthetic (counter-based splitmix64 streams)",
+            "config": {"workload": wl.description, "kernel": wl.kernel_name},
+            "roofline": {"bound": "hbm" if hbm else "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s",
+                         "frac": round(achieved / peak, 4), "traffic": None, "kernel": wl.kernel_name, "avg_launch_us": round(us, 2),
+                         "bytes_per_launch": wl.bytes, "flop_per_launch": wl.flops}}))
         return
 
     # ---------------- headline: config 2, NN ----------------
