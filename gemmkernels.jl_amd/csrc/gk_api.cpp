@@ -313,7 +313,7 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   const gk_operator& op = c->op;
   if (g.M <= 0 || g.N <= 0 || g.K <= 0) return fail(GK_ERR_DIMENSION_MISMATCH, "matmul_shape must be positive, got (%d, %d, %d)", g.M, g.N, g.K);
   if (b.M <= 0 || b.N <= 0 || b.K <= 0) return fail(GK_ERR_BLOCK_SHAPE, "block_shape must be positive");
-  if (kernel < GK_KERNEL_SINGLESTAGE || kernel > GK_KERNEL_PIPELINED_NG) return fail(GK_ERR_INVALID_ARGUMENT, "unknown kernel kind %d", kernel);
+  if (kernel < GK_KERNEL_SINGLESTAGE || kernel > GK_KERNEL_SPLIT_K) return fail(GK_ERR_INVALID_ARGUMENT, "unknown kernel kind %d", kernel);
   const gk_layout* layouts[8] = {&c->global_a_layout, &c->global_b_layout, &c->global_c_layout, &c->global_d_layout,
                                  &c->shared_a_layout, &c->shared_b_layout, &c->shared_c_layout, &c->shared_d_layout};
   for (const gk_layout* l : layouts)
@@ -678,6 +678,38 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   if (rc != GK_OK) return rc;
   gk::FamilyFn fn = family_fn(L.key);
   hipError_t err = hipSuccess;
+  if (kernel == GK_KERNEL_SPLIT_K) {
+    if (L.key.family != gk::FAMILY_MFMA) return fail(GK_ERR_UNSUPPORTED, "the K-split kernel runs the real MFMA operator on aligned layouts");
+    if (conf->global_d_layout.eltype != GK_F32) return fail(GK_ERR_UNSUPPORTED, "the K-split kernel adds partial sums with fp32 atomics: D must be Float32");
+    if ((epilogue && epilogue->kind != GK_EPILOGUE_DEFAULT) || L.args.t[gk::H_RF2SH_D].n > 0 || L.args.t[gk::H_SH2GL_D].n > 0)
+      return fail(GK_ERR_UNSUPPORTED, "the K-split kernel takes no transform on D and no bias (they would apply to partial sums)");
+    // K slices: enough workgroups to fill every CU as far as the LDS lets them share it (small tiles
+    // hide each other's latency, measured best at up to four per CU), each slice at least eight K tiles
+    // long so that its prologue, epilogue and atomic adds stay a small part of it
+    const int tiles = L.gx * L.gy;
+    const int kt = conf->matmul_shape.K / conf->block_shape.K;
+    int per_cu = L.info.lds_bytes > 0 ? (160 * 1024) / L.info.lds_bytes : 1;
+    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+    int slices = (per_cu * gk::kNumCUs + tiles - 1) / tiles;
+    if (slices > kt / 8) slices = kt / 8;
+    gk::InstanceInfo sk_info;
+    // K-split instances exist for the small tiles that skinny products run; anything else (a large
+    // tile, generic A / B hooks) runs unsplit below
+    if (slices > 1 && gk::family_mfma_splitk(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
+      const int per = (kt + slices - 1) / slices;
+      slices = (kt + per - 1) / per;
+      gk::GemmArgs first = L.args;       // slice 0: reads C, writes D
+      first.k_begin = 0; first.k_steps = per; first.atomic_d = 0;
+      gk::family_mfma_splitk(L.key, first, dim3((unsigned)L.gx, (unsigned)L.gy, 1), (hipStream_t)stream, 1, &sk_info, &err);
+      if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
+      gk::GemmArgs rest = L.args;        // slices 1..: start from zero, add into D; stream order puts them after slice 0
+      rest.k_begin = per; rest.k_steps = per; rest.atomic_d = 1; rest.c_mode = 0;
+      rest.t[gk::H_GL2SH_C].n = 0; rest.t[gk::H_SH2RF_C].n = 0;      // the hooks of C belong to slice 0 alone
+      gk::family_mfma_splitk(L.key, rest, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)(slices - 1)), (hipStream_t)stream, 1, &sk_info, &err);
+      if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
+      return GK_OK;
+    }
+  }
   if (!fn || !fn(L.key, L.args, dim3((unsigned)L.gx, (unsigned)L.gy), (hipStream_t)stream, 1, &L.info, &err))
     return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance");
   if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", L.info.name, hipGetErrorString(err));

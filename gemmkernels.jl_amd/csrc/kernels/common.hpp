@@ -21,6 +21,7 @@ typedef int int2v __attribute__((ext_vector_type(2)));
 #define GK_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
 constexpr int kWaveSize = 64;
+constexpr int kNumCUs = 256;      // MI355X
 
 // dtype codes (same values as gk_dtype of the C ABI)
 enum : int { DT_F16 = 0, DT_BF16 = 1, DT_F32 = 2, DT_F64 = 3, DT_I16 = 4, DT_I32 = 5, DT_I64 = 6 };
@@ -86,6 +87,9 @@ struct GemmArgs {
   int fast_scale_a, fast_scale_b;
   float scale_a, scale_b;
   GettDim gm, gn, gk;
+  // K-split launches (0 / 0 / 0 otherwise): workgroup z handles the k_steps tiles of K that start at
+  // tile k_begin + z * k_steps and, with atomic_d, adds its partial result into D atomically
+  int k_begin, k_steps, atomic_d;
 };
 
 // ---------------------------------------------------------------------------------------------

@@ -268,7 +268,7 @@ __device__ __forceinline__ int4v scale_fragment_f16(int4v f, float scale) {
 }
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int A_KIND_, int B_KIND_, typename T_, int FUSE_,
-          bool GETT_ = false, int FIX_ = FIX_NONE>
+          bool GETT_ = false, int FIX_ = FIX_NONE, bool SPLITK_ = false>
 struct MfmaGemmConfig {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr int A_KIND = A_KIND_, B_KIND = B_KIND_, FIX = FIX_;
@@ -280,6 +280,9 @@ struct MfmaGemmConfig {
   static constexpr bool FUSED_AB_GENERIC = FUSE_ == 2;
   static constexpr bool EXPAND_A = (FIX_ != FIX_NONE);   // complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
+  // K-split instances: a workgroup handles one slice of K (blockIdx.z) and may add its partial result
+  // into D with atomics.  A variant of its own so that the plain kernels carry none of it.
+  static constexpr bool SPLITK = SPLITK_;
   static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / 16) % 2 == 0);   // cross-step fragment prefetch
   typedef T_ T;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -300,6 +303,7 @@ struct MfmaGemmConfig {
   static_assert((STAGES - 2) * DMA_PER_TILE <= 63, "vmcnt is a 6-bit counter");
   static_assert(FM * FN > 0, "empty wave tile");
   static_assert(!GETT || (A_KIND != OPK_CROWK && B_KIND != OPK_CROWK && FIX == FIX_NONE), "contractions are real");
+  static_assert(!SPLITK || (!GETT && FIX == FIX_NONE), "K-split instances are plain real GEMMs");
 };
 
 template <class Cfg>
@@ -406,7 +410,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     }
   };
 
-  const int KT = args.K / BK;
+  // K tiles of this workgroup: all of them, or one slice of a K-split launch
+  int KT = args.K / BK;
+  if constexpr (Cfg::SPLITK) {
+    const int kt0 = args.k_begin + (int)blockIdx.z * args.k_steps;
+    KT = (KT - kt0) < args.k_steps ? (KT - kt0) : args.k_steps;
+    if (KT <= 0) return;       // the whole workgroup leaves together, before any barrier
+    ga += (long long)kt0 * a_step;
+    gb += (long long)kt0 * b_step;
+  }
 
   // --- prologue: start the first STAGES-1 tiles on their way ---
 #pragma unroll
@@ -641,6 +653,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         hook_regs<H_SH2GL_D, 16>(args, x);
       }
       // the accumulator is rounded once, to the element type of D
+      if constexpr (Cfg::SPLITK) {
+        if (args.atomic_d) {
+          // partial result of a K slice: fp32 atomic adds (the order of the slices, and with it the
+          // last bits of the sum, is not fixed)
+          float* dp = (float*)args.d + off;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) atomicAdd(&dp[(long long)(8 * (v / 4) + (v % 4)) * ns], x[v]);
+          continue;
+        }
+      }
       if (args.d_dtype == DT_F32) {
         float* dp = (float*)args.d + off;
 #pragma unroll

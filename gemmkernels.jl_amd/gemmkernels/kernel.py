@@ -22,6 +22,9 @@ class KernelKind:
 matmul_singlestage = KernelKind(0, "matmul_singlestage")     # src/kernel.jl:10-129
 matmul_pipelined = KernelKind(1, "matmul_pipelined")         # src/kernel.jl:147-350
 matmul_pipelined_ng = KernelKind(2, "matmul_pipelined_ng")   # src/kernel.jl:368-574
+# no counterpart in the reference: the pipelined kernel with the K range cut into slices that run as
+# separate workgroups (fp32 atomic adds into D), for problems with too few output tiles to fill the chip
+matmul_split_k = KernelKind(3, "matmul_split_k")
 
 
 def shmem_size(conf, kernel: KernelKind = matmul_singlestage) -> int:

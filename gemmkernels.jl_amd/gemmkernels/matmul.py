@@ -382,6 +382,12 @@ def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None)
             raise ConfigError(f"{name} = {value!r} is not representable in binary32, the parameter type of the transform hooks")
     ta = Transform.Elementwise(ops=[] if alpha_c == 1.0 else [(Transform.SCALE, alpha_c, 0.0)])
     tc = Transform.Elementwise(ops=[] if beta_c == 1.0 else [(Transform.SCALE, beta_c, 0.0)])
+    if (kernel is Kernel.matmul_pipelined and conf.operator.kind == Operator.MFMA and from_torch(C.dtype) == Float32):
+        # few output tiles and a long K loop (skinny products): cut K into slices so that every CU gets work
+        bs, ms = conf.block_shape, conf.matmul_shape
+        tiles = -(-ms.M // bs.M) * -(-ms.N // bs.N)
+        if tiles <= 128 and ms.K // bs.K >= 4:
+            kernel = Kernel.matmul_split_k
     return plan(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)
 
 

@@ -148,11 +148,17 @@ typedef struct gk_config {
 } gk_config;
 
 /* Kernels (reference src/kernel.jl: matmul_singlestage :10-129, matmul_pipelined :147-350,
- * matmul_pipelined_ng :368-574). */
+ * matmul_pipelined_ng :368-574).  GK_KERNEL_SPLIT_K has no counterpart in the reference: for
+ * problems with too few output tiles to fill the 256 CUs (skinny M or N, long K) the K range is cut
+ * into slices that run as separate workgroups; the first slice writes D = T_c(C) + its partial sum in
+ * a launch of its own, the others add theirs with fp32 atomics in a second launch.  Real MFMA
+ * operator, fp32 D, no transform on D and no bias; the order of the atomic adds, and so the last
+ * bits of D, can differ between runs.  With enough tiles it is the pipelined kernel. */
 typedef enum gk_kernel_kind {
   GK_KERNEL_SINGLESTAGE = 0,
   GK_KERNEL_PIPELINED = 1,
-  GK_KERNEL_PIPELINED_NG = 2
+  GK_KERNEL_PIPELINED_NG = 2,
+  GK_KERNEL_SPLIT_K = 3
 } gk_kernel_kind;
 
 /* Transform.Elementwise (reference src/transform.jl:20-30) as a closed vocabulary: a hook is a
