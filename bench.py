@@ -35,7 +35,7 @@ def parse_args():
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--no-extras", action="store_true", help="skip the secondary configs and the CPU baseline")
-    p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4b", "5"],
+    p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4b", "5", "skinny"],
                    help="benchmark config to time as the step (default: 2, the headline; the others are for profiling one "
                         "kernel at a time and imply --no-extras)")
     p.add_argument("--variant", default="NN", choices=["NN", "NT", "TN", "TT"], help="transposes of config 2")
@@ -151,7 +151,7 @@ def main():
         result["single_launch_us"] = {"min": round(lo, 2), "median": round(med, 2), "launches": 40}
         # ---------------- the other transposes and configs (outside the timed region) ----------------
         extras = {}
-        for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4b", None), (5, None)]:
+        for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4b", None), (5, None), ("skinny", None)]:
             try:
                 w = configs.benchmark_config(cfg, variant=variant)
                 r = w.prepare()

@@ -304,8 +304,34 @@ def _config5() -> Workload:
         kernel_name=kernel_name(conf, Kernel.matmul_pipelined))
 
 
+def _skinny() -> Workload:
+    """Not one of the five benchmark configurations: a skinny product (few output tiles, long K) that
+    is bound by memory and latency, timed with the K-split kernel kind."""
+    M, N, K = 4096, 64, 4096
+    conf = mfma_config(M, N, K, block_shape=(64, 64, 64))
+
+    def host():
+        return dict(a=rng.matrix("upm1_f16", 6001, (M, K)), b=rng.matrix("upm1_f16", 6002, (K, N)), c=rng.matrix("upm1_f32", 6003, (M, N)))
+
+    def launch(h):
+        import torch
+        a, b, c = colmajor(h["a"]), colmajor(h["b"]), colmajor(h["c"])
+        d = colmajor_empty((M, N), torch.float32)
+        launch_plan = plan(conf, a, b, c, d, kernel=Kernel.matmul_split_k)
+
+        def run():
+            launch_plan()
+        return _attach(run, a=a, b=b, c=c, d=d, conf=conf)
+
+    return Workload(
+        name="skinny",
+        description="skinny product C = A*B + C, M=4096, N=64, K=4096, FP16 A/B, FP32 C/D, 'N','N', K-split kernel (64 tiles x 8 K slices)",
+        flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + 2 * M * N * 4, bound="hbm", make_host=host, make_launch=launch,
+        kernel_name="mfma_gemm_splitk_nn_64x64x64_w2x2_f16")
+
+
 def benchmark_config(n, variant: Optional[str] = None) -> Workload:
-    """The benchmark workloads 1, 2 (variant NN/NT/TN/TT), 3, "4a", "4b", 5."""
+    """The benchmark workloads 1, 2 (variant NN/NT/TN/TT), 3, "4a", "4b", 5, and "skinny"."""
     if n == 2:
         return _config2(variant or "NN")
     if n == 3:
@@ -316,4 +342,4 @@ def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     raise NotImplementedError(f"benchmark config {n}")
 
 
-_LATE_BUILDERS = {1: _config1, "4a": _config4a, "4b": _config4b, 5: _config5}
+_LATE_BUILDERS = {1: _config1, "4a": _config4a, "4b": _config4b, 5: _config5, "skinny": _skinny}
