@@ -151,7 +151,7 @@ def main():
         result["single_launch_us"] = {"min": round(lo, 2), "median": round(med, 2), "launches": 40}
         # ---------------- the other transposes and configs (outside the timed region) ----------------
         extras = {}
-        for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4b", None), (5, None), ("skinny", None)]:
+        for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4a-planar", None), ("4b", None), (5, None), ("skinny", None)]:
             try:
                 w = configs.benchmark_config(cfg, variant=variant)
                 r = w.prepare()

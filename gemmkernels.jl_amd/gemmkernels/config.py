@@ -295,11 +295,14 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
                   global_a_layout, global_b_layout, global_c_layout, global_d_layout,
                   shared_a_layout, shared_b_layout, shared_c_layout, shared_d_layout,
                   operator, is_a_col_major, is_b_col_major, cta_swizzle)
-    if not params.get("specialize", False):
+    planar = global_a_layout.kind in (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
+    if not params.get("specialize", False) and not planar:
         # ``specialize=True``: the block shape need not be in the library's table because the kernel
         # will be compiled at run time (gemmkernels.specialize); that compilation and every launch run
         # the same checks, minus the table lookup
         check_config(conf, params.get("kernel"))
+    # planar complex global layouts: the product is made of real GEMMs on the planes
+    # (gemmkernels.complex_planar), each of which is checked when its own configuration is built
     return conf
 
 

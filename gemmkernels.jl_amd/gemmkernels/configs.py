@@ -245,6 +245,20 @@ def complex_config(M, N, K, ta=False, tb=False, zero_c=True, dual=False, **kw):
     return get_config(**params)
 
 
+def complex_planar_config(M, N, K, ta=False, tb=False, zero_c=True, **kw):
+    """Complex GEMM on planar (split re / im) global arrays of logical shape (rows, cols, 2): the
+    reference's LDS layouts Layout.SplitColMajor / SplitRowMajor (src/layout.jl:340-411) used as global
+    layouts.  The product runs as real GEMMs on the planes (gemmkernels.complex_planar)."""
+    sp = lambda t, T: Layout.SplitRowMajor[T] if t else Layout.SplitColMajor[T]
+    params = dict(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAComplexOp[16, 16, 16, Float16, Float32],
+                  global_a_layout=sp(ta, Float16), global_b_layout=sp(tb, Float16),
+                  global_c_layout=Layout.Zero[Float32] if zero_c else Layout.SplitColMajor[Float32],
+                  global_d_layout=Layout.SplitColMajor[Float32], block_shape=NT(M=64, N=128, K=32),
+                  is_a_col_major=not ta, is_b_col_major=not tb)
+    params.update(kw)
+    return get_config(**params)
+
+
 def complex_matrix(seed, rows, cols):
     """Interleaved Complex{Float16} matrix as a real array of shape (2, rows, cols), column-major:
     re and im ~ U[-1,1) from one stream in storage order."""
@@ -304,6 +318,35 @@ def _config5() -> Workload:
         kernel_name=kernel_name(conf, Kernel.matmul_pipelined))
 
 
+def _config4a_planar() -> Workload:
+    """Config 4a on planar (split re / im) global arrays: real GEMMs on the planes."""
+    M = N = K = 2048
+    conf = complex_planar_config(M, N, K)
+
+    def planar(seed, rows, cols):
+        return rng.matrix("upm1_f16", seed, (rows * cols, 2)).reshape((rows, cols, 2), order="F")
+
+    def host():
+        return dict(a=planar(4001, M, K), b=planar(4002, K, N), c=None)
+
+    def launch(h):
+        import torch
+        a, b = colmajor(h["a"]), colmajor(h["b"])
+        d = colmajor_empty((M, N, 2), torch.float32)
+        launch_plan = plan(conf, a, b, None, d, kernel=Kernel.matmul_pipelined)
+
+        def run():
+            launch_plan()
+        return _attach(run, a=a, b=b, d=d, conf=conf)
+
+    return Workload(
+        name="config 4a planar",
+        description="config 4a on planar global arrays (rows, cols, 2): Complex{Float16} A, B 2048x2048, Complex{Float32} D, no C; "
+                    "three real MFMA GEMMs on the planes",
+        flops=8 * M * N * K, bytes=(M * K + K * N) * 4 + M * N * 8, bound="mfma", make_host=host, make_launch=launch,
+        kernel_name="mfma_gemm_nn_256x128x64_w2x2_s3__Float16 + 2 x mfma_gemm_nn_128x128x64_w2x2_s2__Float16_fused")
+
+
 def _skinny() -> Workload:
     """Not one of the five benchmark configurations: a skinny product (few output tiles, long K) that
     is bound by memory and latency, timed with the K-split kernel kind."""
@@ -342,4 +385,4 @@ def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     raise NotImplementedError(f"benchmark config {n}")
 
 
-_LATE_BUILDERS = {1: _config1, "4a": _config4a, "4b": _config4b, 5: _config5, "skinny": _skinny}
+_LATE_BUILDERS = {1: _config1, "4a": _config4a, "4a-planar": _config4a_planar, "4b": _config4b, 5: _config5, "skinny": _skinny}

@@ -202,6 +202,9 @@ def plan(conf: Config, a, b, c, d, *,
          transform_shared_to_regs_c=None, transform_regs_to_shared_d=None,
          epilogue=None, kernel=Kernel.matmul_singlestage) -> Plan:
     """Same arguments as ``matmul``; returns a ``Plan`` whose call launches on the current stream."""
+    from . import complex_planar
+    if complex_planar.is_planar(conf):
+        return complex_planar.PlanarComplexPlan(conf, a, b, c, d)
     transforms = _collect(dict(transform_global_to_shared_a=transform_global_to_shared_a,
                                transform_global_to_shared_b=transform_global_to_shared_b,
                                transform_global_to_shared_c=transform_global_to_shared_c,
@@ -221,6 +224,9 @@ def matmul(conf: Config, a, b, c, d, *,
            epilogue=None, kernel=Kernel.matmul_singlestage, stream=None):
     """reference src/matmul.jl:7-44: launch geometry, checks (ConfigError) and the asynchronous
     launch on the current stream.  Same positional and keyword arguments as the reference."""
+    from . import complex_planar
+    if complex_planar.is_planar(conf):
+        return complex_planar.PlanarComplexPlan(conf, a, b, c, d)(stream)
     ctrans = None
     if not (transform_global_to_shared_a is None and transform_global_to_shared_b is None and
             transform_global_to_shared_c is None and transform_shared_to_global_d is None and

@@ -91,3 +91,41 @@ def test_config4a_full_size(gpu):
     d = to_c128(gk.to_numpy(r.d))
     ref = (to_c128(h["a"]).astype(np.complex64) @ to_c128(h["b"]).astype(np.complex64))
     assert oracle.rel_frobenius(d, ref) <= TOL
+
+
+def planar(seed, rows, cols, dtype=np.float16):
+    """Planar complex matrix as a real array of logical shape (rows, cols, 2), column-major."""
+    kind = "upm1_f16" if dtype == np.float16 else "upm1_f32"
+    return rng.matrix(kind, seed, (rows * cols, 2)).reshape((rows, cols, 2), order="F")
+
+
+def planar_to_c128(x):
+    return x[:, :, 0].astype(np.float64) + 1j * x[:, :, 1].astype(np.float64)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("zero_c", [True, False])
+def test_planar_global_layouts(gpu, ta, tb, zero_c):
+    """Complex GEMM on split re / im global arrays (Layout.SplitColMajor / SplitRowMajor as global
+    layouts): real GEMMs on the planes with the sign pattern of WMMAComplexOp.mma (src/operator.jl:307-311)."""
+    M, N, K = 256, 384, 192
+    conf = configs.complex_planar_config(M, N, K, ta, tb, zero_c=zero_c)
+    a = planar(81, K if ta else M, M if ta else K)
+    b = planar(82, N if tb else K, K if tb else N)
+    c = None if zero_c else planar(83, M, N, np.float32)
+    ta_, tb_ = gk.colmajor(a), gk.colmajor(b)
+    tc = None if zero_c else gk.colmajor(c)
+    td = gk.colmajor_empty((M, N, 2), torch.float32)
+    td.fill_(float("nan"))
+    gk.matmul(conf, ta_, tb_, tc, td, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    A = planar_to_c128(a).T if ta else planar_to_c128(a)
+    B = planar_to_c128(b).T if tb else planar_to_c128(b)
+    ref = A @ B + (0 if zero_c else planar_to_c128(c))
+    d = planar_to_c128(gk.to_numpy(td))
+    assert np.isfinite(d).all()
+    assert oracle.rel_frobenius(d, ref) <= TOL
+    if not zero_c:      # in place, mul! style: d is c
+        gk.matmul(conf, ta_, tb_, tc, tc, kernel=Kernel.matmul_pipelined)
+        torch.cuda.synchronize()
+        assert oracle.rel_frobenius(planar_to_c128(gk.to_numpy(tc)), ref) <= TOL
