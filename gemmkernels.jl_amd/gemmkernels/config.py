@@ -143,8 +143,10 @@ def adjacent_elements(num: int, parent_size: NT, is_col_major: bool) -> NT:
 # block / waves; every entry is made of 32x32 MFMA blocks.
 _MFMA_TILES = [
     ((256, 256, 64), (2, 4)),
+    ((256, 256, 32), (4, 2)),     # for K that is a multiple of 32 only; on par with 256x256x64 otherwise
     ((256, 128, 64), (2, 2)),
     ((128, 256, 64), (2, 2)),
+    ((128, 128, 32), (2, 2)),     # four stages: measured ahead of 128x128x64 with two stages on 2048-sized problems
     ((128, 128, 64), (2, 2)),
     ((64, 64, 64), (2, 2)),
     ((64, 64, 32), (1, 1)),
@@ -178,7 +180,9 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
     for t in fitting:
         if -(-M // t[0]) * -(-N // t[1]) >= NUM_CUS:
             return NT(M=t[0], N=t[1], K=t[2])
-    return NT(M=fitting[-1][0], N=fitting[-1][1], K=fitting[-1][2])
+    # no tile fills the chip: the smallest tile, with four waves per workgroup when K allows
+    last = (64, 64, 64) if (64, 64, 64) in fitting else fitting[-1]
+    return NT(M=last[0], N=last[1], K=last[2])
 
 
 # complex / dual tiles (complex elements) -> waves

@@ -51,10 +51,14 @@ def mfma_config(M, N, K, ta, tb, block, waves, panel, zero_c=False, ab=Float16, 
 
 def tune_mfma(M: int, N: int, K: int, ta: bool = False, tb: bool = False, zero_c: bool = False,
               candidates: Optional[Iterable] = None, panels: Iterable[int] = SWIZZLE_PANELS,
-              launches: int = 20, warmup: int = 3, verbose: bool = False) -> list:
+              launches: int = 20, warmup: int = 3, rounds: int = 3, verbose: bool = False) -> list:
     """Times every candidate that the library accepts for the problem (the others raise ConfigError,
     like the skipped configurations of the reference's sweep) and returns the measurements, fastest
-    first: dicts with block, waves, panel, us, tflops."""
+    first: dicts with block, waves, panel, us, tflops.
+
+    The part is power-limited, so what a candidate measures depends on what ran just before it.  All
+    candidates are therefore timed in ``rounds`` interleaved passes (after one untimed pass that warms
+    the chip up) and the median of a candidate's passes is its result."""
     import torch
     from .arrays import colmajor, colmajor_empty
     from .matmul import plan
@@ -62,27 +66,37 @@ def tune_mfma(M: int, N: int, K: int, ta: bool = False, tb: bool = False, zero_c
     b = colmajor(rng.matrix("upm1_f16", 2, (N, K) if tb else (K, N)))
     c = None if zero_c else colmajor(rng.matrix("upm1_f32", 3, (M, N)))
     d = colmajor_empty((M, N), torch.float32)
-    results = []
+    steps = []
     for block, waves in (MFMA_CANDIDATES if candidates is None else candidates):
         for panel in panels:
             try:
                 conf = mfma_config(M, N, K, ta, tb, block, waves, panel, zero_c)
             except ConfigError:
                 break                      # the tile does not fit the problem: no panel height will
-            step = plan(conf, a, b, c, d, kernel=Kernel.matmul_pipelined)
-            for _ in range(warmup):
-                step()
-            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            for _ in range(launches):
-                step()
-            stop.record()
-            stop.synchronize()
-            us = start.elapsed_time(stop) * 1e3 / launches
-            results.append(dict(block=list(block), waves=list(waves), panel=panel, us=round(us, 2),
-                                tflops=round(2.0 * M * N * K / us / 1e6, 1)))
-            if verbose:
-                print(results[-1], file=sys.stderr, flush=True)
+            steps.append((block, waves, panel, plan(conf, a, b, c, d, kernel=Kernel.matmul_pipelined)))
+
+    def timed(step, n):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(n):
+            step()
+        stop.record()
+        stop.synchronize()
+        return start.elapsed_time(stop) * 1e3 / n
+
+    for _, _, _, step in steps:            # untimed pass: first launches, clocks and caches settle
+        timed(step, warmup)
+    samples = [[] for _ in steps]
+    for _ in range(max(1, rounds)):
+        for i, (_, _, _, step) in enumerate(steps):
+            samples[i].append(timed(step, launches))
+    results = []
+    for (block, waves, panel, _), s in zip(steps, samples):
+        us = sorted(s)[len(s) // 2]
+        results.append(dict(block=list(block), waves=list(waves), panel=panel, us=round(us, 2),
+                            tflops=round(2.0 * M * N * K / us / 1e6, 1)))
+        if verbose:
+            print(results[-1], file=sys.stderr, flush=True)
     results.sort(key=lambda r: r["us"])
     return results
 

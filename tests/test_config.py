@@ -99,9 +99,11 @@ def test_get_config_defaults_for_the_headline_problem():
 
 def test_default_block_shape_shrinks_to_fill_the_chip():
     assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=4096, N=4096, K=4096)) == NT(M=256, N=256, K=64)
-    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=2048, N=2048, K=2048)) == NT(M=128, N=128, K=64)
-    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=256, N=256, K=256)) == NT(M=64, N=64, K=32)
-    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=4096, N=4096, K=2048 + 32)) == NT(M=64, N=64, K=32)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=4096, N=4096, K=2048)) == NT(M=256, N=256, K=64)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=2048, N=2048, K=2048)) == NT(M=128, N=128, K=32)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=256, N=256, K=256)) == NT(M=64, N=64, K=64)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=256, N=256, K=96)) == NT(M=64, N=64, K=32)
+    assert gk.default_block_shape(Operator.MFMAOp[32, 32, 16, F16, F32], NT(M=4096, N=4096, K=2048 + 32)) == NT(M=256, N=256, K=32)
 
 
 ERROR_CASES = [
