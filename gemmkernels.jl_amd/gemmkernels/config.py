@@ -158,7 +158,11 @@ NUM_CUS = 256
 TUNED = {}
 
 
-def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
+# tiles compiled with tensor-contraction addressing
+_GETT_TILES = [(256, 256, 64), (128, 128, 64), (64, 64, 32)]
+
+
+def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: bool = False) -> NT:
     """MI355X block shape: the largest tile of the table that divides the problem and still gives
     every one of the 256 CUs a workgroup; the smallest dividing tile when none does."""
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
@@ -175,6 +179,8 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True) -> NT:
         t = fitting[-1] if fitting else (64, 64, 32)
         return NT(M=t[0], N=t[1], K=t[2])
     fitting = [t for t, _ in _MFMA_TILES if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
+    if gett:
+        fitting = [t for t in fitting if t in _GETT_TILES]
     if not fitting:
         return NT(M=64, N=64, K=32)
     for t in fitting:
@@ -252,7 +258,8 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
         block_shape = NT(M=64, N=64, K=32 if gemm_shape.K % 32 == 0 else gemm_shape.K)
         params.setdefault("warps_per_block", 4)
         params.setdefault("compute_warp", NT(M=32, N=32, K=16))
-    block_shape = default_block_shape(operator, gemm_shape, tile_sized) if block_shape is None else NT(block_shape)
+    is_gett = any(l.kind == Layout.GETT_KIND for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
+    block_shape = default_block_shape(operator, gemm_shape, tile_sized, is_gett) if block_shape is None else NT(block_shape)
     op_shape = Operator.shape(operator)
 
     checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))

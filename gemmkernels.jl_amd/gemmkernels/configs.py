@@ -344,7 +344,7 @@ def _config4a_planar() -> Workload:
         description="config 4a on planar global arrays (rows, cols, 2): Complex{Float16} A, B 2048x2048, Complex{Float32} D, no C; "
                     "three real MFMA GEMMs on the planes",
         flops=8 * M * N * K, bytes=(M * K + K * N) * 4 + M * N * 8, bound="mfma", make_host=host, make_launch=launch,
-        kernel_name="mfma_gemm_nn_256x128x64_w2x2_s3__Float16 + 2 x mfma_gemm_nn_128x128x64_w2x2_s2__Float16_fused")
+        kernel_name="three real mfma_gemm launches on the planes")
 
 
 def _skinny() -> Workload:

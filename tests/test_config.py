@@ -214,3 +214,28 @@ def test_every_tile_of_the_python_tables_has_a_compiled_instance():
     for (bm, bn, bk), (wm, wn) in cfg._COMPLEX_TILES:
         conf = configs.complex_config(2 * bm, 2 * bn, 4 * bk, block_shape=NT(M=bm, N=bn, K=bk))
         assert f"{bm}x{bn}x{bk}_w{wm}x{wn}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+
+
+@pytest.mark.parametrize("size", [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 768, 128), (2048, 2048, 2048), (4096, 4096, 4096)])
+def test_default_tiles_resolve_to_compiled_instances_for_every_kind_of_config(size):
+    """Whatever tile the defaults pick for a problem, the library holds the instance: plain, with
+    transforms on the fragments (the fused levels), BF16, 16-bit C/D, and tensor-contraction layouts
+    (which are compiled for fewer tiles than the plain kernel)."""
+    from gemmkernels import configs, BFloat16, Transform
+    M, N, K = size
+    for ta in (False, True):
+        for tb in (False, True):
+            conf = configs.mfma_config(M, N, K, ta=ta, tb=tb)
+            assert gk.kernel_name(conf, Kernel.matmul_pipelined).startswith("mfma_gemm_")
+            scale = Transform.Elementwise(lambda x: x * 2.0)
+            for hook in ("transform_shared_to_regs_a", "transform_shared_to_regs_c"):
+                assert gk.kernel_name(conf, Kernel.matmul_pipelined, transforms={hook: scale}).startswith("mfma_gemm_")
+    conf = configs.mfma_config(M, N, K, operator=Operator.MFMAOp[32, 32, 16, BFloat16, F32],
+                               global_a_layout=ACM[BFloat16], global_b_layout=ACM[BFloat16])
+    assert "bf16" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    conf = configs.mfma_config(M, N, K, global_c_layout=ACM[F16], global_d_layout=ACM[F16])
+    assert gk.kernel_name(conf, Kernel.matmul_pipelined).startswith("mfma_gemm_")
+    # a contraction with the same GEMM extents: M = a*b, N = c, K = d
+    ext = dict(a=M // 32, b=32, c=N, d=K)
+    conf, _ = configs.gett_config("bda", "dc", "abc", ext)
+    assert gk.kernel_name(conf, Kernel.matmul_pipelined).endswith("_gett")
