@@ -64,6 +64,7 @@ bool is_row_major(int kind) {
   return kind == GK_LAYOUT_ROW_MAJOR || kind == GK_LAYOUT_ALIGNED_ROW_MAJOR || kind == GK_LAYOUT_INTERLEAVED_ROW_MAJOR ||
          kind == GK_LAYOUT_SPLIT_ROW_MAJOR;
 }
+bool is_split_layout(int kind) { return kind == GK_LAYOUT_SPLIT_COL_MAJOR || kind == GK_LAYOUT_SPLIT_ROW_MAJOR; }
 // reference src/config.jl:175-178
 bool require_tile_sized_global(int kind) { return !(kind == GK_LAYOUT_ZERO || is_checked_layout(kind)); }
 
@@ -110,7 +111,7 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
     case GK_OP_MFMA_COMPLEX:
     case GK_OP_MFMA_DUAL:
       key->family = gk::FAMILY_COMPLEX;
-      key->variant = (c->op.kind == GK_OP_MFMA_DUAL) ? 1 : 0;
+      key->variant = (c->op.kind == GK_OP_MFMA_DUAL) ? 1 : (is_split_layout(ak) ? 2 : 0);
       break;
     default:
       return fail(GK_ERR_INVALID_ARGUMENT, "unknown operator kind %d", c->op.kind);
@@ -172,7 +173,16 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
     // interleaved complex operands seen as real matrices: M and K double, and so does every
     // leading dimension (counted in real elements)
     args->M *= 2; args->K *= 2;
-    args->lda *= 2; args->ldb *= 2; args->ldc *= 2; args->ldd *= 2;
+    if (is_split_layout(c->global_a_layout.kind)) {
+      // planar operands: a matrix is the real array (rows, cols, 2) in column-major order, so the
+      // imaginary plane starts ld * cols elements after the real one; the kernel walks K twice
+      args->plane_a = args->lda * (a_row ? c->matmul_shape.M : c->matmul_shape.K);
+      args->plane_b = args->ldb * (b_row ? c->matmul_shape.K : c->matmul_shape.N);
+      args->plane_c = args->ldc * c->matmul_shape.N;
+      args->plane_d = args->ldd * c->matmul_shape.N;
+    } else {
+      args->lda *= 2; args->ldb *= 2; args->ldc *= 2; args->ldd *= 2;
+    }
   }
   args->swz_kind = c->cta_swizzle.kind;
   args->swz_param = c->cta_swizzle.param;
@@ -393,9 +403,16 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
 
   if (op.kind == GK_OP_MFMA_COMPLEX || op.kind == GK_OP_MFMA_DUAL) {
     auto inter = [](int k) { return k == GK_LAYOUT_INTERLEAVED_COL_MAJOR || k == GK_LAYOUT_INTERLEAVED_ROW_MAJOR; };
-    if (!inter(c->global_a_layout.kind) || !inter(c->global_b_layout.kind) || c->global_d_layout.kind != GK_LAYOUT_INTERLEAVED_COL_MAJOR ||
-        (c->global_c_layout.kind != GK_LAYOUT_INTERLEAVED_COL_MAJOR && c->global_c_layout.kind != GK_LAYOUT_ZERO))
-      return fail(GK_ERR_UNSUPPORTED, "complex and dual operators need Interleaved layouts for A and B and InterleavedColMajor for C and D");
+    const bool all_inter = inter(c->global_a_layout.kind) && inter(c->global_b_layout.kind) &&
+                           c->global_d_layout.kind == GK_LAYOUT_INTERLEAVED_COL_MAJOR &&
+                           (c->global_c_layout.kind == GK_LAYOUT_INTERLEAVED_COL_MAJOR || c->global_c_layout.kind == GK_LAYOUT_ZERO);
+    // planar global matrices (re plane, then im plane) are an addition for the complex operator
+    const bool all_split = op.kind == GK_OP_MFMA_COMPLEX && is_split_layout(c->global_a_layout.kind) &&
+                           is_split_layout(c->global_b_layout.kind) && c->global_d_layout.kind == GK_LAYOUT_SPLIT_COL_MAJOR &&
+                           (c->global_c_layout.kind == GK_LAYOUT_SPLIT_COL_MAJOR || c->global_c_layout.kind == GK_LAYOUT_ZERO);
+    if (!all_inter && !all_split)
+      return fail(GK_ERR_UNSUPPORTED, "complex and dual operators need Interleaved layouts for A and B and InterleavedColMajor for C and D "
+                                      "(the complex operator also takes Split layouts for all of them)");
     if (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT))
       return fail(GK_ERR_UNSUPPORTED, "transforms and bias are not available with the complex and dual operators");
   }
@@ -623,7 +640,7 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
   // aligned layouts move 16-byte vectors (reference src/layout.jl:22-34 traps on the device; here it is a host check)
   auto check_aligned = [&](const gk_layout& l, const void* p, long long ld, const char* what) -> int {
     const bool interleaved = l.kind == GK_LAYOUT_INTERLEAVED_COL_MAJOR || l.kind == GK_LAYOUT_INTERLEAVED_ROW_MAJOR;
-    if (l.kind != GK_LAYOUT_ALIGNED_COL_MAJOR && l.kind != GK_LAYOUT_ALIGNED_ROW_MAJOR && !interleaved) return GK_OK;
+    if (l.kind != GK_LAYOUT_ALIGNED_COL_MAJOR && l.kind != GK_LAYOUT_ALIGNED_ROW_MAJOR && !interleaved && !is_split_layout(l.kind)) return GK_OK;
     const int es = dtype_size(l.eltype);   // ld already counts real elements for interleaved data
     if (es == 0) return fail(GK_ERR_INVALID_ARGUMENT, "unknown element type of %s", what);
     if (((uintptr_t)p & 15u) != 0) return fail(GK_ERR_ALIGNMENT, "%s is not aligned to 16 bytes", what);
@@ -643,17 +660,21 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
   // leading dimensions must cover the operand
   {
     const bool a_row = is_row_major(conf->global_a_layout.kind), b_row = is_row_major(conf->global_b_layout.kind);
+    // extents in the unit the leading dimensions count: real elements (two per complex number of an
+    // interleaved matrix, one per complex number of a plane)
+    const bool planar = is_split_layout(conf->global_a_layout.kind);
+    const long long em = planar ? conf->matmul_shape.M : args.M, ek = planar ? conf->matmul_shape.K : args.K;
     if (!a_zero && conf->global_a_layout.kind != GK_LAYOUT_DIAGONAL && conf->global_a_layout.kind != GK_LAYOUT_GETT &&
-        args.lda < (a_row ? args.K : args.M))
+        args.lda < (a_row ? ek : em))
       return fail(GK_ERR_DIMENSION_MISMATCH, "lda = %lld is smaller than the leading extent of A", args.lda);
-    if (!b_zero && conf->global_b_layout.kind != GK_LAYOUT_GETT && args.ldb < (b_row ? args.N : args.K))
+    if (!b_zero && conf->global_b_layout.kind != GK_LAYOUT_GETT && args.ldb < (b_row ? args.N : ek))
       return fail(GK_ERR_DIMENSION_MISMATCH, "ldb = %lld is smaller than the leading extent of B", args.ldb);
-    if (conf->global_d_layout.kind != GK_LAYOUT_GETT && (args.ldd < args.M || (args.c_mode && args.ldc < args.M)))
+    if (conf->global_d_layout.kind != GK_LAYOUT_GETT && (args.ldd < em || (args.c_mode && args.ldc < em)))
       return fail(GK_ERR_DIMENSION_MISMATCH, "ldc/ldd is smaller than M");
     // the kernels keep per-lane tile offsets in 32 bits
     const long long span_a = (long long)(a_row ? conf->block_shape.M : conf->block_shape.K) * args.lda * 2;
     const long long span_b = (long long)(b_row ? conf->block_shape.K : conf->block_shape.N) * args.ldb * 2;
-    if (span_a >= (1ll << 31) || span_b >= (1ll << 31))
+    if (span_a + 2 * args.plane_a >= (1ll << 31) || span_b >= (1ll << 31))
       return fail(GK_ERR_UNSUPPORTED, "leading dimension too large for 32-bit tile offsets");
   }
 

@@ -90,6 +90,9 @@ struct GemmArgs {
   // K-split launches (0 / 0 / 0 otherwise): workgroup z handles the k_steps tiles of K that start at
   // tile k_begin + z * k_steps and, with atomic_d, adds its partial result into D atomically
   int k_begin, k_steps, atomic_d;
+  // planar complex operands (0 otherwise): distance in elements from the real plane of a matrix to
+  // its imaginary plane
+  long long plane_a, plane_b, plane_c, plane_d;
 };
 
 // ---------------------------------------------------------------------------------------------

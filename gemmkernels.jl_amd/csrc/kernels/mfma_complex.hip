@@ -14,6 +14,7 @@ namespace gk {
 int family_complex(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode, InstanceInfo* info,
                    hipError_t* err) {
   if (key.dtype != DT_F16 || key.fused != 0) return 0;
+  if (key.variant == 2) return family_complex_planar(key, args, grid, stream, mode, info, err);   // planar global matrices
 #define GK_CPLX(bm_, bn_, bk_, wm_, wn_, st_, akm_, bkm_, dual_, NAME)                                                     \
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
       key.a_kmajor == akm_ && key.b_kmajor == bkm_ && key.variant == dual_) {                                             \

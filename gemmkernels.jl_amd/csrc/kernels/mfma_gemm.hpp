@@ -32,7 +32,12 @@ namespace gk {
 // rows, so the tile holds R/2 complex rows.
 // ----------------------------------------------------------------------------------------------
 enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_CROWK = 2 };
-enum : int { FIX_NONE = 0, FIX_COMPLEX = 1, FIX_DUAL = 2 };
+// FIX_PLANAR: complex product on planar (split re / im) matrices.  Nothing is expanded in registers:
+// a workgroup owns BM/2 complex rows, the upper half of its real tile is the real plane of D and the
+// lower half the imaginary plane, and K runs twice: first over B_im with [A_im; A_re] as the A tile,
+// then over B_re with [A_re; A_im].  The upper half starts from -C_re and flips the sign of its
+// accumulators between the two passes, which gives C_re - A_im B_im + A_re B_re.
+enum : int { FIX_NONE = 0, FIX_COMPLEX = 1, FIX_DUAL = 2, FIX_PLANAR = 3 };
 
 template <int R, int BK, int KIND, bool EXPAND>
 struct OperandGeom {
@@ -197,7 +202,7 @@ struct FragReader {
 // (reference src/operator.jl:307-311 and :366-369).
 template <int FIX>
 __device__ __forceinline__ int4v expand_fixup(int4v x, int lane) {
-  if (FIX == FIX_NONE) return x;
+  if (FIX == FIX_NONE || FIX == FIX_PLANAR) return x;
   const bool odd = (lane & 1) != 0;
   const unsigned sel = odd ? 0x01000302u : 0x03020100u;                       // swap halves on odd rows
   const unsigned flip = (FIX == FIX_COMPLEX && !odd) ? 0x80000000u : 0u;       // negate the imaginary half
@@ -278,7 +283,8 @@ struct MfmaGemmConfig {
   static constexpr int FUSE = FUSE_;
   static constexpr bool FUSED = FUSE_ != 0;
   static constexpr bool FUSED_AB_GENERIC = FUSE_ == 2;
-  static constexpr bool EXPAND_A = (FIX_ != FIX_NONE);   // complex / dual A: one complex row feeds two MFMA rows
+  static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
+  static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
   // K-split instances: a workgroup handles one slice of K (blockIdx.z) and may add its partial result
   // into D with atomics.  A variant of its own so that the plain kernels carry none of it.
@@ -304,6 +310,7 @@ struct MfmaGemmConfig {
   static_assert(FM * FN > 0, "empty wave tile");
   static_assert(!GETT || (A_KIND != OPK_CROWK && B_KIND != OPK_CROWK && FIX == FIX_NONE), "contractions are real");
   static_assert(!SPLITK || (!GETT && FIX == FIX_NONE), "K-split instances are plain real GEMMs");
+  static_assert(!PLANAR || (WAVES_M_ % 2 == 0 && FUSE_ == 0), "planar complex: a wave's rows lie in one plane of D; no hooks");
 };
 
 template <class Cfg>
@@ -337,22 +344,36 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const char* gb;
   long long a_step = 0, b_step = 0;
   unsigned offa[DMA_A], offb[DMA_B];
+  unsigned offa2[Cfg::PLANAR ? DMA_A : 1];   // planar complex: the A offsets of the second pass over K
+  int to_switch = 0;                         // planar complex: tiles left to issue in the first pass
   KWalker walk;
   walk.reset();
   if constexpr (!Cfg::GETT) {
     // tile origin and K step in 16-bit elements (lda / ldb are in 16-bit elements as well; an
     // interleaved complex matrix counts two per complex number)
-    const long long a_org = Cfg::A_KIND == OPK_KMAJOR ? (long long)(Cfg::EXPAND_A ? m0 / 2 : m0) * args.lda : (long long)m0;
+    const int m0g = Cfg::EXPAND_A ? m0 / 2 : (Cfg::PLANAR ? m0 / 2 : m0);   // first row of the tile in the stored matrix
+    const long long a_org = Cfg::A_KIND == OPK_KMAJOR ? (long long)m0g * args.lda : (long long)(Cfg::PLANAR ? m0g : m0);
     const long long b_org = Cfg::B_KIND == OPK_KMAJOR ? (long long)n0 * args.ldb : (Cfg::B_KIND == OPK_MMAJOR ? (long long)n0 : 2ll * n0);
     ga = (const char*)args.a + a_org * 2;
     gb = (const char*)args.b + b_org * 2;
+    if constexpr (Cfg::PLANAR) gb += args.plane_b * 2;   // the first pass over K reads B_im
     a_step = (Cfg::A_KIND == OPK_KMAJOR ? (long long)BK : (long long)GA::LDS_ROWS * args.lda) * 2;
     b_step = (Cfg::B_KIND == OPK_KMAJOR ? (long long)BK : (long long)GB::LDS_ROWS * args.ldb) * 2;
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i) {
       int row, col;
       dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
-      offa[i] = (unsigned)(((long long)row * args.lda + col) * 2);
+      if constexpr (Cfg::PLANAR) {
+        // rows [0, BM/2) of the tile come from one plane of A, rows [BM/2, BM) from the other
+        int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
+        const bool lower = m >= BM / 2;
+        if (lower) m -= BM / 2;
+        const unsigned base = (unsigned)(((long long)row * args.lda + col) * 2);
+        offa[i] = base + (lower ? 0u : (unsigned)(args.plane_a * 2));
+        offa2[i] = base + (lower ? (unsigned)(args.plane_a * 2) : 0u);
+      } else {
+        offa[i] = (unsigned)(((long long)row * args.lda + col) * 2);
+      }
     }
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i) {
@@ -391,6 +412,17 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #endif
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
+    if constexpr (Cfg::PLANAR) {
+      if (to_switch == 0) {
+        // second pass: back to k = 0, B_re instead of B_im, the planes of A trade places
+        const long long kh = (args.K / BK) / 2;
+        ga -= kh * a_step;
+        gb -= kh * b_step + args.plane_b * 2;
+#pragma unroll
+        for (int i = 0; i < DMA_A; ++i) offa[i] = offa2[i];
+      }
+      --to_switch;
+    }
     const char* pa = ga;
     const char* pb = gb;
     if constexpr (Cfg::GETT) {
@@ -411,7 +443,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   };
 
   // K tiles of this workgroup: all of them, or one slice of a K-split launch
-  int KT = args.K / BK;
+  int KT = args.K / BK;       // planar complex: args.K counts both passes
+  [[maybe_unused]] const int KH = KT / 2;
+  if constexpr (Cfg::PLANAR) to_switch = KH;
   if constexpr (Cfg::SPLITK) {
     const int kt0 = args.k_begin + (int)blockIdx.z * args.k_steps;
     KT = (KT - kt0) < args.k_steps ? (KT - kt0) : args.k_steps;
@@ -428,13 +462,17 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // --- accumulators: C tile (two transforms) or zeros -------------------------------------------
   // lane l owns rows m = 32*fi + l%32 and columns n = 32*fj + 8*(v/4) + 4*(l/32) + v%4
   float16v acc[FM][FN];
-  const int mrow = m0 + wm * Cfg::WTM + (lane & 31);
+  // planar complex: the wave's rows lie in the real (upper) or the imaginary (lower) plane of C / D
+  [[maybe_unused]] const bool lower_plane = Cfg::PLANAR && (wm * Cfg::WTM >= BM / 2);
+  const int mrow = Cfg::PLANAR ? m0 / 2 + wm * Cfg::WTM - (lower_plane ? BM / 2 : 0) + (lane & 31) : m0 + wm * Cfg::WTM + (lane & 31);
   const int ncol = n0 + wn * Cfg::WTN + 4 * (lane >> 5);
   // element offset of the lane's first element of accumulator block (fi, fj) in C / D, and the
   // stride between its consecutive columns.  With a tensor-contraction map the first M mode and
   // the first N mode cover whole 32-wide blocks, so only the block origin needs the digit walk.
-  auto cd_offset = [&](int fi, int fj, long long ld) -> long long {
-    if constexpr (!Cfg::GETT) {
+  auto cd_offset = [&](int fi, int fj, long long ld, [[maybe_unused]] long long plane) -> long long {
+    if constexpr (Cfg::PLANAR) {
+      return (long long)(mrow + 32 * fi) + (long long)(ncol + 32 * fj) * ld + (lower_plane ? plane : 0ll);
+    } else if constexpr (!Cfg::GETT) {
       return (long long)(mrow + 32 * fi) + (long long)(ncol + 32 * fj) * ld;
     } else {
       long long t0, om, on;
@@ -446,12 +484,18 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   auto cd_nstride = [&](long long ld) -> long long {
     if constexpr (!Cfg::GETT) return ld; else return args.gn.stride1[0];
   };
+  auto negate_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = -acc[fi][fj];
+  };
   if (args.c_mode != 0) {
 #pragma unroll
     for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj) {
-        const long long off = cd_offset(fi, fj, args.ldc);
+        const long long off = cd_offset(fi, fj, args.ldc, args.plane_c);
         const long long ns = cd_nstride(args.ldc);
         if (args.c_dtype == DT_F32) {
           const float* cp = (const float*)args.c + off;
@@ -490,6 +534,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[fi][fj][v] = 0.0f;
+  }
+
+  if constexpr (Cfg::PLANAR) {
+    if (args.c_mode != 0 && !lower_plane) negate_acc();   // the sign comes back between the two passes over K
   }
 
   const bool xf_a = Cfg::FUSED && (hook_present<H_GL2SH_A>(args) || hook_present<H_SH2RF_A>(args));
@@ -572,6 +620,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       // tile kt has landed once at most the DMA of the STAGES-2 younger tiles is outstanding
       if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 2) * DPT>(); else wait_vmcnt<0>();
       block_barrier();   // every wave's share of tile kt is in LDS; every wave is done with tile kt-1
+      if constexpr (Cfg::PLANAR) {
+        if (kt == KH && !lower_plane) negate_acc();
+      }
       const unsigned stage_addr = lds_base + (unsigned)(kt % STAGES) * Cfg::STAGE_BYTES;
       ra.set_stage(stage_addr);
       rb.set_stage(stage_addr + GA::BYTES);
@@ -601,6 +652,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       // tiles <= kt+1 have landed once at most the STAGES-3 younger tiles are outstanding
       if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 3) * DPT>(); else wait_vmcnt<0>();
       block_barrier();   // tile kt+1 is visible; every wave is done reading tile kt-1
+      if constexpr (Cfg::PLANAR) {
+        if (kt == KH && !lower_plane) negate_acc();
+      }
       const bool issue = (kt + STAGES - 1 < KT);
       const bool last = (kt + 1 >= KT);
       static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
@@ -635,7 +689,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
     for (int fj = 0; fj < FN; ++fj) {
-      const long long off = cd_offset(fi, fj, args.ldd);
+      const long long off = cd_offset(fi, fj, args.ldd, args.plane_d);
       const long long ns = cd_nstride(args.ldd);
       float x[16];
 #pragma unroll

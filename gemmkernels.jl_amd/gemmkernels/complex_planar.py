@@ -7,10 +7,13 @@ real part -- a complex product is four real products on whole planes,
 
     D_re = A_re B_re - A_im B_im + C_re          D_im = A_re B_im + A_im B_re + C_im
 
-(the sign pattern of WMMAComplexOp.mma, src/operator.jl:307-311), each of which is an ordinary aligned
-FP16 x FP16 -> FP32 GEMM: no expansion in registers, no special kernel.  The minus sign rides on the
-A-side transform hook as an exact FP16 scale by -1.  With 'N' B the two products that share an A plane
-run as one GEMM of width 2N on the (K, 2N) view of planar B, so a product is three launches.
+(the sign pattern of WMMAComplexOp.mma, src/operator.jl:307-311).  When the two planes of every
+operand are adjacent in memory (the array is contiguous in its third dimension) the library runs the
+whole product as ONE launch of a kernel that walks K twice (``gemmkernels.matmul`` goes there
+directly).  This module is the path for operands whose planes lie apart: each of the four products is
+an ordinary aligned FP16 x FP16 -> FP32 GEMM, the minus sign rides on the A-side transform hook as an
+exact FP16 scale by -1, and with 'N' B the two products that share an A plane run as one GEMM of
+width 2N when B, C and D happen to have adjacent planes, so a product is three or four launches.
 """
 from __future__ import annotations
 
@@ -28,6 +31,17 @@ _NEGATE = Transform.Elementwise(ops=[(Transform.SCALE, -1.0, 0.0)])
 
 def is_planar(conf) -> bool:
     return conf.global_a_layout.kind in (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
+
+
+def planes_adjacent(*operands) -> bool:
+    """True when every operand is a (rows, cols, 2) tensor whose imaginary plane starts where the real
+    plane ends: what the single-launch kernel of the library addresses."""
+    for x in operands:
+        if x is None:
+            continue
+        if x.dim() != 3 or x.size(2) != 2 or x.stride(2) != x.stride(1) * x.size(1):
+            return False
+    return True
 
 
 def _plane(x, i):

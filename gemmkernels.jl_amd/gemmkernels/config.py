@@ -162,7 +162,7 @@ TUNED = {}
 _GETT_TILES = [(256, 256, 64), (128, 128, 64), (64, 64, 32)]
 
 
-def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: bool = False) -> NT:
+def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: bool = False, planar: bool = False) -> NT:
     """MI355X block shape: the largest tile of the table that divides the problem and still gives
     every one of the 256 CUs a workgroup; the smallest dividing tile when none does."""
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
@@ -170,7 +170,8 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
     M, N, K = gemm_shape["M"], gemm_shape["N"], gemm_shape["K"]
     if operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
         # complex tiles, in complex elements; every MFMA row pair is one complex row
-        fitting = [t for t, _ in _COMPLEX_TILES if M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0]
+        table = _PLANAR_TILES if planar else _COMPLEX_TILES
+        fitting = [t for t, _ in table if M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0]
         if operator.kind == Operator.MFMA_DUAL:
             fitting = [t for t in fitting if t in ((64, 128, 32), (64, 64, 32))]
         for t in fitting:
@@ -194,19 +195,23 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
 # complex / dual tiles (complex elements) -> waves
 _COMPLEX_TILES = [((128, 256, 32), (2, 4)), ((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 
+# complex tiles (complex elements) of the kernel for planar global matrices -> waves; a workgroup's real
+# tile has twice as many rows (both planes of D)
+_PLANAR_TILES = [((128, 256, 64), (2, 4)), ((64, 128, 64), (2, 2)), ((128, 128, 64), (2, 2)), ((64, 128, 32), (2, 2)), ((64, 64, 32), (2, 2))]
+
 # tiles of the vector-ALU kernel and of the bounds-checked MFMA kernel
 _FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2))]
 _CHECKED_TILES = [((64, 64, 32), (2, 2))]
 
 
-def _default_waves(operator, block_shape, checked=False):
+def _default_waves(operator, block_shape, checked=False, planar=False):
     key = (block_shape["M"], block_shape["N"], block_shape["K"])
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         table = _FPU_TILES
     elif operator.kind == Operator.MFMA and checked:
         table = _CHECKED_TILES
     elif operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
-        table = _COMPLEX_TILES
+        table = _PLANAR_TILES if planar else _COMPLEX_TILES
     else:
         table = _MFMA_TILES
     for t, w in table:
@@ -259,11 +264,12 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
         params.setdefault("warps_per_block", 4)
         params.setdefault("compute_warp", NT(M=32, N=32, K=16))
     is_gett = any(l.kind == Layout.GETT_KIND for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
-    block_shape = default_block_shape(operator, gemm_shape, tile_sized, is_gett) if block_shape is None else NT(block_shape)
+    planar = global_a_layout.kind in (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
+    block_shape = default_block_shape(operator, gemm_shape, tile_sized, is_gett, planar) if block_shape is None else NT(block_shape)
     op_shape = Operator.shape(operator)
 
     checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
-    waves = _default_waves(operator, block_shape, checked)
+    waves = _default_waves(operator, block_shape, checked, planar)
     if waves is not None:
         warps_default = waves[0] * waves[1]
         compute_warp_default = NT(M=block_shape.M // waves[0], N=block_shape.N // waves[1], K=op_shape.K)
@@ -306,14 +312,11 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
                   global_a_layout, global_b_layout, global_c_layout, global_d_layout,
                   shared_a_layout, shared_b_layout, shared_c_layout, shared_d_layout,
                   operator, is_a_col_major, is_b_col_major, cta_swizzle)
-    planar = global_a_layout.kind in (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
-    if not params.get("specialize", False) and not planar:
+    if not params.get("specialize", False):
         # ``specialize=True``: the block shape need not be in the library's table because the kernel
         # will be compiled at run time (gemmkernels.specialize); that compilation and every launch run
         # the same checks, minus the table lookup
         check_config(conf, params.get("kernel"))
-    # planar complex global layouts: the product is made of real GEMMs on the planes
-    # (gemmkernels.complex_planar), each of which is checked when its own configuration is built
     return conf
 
 

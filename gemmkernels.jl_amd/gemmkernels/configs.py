@@ -248,12 +248,13 @@ def complex_config(M, N, K, ta=False, tb=False, zero_c=True, dual=False, **kw):
 def complex_planar_config(M, N, K, ta=False, tb=False, zero_c=True, **kw):
     """Complex GEMM on planar (split re / im) global arrays of logical shape (rows, cols, 2): the
     reference's LDS layouts Layout.SplitColMajor / SplitRowMajor (src/layout.jl:340-411) used as global
-    layouts.  The product runs as real GEMMs on the planes (gemmkernels.complex_planar)."""
+    layouts.  One launch when the planes of every operand are adjacent in memory, real GEMMs on the
+    planes otherwise (gemmkernels.complex_planar)."""
     sp = lambda t, T: Layout.SplitRowMajor[T] if t else Layout.SplitColMajor[T]
     params = dict(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAComplexOp[16, 16, 16, Float16, Float32],
                   global_a_layout=sp(ta, Float16), global_b_layout=sp(tb, Float16),
                   global_c_layout=Layout.Zero[Float32] if zero_c else Layout.SplitColMajor[Float32],
-                  global_d_layout=Layout.SplitColMajor[Float32], block_shape=NT(M=64, N=128, K=32),
+                  global_d_layout=Layout.SplitColMajor[Float32],
                   is_a_col_major=not ta, is_b_col_major=not tb)
     params.update(kw)
     return get_config(**params)
@@ -319,7 +320,7 @@ def _config5() -> Workload:
 
 
 def _config4a_planar() -> Workload:
-    """Config 4a on planar (split re / im) global arrays: real GEMMs on the planes."""
+    """Config 4a on planar (split re / im) global arrays: one launch that walks K twice."""
     M = N = K = 2048
     conf = complex_planar_config(M, N, K)
 
@@ -342,9 +343,9 @@ def _config4a_planar() -> Workload:
     return Workload(
         name="config 4a planar",
         description="config 4a on planar global arrays (rows, cols, 2): Complex{Float16} A, B 2048x2048, Complex{Float32} D, no C; "
-                    "three real MFMA GEMMs on the planes",
+                    "one launch, two passes over K",
         flops=8 * M * N * K, bytes=(M * K + K * N) * 4 + M * N * 8, bound="mfma", make_host=host, make_launch=launch,
-        kernel_name="three real mfma_gemm launches on the planes")
+        kernel_name=kernel_name(conf, Kernel.matmul_pipelined))
 
 
 def _skinny() -> Workload:

@@ -41,6 +41,9 @@ _NO_LD = (Layout.ZERO, Layout.DIAGONAL, Layout.GETT_KIND)
 _INTERLEAVED = (Layout.INTERLEAVED_COL_MAJOR, Layout.INTERLEAVED_ROW_MAJOR)
 
 
+_SPLIT = (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
+
+
 def _leading_dim(x, layout) -> int:
     """Leading dimension, in elements, of a column-major device matrix."""
     kind = layout.kind
@@ -57,6 +60,12 @@ def _leading_dim(x, layout) -> int:
         if len(shape) != 3 or shape[0] != 2 or stride[0] != 1 or (shape[1] > 1 and stride[1] != 2):
             raise ConfigError("interleaved complex operands must have shape (2, rows, cols) in column-major order")
         return int(stride[2]) // 2 if shape[2] > 1 else max(int(shape[1]), 1)
+    if kind in _SPLIT:
+        # planar complex data: a real tensor of logical shape (rows, cols, 2), column-major, the
+        # imaginary plane right behind the real one
+        if len(shape) != 3 or shape[2] != 2 or (shape[0] > 1 and stride[0] != 1) or stride[2] != stride[1] * shape[1]:
+            raise ConfigError("planar complex operands must have shape (rows, cols, 2) in column-major order")
+        return int(stride[1])
     if len(shape) != 2:
         raise ConfigError("matrix operands must be 2-dimensional")
     if shape[0] > 1 and stride[0] != 1:
@@ -203,7 +212,7 @@ def plan(conf: Config, a, b, c, d, *,
          epilogue=None, kernel=Kernel.matmul_singlestage) -> Plan:
     """Same arguments as ``matmul``; returns a ``Plan`` whose call launches on the current stream."""
     from . import complex_planar
-    if complex_planar.is_planar(conf):
+    if complex_planar.is_planar(conf) and not complex_planar.planes_adjacent(a, b, c, d):
         return complex_planar.PlanarComplexPlan(conf, a, b, c, d)
     transforms = _collect(dict(transform_global_to_shared_a=transform_global_to_shared_a,
                                transform_global_to_shared_b=transform_global_to_shared_b,
@@ -225,7 +234,7 @@ def matmul(conf: Config, a, b, c, d, *,
     """reference src/matmul.jl:7-44: launch geometry, checks (ConfigError) and the asynchronous
     launch on the current stream.  Same positional and keyword arguments as the reference."""
     from . import complex_planar
-    if complex_planar.is_planar(conf):
+    if complex_planar.is_planar(conf) and not complex_planar.planes_adjacent(a, b, c, d):
         return complex_planar.PlanarComplexPlan(conf, a, b, c, d)(stream)
     ctrans = None
     if not (transform_global_to_shared_a is None and transform_global_to_shared_b is None and

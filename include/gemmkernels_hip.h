@@ -86,8 +86,11 @@ typedef enum gk_layout_kind {
   GK_LAYOUT_DIAGONAL = 5,               /* :225-236 A given by its diagonal */
   GK_LAYOUT_INTERLEAVED_COL_MAJOR = 6,  /* :276-302 Complex{T}, re/im adjacent */
   GK_LAYOUT_INTERLEAVED_ROW_MAJOR = 7,  /* :310-334 */
-  GK_LAYOUT_SPLIT_COL_MAJOR = 8,        /* :340-372 planar re/im (LDS) */
-  GK_LAYOUT_SPLIT_ROW_MAJOR = 9,        /* :380-411 */
+  GK_LAYOUT_SPLIT_COL_MAJOR = 8,        /* :340-372 planar re/im.  The reference uses it in shared memory only; here it is
+                                           also a global layout of the complex operator: the matrix is the real array
+                                           (rows, cols, 2) in column-major order, i.e. the imaginary plane starts
+                                           ld * cols elements after the real one, and ld counts elements of a plane */
+  GK_LAYOUT_SPLIT_ROW_MAJOR = 9,        /* :380-411 (as a global layout: the planar array of the transpose) */
   GK_LAYOUT_GETT = 10                   /* tensor-contraction index map, see gk_gett */
 } gk_layout_kind;
 

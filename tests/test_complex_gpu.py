@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import gemmkernels as gk
-from gemmkernels import Kernel, configs, rng
+from gemmkernels import Kernel, NT, configs, rng
 import helpers
 from oracle import oracle
 
@@ -129,3 +129,61 @@ def test_planar_global_layouts(gpu, ta, tb, zero_c):
         gk.matmul(conf, ta_, tb_, tc, tc, kernel=Kernel.matmul_pipelined)
         torch.cuda.synchronize()
         assert oracle.rel_frobenius(planar_to_c128(gk.to_numpy(tc)), ref) <= TOL
+
+
+def _run_planar(M, N, K, ta, tb, zero_c, block=None, seed=90):
+    kw = {} if block is None else dict(block_shape=NT(M=block[0], N=block[1], K=block[2]))
+    conf = configs.complex_planar_config(M, N, K, ta, tb, zero_c=zero_c, **kw)
+    a = planar(seed + 1, K if ta else M, M if ta else K)
+    b = planar(seed + 2, N if tb else K, K if tb else N)
+    c = None if zero_c else planar(seed + 3, M, N, np.float32)
+    ta_, tb_ = gk.colmajor(a), gk.colmajor(b)
+    tc = None if zero_c else gk.colmajor(c)
+    td = gk.colmajor_empty((M, N, 2), torch.float32)
+    td.fill_(float("nan"))
+    gk.matmul(conf, ta_, tb_, tc, td, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    A = planar_to_c128(a).T if ta else planar_to_c128(a)
+    B = planar_to_c128(b).T if tb else planar_to_c128(b)
+    ref = A @ B + (0 if zero_c else planar_to_c128(c))
+    d = planar_to_c128(gk.to_numpy(td))
+    assert np.isfinite(d).all()
+    return conf, oracle.rel_frobenius(d, ref), oracle.rel_frobenius(d.real, ref.real), oracle.rel_frobenius(d.imag, ref.imag)
+
+
+@pytest.mark.parametrize("block", [(128, 256, 64), (128, 128, 64), (64, 128, 32), (64, 128, 64), (64, 64, 32)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_planar_kernel_every_tile(gpu, block, ta, tb):
+    """The single-launch kernel for planar matrices, every compiled tile and transpose, C read: each
+    plane of D is checked on its own (a wrong sign or a swapped plane leaves the other one intact)."""
+    M, N, K = 2 * block[0], 3 * block[1], 5 * block[2]
+    conf, err, err_re, err_im = _run_planar(M, N, K, ta, tb, False, block)
+    assert "planar" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    assert err <= TOL and err_re <= TOL and err_im <= TOL
+
+
+@pytest.mark.parametrize("ktiles", [1, 2, 3])
+def test_planar_kernel_short_k(gpu, ktiles):
+    """K of one to three tiles: the switch from the first pass over K to the second falls into the
+    prologue of the pipeline."""
+    for block in [(128, 256, 64), (64, 128, 32)]:
+        _, err, err_re, err_im = _run_planar(block[0], block[1], ktiles * block[2], False, False, True, block, seed=95)
+        assert err <= TOL and err_re <= TOL and err_im <= TOL
+
+
+def test_planar_operands_with_separate_planes_fall_back_to_real_gemms(gpu):
+    """Planes that do not follow each other in memory (a view into a wider array) run as real GEMMs on
+    the planes; same result."""
+    M, N, K = 128, 256, 96
+    conf = configs.complex_planar_config(M, N, K, False, False, zero_c=True)
+    a, b = planar(101, M, K), planar(102, K, N)
+    wide_a = gk.colmajor_empty((M, K + 8, 2), torch.float16)
+    wide_a.zero_()
+    wide_a[:, :K, :] = gk.colmajor(a)
+    ta_ = wide_a[:, :K, :]
+    assert ta_.stride(2) != ta_.stride(1) * ta_.size(1)
+    td = gk.colmajor_empty((M, N, 2), torch.float32)
+    gk.matmul(conf, ta_, gk.colmajor(b), None, td, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    ref = planar_to_c128(a) @ planar_to_c128(b)
+    assert oracle.rel_frobenius(planar_to_c128(gk.to_numpy(td)), ref) <= TOL
