@@ -184,6 +184,18 @@ def main():
             torch.cuda.empty_cache()
         except Exception as e:
             extras.setdefault("config 4b", {})["rotating_buffers"] = {"error": f"{type(e).__name__}: {e}"}
+        # the skinny product in place (mul!(C, A, B, 1, 1): d is c), which the K-split kind runs as one launch
+        try:
+            from gemmkernels import Kernel, plan
+            w = configs.benchmark_config("skinny")
+            r = w.prepare()
+            in_place = plan(r.conf, r.a, r.b, r.c, r.c, kernel=Kernel.matmul_split_k)
+            u, _ = time_launches(in_place, 50, 10)
+            extras["skinny"]["in_place"] = {"us": round(u, 2), "GB/s": round(w.bytes / u / 1e3, 1),
+                                            "frac_of_hbm_peak": round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)}
+            del r, w, in_place
+        except Exception as e:
+            extras.setdefault("skinny", {})["in_place"] = {"error": f"{type(e).__name__}: {e}"}
         # the vendor library on the headline shape, for orientation only: FP16 in, FP16 out, no C read
         # (torch.mm -> hipBLASLt), so it moves 96 MiB less per launch than config 2 does
         try:

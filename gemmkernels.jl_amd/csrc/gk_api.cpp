@@ -719,6 +719,16 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
     if (slices > 1 && gk::family_mfma_splitk(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
       const int per = (kt + slices - 1) / slices;
       slices = (kt + per - 1) / per;
+      if (L.args.c_mode != 0 && c == d && L.args.ldc == L.args.ldd && conf->global_c_layout.eltype == GK_F32 &&
+          L.args.t[gk::H_GL2SH_C].n == 0 && L.args.t[gk::H_SH2RF_C].n == 0) {
+        // in place with an untouched C (C = A*B + C): D holds its starting value already, so every
+        // slice adds its partial sum and one launch does it all
+        gk::GemmArgs all = L.args;
+        all.k_begin = 0; all.k_steps = per; all.atomic_d = 1; all.c_mode = 0;
+        gk::family_mfma_splitk(L.key, all, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)slices), (hipStream_t)stream, 1, &sk_info, &err);
+        if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
+        return GK_OK;
+      }
       gk::GemmArgs first = L.args;       // slice 0: reads C, writes D
       first.k_begin = 0; first.k_steps = per; first.atomic_d = 0;
       gk::family_mfma_splitk(L.key, first, dim3((unsigned)L.gx, (unsigned)L.gy, 1), (hipStream_t)stream, 1, &sk_info, &err);

@@ -41,6 +41,23 @@ def test_skinny_products(gpu, dims, block, ta, tb):
     assert oracle.rel_frobenius(gk.to_numpy(C), ref2) <= TOL
 
 
+@pytest.mark.parametrize("dims,block", [((4096, 64, 4096), (64, 64, 64)), ((256, 256, 8192), (128, 128, 64))])
+def test_in_place_with_an_untouched_c_is_one_launch_of_atomic_adds(gpu, dims, block):
+    """C = A*B + C in place (mul!(C, A, B, 1, 1)): D already holds C, every K slice adds into it."""
+    M, N, K = dims
+    conf = configs.mfma_config(M, N, K, block_shape=block)
+    a, b, c = operands(M, N, K, False, False, 4300)
+    A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
+    gk.matmul(conf, A, B, C, C, kernel=Kernel.matmul_split_k)
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(gk.to_numpy(C), oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False)) <= TOL
+    # a second product on top, with a scale on A (the hook applies in every slice)
+    gk.matmul(conf, A, B, C, C, kernel=Kernel.matmul_split_k, transform_shared_to_regs_a=Transform.Elementwise(lambda x: x * -2.0))
+    torch.cuda.synchronize()
+    ref = oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False) + oracle.gemm_f64(a, b, None, -2.0, 0.0, False, False)
+    assert oracle.rel_frobenius(gk.to_numpy(C), ref) <= TOL
+
+
 def test_what_the_k_split_kernel_refuses(gpu):
     M, N, K = 128, 128, 2048
     conf = configs.mfma_config(M, N, K, block_shape=(64, 64, 64))
