@@ -290,6 +290,11 @@ struct MfmaGemmConfig {
   // into D with atomics.  A variant of its own so that the plain kernels carry none of it.
   static constexpr bool SPLITK = SPLITK_;
   static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / 16) % 2 == 0);   // cross-step fragment prefetch
+  // The DMA instructions of a tile are issued a few per k-step instead of all at once: a wave whose
+  // DMA instruction waits for room in the memory pipeline cannot issue its MFMAs either, and a burst
+  // from every wave right after the barrier makes all of them wait together (measured on 4096^3:
+  // 3031 -> 2903 shader clocks per 64 of K for 256x256x64, 2985 -> 2767 for 256x256x32 with four stages).
+  static constexpr bool SPREAD = !GETT_ && FIX_ != FIX_PLANAR;
   typedef T_ T;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int THREADS = NWAVES * kWaveSize;
@@ -437,6 +442,26 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     for (int i = 0; i < DMA_B; ++i)
       __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
     if constexpr (!Cfg::GETT) {
+      ga += a_step;
+      gb += b_step;
+    }
+  };
+
+  // part P of NP of the same DMA (Cfg::SPREAD); the tile pointers move on with the last part
+  auto issue_part = [&](auto p_c, auto np_c, int stage) __attribute__((always_inline)) {
+#ifdef GK_ABLATE_DMA
+    (void)p_c; (void)np_c; (void)stage; return;
+#endif
+    constexpr int P = decltype(p_c)::value, NP = decltype(np_c)::value;
+    char* sa = smem + stage * Cfg::STAGE_BYTES;
+    char* sb = sa + GA::BYTES;
+#pragma unroll
+    for (int i = 0; i < DMA_A; ++i)
+      if ((i % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < DMA_B; ++i)
+      if (((DMA_A + i) % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+    if constexpr (P == NP - 1) {
       ga += a_step;
       gb += b_step;
     }
@@ -627,10 +652,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       ra.set_stage(stage_addr);
       rb.set_stage(stage_addr + GA::BYTES);
       load_frags<0>(ra, rb, fa[0], fb[0]);
-      if (kt + STAGES - 1 < KT) issue_tile((kt + STAGES - 1) % STAGES);
+      const bool issue = (kt + STAGES - 1 < KT);
+      if constexpr (!Cfg::SPREAD) {
+        if (issue) issue_tile((kt + STAGES - 1) % STAGES);
+      }
       static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
         constexpr bool more = (ks + 1 < Cfg::KSTEPS);
+        if constexpr (Cfg::SPREAD) {
+          if (issue) issue_part(ks_c, std::integral_constant<int, Cfg::KSTEPS>{}, (kt + STAGES - 1) % STAGES);
+        }
         if constexpr (more) load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
         wait_lgkmcnt<more ? FRAG_OPS : 0>();
         compute(ks_c);
@@ -662,7 +693,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         if constexpr (ks + 1 < Cfg::KSTEPS) {
           load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
           wait_lgkmcnt<FRAG_OPS>();
-          if constexpr (ks == 0) {
+          if constexpr (ks == 0 && !Cfg::SPREAD) {
             if (issue) issue_tile((kt + STAGES - 1) % STAGES);
           }
         } else {
@@ -675,6 +706,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           } else {
             wait_lgkmcnt<0>();
           }
+        }
+        if constexpr (Cfg::SPREAD) {
+          if (issue) issue_part(ks_c, std::integral_constant<int, Cfg::KSTEPS>{}, (kt + STAGES - 1) % STAGES);
         }
         compute(ks_c);
       });
