@@ -284,6 +284,10 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+#ifdef GK_ABLATE_BARRIER
+__device__ __forceinline__ void block_barrier() { asm volatile("" ::: "memory"); }   // development aid (timing only, wrong results)
+#else
 __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
+#endif
 
 }  // namespace gk
