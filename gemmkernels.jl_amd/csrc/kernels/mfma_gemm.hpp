@@ -297,7 +297,7 @@ struct MfmaGemmConfig {
   // DMA instruction waits for room in the memory pipeline cannot issue its MFMAs either, and a burst
   // from every wave right after the barrier makes all of them wait together (measured on 4096^3:
   // 3031 -> 2903 shader clocks per 64 of K for 256x256x64, 2985 -> 2767 for 256x256x32 with four stages).
-  static constexpr bool SPREAD = !GETT_ && FIX_ != FIX_PLANAR;
+  static constexpr bool SPREAD = true;
   typedef T_ T;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int THREADS = NWAVES * kWaveSize;
@@ -450,6 +450,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     }
   };
 
+  [[maybe_unused]] const char* part_a = nullptr;
+  [[maybe_unused]] const char* part_b = nullptr;
   // part P of NP of the same DMA (Cfg::SPREAD); the tile pointers move on with the last part
   auto issue_part = [&](auto p_c, auto np_c, int stage) __attribute__((always_inline)) {
 #ifdef GK_ABLATE_DMA
@@ -458,13 +460,32 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     constexpr int P = decltype(p_c)::value, NP = decltype(np_c)::value;
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
+    if constexpr (Cfg::PLANAR && P == 0) {
+      if (to_switch == 0) {
+        // second pass: back to k = 0, B_re instead of B_im, the planes of A trade places
+        const long long kh = (args.K / BK) / 2;
+        ga -= kh * a_step;
+        gb -= kh * b_step + args.plane_b * 2;
+#pragma unroll
+        for (int i = 0; i < DMA_A; ++i) offa[i] = offa2[i];
+      }
+      --to_switch;
+    }
+    if constexpr (Cfg::GETT && P == 0) {
+      // tile base of the tensor walk, the same for every part of this tile
+      part_a = ga + walk.offset(args.gk, args.gk.stride0) * 2;
+      part_b = gb + walk.offset(args.gk, args.gk.stride1) * 2;
+      walk.advance(args.gk, BK);
+    }
+    const char* pa = Cfg::GETT ? part_a : ga;
+    const char* pb = Cfg::GETT ? part_b : gb;
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i)
-      if ((i % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      if ((i % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i)
-      if (((DMA_A + i) % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
-    if constexpr (P == NP - 1) {
+      if (((DMA_A + i) % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+    if constexpr (P == NP - 1 && !Cfg::GETT) {
       ga += a_step;
       gb += b_step;
     }

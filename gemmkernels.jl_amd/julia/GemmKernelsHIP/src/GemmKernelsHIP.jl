@@ -55,7 +55,7 @@ const DTYPE = Dict(Float16 => 0, Float32 => 2, Float64 => 3)          # BFloat16
 const LAYOUT_KIND = Dict(:Zero => 0, :ColMajor => 1, :RowMajor => 2, :UnsafeAlignedColMajor => 3,
                          :UnsafeAlignedRowMajor => 4, :Diagonal => 5, :InterleavedColMajor => 6,
                          :InterleavedRowMajor => 7, :SplitColMajor => 8, :SplitRowMajor => 9, :GETT => 10)
-const KERNEL_KIND = Dict(:matmul_singlestage => 0, :matmul_pipelined => 1, :matmul_pipelined_ng => 2)
+const KERNEL_KIND = Dict(:matmul_singlestage => 0, :matmul_pipelined => 1, :matmul_pipelined_ng => 2, :matmul_split_k => 3)
 const OP_KIND = Dict(:identity => 0, :scale => 1, :add => 2, :relu => 3, :neg => 4, :abs => 5, :clamp => 6, :square => 7)
 
 shape(nt) = GkShape(get(nt, :M, 0), get(nt, :N, 0), get(nt, :K, 0))
@@ -119,6 +119,44 @@ function heuristic_block_shape(shared_a::Type, shared_b::Type, shared_c::Type, s
                Ref(lower_layout(shared_a)), Ref(lower_layout(shared_b)), Ref(lower_layout(shared_c)), Ref(lower_layout(shared_d)), out)
     rc == 0 || throw(ConfigError(last_error(), rc))
     (M = Int(out[].M), N = Int(out[].N), K = Int(out[].K))
+end
+
+"""
+    specialize(conf::GkConfig, hooks; kernel = :matmul_pipelined) -> SpecializedKernel
+
+A kernel compiled at run time for `conf` with its transform hooks inlined: the counterpart of the
+reference's JIT-compiled kernel per `Config` with arbitrary functors (src/matmul.jl:38,
+src/transform.jl:26-30).  `hooks` is a tuple of 8 entries in the keyword order of the reference launcher
+(src/matmul.jl:8-15), each `nothing` (identity) or a C expression in the Float32 variable `x`, e.g.
+`"x > 0.0f ? x : 0.01f * x"`.  The block shape of `conf` may be any tile the kernel template accepts.
+"""
+struct SpecializedKernel
+    handle::Ptr{Cvoid}
+    conf::GkConfig
+end
+
+function specialize(conf::GkConfig, hooks::NTuple{8,Union{Nothing,String}}; kernel::Symbol = :matmul_pipelined)
+    strs = [h === nothing ? C_NULL : Base.unsafe_convert(Cstring, Base.cconvert(Cstring, h)) for h in hooks]
+    handle = Ref{Ptr{Cvoid}}(C_NULL)
+    GC.@preserve hooks begin
+        check(ccall((:gk_rtc_compile, libgk[]), Cint, (Ref{GkConfig}, Ptr{Cstring}, Int32, Ref{Ptr{Cvoid}}),
+                    Ref(conf), strs, KERNEL_KIND[kernel], handle))
+    end
+    SpecializedKernel(handle[], conf)
+end
+
+function kernel_name(k::SpecializedKernel)
+    buf = Vector{UInt8}(undef, 256)
+    check(ccall((:gk_rtc_kernel_name, libgk[]), Cint, (Ptr{Cvoid}, Ptr{UInt8}, Csize_t), k.handle, buf, length(buf)))
+    unsafe_string(pointer(buf))
+end
+
+"Launch a specialised kernel; same operands, epilogue and stream as `matmul`."
+function (k::SpecializedKernel)(a, b, c, d; epilogue::GkEpilogue = GkEpilogue(0, 0, C_NULL), stream::Ptr{Cvoid} = C_NULL)
+    check(ccall((:gk_rtc_matmul, libgk[]), Cint,
+                (Ptr{Cvoid}, Ref{GkConfig}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ref{GkEpilogue}, Ptr{Cvoid}),
+                k.handle, Ref(k.conf), a, b, c, d, Ref(epilogue), stream))
+    return d
 end
 
 # Device memory without AMDGPU.jl: the library's own thin wrappers over hipMalloc / hipMemcpy.
