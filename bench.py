@@ -182,6 +182,20 @@ def main():
                                                        "frac_of_hbm_peak": round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)}
             del runs
             torch.cuda.empty_cache()
+            # orientation: torch's converting copy FP16 -> FP32 of a 4096 x 4096 matrix moves exactly the same
+            # bytes per launch (32 MiB read, 64 MiB written); four buffer pairs in rotation as well
+            pairs = [(torch.ones(4096, 4096, dtype=torch.float16, device="cuda"), torch.empty(4096, 4096, dtype=torch.float32, device="cuda"))
+                     for _ in range(4)]
+
+            def copy_rotate():
+                src, dst = pairs[state["i"] & 3]
+                dst.copy_(src)
+                state["i"] += 1
+            u, _ = time_launches(copy_rotate, 48, 8)
+            extras["config 4b"]["converting_copy_same_bytes_rotating"] = {"us": round(u, 2), "GB/s": round(w.bytes / u / 1e3, 1),
+                                                                          "frac_of_hbm_peak": round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)}
+            del pairs
+            torch.cuda.empty_cache()
         except Exception as e:
             extras.setdefault("config 4b", {})["rotating_buffers"] = {"error": f"{type(e).__name__}: {e}"}
         # the skinny product in place (mul!(C, A, B, 1, 1): d is c), which the K-split kind runs as one launch

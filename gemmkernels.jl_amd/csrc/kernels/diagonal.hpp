@@ -11,6 +11,13 @@
 #include "common.hpp"
 #include <type_traits>
 
+#ifndef GK_DIAG_U
+#define GK_DIAG_U 8      // 4-row chunks in flight per lane without C
+#endif
+#ifndef GK_DIAG_U_C
+#define GK_DIAG_U_C 4    // ... and with C
+#endif
+
 namespace gk {
 
 // B_ROWMAJOR: B is the 'T' operand, stored N x K with K = M contiguous along j ... i.e. element
@@ -131,12 +138,46 @@ __global__ void __launch_bounds__(1024) diagonal_gemm_kernel(const GemmArgs args
         }
       }
     };
+    // No transform and no bias: chunks of 4 rows, so that one store instruction of a wave writes 1 KiB
+    // of consecutive addresses (with 8-row chunks the two 16-byte stores of a lane each fill every other
+    // half of the 32-byte pieces, i.e. partial lines per instruction) and one load reads 512 B.
+    auto sweep4 = [&](auto u_c) {
+      constexpr int U = decltype(u_c)::value;
+      typedef T vec4 __attribute__((ext_vector_type(4)));
+      const int chunks4 = BM / 4, total4 = chunks4 * BN;
+      const int stride = (int)blockDim.x;
+      for (int q0 = (int)threadIdx.x; q0 < total4; q0 += U * stride) {
+        vec4 bq[U], aq[U];
+        float4v cq[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int q = q0 + u * stride;
+          if (q < total4) {
+            const int i = m0 + (q % chunks4) * 4, j = n0 + q / chunks4;
+            bq[u] = *(const vec4*)&B[i + (long long)j * args.ldb];
+            aq[u] = *(const vec4*)&A[i];
+            if (args.c_mode != 0) cq[u] = *(const float4v*)&C[i + (long long)j * args.ldc];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int q = q0 + u * stride;
+          if (q < total4) {
+            const int i = m0 + (q % chunks4) * 4, j = n0 + q / chunks4;
+            float4v x;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = __builtin_fmaf((float)aq[u][e], (float)bq[u][e], args.c_mode != 0 ? cq[u][e] : 0.0f);
+            *(float4v*)&D[i + (long long)j * args.ldd] = x;
+          }
+        }
+      }
+    };
     typedef std::true_type Plain;
     typedef std::false_type Generic;
-    // chunks in flight per lane: four measured best without C (eight was 10-15 % slower)
+    (void)Plain{};
     if (xf_a || xf_b || xf_c || xf_d) sweep(std::integral_constant<int, 1>{}, Generic{});
-    else if (args.c_mode != 0) sweep(std::integral_constant<int, 2>{}, Plain{});
-    else sweep(std::integral_constant<int, 4>{}, Plain{});
+    else if (args.c_mode != 0) sweep4(std::integral_constant<int, GK_DIAG_U_C>{});
+    else sweep4(std::integral_constant<int, GK_DIAG_U>{});
   } else {
     // transpose 64 (i) x 64 (j) sub-tiles of B through LDS so that both the loads (along j) and the
     // stores (along i) are 16-byte vectors

@@ -263,6 +263,9 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
         block_shape = NT(M=64, N=64, K=32 if gemm_shape.K % 32 == 0 else gemm_shape.K)
         params.setdefault("warps_per_block", 4)
         params.setdefault("compute_warp", NT(M=32, N=32, K=16))
+        # consecutive workgroups on consecutive pieces of memory: the XCD-aware walk (made for tiles that
+        # share operands) costs a streaming kernel 8 % here
+        params.setdefault("cta_swizzle", CTASwizzle.Identity)
     is_gett = any(l.kind == Layout.GETT_KIND for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
     planar = global_a_layout.kind in (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
     block_shape = default_block_shape(operator, gemm_shape, tile_sized, is_gett, planar) if block_shape is None else NT(block_shape)

@@ -187,3 +187,18 @@ def test_planar_operands_with_separate_planes_fall_back_to_real_gemms(gpu):
     torch.cuda.synchronize()
     ref = planar_to_c128(a) @ planar_to_c128(b)
     assert oracle.rel_frobenius(planar_to_c128(gk.to_numpy(td)), ref) <= TOL
+
+
+def test_config4a_planar_full_size(gpu):
+    """Benchmark config 4a on planar arrays at its full size (2048^3), one launch; both planes checked
+    against a complex64 product of the same inputs."""
+    w = configs.benchmark_config("4a-planar")
+    assert "planar" in w.kernel_name
+    r = w.prepare()
+    r()
+    torch.cuda.synchronize()
+    h = w.host()
+    d = planar_to_c128(gk.to_numpy(r.d))
+    ref = planar_to_c128(h["a"]).astype(np.complex64) @ planar_to_c128(h["b"]).astype(np.complex64)
+    assert oracle.rel_frobenius(d.real, ref.real) <= TOL
+    assert oracle.rel_frobenius(d.imag, ref.imag) <= TOL
