@@ -239,3 +239,25 @@ def test_default_tiles_resolve_to_compiled_instances_for_every_kind_of_config(si
     ext = dict(a=M // 32, b=32, c=N, d=K)
     conf, _ = configs.gett_config("bda", "dc", "abc", ext)
     assert gk.kernel_name(conf, Kernel.matmul_pipelined).endswith("_gett")
+
+
+def test_complex_layout_rules_of_the_library():
+    """Complex matrices are interleaved (the reference's global form) or planar, never a mix; planar
+    ones are for the complex operator only, and only for tiles compiled with planar addressing."""
+    from gemmkernels import configs
+    M, N, K = 256, 256, 128
+    conf = configs.complex_planar_config(M, N, K)
+    assert "mfma_complex_planar_nn_" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    assert "mfma_complex_nn_" in gk.kernel_name(configs.complex_config(M, N, K), Kernel.matmul_pipelined)
+    cases = [
+        dict(global_b_layout=Layout.InterleavedColMajor[F16]),                                   # planar A, interleaved B
+        dict(global_d_layout=Layout.InterleavedColMajor[F32]),                                   # planar inputs, interleaved D
+        dict(operator=Operator.MFMADualOp[16, 16, 16, F16, F32]),                                # dual numbers have no planar form
+        dict(block_shape=NT(M=32, N=64, K=32)),                                                  # an interleaved-only tile
+    ]
+    for over in cases:
+        with pytest.raises(ConfigError) as ei:
+            configs.complex_planar_config(M, N, K, **over)
+        assert ei.value.status in (_lib.GK_ERR_UNSUPPORTED, _lib.GK_ERR_BLOCK_SHAPE), ei.value.message
+    with pytest.raises(ConfigError):                                                            # K not a multiple of the tile
+        configs.complex_planar_config(M, N, 48)
