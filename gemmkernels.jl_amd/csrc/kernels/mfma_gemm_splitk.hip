@@ -25,7 +25,7 @@ int family_mfma_splitk(const InstanceKey& key, const GemmArgs& args, dim3 grid, 
   GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, _Float16, DT_F16, 1, "_f16_fused")  \
   GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, __bf16, DT_BF16, 0, "_bf16")
   GK_SK_TILE(128, 128, 64, 2, 2, 2)
-  GK_SK_TILE(64, 64, 64, 2, 2, 2)
+  GK_SK_TILE(64, 64, 64, 2, 2, 4)
   GK_SK_TILE(64, 64, 32, 1, 1, 2)
 #undef GK_SK_TILE
 #undef GK_SK_T
