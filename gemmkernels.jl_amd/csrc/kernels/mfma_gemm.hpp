@@ -164,8 +164,20 @@ struct FragReader {
 #pragma unroll
     for (int i = 0; i < NBASE; ++i) cur[i] = base[i] + tile_lds_addr;
   }
-  template <int FI, int KS>
+  // SYNC: the wait for the data is part of the same assembly statement, so that the registers are
+  // valid wherever the compiler may look at them (kernels that spill registers use this form: a
+  // spill store between an asynchronous read and its wait would save stale values)
+  template <int FI, int KS, bool SYNC = false>
   __device__ __forceinline__ void read(Raw& r) const {
+    if constexpr (SYNC && KIND == OPK_KMAJOR) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
+      return;
+    } else if constexpr (SYNC && KIND == OPK_MMAJOR) {
+      asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
+                   : "=&v"(r.lo), "=&v"(r.hi)
+                   : "v"(cur[FI < NBASE ? FI : 0]), "n"((KS * 16) * G::ROW_BYTES), "n"((KS * 16 + 4) * G::ROW_BYTES) : "memory");
+      return;
+    }
     if (KIND == OPK_KMAJOR) {
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
     } else if (KIND == OPK_MMAJOR) {
@@ -223,13 +235,13 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
-template <int KS, class RA, class RB, int FM, int FN>
+template <int KS, bool SYNC = false, class RA, class RB, int FM, int FN>
 __device__ __forceinline__ void load_frags(const RA& ra, const RB& rb, typename RA::Raw (&fa)[FM], typename RB::Raw (&fb)[FN]) {
 #ifdef GK_ABLATE_LDS
   (void)ra; (void)rb; (void)fa; (void)fb; return;   // development aid (timing only, wrong results)
 #endif
-  static_for<0, FM>([&](auto fi) { ra.template read<decltype(fi)::value, KS>(fa[decltype(fi)::value]); });
-  static_for<0, FN>([&](auto fj) { rb.template read<decltype(fj)::value, KS>(fb[decltype(fj)::value]); });
+  static_for<0, FM>([&](auto fi) { ra.template read<decltype(fi)::value, KS, SYNC>(fa[decltype(fi)::value]); });
+  static_for<0, FN>([&](auto fj) { rb.template read<decltype(fj)::value, KS, SYNC>(fb[decltype(fj)::value]); });
 }
 
 template <typename T> struct Mfma;
@@ -286,6 +298,10 @@ struct MfmaGemmConfig {
   static constexpr int FUSE = FUSE_;
   static constexpr bool FUSED = FUSE_ != 0;
   static constexpr bool FUSED_AB_GENERIC = FUSE_ == 2;
+  // the generic A / B hooks, and wave tiles of more than eight 32x32 blocks (256 accumulator registers),
+  // need so many registers that the kernel spills: their fragment reads wait for their data inside the
+  // assembly statement that issues them (see FragReader::read)
+  static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8);
   static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
@@ -675,7 +691,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       const unsigned stage_addr = lds_base + (unsigned)(kt % STAGES) * Cfg::STAGE_BYTES;
       ra.set_stage(stage_addr);
       rb.set_stage(stage_addr + GA::BYTES);
-      load_frags<0>(ra, rb, fa[0], fb[0]);
+      load_frags<0, Cfg::SYNC_FRAGS>(ra, rb, fa[0], fb[0]);
       const bool issue = (kt + STAGES - 1 < KT);
       if constexpr (!Cfg::SPREAD) {
         if (issue) issue_tile((kt + STAGES - 1) % STAGES);
@@ -686,7 +702,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         if constexpr (Cfg::SPREAD) {
           if (issue) issue_part(ks_c, std::integral_constant<int, Cfg::KSTEPS>{}, (kt + STAGES - 1) % STAGES);
         }
-        if constexpr (more) load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+        if constexpr (more) load_frags<ks + 1, Cfg::SYNC_FRAGS>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
         wait_lgkmcnt<more ? FRAG_OPS : 0>();
         compute(ks_c);
       });
@@ -702,7 +718,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     block_barrier();
     ra.set_stage(lds_base);
     rb.set_stage(lds_base + GA::BYTES);
-    load_frags<0>(ra, rb, fa[0], fb[0]);
+    load_frags<0, Cfg::SYNC_FRAGS>(ra, rb, fa[0], fb[0]);
     for (int kt = 0; kt < KT; ++kt) {
       // tiles <= kt+1 have landed once at most the STAGES-3 younger tiles are outstanding
       if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 3) * DPT>(); else wait_vmcnt<0>();
@@ -715,7 +731,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
         if constexpr (ks + 1 < Cfg::KSTEPS) {
-          load_frags<ks + 1>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+          load_frags<ks + 1, Cfg::SYNC_FRAGS>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
           wait_lgkmcnt<FRAG_OPS>();
           if constexpr (ks == 0 && !Cfg::SPREAD) {
             if (issue) issue_tile((kt + STAGES - 1) % STAGES);
@@ -725,7 +741,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             const unsigned stage_addr = lds_base + (unsigned)((kt + 1) % STAGES) * Cfg::STAGE_BYTES;
             ra.set_stage(stage_addr);
             rb.set_stage(stage_addr + GA::BYTES);
-            load_frags<0>(ra, rb, fa[0], fb[0]);
+            load_frags<0, Cfg::SYNC_FRAGS>(ra, rb, fa[0], fb[0]);
             wait_lgkmcnt<FRAG_OPS>();
           } else {
             wait_lgkmcnt<0>();

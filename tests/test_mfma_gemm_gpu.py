@@ -14,9 +14,7 @@ TOL = 1e-3
 
 TILES = [  # block shape, (waves_m, waves_n)
     ((256, 256, 64), (2, 4)),
-    ((256, 256, 64), (2, 2)),
     ((256, 256, 32), (2, 4)),
-    ((256, 256, 32), (2, 2)),
     ((256, 256, 32), (4, 2)),
     ((256, 128, 64), (2, 2)),
     ((128, 256, 64), (2, 2)),
