@@ -138,33 +138,40 @@ int gk_rtc_compile(const gk_config* conf, const char* const hooks[8], int32_t ke
   auto hit = g_cache.find(cache_key);
   if (hit != g_cache.end()) { *out = hit->second; return GK_OK; }
 
-  hiprtcProgram prog;
-  const char* header_names[2] = {"common.hpp", "mfma_gemm.hpp"};
-  const char* header_text[2] = {kEmbedded_common_hpp, kEmbedded_mfma_gemm_hpp};
-  hiprtcResult r = hiprtcCreateProgram(&prog, src.c_str(), "gk_user_kernel.hip", 2, header_text, header_names);
-  if (r != HIPRTC_SUCCESS) return fail(GK_ERR_HIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
-  const char* name_expr = "&gk::mfma_gemm_kernel<GkUserCfg>";
-  hiprtcAddNameExpression(prog, name_expr);
-  const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off"};
-  r = hiprtcCompileProgram(prog, 4, opts);
-  if (r != HIPRTC_SUCCESS) {
-    size_t n = 0;
-    hiprtcGetProgramLogSize(prog, &n);
-    std::string log(n ? n : 1, '\0');
-    if (n) hiprtcGetProgramLog(prog, &log[0]);
+  // compiles one source text; the code object and the mangled kernel name come back
+  auto compile = [](const std::string& text, std::string& code, std::string& lowered_name) -> int {
+    hiprtcProgram prog;
+    const char* header_names[2] = {"common.hpp", "mfma_gemm.hpp"};
+    const char* header_text[2] = {kEmbedded_common_hpp, kEmbedded_mfma_gemm_hpp};
+    hiprtcResult r = hiprtcCreateProgram(&prog, text.c_str(), "gk_user_kernel.hip", 2, header_text, header_names);
+    if (r != HIPRTC_SUCCESS) return fail(GK_ERR_HIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+    const char* name_expr = "&gk::mfma_gemm_kernel<GkUserCfg>";
+    hiprtcAddNameExpression(prog, name_expr);
+    const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off"};
+    r = hiprtcCompileProgram(prog, 4, opts);
+    if (r != HIPRTC_SUCCESS) {
+      size_t n = 0;
+      hiprtcGetProgramLogSize(prog, &n);
+      std::string log(n ? n : 1, '\0');
+      if (n) hiprtcGetProgramLog(prog, &log[0]);
+      hiprtcDestroyProgram(&prog);
+      // a failed static_assert of the tile geometry or a malformed expression: the compiler says which
+      return fail(GK_ERR_UNSUPPORTED, "run-time compilation failed: %.1800s", log.c_str());
+    }
+    const char* lowered = nullptr;
+    r = hiprtcGetLoweredName(prog, name_expr, &lowered);
+    size_t code_size = 0;
+    if (r == HIPRTC_SUCCESS) r = hiprtcGetCodeSize(prog, &code_size);
+    code.assign(code_size, '\0');
+    if (r == HIPRTC_SUCCESS) r = hiprtcGetCode(prog, &code[0]);
+    lowered_name = lowered ? lowered : "";
     hiprtcDestroyProgram(&prog);
-    // a failed static_assert of the tile geometry or a malformed expression: the compiler says which
-    return fail(GK_ERR_UNSUPPORTED, "run-time compilation failed: %.1800s", log.c_str());
-  }
-  const char* lowered = nullptr;
-  r = hiprtcGetLoweredName(prog, name_expr, &lowered);
-  size_t code_size = 0;
-  if (r == HIPRTC_SUCCESS) r = hiprtcGetCodeSize(prog, &code_size);
-  std::string code(code_size, '\0');
-  if (r == HIPRTC_SUCCESS) r = hiprtcGetCode(prog, &code[0]);
-  std::string lowered_name = lowered ? lowered : "";
-  hiprtcDestroyProgram(&prog);
-  if (r != HIPRTC_SUCCESS || lowered_name.empty()) return fail(GK_ERR_HIP, "hipRTC produced no code object: %s", hiprtcGetErrorString(r));
+    if (r != HIPRTC_SUCCESS || lowered_name.empty()) return fail(GK_ERR_HIP, "hipRTC produced no code object: %s", hiprtcGetErrorString(r));
+    return GK_OK;
+  };
+  std::string code, lowered_name;
+  int rc_compile = compile(src, code, lowered_name);
+  if (rc_compile != GK_OK) return rc_compile;
 
   gk_rtc_kernel* k = new gk_rtc_kernel();
   k->BM = b.M; k->BN = b.N; k->BK = b.K; k->waves_m = wm; k->waves_n = wn; k->stages = stages;
@@ -177,8 +184,29 @@ int gk_rtc_compile(const gk_config* conf, const char* const hooks[8], int32_t ke
   k->info.lds_bytes = (int)((long long)(b.M + b.N) * b.K * 2 * stages);
   k->info.threads = nwaves * gk::kWaveSize;
   if (device >= 0) {
-    hipError_t e = hipModuleLoadData(&k->module, code.data());
-    if (e == hipSuccess) e = hipModuleGetFunction(&k->function, k->module, lowered_name.c_str());
+    auto load = [&]() -> hipError_t {
+      hipError_t e = hipModuleLoadData(&k->module, code.data());
+      if (e == hipSuccess) e = hipModuleGetFunction(&k->function, k->module, lowered_name.c_str());
+      return e;
+    };
+    hipError_t e = load();
+    // The fragment reads of the kernel are asynchronous with hand-placed waits, which is sound only
+    // while no register is spilled (a spill store between a read and its wait would save stale
+    // values).  A tile that makes this kernel use scratch memory is compiled again with reads that
+    // wait inside the assembly statement that issues them.
+    const bool sync_already = fuse == 2 || (w.M / 32) * (w.N / 32) > 8;     // MfmaGemmConfig::SYNC_FRAGS
+    int scratch_bytes = 0;
+    if (e == hipSuccess && !sync_already &&
+        hipFuncGetAttribute(&scratch_bytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, k->function) == hipSuccess && scratch_bytes > 0) {
+      (void)hipModuleUnload(k->module);
+      k->module = nullptr;
+      k->function = nullptr;
+      int rc2 = compile("#define GK_FORCE_SYNC_FRAGS 1\n" + src, code, lowered_name);
+      if (rc2 != GK_OK) { delete k; return rc2; }
+      e = load();
+      k->name += "_sync";
+      k->info.name = k->name.c_str();
+    }
     if (e != hipSuccess) {
       if (k->module) (void)hipModuleUnload(k->module);
       delete k;

@@ -287,6 +287,10 @@ __device__ __forceinline__ int4v scale_fragment_f16(int4v f, float scale) {
   return __builtin_bit_cast(int4v, v);
 }
 
+#ifndef GK_FORCE_SYNC_FRAGS
+#define GK_FORCE_SYNC_FRAGS 0     // set by the run-time compiler for a tile that turned out to spill registers
+#endif
+
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int A_KIND_, int B_KIND_, typename T_, int FUSE_,
           bool GETT_ = false, int FIX_ = FIX_NONE, bool SPLITK_ = false>
 struct MfmaGemmConfig {
@@ -301,7 +305,7 @@ struct MfmaGemmConfig {
   // the generic A / B hooks, and wave tiles of more than eight 32x32 blocks (256 accumulator registers),
   // need so many registers that the kernel spills: their fragment reads wait for their data inside the
   // assembly statement that issues them (see FragReader::read)
-  static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8);
+  static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
   static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps

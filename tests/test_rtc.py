@@ -114,3 +114,23 @@ def test_block_shapes_outside_the_compiled_table(gpu, block, waves):
     torch.cuda.synchronize()
     ref = oracle.gemm_f64((a.astype(np.float32) ** 2).astype(np.float16), b, c, 1.0, 1.0, False, True)
     assert oracle.rel_frobenius(gk.to_numpy(D), ref) <= 1e-3
+
+
+@pytest.mark.gpu
+def test_wave_tile_of_sixteen_blocks_runs_with_synchronous_fragment_reads(gpu):
+    """A 256x256 tile on 2x2 waves keeps 256 accumulator registers per lane and spills; kernels like
+    that read their fragments synchronously (a spill between an asynchronous read and its wait would
+    save stale values).  Only a hook on D here, so the K loop is the plain one."""
+    import torch
+    from oracle import oracle
+    M, N, K = 512, 512, 192
+    conf = gk.get_config(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+                         global_a_layout=Layout.UnsafeAlignedColMajor[Float16], global_c_layout=Layout.UnsafeAlignedColMajor[Float32],
+                         block_shape=NT(M=256, N=256, K=32), warps_per_block=4, compute_warp=NT(M=128, N=128, K=16), specialize=True)
+    a, b, c = rng.matrix("upm1_f16", 31, (M, K)), rng.matrix("upm1_f16", 32, (K, N)), rng.matrix("upm1_f32", 33, (M, N))
+    A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
+    D = gk.colmajor_empty((M, N), torch.float32)
+    D.fill_(float("nan"))
+    gk.specialize(conf, transform_shared_to_global_d="2.0f * x")(A, B, C, D)
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(gk.to_numpy(D), 2.0 * oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False)) <= 1e-3
