@@ -154,7 +154,8 @@ typedef struct gk_config {
  * matmul_pipelined_ng :368-574).  GK_KERNEL_SPLIT_K has no counterpart in the reference: for
  * problems with too few output tiles to fill the 256 CUs (skinny M or N, long K) the K range is cut
  * into slices that run as separate workgroups; the first slice writes D = T_c(C) + its partial sum in
- * a launch of its own, the others add theirs with fp32 atomics in a second launch.  Real MFMA
+ * a launch of its own, the others add theirs with fp32 atomics in a second launch (when d == c and C
+ * has no transform, D holds its starting value already and all slices add in one launch).  Real MFMA
  * operator, fp32 D, no transform on D and no bias; the order of the atomic adds, and so the last
  * bits of D, can differ between runs.  With enough tiles it is the pipelined kernel. */
 typedef enum gk_kernel_kind {
