@@ -45,6 +45,16 @@ def parse_args():
     return p.parse_args()
 
 
+def gk_f32():
+    from gemmkernels import Float32
+    return Float32
+
+
+def gk_name(conf):
+    from gemmkernels import Kernel, kernel_name
+    return kernel_name(conf, Kernel.matmul_pipelined)
+
+
 def time_launches(fn, steps, warmup):
     """Average duration in microseconds of `steps` back-to-back launches, HIP events on the launch stream."""
     import torch
@@ -198,6 +208,29 @@ def main():
             torch.cuda.empty_cache()
         except Exception as e:
             extras.setdefault("config 4b", {})["rotating_buffers"] = {"error": f"{type(e).__name__}: {e}"}
+        # the headline shape with the other element types of the MFMA kernels: BF16 multiplicands, and FP16 C / D
+        try:
+            from gemmkernels import BFloat16, Float16, Kernel, Layout, Operator, plan
+            w = configs.benchmark_config(2, variant="NN")
+            r = w.prepare()
+            M = N = K = 4096
+            acm = Layout.UnsafeAlignedColMajor
+            conf_bf = configs.mfma_config(M, N, K, operator=Operator.MFMAOp[32, 32, 16, BFloat16, gk_f32()], global_a_layout=acm[BFloat16],
+                                          global_b_layout=acm[BFloat16])
+            a_bf, b_bf = r.a.to(torch.bfloat16), r.b.to(torch.bfloat16)
+            run_bf = plan(conf_bf, a_bf, b_bf, r.c, r.d, kernel=Kernel.matmul_pipelined)
+            u, _ = time_launches(run_bf, 50, 10)
+            extras["config 2 NN, BF16 A/B"] = {"us": round(u, 2), "kernel": gk_name(conf_bf), "TFLOP/s": round(w.flops / u / 1e6, 2)}
+            conf_h = configs.mfma_config(M, N, K, global_c_layout=acm[Float16], global_d_layout=acm[Float16])
+            c_h = r.c.to(torch.float16)
+            d_h = torch.empty_like(c_h)
+            run_h = plan(conf_h, r.a, r.b, c_h, d_h, kernel=Kernel.matmul_pipelined)
+            u, _ = time_launches(run_h, 50, 10)
+            extras["config 2 NN, FP16 C/D"] = {"us": round(u, 2), "kernel": gk_name(conf_h), "TFLOP/s": round(w.flops / u / 1e6, 2)}
+            del r, w, run_bf, run_h, a_bf, b_bf, c_h, d_h
+            torch.cuda.empty_cache()
+        except Exception as e:
+            extras["config 2 NN, other element types"] = {"error": f"{type(e).__name__}: {e}"}
         # the skinny product in place (mul!(C, A, B, 1, 1): d is c), which the K-split kind runs as one launch
         try:
             from gemmkernels import Kernel, plan
