@@ -32,8 +32,11 @@ MEASURED_TRAFFIC_BYTES = 335_872_000   # profiles/mfma_gemm_config2_hbm_traffic.
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=200)
-    p.add_argument("--warmup", type=int, default=20)
+    # defaults: 2000 warm-up launches (0.27 s) because the clock and power management of the device needs
+    # a tenth of a second of load to settle after the idle time in which the inputs are generated (measured:
+    # 1029 TFLOP/s after 20 warm-up launches, 1045 after 200, 1051 after 2000 and after 5000); 1000 timed launches
+    p.add_argument("--steps", type=int, default=1000)
+    p.add_argument("--warmup", type=int, default=2000)
     p.add_argument("--no-extras", action="store_true", help="skip the secondary configs and the CPU baseline")
     p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4a-planar", "4b", "5", "skinny"],
                    help="benchmark config to time as the step (default: 2, the headline; the others are for profiling one "
@@ -55,11 +58,65 @@ def gk_name(conf):
     return kernel_name(conf, Kernel.matmul_pipelined)
 
 
-def time_launches(fn, steps, warmup):
-    """Average duration in microseconds of `steps` back-to-back launches, HIP events on the launch stream."""
+def observe_device(fn, bursts=100, launches_per_burst=100):
+    """Shader clock, power and temperature the driver reports (sysfs of the first card) while `fn` runs
+    back to back for a good second (the power reading is a moving average: the second half of the
+    samples is what is reported); outside every timed region.  None where the files are not there."""
+    import glob
+    import statistics
+    import torch
+    dev = "/sys/class/drm/card0/device"
+
+    def read(path):
+        try:
+            with open(path) as f:
+                return f.read()
+        except OSError:
+            return None
+
+    hwmon = (glob.glob(dev + "/hwmon/hwmon*") or [None])[0]
+    clocks, watts, temps = [], [], []
+    for _ in range(bursts):
+        for _ in range(launches_per_burst):
+            fn()
+        torch.cuda.synchronize()
+        text = read(dev + "/pp_dpm_sclk")
+        if text:
+            for line in text.splitlines():
+                if line.rstrip().endswith("*"):
+                    clocks.append(int("".join(ch for ch in line.split(":")[1] if ch.isdigit())))
+        if hwmon:
+            w = read(hwmon + "/power1_input") or read(hwmon + "/power1_average")
+            if w:
+                watts.append(int(w) / 1e6)
+            t = read(hwmon + "/temp2_input") or read(hwmon + "/temp1_input")
+            if t:
+                temps.append(int(t) / 1e3)
+    torch.cuda.synchronize()
+    if not clocks and not watts:
+        return None
+    clocks, watts = clocks[len(clocks) // 2:], watts[len(watts) // 2:]
+    cap = read(hwmon + "/power1_cap") if hwmon else None
+    return {"sclk_mhz_median": statistics.median(clocks) if clocks else None, "sclk_mhz_min": min(clocks) if clocks else None,
+            "power_w_median": round(statistics.median(watts), 1) if watts else None,
+            "power_cap_w": round(int(cap) / 1e6, 1) if cap else None,
+            "temperature_c_max": max(temps) if temps else None, "samples": max(len(clocks), len(watts)),
+            "note": "driver readings while the headline kernel runs back to back (spec clock 2400 MHz)"}
+
+
+def time_launches(fn, steps, warmup, settle_seconds=0.0):
+    """Average duration in microseconds of `steps` back-to-back launches, HIP events on the launch stream.
+    settle_seconds: keep launching for at least this long before timing (on top of `warmup`), so that a
+    secondary workload is not timed while the device clock is still coming up from idle."""
     import torch
     for _ in range(warmup):
         fn()
+    if settle_seconds > 0:
+        t_end = time.perf_counter() + settle_seconds
+        while time.perf_counter() < t_end:
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -159,13 +216,17 @@ def main():
     if not args.no_extras:
         lo, med = launch_distribution(run)
         result["single_launch_us"] = {"min": round(lo, 2), "median": round(med, 2), "launches": 40}
+        try:
+            result["observed_device"] = observe_device(run)
+        except Exception as e:      # readings are for orientation; never fail the benchmark over them
+            result["observed_device"] = {"error": f"{type(e).__name__}: {e}"}
         # ---------------- the other transposes and configs (outside the timed region) ----------------
         extras = {}
         for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4a-planar", None), ("4b", None), (5, None), ("skinny", None)]:
             try:
                 w = configs.benchmark_config(cfg, variant=variant)
                 r = w.prepare()
-                u, _ = time_launches(r, 50, 10)
+                u, _ = time_launches(r, 50, 10, 0.15)
                 entry = {"us": round(u, 2), "kernel": w.kernel_name}
                 if w.bound == "hbm":
                     entry["GB/s"] = round(w.bytes / u / 1e3, 1)
@@ -187,7 +248,7 @@ def main():
             def rotate():
                 runs[state["i"] & 3]()
                 state["i"] += 1
-            u, _ = time_launches(rotate, 48, 8)
+            u, _ = time_launches(rotate, 48, 8, 0.15)
             extras["config 4b"]["rotating_buffers"] = {"us": round(u, 2), "GB/s": round(w.bytes / u / 1e3, 1),
                                                        "frac_of_hbm_peak": round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)}
             del runs
@@ -201,7 +262,7 @@ def main():
                 src, dst = pairs[state["i"] & 3]
                 dst.copy_(src)
                 state["i"] += 1
-            u, _ = time_launches(copy_rotate, 48, 8)
+            u, _ = time_launches(copy_rotate, 48, 8, 0.15)
             extras["config 4b"]["converting_copy_same_bytes_rotating"] = {"us": round(u, 2), "GB/s": round(w.bytes / u / 1e3, 1),
                                                                           "frac_of_hbm_peak": round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)}
             del pairs
@@ -219,13 +280,13 @@ def main():
                                           global_b_layout=acm[BFloat16])
             a_bf, b_bf = r.a.to(torch.bfloat16), r.b.to(torch.bfloat16)
             run_bf = plan(conf_bf, a_bf, b_bf, r.c, r.d, kernel=Kernel.matmul_pipelined)
-            u, _ = time_launches(run_bf, 50, 10)
+            u, _ = time_launches(run_bf, 50, 10, 0.15)
             extras["config 2 NN, BF16 A/B"] = {"us": round(u, 2), "kernel": gk_name(conf_bf), "TFLOP/s": round(w.flops / u / 1e6, 2)}
             conf_h = configs.mfma_config(M, N, K, global_c_layout=acm[Float16], global_d_layout=acm[Float16])
             c_h = r.c.to(torch.float16)
             d_h = torch.empty_like(c_h)
             run_h = plan(conf_h, r.a, r.b, c_h, d_h, kernel=Kernel.matmul_pipelined)
-            u, _ = time_launches(run_h, 50, 10)
+            u, _ = time_launches(run_h, 50, 10, 0.15)
             extras["config 2 NN, FP16 C/D"] = {"us": round(u, 2), "kernel": gk_name(conf_h), "TFLOP/s": round(w.flops / u / 1e6, 2)}
             del r, w, run_bf, run_h, a_bf, b_bf, c_h, d_h
             torch.cuda.empty_cache()
@@ -237,7 +298,7 @@ def main():
             w = configs.benchmark_config("skinny")
             r = w.prepare()
             in_place = plan(r.conf, r.a, r.b, r.c, r.c, kernel=Kernel.matmul_split_k)
-            u, _ = time_launches(in_place, 50, 10)
+            u, _ = time_launches(in_place, 50, 10, 0.15)
             extras["skinny"]["in_place"] = {"us": round(u, 2), "GB/s": round(w.bytes / u / 1e3, 1),
                                             "frac_of_hbm_peak": round(w.bytes / u / 1e3 / PEAK_HBM_GBS, 4)}
             del r, w, in_place
@@ -249,7 +310,7 @@ def main():
             x = torch.randn(4096, 4096, device="cuda").to(torch.float16)
             y = torch.randn(4096, 4096, device="cuda").to(torch.float16)
             out = torch.empty(4096, 4096, device="cuda", dtype=torch.float16)
-            u, _ = time_launches(lambda: torch.mm(x, y, out=out), 50, 10)
+            u, _ = time_launches(lambda: torch.mm(x, y, out=out), 50, 10, 0.15)
             extras["vendor_library_fp16_out_no_c"] = {"us": round(u, 2), "TFLOP/s": round(wl.flops / u / 1e6, 2)}
             del x, y, out
         except Exception as e:
