@@ -78,7 +78,7 @@ std::string build_source(const gk_config* c, const char* const hooks[8], int sta
   src += "    return x;\n  }\n};\n}\n#include \"mfma_gemm.hpp\"\n";
   char buf[512];
   snprintf(buf, sizeof(buf),
-           "typedef gk::MfmaGemmConfig<%d, %d, %d, %d, %d, %d, %d, %d, %s, %d> GkUserCfg;\n"
+           "typedef gk::MfmaGemmConfig<%d, %d, %d, %d, %d, %d, %d, %d, %s, %d, false, gk::FIX_NONE, false, 16> GkUserCfg;\n"
            "template __global__ void gk::mfma_gemm_kernel<GkUserCfg>(const gk::GemmArgs);\n",
            c->block_shape.M, c->block_shape.N, c->block_shape.K, c->block_shape.M / c->compute_warp.M,
            c->block_shape.N / c->compute_warp.N, stages, a_kind, b_kind, type, fuse);

@@ -21,7 +21,7 @@ int family_complex_planar(const InstanceKey& key, const GemmArgs& args, dim3 gri
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
       key.a_kmajor == akm_ && key.b_kmajor == bkm_) {                                                                     \
     typedef MfmaGemmConfig<2 * bm_, bn_, bk_, wm_, wn_, st_, (akm_ ? OPK_KMAJOR : OPK_MMAJOR),                             \
-                           (bkm_ ? OPK_KMAJOR : OPK_MMAJOR), _Float16, 0, false, FIX_PLANAR> Cfg;                          \
+                           (bkm_ ? OPK_KMAJOR : OPK_MMAJOR), _Float16, 0, false, FIX_PLANAR, false, 16> Cfg;                          \
     return run_instance<Cfg>(mfma_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
 #define GK_PLANAR_T(bm_, bn_, bk_, wm_, wn_, st_)                                                               \

@@ -55,6 +55,8 @@ struct OperandGeom {
   static constexpr int GROUPS = CPR / 4;
   static constexpr int GMASK = (GROUPS - 1) < 3 ? (GROUPS - 1) : 3;
   __device__ static __forceinline__ int swz_m(int k) { return (k / RP256) & GMASK; }
+  // ... and the two 32-byte halves of a 64-byte group trade places on every other block of 8 k rows, so
+  // that the 16-lane groups of a transposing read for 16-row fragments (k, k + 8, ...) use both halves
   static_assert((CPR & (CPR - 1)) == 0, "chunks per row must be a power of two");
   static_assert(KIND != OPK_MMAJOR || CPR >= 4, "M-major tiles need at least 32 rows");
   static_assert(BYTES % 1024 == 0, "tile must be a whole number of DMA instructions");
@@ -70,7 +72,7 @@ __device__ __forceinline__ void dma_lane_coords(int q, int lane, int& row, int& 
   row = p / G::CPR;
   const int cs = p % G::CPR;
   if (KIND == OPK_KMAJOR) col = (cs ^ G::swz_k(row)) * 8;
-  else if (KIND == OPK_MMAJOR) col = (((cs >> 2) ^ G::swz_m(row)) * 4 + (cs & 3)) * 8;
+  else if (KIND == OPK_MMAJOR) col = (((cs >> 2) ^ G::swz_m(row)) * 4 + ((cs & 3) ^ (((row >> 3) & 1) << 1))) * 8;
   else col = cs * 8;
 }
 
@@ -120,49 +122,59 @@ __device__ __forceinline__ void wait_lgkmcnt() {
 // apart), which serialises the pipeline.  Their completion is therefore tracked by hand:
 // read() only issues, the registers it names (Raw) must not be looked at before
 // wait_lgkmcnt<N>() + pin_raw(), and finish() turns them into the MFMA operand afterwards.
-template <int R, int BK, int KIND, bool EXPAND, int F>
+template <int R, int BK, int KIND, bool EXPAND, int F, int MI = 32>
 struct FragReader {
   typedef OperandGeom<R, BK, KIND, EXPAND> G;
-  static constexpr int KSTEPS = BK / 16;
-  static constexpr int NBASE = KIND == OPK_KMAJOR ? KSTEPS : (KIND == OPK_MMAJOR ? F : 1);
+  // MI = 32: fragments of 32 rows x 16 k (v_mfma_f32_32x32x16); MI = 16: 16 rows x 32 k (v_mfma_f32_16x16x32),
+  // lane l holds the 8 k-values 8*(l/MI)..+7 of row l%MI in both cases
+  static constexpr int KSTEP_K = MI == 32 ? 16 : 32;
+  static constexpr int KSTEPS = BK / KSTEP_K;
+  // M-major, 16-row fragments: fragments 2j and 2j+1 are the two 32-byte halves of one 64-byte group, so one
+  // address serves both (the odd one is the even one with bit 5 flipped)
+  static constexpr bool PAIRED = KIND == OPK_MMAJOR && MI == 16 && F % 2 == 0;
+  static constexpr int NBASE = KIND == OPK_KMAJOR ? KSTEPS : (KIND == OPK_MMAJOR ? (PAIRED ? F / 2 : F) : 1);
   static constexpr int OPS = KIND == OPK_KMAJOR ? 1 : (KIND == OPK_MMAJOR ? 2 : 4);   // LDS instructions per fragment
-  static constexpr int FRAG_ROWS = EXPAND ? 16 : 32;           // tile rows (complex rows when EXPAND) per fragment
+  static constexpr int FRAG_ROWS = EXPAND ? MI / 2 : MI;       // tile rows (complex rows when EXPAND) per fragment
   struct Raw {
     int4v q;          // OPK_KMAJOR
     int2v lo, hi;     // OPK_MMAJOR
     int x0, x1, x2, x3;   // OPK_CROWK
   };
-  unsigned base[NBASE];                         // lane-dependent byte offsets inside a tile
-  unsigned cur[NBASE];                          // the same, relative to the current stage
+  unsigned cur[NBASE];                          // lane-dependent byte addresses inside the tile of the current stage
+  unsigned stage_addr;                          // LDS address of that tile (wave-uniform)
 
   // row0: first MFMA row of the wave inside the block tile (multiple of 32)
   __device__ __forceinline__ void init(int row0, int lane) {
     if (KIND == OPK_KMAJOR) {
-      const int row = EXPAND ? ((row0 + (lane & 31)) >> 1) : (row0 + (lane & 31));
+      const int row = EXPAND ? ((row0 + (lane % MI)) >> 1) : (row0 + (lane % MI));
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int c = ks * 2 + (lane >> 5);
-        base[ks < NBASE ? ks : 0] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_k(row)));
+        const int c = ks * (KSTEP_K / 8) + (lane / MI);
+        cur[ks < NBASE ? ks : 0] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_k(row)));
       }
     } else if (KIND == OPK_MMAJOR) {
       const int i = lane & 15;
-      const int k = 8 * (lane >> 5) + (i >> 2);
-      const int m = (lane & 16) + 4 * (i & 3);          // offset inside the 32-row fragment
-      const int c = m >> 3;
-      const unsigned lane_part = (unsigned)(k * G::ROW_BYTES + (c & 3) * 16 + (m & 4) * 2);
+      const int k = 8 * (lane / MI) + (i >> 2);
+      const int m = (MI == 32 ? (lane & 16) : 0) + 4 * (i & 3);          // offset inside the fragment
 #pragma unroll
-      for (int fi = 0; fi < F; ++fi) {
-        const int g = ((row0 >> 5) + fi) ^ G::swz_m(k);
-        base[fi < NBASE ? fi : 0] = lane_part + (unsigned)g * 64u;
+      for (int fi = 0; fi < F; fi += (PAIRED ? 2 : 1)) {
+        const int rowf = row0 + fi * MI;                 // first row of the fragment inside the block tile
+        const int mm = (rowf & 31) + m;                  // offset inside the 32-row (64-byte) group
+        const int g = (rowf >> 5) ^ G::swz_m(k);
+        const int c = ((mm >> 3) & 3) ^ (((k >> 3) & 1) << 1);
+        cur[(PAIRED ? fi / 2 : fi) < NBASE ? (PAIRED ? fi / 2 : fi) : 0] = (unsigned)(k * G::ROW_BYTES + g * 64 + c * 16 + (mm & 4) * 2);
       }
     } else {
-      const int elem = EXPAND ? ((row0 + (lane & 31)) >> 1) : (row0 + (lane & 31));
-      base[0] = (unsigned)(4 * (lane >> 5) * G::ROW_BYTES + elem * 4);
+      const int elem = EXPAND ? ((row0 + (lane % MI)) >> 1) : (row0 + (lane % MI));
+      cur[0] = (unsigned)(4 * (lane / MI) * G::ROW_BYTES + elem * 4);
     }
+    stage_addr = 0;
   }
   __device__ __forceinline__ void set_stage(unsigned tile_lds_addr) {
+    const unsigned delta = tile_lds_addr - stage_addr;     // one register per address: the offsets move with the stage
 #pragma unroll
-    for (int i = 0; i < NBASE; ++i) cur[i] = base[i] + tile_lds_addr;
+    for (int i = 0; i < NBASE; ++i) cur[i] += delta;
+    stage_addr = tile_lds_addr;
   }
   // SYNC: the wait for the data is part of the same assembly statement, so that the registers are
   // valid wherever the compiler may look at them (kernels that spill registers use this form: a
@@ -175,20 +187,25 @@ struct FragReader {
     } else if constexpr (SYNC && KIND == OPK_MMAJOR) {
       asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
                    : "=&v"(r.lo), "=&v"(r.hi)
-                   : "v"(cur[FI < NBASE ? FI : 0]), "n"((KS * 16) * G::ROW_BYTES), "n"((KS * 16 + 4) * G::ROW_BYTES) : "memory");
+                   : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K) * G::ROW_BYTES), "n"((KS * KSTEP_K + 4) * G::ROW_BYTES) : "memory");
       return;
     }
     if (KIND == OPK_KMAJOR) {
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
     } else if (KIND == OPK_MMAJOR) {
-      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.lo) : "v"(cur[FI < NBASE ? FI : 0]), "n"((KS * 16) * G::ROW_BYTES) : "memory");
-      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.hi) : "v"(cur[FI < NBASE ? FI : 0]), "n"((KS * 16 + 4) * G::ROW_BYTES) : "memory");
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.lo) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K) * G::ROW_BYTES) : "memory");
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.hi) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K + 4) * G::ROW_BYTES) : "memory");
     } else {
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x0) : "v"(cur[0]), "n"((KS * 8 + 0) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x1) : "v"(cur[0]), "n"((KS * 8 + 1) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x2) : "v"(cur[0]), "n"((KS * 8 + 2) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x3) : "v"(cur[0]), "n"((KS * 8 + 3) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x0) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 0) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x1) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 1) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x2) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 2) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x3) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 3) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
     }
+  }
+  template <int FI>
+  __device__ __forceinline__ unsigned mmajor_addr() const {
+    if constexpr (PAIRED) return (FI & 1) ? (cur[FI / 2] ^ 32u) : cur[FI / 2];
+    else return cur[FI < NBASE ? FI : 0];
   }
   __device__ static __forceinline__ void pin_raw(Raw& r) {
     if (KIND == OPK_KMAJOR) pin(r.q);
@@ -202,9 +219,10 @@ struct FragReader {
     else { v[0] = r.x0; v[1] = r.x1; v[2] = r.x2; v[3] = r.x3; }
     return v;
   }
-  static_assert(KIND != OPK_MMAJOR || (KSTEPS * 16 + 4) * G::ROW_BYTES < 65536, "LDS immediate offset is 16 bits");
+  static_assert(KIND != OPK_MMAJOR || (KSTEPS * KSTEP_K + 4) * G::ROW_BYTES < 65536, "LDS immediate offset is 16 bits");
   static_assert(KIND != OPK_KMAJOR || F * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
-  static_assert(KIND != OPK_CROWK || (KSTEPS * 8) * G::ROW_BYTES + F * FRAG_ROWS * 4 <= 65536, "LDS immediate offset is 16 bits");
+  static_assert(KIND != OPK_CROWK || (KSTEPS * (KSTEP_K / 2)) * G::ROW_BYTES + F * FRAG_ROWS * 4 <= 65536, "LDS immediate offset is 16 bits");
+  static_assert(MI == 32 || MI == 16, "fragments of 32 or 16 rows");
 };
 
 // The A operand of a complex product D = A * B computed as the real product of the expanded
@@ -244,15 +262,31 @@ __device__ __forceinline__ void load_frags(const RA& ra, const RB& rb, typename 
   static_for<0, FN>([&](auto fj) { rb.template read<decltype(fj)::value, KS, SYNC>(fb[decltype(fj)::value]); });
 }
 
-template <typename T> struct Mfma;
-template <> struct Mfma<_Float16> {
+template <typename T, int MI = 32> struct Mfma;
+template <> struct Mfma<_Float16, 32> {
+  typedef float16v Acc;
   __device__ static __forceinline__ float16v run(int4v a, int4v b, float16v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
   }
 };
-template <> struct Mfma<__bf16> {
+template <> struct Mfma<__bf16, 32> {
+  typedef float16v Acc;
   __device__ static __forceinline__ float16v run(int4v a, int4v b, float16v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+// 16x16x32: the same flop per operand byte; on U[-1,1) data the matrix cores hold a 14 % higher clock
+// with it under the power limit (register-only loop: 1.98 against 1.74 PFLOP/s)
+template <> struct Mfma<_Float16, 16> {
+  typedef float4v Acc;
+  __device__ static __forceinline__ float4v run(int4v a, int4v b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<__bf16, 16> {
+  typedef float4v Acc;
+  __device__ static __forceinline__ float4v run(int4v a, int4v b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
 };
 
@@ -292,8 +326,10 @@ __device__ __forceinline__ int4v scale_fragment_f16(int4v f, float scale) {
 #endif
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_, int A_KIND_, int B_KIND_, typename T_, int FUSE_,
-          bool GETT_ = false, int FIX_ = FIX_NONE, bool SPLITK_ = false>
+          bool GETT_ = false, int FIX_ = FIX_NONE, bool SPLITK_ = false, int MI_ = 32>
 struct MfmaGemmConfig {
+  static constexpr int MI = MI_;                         // rows of an MFMA block: 32 (32x32x16) or 16 (16x16x32)
+  static constexpr int KSTEP_K = MI_ == 32 ? 16 : 32;    // k-values per MFMA
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr int A_KIND = A_KIND_, B_KIND = B_KIND_, FIX = FIX_;
   // 0: no transform and no bias; 1: C / D hooks, bias and at most one exact 16-bit scale on A and on B
@@ -312,7 +348,7 @@ struct MfmaGemmConfig {
   // K-split instances: a workgroup handles one slice of K (blockIdx.z) and may add its partial result
   // into D with atomics.  A variant of its own so that the plain kernels carry none of it.
   static constexpr bool SPLITK = SPLITK_;
-  static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / 16) % 2 == 0);   // cross-step fragment prefetch
+  static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / KSTEP_K) % 2 == 0);   // cross-step fragment prefetch
   // The DMA instructions of a tile are issued a few per k-step instead of all at once: a wave whose
   // DMA instruction waits for room in the memory pipeline cannot issue its MFMAs either, and a burst
   // from every wave right after the barrier makes all of them wait together (measured on 4096^3:
@@ -322,8 +358,8 @@ struct MfmaGemmConfig {
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int THREADS = NWAVES * kWaveSize;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
-  static constexpr int FM = WTM / 32, FN = WTN / 32;             // 32x32 accumulator blocks per wave
-  static constexpr int KSTEPS = BK / 16;
+  static constexpr int FM = WTM / MI, FN = WTN / MI;             // MI x MI accumulator blocks per wave
+  static constexpr int KSTEPS = BK / KSTEP_K;
   typedef OperandGeom<BM, BK, A_KIND, EXPAND_A> GA;
   typedef OperandGeom<BN, BK, B_KIND, false> GB;
   static constexpr int STAGE_BYTES = GA::BYTES + GB::BYTES;
@@ -333,6 +369,7 @@ struct MfmaGemmConfig {
   static constexpr int DMA_PER_TILE = DMA_A + DMA_B;
   static_assert(GA::NDMA % NWAVES == 0 && GB::NDMA % NWAVES == 0, "every wave issues the same number of DMA instructions");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
+  static_assert(BK_ % KSTEP_K == 0, "BLOCK_K is a whole number of MFMA k-steps");
   static_assert(STAGES >= 2, "at least two LDS stages");
   static_assert((STAGES - 2) * DMA_PER_TILE <= 63, "vmcnt is a 6-bit counter");
   static_assert(FM * FN > 0, "empty wave tile");
@@ -529,25 +566,30 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if (s < KT) issue_tile(s);
 
   // --- accumulators: C tile (two transforms) or zeros -------------------------------------------
-  // lane l owns rows m = 32*fi + l%32 and columns n = 32*fj + 8*(v/4) + 4*(l/32) + v%4
-  float16v acc[FM][FN];
+  // 32x32 blocks: lane l owns row m = 32*fi + l%32 and columns n = 32*fj + 8*(v/4) + 4*(l/32) + v%4, v < 16;
+  // 16x16 blocks: row m = 16*fi + l%16 and columns n = 16*fj + 4*(l/16) + v, v < 4
+  constexpr int MI = Cfg::MI;
+  constexpr int NV = MI == 32 ? 16 : 4;                       // accumulator values per lane and block
+  typedef typename Mfma<T, MI>::Acc AccV;
+  auto vcol = [](int v) { return MI == 32 ? 8 * (v / 4) + (v % 4) : v; };   // column of value v inside a block, from the lane's first
+  AccV acc[FM][FN];
   // planar complex: the wave's rows lie in the real (upper) or the imaginary (lower) plane of C / D
   [[maybe_unused]] const bool lower_plane = Cfg::PLANAR && (wm * Cfg::WTM >= BM / 2);
-  const int mrow = Cfg::PLANAR ? m0 / 2 + wm * Cfg::WTM - (lower_plane ? BM / 2 : 0) + (lane & 31) : m0 + wm * Cfg::WTM + (lane & 31);
-  const int ncol = n0 + wn * Cfg::WTN + 4 * (lane >> 5);
+  const int mrow = Cfg::PLANAR ? m0 / 2 + wm * Cfg::WTM - (lower_plane ? BM / 2 : 0) + (lane % MI) : m0 + wm * Cfg::WTM + (lane % MI);
+  const int ncol = n0 + wn * Cfg::WTN + 4 * (lane / MI);
   // element offset of the lane's first element of accumulator block (fi, fj) in C / D, and the
   // stride between its consecutive columns.  With a tensor-contraction map the first M mode and
   // the first N mode cover whole 32-wide blocks, so only the block origin needs the digit walk.
   auto cd_offset = [&](int fi, int fj, long long ld, [[maybe_unused]] long long plane) -> long long {
     if constexpr (Cfg::PLANAR) {
-      return (long long)(mrow + 32 * fi) + (long long)(ncol + 32 * fj) * ld + (lower_plane ? plane : 0ll);
+      return (long long)(mrow + MI * fi) + (long long)(ncol + MI * fj) * ld + (lower_plane ? plane : 0ll);
     } else if constexpr (!Cfg::GETT) {
-      return (long long)(mrow + 32 * fi) + (long long)(ncol + 32 * fj) * ld;
+      return (long long)(mrow + MI * fi) + (long long)(ncol + MI * fj) * ld;
     } else {
       long long t0, om, on;
-      gett_offsets(args.gm, m0 + wm * Cfg::WTM + 32 * fi, t0, om);
-      gett_offsets(args.gn, n0 + wn * Cfg::WTN + 32 * fj, t0, on);
-      return om + (long long)(lane & 31) * args.gm.stride1[0] + on + (long long)(4 * (lane >> 5)) * args.gn.stride1[0];
+      gett_offsets(args.gm, m0 + wm * Cfg::WTM + MI * fi, t0, om);
+      gett_offsets(args.gn, n0 + wn * Cfg::WTN + MI * fj, t0, on);
+      return om + (long long)(lane % MI) * args.gm.stride1[0] + on + (long long)(4 * (lane / MI)) * args.gn.stride1[0];
     }
   };
   auto cd_nstride = [&](long long ld) -> long long {
@@ -569,15 +611,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         if (args.c_dtype == DT_F32) {
           const float* cp = (const float*)args.c + off;
 #pragma unroll
-          for (int v = 0; v < 16; ++v) acc[fi][fj][v] = cp[(long long)(8 * (v / 4) + (v % 4)) * ns];
+          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = cp[(long long)vcol(v) * ns];
         } else if (args.c_dtype == DT_F16) {
           const _Float16* cp = (const _Float16*)args.c + off;
 #pragma unroll
-          for (int v = 0; v < 16; ++v) acc[fi][fj][v] = (float)cp[(long long)(8 * (v / 4) + (v % 4)) * ns];
+          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = (float)cp[(long long)vcol(v) * ns];
         } else {
           const __bf16* cp = (const __bf16*)args.c + off;
 #pragma unroll
-          for (int v = 0; v < 16; ++v) acc[fi][fj][v] = (float)cp[(long long)(8 * (v / 4) + (v % 4)) * ns];
+          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = (float)cp[(long long)vcol(v) * ns];
         }
       }
     if (Cfg::FUSED) {
@@ -586,13 +628,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
           for (int fj = 0; fj < FN; ++fj) {
-            float x[16];
+            float x[NV];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
-            hook_regs<H_GL2SH_C, 16>(args, x);
-            hook_regs<H_SH2RF_C, 16>(args, x);
+            for (int v = 0; v < NV; ++v) x[v] = acc[fi][fj][v];
+            hook_regs<H_GL2SH_C, NV>(args, x);
+            hook_regs<H_SH2RF_C, NV>(args, x);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[fi][fj][v] = x[v];
+            for (int v = 0; v < NV; ++v) acc[fi][fj][v] = x[v];
           }
       }
     }
@@ -602,7 +644,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[fi][fj][v] = 0.0f;
+        for (int v = 0; v < NV; ++v) acc[fi][fj][v] = 0.0f;
   }
 
   if constexpr (Cfg::PLANAR) {
@@ -617,8 +659,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const bool fast_b = std::is_same<T, _Float16>::value && args.fast_scale_b != 0;
   const float scale_a = args.scale_a, scale_b = args.scale_b;
 
-  typedef FragReader<BM, BK, Cfg::A_KIND, Cfg::EXPAND_A, FM> RA;
-  typedef FragReader<BN, BK, Cfg::B_KIND, false, FN> RB;
+  typedef FragReader<BM, BK, Cfg::A_KIND, Cfg::EXPAND_A, FM, MI> RA;
+  typedef FragReader<BN, BK, Cfg::B_KIND, false, FN, MI> RB;
   RA ra;
   RB rb;
   ra.init(wm * Cfg::WTM, lane);
@@ -677,7 +719,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #ifdef GK_ABLATE_MFMA
         acc[fi][fj][0] += __builtin_bit_cast(float, vb[fj][0] ^ va[fi][0]);
 #else
-        acc[fi][fj] = Mfma<T>::run(vb[fj], va[fi], acc[fi][fj]);
+        acc[fi][fj] = Mfma<T, MI>::run(vb[fj], va[fi], acc[fi][fj]);
 #endif
       }
   };
@@ -769,20 +811,20 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     for (int fj = 0; fj < FN; ++fj) {
       const long long off = cd_offset(fi, fj, args.ldd, args.plane_d);
       const long long ns = cd_nstride(args.ldd);
-      float x[16];
+      float x[NV];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) x[v] = acc[fi][fj][v];
+      for (int v = 0; v < NV; ++v) x[v] = acc[fi][fj][v];
       if (Cfg::FUSED) {
-        hook_regs<H_RF2SH_D, 16>(args, x);
+        hook_regs<H_RF2SH_D, NV>(args, x);
         if (args.epi_kind == 1) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) x[v] = x[v] + args.bias[ncol + 32 * fj + 8 * (v / 4) + (v % 4)];
+          for (int v = 0; v < NV; ++v) x[v] = x[v] + args.bias[ncol + MI * fj + vcol(v)];
         } else if (args.epi_kind == 2) {
-          const float bv = args.bias[mrow + 32 * fi];
+          const float bv = args.bias[mrow + MI * fi];
 #pragma unroll
-          for (int v = 0; v < 16; ++v) x[v] = x[v] + bv;
+          for (int v = 0; v < NV; ++v) x[v] = x[v] + bv;
         }
-        hook_regs<H_SH2GL_D, 16>(args, x);
+        hook_regs<H_SH2GL_D, NV>(args, x);
       }
       // the accumulator is rounded once, to the element type of D
       if constexpr (Cfg::SPLITK) {
@@ -791,22 +833,22 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           // last bits of the sum, is not fixed)
           float* dp = (float*)args.d + off;
 #pragma unroll
-          for (int v = 0; v < 16; ++v) atomicAdd(&dp[(long long)(8 * (v / 4) + (v % 4)) * ns], x[v]);
+          for (int v = 0; v < NV; ++v) atomicAdd(&dp[(long long)vcol(v) * ns], x[v]);
           continue;
         }
       }
       if (args.d_dtype == DT_F32) {
         float* dp = (float*)args.d + off;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) dp[(long long)(8 * (v / 4) + (v % 4)) * ns] = x[v];
+        for (int v = 0; v < NV; ++v) dp[(long long)vcol(v) * ns] = x[v];
       } else if (args.d_dtype == DT_F16) {
         _Float16* dp = (_Float16*)args.d + off;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) dp[(long long)(8 * (v / 4) + (v % 4)) * ns] = (_Float16)x[v];
+        for (int v = 0; v < NV; ++v) dp[(long long)vcol(v) * ns] = (_Float16)x[v];
       } else {
         __bf16* dp = (__bf16*)args.d + off;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) dp[(long long)(8 * (v / 4) + (v % 4)) * ns] = (__bf16)x[v];
+        for (int v = 0; v < NV; ++v) dp[(long long)vcol(v) * ns] = (__bf16)x[v];
       }
     }
 #ifdef GK_PHASE_TRACE
