@@ -9,6 +9,13 @@
 #include "mfma_gemm.hpp"
 #include "registry.hpp"
 
+#ifndef GK_CPLX_MI
+// MFMA block of the complex / dual instances with A contiguous along m (16: v_mfma_f32_16x16x32).  With a
+// K-major A (one complex row feeds two MFMA rows) a 16-row fragment spans 8 tile rows, which the row swizzle
+// of the tile does not leave invariant under the immediate offsets of the reads: those stay with 32.
+#define GK_CPLX_MI 16
+#endif
+
 namespace gk {
 
 int family_complex(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode, InstanceInfo* info,
@@ -19,7 +26,7 @@ int family_complex(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipS
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
       key.a_kmajor == akm_ && key.b_kmajor == bkm_ && key.variant == dual_) {                                             \
     typedef MfmaGemmConfig<2 * bm_, bn_, 2 * bk_, wm_, wn_, st_, (akm_ ? OPK_KMAJOR : OPK_CROWK),                          \
-                           (bkm_ ? OPK_KMAJOR : OPK_CROWK), _Float16, 0, false, (dual_ ? FIX_DUAL : FIX_COMPLEX)> Cfg; \
+                           (bkm_ ? OPK_KMAJOR : OPK_CROWK), _Float16, 0, false, (dual_ ? FIX_DUAL : FIX_COMPLEX), false, (akm_ ? 32 : GK_CPLX_MI)> Cfg; \
     return run_instance<Cfg>(mfma_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
 #define GK_CPLX_T(bm_, bn_, bk_, wm_, wn_, st_, dual_, TAG)                                     \

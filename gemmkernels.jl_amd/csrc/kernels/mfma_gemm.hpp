@@ -223,6 +223,7 @@ struct FragReader {
   static_assert(KIND != OPK_KMAJOR || F * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
   static_assert(KIND != OPK_CROWK || (KSTEPS * (KSTEP_K / 2)) * G::ROW_BYTES + F * FRAG_ROWS * 4 <= 65536, "LDS immediate offset is 16 bits");
   static_assert(MI == 32 || MI == 16, "fragments of 32 or 16 rows");
+  static_assert(!(EXPAND && KIND == OPK_KMAJOR && MI == 16), "expanded K-major fragments of 8 tile rows break the swizzle invariance of the read offsets");
 };
 
 // The A operand of a complex product D = A * B computed as the real product of the expanded
@@ -580,16 +581,31 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // element offset of the lane's first element of accumulator block (fi, fj) in C / D, and the
   // stride between its consecutive columns.  With a tensor-contraction map the first M mode and
   // the first N mode cover whole 32-wide blocks, so only the block origin needs the digit walk.
+  // contractions: origins of the blocks of the wave tile in C / D, one digit walk per 32 rows (columns);
+  // filled before the C load and again before the D store (not kept across the K loop)
+  [[maybe_unused]] long long gett_om[Cfg::GETT ? FM : 1], gett_on[Cfg::GETT ? FN : 1];
+  [[maybe_unused]] auto gett_origins = [&]() __attribute__((always_inline)) {
+    if constexpr (Cfg::GETT) {
+      long long t0;
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi) {
+        if (MI == 16 && (fi & 1)) gett_om[fi] = gett_om[fi - 1] + 16 * args.gm.stride1[0];
+        else gett_offsets(args.gm, m0 + wm * Cfg::WTM + MI * fi, t0, gett_om[fi]);
+      }
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) {
+        if (MI == 16 && (fj & 1)) gett_on[fj] = gett_on[fj - 1] + 16 * args.gn.stride1[0];
+        else gett_offsets(args.gn, n0 + wn * Cfg::WTN + MI * fj, t0, gett_on[fj]);
+      }
+    }
+  };
   auto cd_offset = [&](int fi, int fj, long long ld, [[maybe_unused]] long long plane) -> long long {
     if constexpr (Cfg::PLANAR) {
       return (long long)(mrow + MI * fi) + (long long)(ncol + MI * fj) * ld + (lower_plane ? plane : 0ll);
     } else if constexpr (!Cfg::GETT) {
       return (long long)(mrow + MI * fi) + (long long)(ncol + MI * fj) * ld;
     } else {
-      long long t0, om, on;
-      gett_offsets(args.gm, m0 + wm * Cfg::WTM + MI * fi, t0, om);
-      gett_offsets(args.gn, n0 + wn * Cfg::WTN + MI * fj, t0, on);
-      return om + (long long)(lane % MI) * args.gm.stride1[0] + on + (long long)(4 * (lane / MI)) * args.gn.stride1[0];
+      return gett_om[fi] + (long long)(lane % MI) * args.gm.stride1[0] + gett_on[fj] + (long long)(4 * (lane / MI)) * args.gn.stride1[0];
     }
   };
   auto cd_nstride = [&](long long ld) -> long long {
@@ -602,6 +618,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = -acc[fi][fj];
   };
   if (args.c_mode != 0) {
+    gett_origins();
 #pragma unroll
     for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
@@ -805,6 +822,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   trace_t[2] = clock64();
 #endif
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
+  gett_origins();
 #pragma unroll
   for (int fi = 0; fi < FM; ++fi)
 #pragma unroll

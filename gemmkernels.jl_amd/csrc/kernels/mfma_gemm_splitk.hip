@@ -12,7 +12,7 @@ int family_mfma_splitk(const InstanceKey& key, const GemmArgs& args, dim3 grid, 
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ && key.dtype == DT &&   \
       key.fused == FUSED && key.a_kmajor == akm_ && key.b_kmajor == bkm_) {                                               \
     typedef MfmaGemmConfig<bm_, bn_, bk_, wm_, wn_, st_, (akm_ ? OPK_KMAJOR : OPK_MMAJOR), (bkm_ ? OPK_KMAJOR : OPK_MMAJOR), \
-                           TYPE, FUSED, false, FIX_NONE, true> Cfg;                                                        \
+                           TYPE, FUSED, false, FIX_NONE, true, 16> Cfg;                                                        \
     return run_instance<Cfg>(mfma_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
 #define GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, TYPE, DT, FUSED, TAG)                                                                  \
