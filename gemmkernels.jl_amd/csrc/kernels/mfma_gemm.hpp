@@ -349,7 +349,12 @@ struct MfmaGemmConfig {
   // K-split instances: a workgroup handles one slice of K (blockIdx.z) and may add its partial result
   // into D with atomics.  A variant of its own so that the plain kernels carry none of it.
   static constexpr bool SPLITK = SPLITK_;
-  static constexpr bool PREFETCH = (STAGES_ >= 3) && ((BK_ / KSTEP_K) % 2 == 0);   // cross-step fragment prefetch
+  // 16-row blocks: a k-step of 32 holds twice the fragments of a 16-wide one, so the A fragments are read
+  // and consumed in two halves (rows fi < FM/2, then the rest) with the reads of one half in flight under
+  // the MFMAs of the other: 32 registers fewer than two whole buffers, and never more than 12 LDS reads
+  // outstanding (the wait counter holds 15)
+  static constexpr bool SPLIT_A = MI_ == 16 && ((BM_ / WAVES_M_ / MI_) % 2 == 0);
+  static constexpr bool PREFETCH = !SPLIT_A && (STAGES_ >= 3) && ((BK_ / KSTEP_K) % 2 == 0);   // cross-step fragment prefetch
   // The DMA instructions of a tile are issued a few per k-step instead of all at once: a wave whose
   // DMA instruction waits for room in the memory pipeline cannot issue its MFMAs either, and a burst
   // from every wave right after the barrier makes all of them wait together (measured on 4096^3:
@@ -696,13 +701,19 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr int FRAG_OPS = FM * RA::OPS + FN * RB::OPS;
 
   // runs after the wait that covers the reads of buffer ks & 1
-  auto compute = [&](auto ks_c) {
+  // With Cfg::SPLIT_A the A fragments live in two half buffers fa[h][0 .. FM/2) and `half_c` says which half
+  // (rows fi = h * FM/2 + i) this call multiplies; otherwise fa[ks & 1] holds all FM fragments and half_c is -1.
+  auto compute = [&](auto ks_c, auto half_c) {
     constexpr int ks = decltype(ks_c)::value;
-    int4v va[FM], vb[FN];
+    constexpr int half = decltype(half_c)::value;
+    constexpr int NA = half < 0 ? FM : FM / 2;             // A fragments of this call
+    constexpr int FI0 = half < 0 ? 0 : half * (FM / 2);     // the accumulator row block of the first one
+    constexpr int ABUF = half < 0 ? (ks & 1) : half;
+    int4v va[NA], vb[FN];
 #pragma unroll
-    for (int fi = 0; fi < FM; ++fi) {
-      RA::pin_raw(fa[ks & 1][fi]);
-      va[fi] = expand_fixup<Cfg::FIX>(RA::finish(fa[ks & 1][fi]), lane);
+    for (int fi = 0; fi < NA; ++fi) {
+      RA::pin_raw(fa[ABUF][fi]);
+      va[fi] = expand_fixup<Cfg::FIX>(RA::finish(fa[ABUF][fi]), lane);
     }
 #pragma unroll
     for (int fj = 0; fj < FN; ++fj) {
@@ -713,10 +724,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       if (xf_a) {
         if (fast_a) {
 #pragma unroll
-          for (int fi = 0; fi < FM; ++fi) va[fi] = scale_fragment_f16(va[fi], scale_a);
+          for (int fi = 0; fi < NA; ++fi) va[fi] = scale_fragment_f16(va[fi], scale_a);
         } else if constexpr (Cfg::FUSED_AB_GENERIC) {
 #pragma unroll
-          for (int fi = 0; fi < FM; ++fi) va[fi] = transform_fragment<T, H_GL2SH_A, H_SH2RF_A>(va[fi], args);
+          for (int fi = 0; fi < NA; ++fi) va[fi] = transform_fragment<T, H_GL2SH_A, H_SH2RF_A>(va[fi], args);
         }
       }
       if (xf_b) {
@@ -730,16 +741,17 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       }
     }
 #pragma unroll
-    for (int fi = 0; fi < FM; ++fi)
+    for (int fi = 0; fi < NA; ++fi)
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj) {
 #ifdef GK_ABLATE_MFMA
-        acc[fi][fj][0] += __builtin_bit_cast(float, vb[fj][0] ^ va[fi][0]);
+        acc[FI0 + fi][fj][0] += __builtin_bit_cast(float, vb[fj][0] ^ va[fi][0]);
 #else
-        acc[fi][fj] = Mfma<T, MI>::run(vb[fj], va[fi], acc[fi][fj]);
+        acc[FI0 + fi][fj] = Mfma<T, MI>::run(vb[fj], va[fi], acc[FI0 + fi][fj]);
 #endif
       }
   };
+  typedef std::integral_constant<int, -1> Whole;
 
   if constexpr (!Cfg::PREFETCH) {
     // Two LDS stages: the DMA of tile kt+1 runs while tile kt is consumed; the first fragments of a
@@ -754,8 +766,46 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       const unsigned stage_addr = lds_base + (unsigned)(kt % STAGES) * Cfg::STAGE_BYTES;
       ra.set_stage(stage_addr);
       rb.set_stage(stage_addr + GA::BYTES);
-      load_frags<0, Cfg::SYNC_FRAGS>(ra, rb, fa[0], fb[0]);
       const bool issue = (kt + STAGES - 1 < KT);
+      if constexpr (Cfg::SPLIT_A) {
+        constexpr int HF = FM / 2;
+        constexpr int OPS_AH = HF * RA::OPS, OPS_B = FN * RB::OPS;
+        // reads of A half H of k-step KS into fa[H], of B of k-step KS into fb[KS & 1]
+        auto load_a_half = [&](auto ks2_c, auto h_c) __attribute__((always_inline)) {
+          constexpr int KS2 = decltype(ks2_c)::value, H = decltype(h_c)::value;
+          static_for<0, HF>([&](auto i_c) {
+            constexpr int I = decltype(i_c)::value;
+            ra.template read<H * HF + I, KS2, Cfg::SYNC_FRAGS>(fa[H][I]);
+          });
+        };
+        auto load_b = [&](auto ks2_c) __attribute__((always_inline)) {
+          constexpr int KS2 = decltype(ks2_c)::value;
+          static_for<0, FN>([&](auto j_c) {
+            constexpr int J = decltype(j_c)::value;
+            rb.template read<J, KS2, Cfg::SYNC_FRAGS>(fb[KS2 & 1][J]);
+          });
+        };
+        load_a_half(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+        load_b(std::integral_constant<int, 0>{});
+        static_for<0, 2 * Cfg::KSTEPS>([&](auto u_c) {
+          constexpr int u = decltype(u_c)::value;
+          constexpr int ks = u / 2, h = u % 2;
+          if (issue) issue_part(u_c, std::integral_constant<int, 2 * Cfg::KSTEPS>{}, (kt + STAGES - 1) % STAGES);
+          if constexpr (h == 0) {
+            load_a_half(std::integral_constant<int, ks>{}, std::integral_constant<int, 1>{});
+            wait_lgkmcnt<OPS_AH>();                     // half 0 and B of this k-step have arrived
+          } else if constexpr (ks + 1 < Cfg::KSTEPS) {
+            load_a_half(std::integral_constant<int, ks + 1>{}, std::integral_constant<int, 0>{});
+            load_b(std::integral_constant<int, ks + 1>{});
+            wait_lgkmcnt<OPS_AH + OPS_B>();             // half 1 of this k-step has arrived
+          } else {
+            wait_lgkmcnt<0>();                          // all LDS reads of this stage are complete before the next barrier
+          }
+          compute(std::integral_constant<int, ks>{}, std::integral_constant<int, h>{});
+        });
+        continue;
+      }
+      load_frags<0, Cfg::SYNC_FRAGS>(ra, rb, fa[0], fb[0]);
       if constexpr (!Cfg::SPREAD) {
         if (issue) issue_tile((kt + STAGES - 1) % STAGES);
       }
@@ -767,7 +817,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
         if constexpr (more) load_frags<ks + 1, Cfg::SYNC_FRAGS>(ra, rb, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
         wait_lgkmcnt<more ? FRAG_OPS : 0>();
-        compute(ks_c);
+        compute(ks_c, Whole{});
       });
       // the last wait above was lgkmcnt(0): all LDS reads of this stage are complete before the
       // next barrier lets a DMA overwrite it
@@ -813,7 +863,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         if constexpr (Cfg::SPREAD) {
           if (issue) issue_part(ks_c, std::integral_constant<int, Cfg::KSTEPS>{}, (kt + STAGES - 1) % STAGES);
         }
-        compute(ks_c);
+        compute(ks_c, Whole{});
       });
     }
   }
