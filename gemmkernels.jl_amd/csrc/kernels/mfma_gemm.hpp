@@ -624,10 +624,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   };
   if (args.c_mode != 0) {
     gett_origins();
+    // column blocks outermost: with 16-row blocks the two halves of a 128-byte line of C / D belong to
+    // neighbouring row blocks, which are then read (and, below, written) right after each other
 #pragma unroll
-    for (int fi = 0; fi < FM; ++fi)
+    for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) {
+      for (int fi = 0; fi < FM; ++fi) {
         const long long off = cd_offset(fi, fj, args.ldc, args.plane_c);
         const long long ns = cd_nstride(args.ldc);
         if (args.c_dtype == DT_F32) {
@@ -874,9 +876,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   gett_origins();
 #pragma unroll
-  for (int fi = 0; fi < FM; ++fi)
+  for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
-    for (int fj = 0; fj < FN; ++fj) {
+    for (int fi = 0; fi < FM; ++fi) {
       const long long off = cd_offset(fi, fj, args.ldd, args.plane_d);
       const long long ns = cd_nstride(args.ldd);
       float x[NV];
