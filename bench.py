@@ -26,7 +26,7 @@ PEAK_FP16_TFLOPS = 2516.6     # MI355X dense FP16/BF16 matrix peak (256 CU x 4 S
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the headline kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # summarised in profiles/ (None until measured)
-MEASURED_TRAFFIC_BYTES = 335_872_000   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131232.3 * 2.0 + 65536.0) KiB
+MEASURED_TRAFFIC_BYTES = 337_066_424   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131278.7 * 2.0 + 66633.0) KiB
 
 
 def parse_args():
