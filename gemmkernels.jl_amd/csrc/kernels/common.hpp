@@ -192,45 +192,31 @@ __device__ __forceinline__ float apply_list(const OpList& t, float x) {
   return x;
 }
 
-// Applies a list to an array of registers with the op switch outside the element loop, so that
-// the (wave-uniform) dispatch is paid once per op and not once per element.
+// One op of a list handed to `each` as an elementwise function: the (wave-uniform) switch on the op
+// is paid once per call of `each`, which applies the function to as many registers as the caller
+// holds (a fragment, or all accumulators of a lane).
+template <typename Each>
+__device__ __forceinline__ void dispatch_op(int kind, float p0, float p1, Each&& each) {
+  switch (kind) {
+    case T_SCALE:  each([=](float x) { return x * p0; }); break;
+    case T_ADD:    each([=](float x) { return x + p0; }); break;
+    case T_RELU:   each([=](float x) { return x > 0.0f ? x : 0.0f; }); break;
+    case T_NEG:    each([=](float x) { return -x; }); break;
+    case T_ABS:    each([=](float x) { return __builtin_fabsf(x); }); break;
+    case T_CLAMP:  each([=](float x) { return x < p0 ? p0 : (x > p1 ? p1 : x); }); break;
+    case T_SQUARE: each([=](float x) { return x * x; }); break;
+    default: break;
+  }
+}
+
+// Applies a list to an array of registers with the op switch outside the element loop.
 template <int COUNT>
 __device__ __forceinline__ void apply_list_regs(const OpList& t, float (&x)[COUNT]) {
-  for (int i = 0; i < t.n; ++i) {
-    const float p0 = t.p0[i], p1 = t.p1[i];
-    switch (t.kind[i]) {
-      case T_SCALE:
+  for (int i = 0; i < t.n; ++i)
+    dispatch_op(t.kind[i], t.p0[i], t.p1[i], [&](auto f) {
 #pragma unroll
-        for (int e = 0; e < COUNT; ++e) x[e] = x[e] * p0;
-        break;
-      case T_ADD:
-#pragma unroll
-        for (int e = 0; e < COUNT; ++e) x[e] = x[e] + p0;
-        break;
-      case T_RELU:
-#pragma unroll
-        for (int e = 0; e < COUNT; ++e) x[e] = x[e] > 0.0f ? x[e] : 0.0f;
-        break;
-      case T_NEG:
-#pragma unroll
-        for (int e = 0; e < COUNT; ++e) x[e] = -x[e];
-        break;
-      case T_ABS:
-#pragma unroll
-        for (int e = 0; e < COUNT; ++e) x[e] = __builtin_fabsf(x[e]);
-        break;
-      case T_CLAMP:
-#pragma unroll
-        for (int e = 0; e < COUNT; ++e) x[e] = x[e] < p0 ? p0 : (x[e] > p1 ? p1 : x[e]);
-        break;
-      case T_SQUARE:
-#pragma unroll
-        for (int e = 0; e < COUNT; ++e) x[e] = x[e] * x[e];
-        break;
-      default:
-        break;
-    }
-  }
+      for (int e = 0; e < COUNT; ++e) x[e] = f(x[e]);
+    });
 }
 
 // ---------------------------------------------------------------------------------------------

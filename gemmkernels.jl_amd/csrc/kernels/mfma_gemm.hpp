@@ -219,6 +219,12 @@ struct FragReader {
     else { v[0] = r.x0; v[1] = r.x1; v[2] = r.x2; v[3] = r.x3; }
     return v;
   }
+  // puts a (transformed) operand back into the registers of its fragment
+  __device__ static __forceinline__ void store(Raw& r, int4v v) {
+    if (KIND == OPK_KMAJOR) r.q = v;
+    else if (KIND == OPK_MMAJOR) { r.lo[0] = v[0]; r.lo[1] = v[1]; r.hi[0] = v[2]; r.hi[1] = v[3]; }
+    else { r.x0 = v[0]; r.x1 = v[1]; r.x2 = v[2]; r.x3 = v[3]; }
+  }
   static_assert(KIND != OPK_MMAJOR || (KSTEPS * KSTEP_K + 4) * G::ROW_BYTES < 65536, "LDS immediate offset is 16 bits");
   static_assert(KIND != OPK_KMAJOR || F * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
   static_assert(KIND != OPK_CROWK || (KSTEPS * (KSTEP_K / 2)) * G::ROW_BYTES + F * FRAG_ROWS * 4 <= 65536, "LDS immediate offset is 16 bits");
@@ -622,6 +628,24 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = -acc[fi][fj];
   };
+  // One hook over the accumulators of column block fj (FM blocks): the dispatch on the op is paid once per
+  // op and column block, not once per 16x16 block.  (Over all accumulators at once the cases of the
+  // dispatch meet in more registers than a lane has.)
+  [[maybe_unused]] auto hook_col = [&](auto h_c, int fj) __attribute__((always_inline)) {
+    constexpr int H = decltype(h_c)::value;
+    auto each = [&](auto f) __attribute__((always_inline)) {
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[fi][fj][v] = f(acc[fi][fj][v]);
+    };
+#ifdef GK_USER_HOOKS
+    if constexpr (UserHooks::present[H]) each([](float x) { return UserHooks::template apply<H>(x); });
+#else
+    const OpList& t = args.t[H];
+    for (int i = 0; i < t.n; ++i) dispatch_op(t.kind[i], t.p0[i], t.p1[i], each);
+#endif
+  };
   if (args.c_mode != 0) {
     gett_origins();
     // column blocks outermost: with 16-row blocks the two halves of a 128-byte line of C / D belong to
@@ -647,19 +671,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
       }
     if (Cfg::FUSED) {
-      if (hook_present<H_GL2SH_C>(args) || hook_present<H_SH2RF_C>(args)) {
 #pragma unroll
-        for (int fi = 0; fi < FM; ++fi)
-#pragma unroll
-          for (int fj = 0; fj < FN; ++fj) {
-            float x[NV];
-#pragma unroll
-            for (int v = 0; v < NV; ++v) x[v] = acc[fi][fj][v];
-            hook_regs<H_GL2SH_C, NV>(args, x);
-            hook_regs<H_SH2RF_C, NV>(args, x);
-#pragma unroll
-            for (int v = 0; v < NV; ++v) acc[fi][fj][v] = x[v];
-          }
+      for (int fj = 0; fj < FN; ++fj) {
+        hook_col(std::integral_constant<int, H_GL2SH_C>{}, fj);
+        hook_col(std::integral_constant<int, H_SH2RF_C>{}, fj);
       }
     }
   } else {
@@ -702,6 +717,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   typename RB::Raw fb[2][FN];
   constexpr int FRAG_OPS = FM * RA::OPS + FN * RB::OPS;
 
+  // The whole K loop is a generic lambda whose MODE says at compile time what happens to the fragments
+  // (bits 0 / 1: A / B multiplied by an FP16 factor): a flag tested inside the loop costs a branch around
+  // every group of MFMAs.  MODE -1 reads the flags at run time (kernels without hooks, where they fold
+  // away, and the generic functor kernels).
+  auto k_loop = [&](auto mode_c) __attribute__((always_inline)) {
+  constexpr int MODE = decltype(mode_c)::value;
   // runs after the wait that covers the reads of buffer ks & 1
   // With Cfg::SPLIT_A the A fragments live in two half buffers fa[h][0 .. FM/2) and `half_c` says which half
   // (rows fi = h * FM/2 + i) this call multiplies; otherwise fa[ks & 1] holds all FM fragments and half_c is -1.
@@ -722,7 +743,29 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       RB::pin_raw(fb[ks & 1][fj]);
       vb[fj] = RB::finish(fb[ks & 1][fj]);
     }
-    if (Cfg::FUSED) {
+    if constexpr (MODE >= 0) {
+      // A is scaled one fragment ahead of the MFMAs that use it: in this order the compiler lets part of
+      // the multiplications issue in the shadow of MFMAs (with all of them written up front the loop is 5 %
+      // slower; pinning a finer interleaving with scheduling barriers is slower still).  B is scaled once
+      // per k-step: the call for the second half of A finds it scaled.
+      if constexpr ((MODE & 2) != 0 && half <= 0) {
+#pragma unroll
+        for (int fj = 0; fj < FN; ++fj) {
+          vb[fj] = scale_fragment_f16(vb[fj], scale_b);
+          if constexpr (half == 0) RB::store(fb[ks & 1][fj], vb[fj]);
+        }
+      }
+      if constexpr ((MODE & 1) != 0) va[0] = scale_fragment_f16(va[0], scale_a);
+#pragma unroll
+      for (int fi = 0; fi < NA; ++fi) {
+#pragma unroll
+        for (int fj = 0; fj < FN; ++fj) acc[FI0 + fi][fj] = Mfma<T, MI>::run(vb[fj], va[fi], acc[FI0 + fi][fj]);
+        if constexpr ((MODE & 1) != 0) {
+          if (fi + 1 < NA) va[fi + 1] = scale_fragment_f16(va[fi + 1], scale_a);
+        }
+      }
+      return;
+    } else if (Cfg::FUSED) {
       if (xf_a) {
         if (fast_a) {
 #pragma unroll
@@ -869,6 +912,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       });
     }
   }
+  };   // k_loop
+  if constexpr (Cfg::FUSE == 1) {
+    // FP16 operands whose hooks are at most one multiplication by a factor that is exact in FP16 (the host
+    // passes 1 for an operand without one): both multiplications always run.  Separate copies of the loop
+    // per combination cost more than the multiplications save (the accumulators of the copies meet in
+    // registers the compiler then has to spill).
+    k_loop(std::integral_constant<int, 3>{});
+  } else {
+    k_loop(std::integral_constant<int, -1>{});
+  }
 
 #ifdef GK_PHASE_TRACE
   trace_t[2] = clock64();
@@ -876,7 +929,27 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   gett_origins();
 #pragma unroll
-  for (int fj = 0; fj < FN; ++fj)
+  for (int fj = 0; fj < FN; ++fj) {
+    if (Cfg::FUSED) {
+      hook_col(std::integral_constant<int, H_RF2SH_D>{}, fj);
+      if (args.epi_kind == 1) {          // one bias value per column of D
+        float bv[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) bv[v] = args.bias[ncol + MI * fj + vcol(v)];
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = acc[fi][fj][v] + bv[v];
+      } else if (args.epi_kind == 2) {   // one bias value per row of D
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          const float bv = args.bias[mrow + MI * fi];
+#pragma unroll
+          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = acc[fi][fj][v] + bv;
+        }
+      }
+      hook_col(std::integral_constant<int, H_SH2GL_D>{}, fj);
+    }
 #pragma unroll
     for (int fi = 0; fi < FM; ++fi) {
       const long long off = cd_offset(fi, fj, args.ldd, args.plane_d);
@@ -884,18 +957,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       float x[NV];
 #pragma unroll
       for (int v = 0; v < NV; ++v) x[v] = acc[fi][fj][v];
-      if (Cfg::FUSED) {
-        hook_regs<H_RF2SH_D, NV>(args, x);
-        if (args.epi_kind == 1) {
-#pragma unroll
-          for (int v = 0; v < NV; ++v) x[v] = x[v] + args.bias[ncol + MI * fj + vcol(v)];
-        } else if (args.epi_kind == 2) {
-          const float bv = args.bias[mrow + MI * fi];
-#pragma unroll
-          for (int v = 0; v < NV; ++v) x[v] = x[v] + bv;
-        }
-        hook_regs<H_SH2GL_D, NV>(args, x);
-      }
       // the accumulator is rounded once, to the element type of D
       if constexpr (Cfg::SPLITK) {
         if (args.atomic_d) {
@@ -921,6 +982,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         for (int v = 0; v < NV; ++v) dp[(long long)vcol(v) * ns] = (__bf16)x[v];
       }
     }
+  }
 #ifdef GK_PHASE_TRACE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   trace_t[3] = clock64();
