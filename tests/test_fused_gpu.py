@@ -62,6 +62,33 @@ def test_exact_scaling_and_relu_idempotence(gpu):
 
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("block", [(256, 256, 64), (128, 128, 64), (64, 64, 32)])
+def test_fp16_scales_on_a_and_b_equal_prescaled_operands_bit_for_bit(gpu, block, ta, tb):
+    """A factor that is exact in FP16, on either operand or on both, is applied inside the K loop with one
+    rounding to FP16 per element: the result equals, bit for bit, what the same tile computes from operands
+    scaled (and rounded to FP16) beforehand.  Factors 1.5 and -0.375 are not powers of two, so the rounding
+    of the scaled operand is visible."""
+    BM, BN, BK = block
+    M, N, K = 2 * BM, BN, 4 * BK
+    conf = configs.mfma_config(M, N, K, ta, tb, block_shape=block)
+    a = rng.matrix("upm1_f16", 71, (K, M) if ta else (M, K))
+    b = rng.matrix("upm1_f16", 72, (N, K) if tb else (K, N))
+    c = rng.matrix("upm1_f32", 73, (M, N))
+    sa, sb = np.float16(1.5), np.float16(-0.375)
+    a_s = np.asfortranarray((a.astype(np.float32) * np.float32(sa)).astype(np.float16))
+    b_s = np.asfortranarray((b.astype(np.float32) * np.float32(sb)).astype(np.float16))
+    cases = [(dict(transform_shared_to_regs_b=E(lambda x: x * -0.375)), a, b_s),
+             (dict(transform_global_to_shared_a=E(lambda x: x * 1.5), transform_global_to_shared_b=E(lambda x: x * -0.375)), a_s, b_s),
+             (dict(transform_shared_to_regs_a=E(lambda x: x * 1.5)), a_s, b)]
+    for tr, a_ref, b_ref in cases:
+        name = gk.kernel_name(conf, Kernel.matmul_pipelined, tr)
+        assert name.endswith("_fused"), name        # the kernels with the packed FP16 multiply, not the per-element interpreter
+        d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=tr, kernel=Kernel.matmul_pipelined)
+        want = helpers.run_gpu(conf, a_ref, b_ref, c, (M, N), kernel=Kernel.matmul_pipelined)
+        assert np.array_equal(d, want), sorted(tr)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
 def test_all_eight_hooks(gpu, ta, tb):
     """Every hook carries a different op list; the oracle applies them at the same points with the
     same rounding (alpha on A in FP16, beta on C in FP32 as matmatmul! does, src/matmul.jl:196-201)."""
