@@ -700,7 +700,8 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   gk::FamilyFn fn = family_fn(L.key);
   hipError_t err = hipSuccess;
   if (kernel == GK_KERNEL_SPLIT_K) {
-    if (L.key.family != gk::FAMILY_MFMA) return fail(GK_ERR_UNSUPPORTED, "the K-split kernel runs the real MFMA operator on aligned layouts");
+    if (L.key.family != gk::FAMILY_MFMA && L.key.family != gk::FAMILY_MFMA_CHECKED)
+      return fail(GK_ERR_UNSUPPORTED, "the K-split kernel runs the real MFMA operator");
     if (conf->global_d_layout.eltype != GK_F32) return fail(GK_ERR_UNSUPPORTED, "the K-split kernel adds partial sums with fp32 atomics: D must be Float32");
     if ((epilogue && epilogue->kind != GK_EPILOGUE_DEFAULT) || L.args.t[gk::H_RF2SH_D].n > 0 || L.args.t[gk::H_SH2GL_D].n > 0)
       return fail(GK_ERR_UNSUPPORTED, "the K-split kernel takes no transform on D and no bias (they would apply to partial sums)");
@@ -708,7 +709,7 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
     // hide each other's latency, measured best at up to four per CU), each slice at least eight K tiles
     // long so that its prologue, epilogue and atomic adds stay a small part of it
     const int tiles = L.gx * L.gy;
-    const int kt = conf->matmul_shape.K / conf->block_shape.K;
+    const int kt = (conf->matmul_shape.K + conf->block_shape.K - 1) / conf->block_shape.K;   // bounds-checked layouts: the last tile may be partial
     int per_cu = L.info.lds_bytes > 0 ? (160 * 1024) / L.info.lds_bytes : 1;
     per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
     int slices = (per_cu * gk::kNumCUs + tiles - 1) / tiles;
@@ -716,7 +717,10 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
     gk::InstanceInfo sk_info;
     // K-split instances exist for the small tiles that skinny products run; anything else (a large
     // tile, generic A / B hooks) runs unsplit below
-    if (slices > 1 && gk::family_mfma_splitk(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
+    // the bounds-checked kernel takes its K range from the launch arguments, the aligned kernels have
+    // instances of their own for it
+    gk::FamilyFn sk_fn = L.key.family == gk::FAMILY_MFMA_CHECKED ? fn : gk::family_mfma_splitk;
+    if (slices > 1 && sk_fn && sk_fn(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
       const int per = (kt + slices - 1) / slices;
       slices = (kt + per - 1) / per;
       if (L.args.c_mode != 0 && c == d && L.args.ldc == L.args.ldd && conf->global_c_layout.eltype == GK_F32 &&
@@ -725,18 +729,18 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
         // slice adds its partial sum and one launch does it all
         gk::GemmArgs all = L.args;
         all.k_begin = 0; all.k_steps = per; all.atomic_d = 1; all.c_mode = 0;
-        gk::family_mfma_splitk(L.key, all, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)slices), (hipStream_t)stream, 1, &sk_info, &err);
+        sk_fn(L.key, all, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)slices), (hipStream_t)stream, 1, &sk_info, &err);
         if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
         return GK_OK;
       }
       gk::GemmArgs first = L.args;       // slice 0: reads C, writes D
       first.k_begin = 0; first.k_steps = per; first.atomic_d = 0;
-      gk::family_mfma_splitk(L.key, first, dim3((unsigned)L.gx, (unsigned)L.gy, 1), (hipStream_t)stream, 1, &sk_info, &err);
+      sk_fn(L.key, first, dim3((unsigned)L.gx, (unsigned)L.gy, 1), (hipStream_t)stream, 1, &sk_info, &err);
       if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
       gk::GemmArgs rest = L.args;        // slices 1..: start from zero, add into D; stream order puts them after slice 0
       rest.k_begin = per; rest.k_steps = per; rest.atomic_d = 1; rest.c_mode = 0;
       rest.t[gk::H_GL2SH_C].n = 0; rest.t[gk::H_SH2RF_C].n = 0;      // the hooks of C belong to slice 0 alone
-      gk::family_mfma_splitk(L.key, rest, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)(slices - 1)), (hipStream_t)stream, 1, &sk_info, &err);
+      sk_fn(L.key, rest, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)(slices - 1)), (hipStream_t)stream, 1, &sk_info, &err);
       if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
       return GK_OK;
     }

@@ -3,7 +3,9 @@
 // (src/kernel.jl:10-129, src/layout.jl:117-184).  Elements are loaded one by one (out-of-range
 // reads give 0), written to LDS in the K-major swizzled tile layout of the fast kernel, and the
 // same fragment reader and MFMA sequence consume them; out-of-range stores are dropped.  One LDS
-// stage: load, barrier, compute, barrier.  Slow by design, like the reference's checked layouts.
+// stage; the element loads of the next four tiles are in flight (in registers) while the current
+// one is multiplied.  Scalar accesses make it several times slower than the aligned kernels, like the
+// reference's checked layouts.
 #pragma once
 #include "mfma_gemm.hpp"
 
@@ -66,29 +68,72 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
       }
 
   // element e of a tile: K-major memory walks k fastest, M-major memory walks the row fastest, so
-  // that consecutive threads touch consecutive addresses
-  auto load_tile = [&](const T* base, long long ld, bool kmajor, int R, int r0, int r_limit, int k0, char* dst, int per_thread,
-                       bool xf, const OpList& t0, const OpList& t1, int cpr_shift_rows) {
-    (void)cpr_shift_rows;
-    for (int i = 0; i < per_thread; ++i) {
-      const int e = tid + i * Cfg::THREADS;
+  // that consecutive threads touch consecutive addresses.  fetch() only issues the loads of a tile
+  // (all of them before anything waits); stash() runs the hooks and writes the tile to LDS.
+  auto coords = [&](auto kmajor_c, auto rows_c, int i, int& r, int& k) __attribute__((always_inline)) {
+    constexpr bool KMAJOR = decltype(kmajor_c)::value;
+    constexpr int R = decltype(rows_c)::value;
+    const int e = tid + i * Cfg::THREADS;
+    if (KMAJOR) { r = e / BK; k = e % BK; } else { k = e / R; r = e % R; }
+  };
+  auto fetch = [&](const T* base, long long ld, auto kmajor_c, auto rows_c, int r0, int r_limit, int k0, auto& regs) __attribute__((always_inline)) {
+    constexpr bool KMAJOR = decltype(kmajor_c)::value;
+    constexpr int PER = decltype(rows_c)::value * BK / Cfg::THREADS;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
       int r, k;
-      if (kmajor) { r = e / BK; k = e % BK; } else { k = e / R; r = e % R; }
-      T x = (T)0.0f;
+      coords(kmajor_c, rows_c, i, r, k);
       const int gr = r0 + r, gk_ = k0 + k;
-      if (!zero_ab && gr < r_limit && gk_ < args.K) x = base[kmajor ? (long long)gr * ld + gk_ : (long long)gk_ * ld + gr];
-      if (xf) {
-        float f = (float)x;
-        if (t0.n > 0) f = (float)(T)apply_list(t0, f);
-        if (t1.n > 0) f = (float)(T)apply_list(t1, f);
-        x = (T)f;
+      T x = (T)0.0f;
+      if (!zero_ab && gr < r_limit && gk_ < args.K) x = base[KMAJOR ? (long long)gr * ld + gk_ : (long long)gk_ * ld + gr];
+      regs[i] = x;
+    }
+  };
+  auto stash = [&](auto kmajor_c, auto rows_c, const auto& regs, char* dst, bool xf, auto h0_c, auto h1_c) __attribute__((always_inline)) {
+    const OpList& t0 = args.t[decltype(h0_c)::value];
+    const OpList& t1 = args.t[decltype(h1_c)::value];
+    constexpr int PER = decltype(rows_c)::value * BK / Cfg::THREADS;
+    T vals[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) vals[i] = regs[i];
+    if (xf) {
+      // each of the two hooks is evaluated in fp32 and rounded to the operand's type; the dispatch on the
+      // op runs once per list, not once per element
+      float f[PER];
+#pragma unroll
+      for (int i = 0; i < PER; ++i) f[i] = (float)vals[i];
+      if (t0.n > 0) {
+        apply_list_regs<PER>(t0, f);
+#pragma unroll
+        for (int i = 0; i < PER; ++i) f[i] = (float)(T)f[i];
       }
+      if (t1.n > 0) {
+        apply_list_regs<PER>(t1, f);
+#pragma unroll
+        for (int i = 0; i < PER; ++i) f[i] = (float)(T)f[i];
+      }
+#pragma unroll
+      for (int i = 0; i < PER; ++i) vals[i] = (T)f[i];
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      int r, k;
+      coords(kmajor_c, rows_c, i, r, k);
+      const T x = vals[i];
       constexpr int CPR = BK / 8;
       const int c = k >> 3;
       const int swz = (r / OperandGeom<64, BK, OPK_KMAJOR, false>::RP256) & (CPR - 1);
       *(T*)(dst + 16 * (r * CPR + (c ^ swz)) + (k & 7) * 2) = x;
     }
   };
+  typedef std::integral_constant<bool, Cfg::A_KMAJOR> AKM;
+  typedef std::integral_constant<bool, Cfg::B_KMAJOR> BKM;
+  typedef std::integral_constant<int, BM> RowsA;
+  typedef std::integral_constant<int, BN> RowsB;
+  // tiles in flight: a workgroup at the rim of a cut-up product runs alone on its CU and its K loop is
+  // as long as the memory latency times the number of tiles divided by this depth
+  constexpr int DEPTH = 4;
+  T ga[DEPTH][Cfg::A_PER_THREAD], gb[DEPTH][Cfg::B_PER_THREAD];
 
   typedef FragReader<BM, BK, OPK_KMAJOR, false, FM> RA;
   typedef FragReader<BN, BK, OPK_KMAJOR, false, FN> RB;
@@ -100,11 +145,32 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
   ra.set_stage(lds_base);
   rb.set_stage(lds_base + GA::BYTES);
 
-  const int KT = (args.K + BK - 1) / BK;
-  for (int kt = 0; kt < KT; ++kt) {
-    load_tile(A, args.lda, Cfg::A_KMAJOR, BM, m0, args.M, kt * BK, sa, Cfg::A_PER_THREAD, xf_a, args.t[H_GL2SH_A], args.t[H_SH2RF_A], 0);
-    load_tile(B, args.ldb, Cfg::B_KMAJOR, BN, n0, args.N, kt * BK, sb, Cfg::B_PER_THREAD, xf_b, args.t[H_GL2SH_B], args.t[H_SH2RF_B], 0);
+  // K tiles of this workgroup: all of them, or (k_steps > 0) the slice blockIdx.z of a K-split launch
+  int kt_first = 0, KT = (args.K + BK - 1) / BK;
+  if (args.k_steps > 0) {
+    kt_first = args.k_begin + (int)blockIdx.z * args.k_steps;
+    KT = KT < kt_first + args.k_steps ? KT : kt_first + args.k_steps;
+    if (kt_first >= KT) return;       // the whole workgroup leaves together, before any barrier
+  }
+  static_for<0, DEPTH>([&](auto j_c) __attribute__((always_inline)) {
+    constexpr int j = decltype(j_c)::value;
+    if (kt_first + j < KT) {
+      fetch(A, args.lda, AKM{}, RowsA{}, m0, args.M, (kt_first + j) * BK, ga[j]);
+      fetch(B, args.ldb, BKM{}, RowsB{}, n0, args.N, (kt_first + j) * BK, gb[j]);
+    }
+  });
+  for (int kt0 = kt_first; kt0 < KT; kt0 += DEPTH)
+  static_for<0, DEPTH>([&](auto j_c) __attribute__((always_inline)) {
+    constexpr int j = decltype(j_c)::value;       // register buffer of tile kt
+    const int kt = kt0 + j;
+    if (kt < KT) {
+    stash(AKM{}, RowsA{}, ga[j], sa, xf_a, std::integral_constant<int, H_GL2SH_A>{}, std::integral_constant<int, H_SH2RF_A>{});
+    stash(BKM{}, RowsB{}, gb[j], sb, xf_b, std::integral_constant<int, H_GL2SH_B>{}, std::integral_constant<int, H_SH2RF_B>{});
     __syncthreads();
+    if (kt + DEPTH < KT) {     // its buffer is free again: tile kt + DEPTH starts to travel
+      fetch(A, args.lda, AKM{}, RowsA{}, m0, args.M, (kt + DEPTH) * BK, ga[j]);
+      fetch(B, args.ldb, BKM{}, RowsB{}, n0, args.N, (kt + DEPTH) * BK, gb[j]);
+    }
     static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
       constexpr int ks = decltype(ks_c)::value;
       typename RA::Raw fa[FM];
@@ -122,7 +188,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
         for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = Mfma<T>::run(vb[fj], va[fi], acc[fi][fj]);
     });
     __syncthreads();
-  }
+    }
+  });
 
 #pragma unroll
   for (int fi = 0; fi < FM; ++fi)
@@ -135,7 +202,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
         if (args.epi_kind == 1) x = x + args.bias[cc < args.N ? cc : 0];
         else if (args.epi_kind == 2) x = x + args.bias[r < args.M ? r : 0];
         x = apply_list(args.t[H_SH2GL_D], x);
-        if (r < args.M && cc < args.N) store_cd(args.d, args.d_dtype, r + (long long)cc * args.ldd, x);
+        if (r < args.M && cc < args.N) {
+          // partial result of a K slice: fp32 atomic add (the host only asks for it with a Float32 D and no hook on D)
+          if (args.atomic_d) atomicAdd((float*)args.d + r + (long long)cc * args.ldd, x);
+          else store_cd(args.d, args.d_dtype, r + (long long)cc * args.ldd, x);
+        }
       }
 }
 

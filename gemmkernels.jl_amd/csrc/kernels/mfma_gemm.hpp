@@ -4,8 +4,9 @@
 // Operator.WMMAOp (src/operator.jl:163-245) and the UnsafeAligned{Col,Row}Major layouts
 // (src/layout.jl:192-219, 244-270), re-designed for gfx950:
 //
-//  * one v_mfma_f32_32x32x16 per 32x32x16 product, 64-lane waves, accumulators stay in
-//    registers from the C load to the D store (the reference round-trips them through LDS);
+//  * one v_mfma_f32_16x16x32 per 16x16x32 product (v_mfma_f32_32x32x16 where MI = 32 is asked for),
+//    64-lane waves, accumulators stay in registers from the C load to the D store (the reference
+//    round-trips them through LDS);
 //  * A and B tiles travel global -> LDS with global_load_lds_dwordx4 (no register staging),
 //    STAGES tiles deep, one s_barrier per K step;
 //  * LDS tiles are XOR-swizzled in 16-byte chunks so that both the DMA writes and the fragment
@@ -13,8 +14,9 @@
 //  * operands whose K index is contiguous in memory ("K-major": A of a 'T' GEMM, B of an 'N'
 //    GEMM) are read with ds_read_b128, the others ("M-major") with the transposing
 //    ds_read_b64_tr_b16, so all four transposes run at the same speed;
-//  * the MFMA is issued with swapped operands (B fragment first) so that a lane owns 32
-//    consecutive rows m of D and a half-wave writes whole 128-byte lines of column-major D.
+//  * the MFMA is issued with swapped operands (B fragment first) so that 16 (32) consecutive lanes
+//    own consecutive rows m of D and write 64 (128) contiguous bytes of a column of D; the blocks
+//    of a wave tile are walked so that the two halves of a 128-byte line follow each other.
 #pragma once
 #include "common.hpp"
 #include <type_traits>
@@ -114,8 +116,9 @@ __device__ __forceinline__ void wait_lgkmcnt() {
   asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N < 15 ? N : 15) : "memory");
 }
 
-// Fragment of 32 MFMA rows x 16 k-values: lane l receives the 8 k-values 8*(l/32)..+7 of row
-// row0 + l%32, which is the operand layout of v_mfma_f32_32x32x16.
+// Fragment of MI MFMA rows x 512/MI k-values: lane l receives the 8 k-values 8*(l/MI)..+7 of row
+// row0 + l%MI, which is the operand layout of v_mfma_f32_16x16x32 (MI = 16) and of
+// v_mfma_f32_32x32x16 (MI = 32).
 //
 // The reads are issued from inline assembly: the compiler would otherwise make every
 // transposing LDS read wait for all outstanding global->LDS DMA (it cannot tell the stages
@@ -380,7 +383,7 @@ struct MfmaGemmConfig {
   static constexpr int DMA_B = (GB::NDMA + NWAVES - 1) / NWAVES;
   static constexpr int DMA_PER_TILE = DMA_A + DMA_B;
   static_assert(GA::NDMA % NWAVES == 0 && GB::NDMA % NWAVES == 0, "every wave issues the same number of DMA instructions");
-  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tiles are multiples of 32 x 32 (two 16-row blocks share a 64-byte group of an M-major tile)");
   static_assert(BK_ % KSTEP_K == 0, "BLOCK_K is a whole number of MFMA k-steps");
   static_assert(STAGES >= 2, "at least two LDS stages");
   static_assert((STAGES - 2) * DMA_PER_TILE <= 63, "vmcnt is a 6-bit counter");

@@ -163,8 +163,8 @@ _GETT_TILES = [(256, 256, 64), (128, 128, 64), (64, 64, 32)]
 
 
 def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: bool = False, planar: bool = False) -> NT:
-    """MI355X block shape: the largest tile of the table that divides the problem and still gives
-    every one of the 256 CUs a workgroup; the smallest dividing tile when none does."""
+    """MI355X block shape: of the tiles of the table that divide the problem, the one with the shortest
+    estimated launch (tiles per CU times the cost of a tile)."""
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         return NT(M=64, N=64, K=32)
     M, N, K = gemm_shape["M"], gemm_shape["N"], gemm_shape["K"]
@@ -184,12 +184,19 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
         fitting = [t for t in fitting if t in _GETT_TILES]
     if not fitting:
         return NT(M=64, N=64, K=32)
-    for t in fitting:
-        if -(-M // t[0]) * -(-N // t[1]) >= NUM_CUS:
-            return NT(M=t[0], N=t[1], K=t[2])
-    # no tile fills the chip: the smallest tile, with four waves per workgroup when K allows
-    last = (64, 64, 64) if (64, 64, 64) in fitting else fitting[-1]
-    return NT(M=last[0], N=last[1], K=last[2])
+    # time of the launch in units of "one CU multiplying at the rate of the 256 x 256 x 64 tile": every CU
+    # works through ceil(tiles / 256) tiles one after the other, a tile costs its area over the measured
+    # relative rate of its kernel (ties go to the tile listed first)
+    def cost(t):
+        tiles = -(-M // t[0]) * -(-N // t[1])
+        return -(-tiles // NUM_CUS) * t[0] * t[1] / _MFMA_TILE_RATE.get(t, 0.5)
+    best = min(fitting, key=lambda t: (cost(t), fitting.index(t)))
+    return NT(M=best[0], N=best[1], K=best[2])
+
+
+# throughput of a CU running each tile, relative to 256 x 256 x 64 (from 4096 x 4096 x 2048 and 4032^3 timings)
+_MFMA_TILE_RATE = {(256, 256, 64): 1.0, (256, 256, 32): 0.95, (256, 128, 64): 0.81, (128, 256, 64): 0.82,
+                   (128, 128, 32): 0.86, (128, 128, 64): 0.86, (64, 64, 64): 0.47, (64, 64, 32): 0.30}
 
 
 # complex / dual tiles (complex elements) -> waves

@@ -168,7 +168,7 @@ class Plan:
     other means while it is in use.  For loops that launch the same GEMM many times, where the
     microseconds a general ``matmul`` call spends on lowering would rival the kernel itself."""
 
-    __slots__ = ("_fn", "_conf", "_trans", "_epi", "_args", "_keep", "d")
+    __slots__ = ("_fn", "_conf", "_trans", "_epi", "_args", "_keep", "d", "kernel_names")
 
     def __init__(self, conf: Config, a, b, c, d, transforms: dict, epilogue, kernel, specialized=None):
         if specialized is None and any(t.expr is not None for t in transforms.values()):
@@ -192,6 +192,7 @@ class Plan:
                           ctypes.byref(self._trans) if self._trans is not None else None, epi_ref, kernel.code)
         self._keep = (a, b, c, d, epilogue, specialized)
         self.d = d
+        self.kernel_names = ()      # filled in by the BLAS-level front end
 
     def __call__(self, stream=None):
         rc = self._fn(*self._args, _current_stream() if stream is None else int(stream))
@@ -380,9 +381,8 @@ def _round_to(dtype: DType, x: float) -> float:
     return float(x)
 
 
-def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None) -> Plan:
-    """The launch ``matmatmul_`` would make, as a ``Plan`` to call any number of times."""
-    tA, tB = transA == 'T', transB == 'T'
+def _single_plan(C, tA: bool, tB: bool, A, B, alpha, beta, wmma=None) -> Plan:
+    """One launch for C = alpha * op(A) * op(B) + beta * C: the configuration ``create_config`` picks."""
     conf, compute_type, kernel = get_config(
         from_torch(A.dtype), tuple(A.shape), tuple(A.stride()), tA,
         from_torch(B.dtype), tuple(B.shape), tuple(B.stride()), tB,
@@ -395,15 +395,131 @@ def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None)
             # transform parameters travel as binary32; Float64 (or large integer) factors that do not
             # fit would silently change the result
             raise ConfigError(f"{name} = {value!r} is not representable in binary32, the parameter type of the transform hooks")
+    # beta = 0 has already turned C into a Zero layout: nothing is loaded, nothing to scale
     ta = Transform.Elementwise(ops=[] if alpha_c == 1.0 else [(Transform.SCALE, alpha_c, 0.0)])
-    tc = Transform.Elementwise(ops=[] if beta_c == 1.0 else [(Transform.SCALE, beta_c, 0.0)])
-    if (kernel is Kernel.matmul_pipelined and conf.operator.kind == Operator.MFMA and from_torch(C.dtype) == Float32):
-        # few output tiles and a long K loop (skinny products): cut K into slices so that every CU gets work
+    tc = Transform.Elementwise(ops=[] if beta_c == 1.0 or beta == 0 else [(Transform.SCALE, beta_c, 0.0)])
+    if conf.operator.kind == Operator.MFMA and from_torch(C.dtype) == Float32:
+        # few output tiles and a long K loop (skinny products, the rims of a cut-up product): cut K into
+        # slices so that every CU gets work
         bs, ms = conf.block_shape, conf.matmul_shape
         tiles = -(-ms.M // bs.M) * -(-ms.N // bs.N)
-        if tiles <= 128 and ms.K // bs.K >= 4:
+        if kernel is Kernel.matmul_pipelined and tiles <= 128 and ms.K // bs.K >= 4:
             kernel = Kernel.matmul_split_k
-    return plan(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)
+        elif kernel is Kernel.matmul_singlestage and tiles <= 128 and ms.K // bs.K >= 16:
+            kernel = Kernel.matmul_split_k          # the bounds-checked kernel: slices of at least eight K tiles
+    p = plan(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)
+    p.kernel_names = (kernel_name(conf, kernel, dict(transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc)),)
+    return p
+
+
+class PlanSequence:
+    """Several launches on one stream that together compute one product (``matmatmul_plan`` for sizes
+    that are not whole tiles).  Called like a ``Plan``."""
+
+    def __init__(self, plans, d):
+        self.plans = list(plans)
+        self.d = d
+        self.kernel_names = tuple(n for p in self.plans for n in p.kernel_names)
+
+    def __call__(self, stream=None):
+        for p in self.plans:
+            p(stream)
+        return self.d
+
+
+_REGION_TILES = (256, 128, 64)
+
+
+def output_regions(M: int, N: int):
+    """Cuts an M x N output into disjoint rectangles ``(m0, m, n0, n, whole_tiles)``.  The first is the
+    largest top-left block made of 256 x 256 tiles; the strip to its right (all rows) and the strip below
+    it are cut the same way with 128 and then 64; what is left over, or narrower than 64, is marked
+    ``whole_tiles = False`` and goes to the bounds-checked kernel.  Offsets of rectangles with whole tiles
+    are multiples of 64 elements, so 16-byte aligned columns stay 16-byte aligned."""
+    out = []
+
+    def cut(m0, m, n0, n, level):
+        if m <= 0 or n <= 0:
+            return
+        while level < len(_REGION_TILES) and (m < _REGION_TILES[level] or n < _REGION_TILES[level]):
+            level += 1
+        if level == len(_REGION_TILES):
+            out.append((m0, m, n0, n, False))
+            return
+        t = _REGION_TILES[level]
+        mi, ni = m // t * t, n // t * t
+        out.append((m0, mi, n0, ni, True))
+        cut(m0, m, n0 + ni, n - ni, level + 1)       # right of the block: every row
+        cut(m0 + mi, m - mi, n0, ni, level + 1)      # below the block
+    cut(0, M, 0, N, 0)
+    return out
+
+
+def _estimate_us(operator, M: int, N: int, K: int, whole_tiles: bool) -> float:
+    """Rough duration of one launch, from two measured rates: a CU multiplies a 256 x 256 x 64 tile over
+    K = 4096 in 108 us (other tiles by ``config._MFMA_TILE_RATE``), and the bounds-checked kernel spends
+    0.53 us per CU on a 64 x 64 x 32 step; a launch costs a few microseconds whatever it does, a K-split
+    rim two launches and the atomic adds."""
+    from .config import _MFMA_TILE_RATE, NUM_CUS, default_block_shape
+    if whole_tiles:
+        bs = default_block_shape(operator, NT(M=M, N=N, K=K))
+        tiles = -(-M // bs.M) * -(-N // bs.N)
+        per_cu = -(-tiles // NUM_CUS) * bs.M * bs.N / _MFMA_TILE_RATE.get((bs.M, bs.N, bs.K), 0.5)
+        return per_cu * K / (65536.0 * 4096.0) * 108.0 + 6.0
+    steps = -(-M // 64) * -(-N // 64) * -(-K // 32)
+    return max(-(-steps // NUM_CUS), 8) * 0.53 + 25.0
+
+
+def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None, regions=None):
+    """The launches ``matmatmul_`` would make, as a ``Plan`` (or a ``PlanSequence``) to call any number of
+    times.
+
+    Sizes that are whole tiles, and everything the matrix cores do not run, take one launch of the
+    configuration ``create_config`` picks (reference src/matmul.jl:185-204).  A large 16-bit product whose
+    sizes are *not* whole tiles would run entirely on the bounds-checked kernel, at a tenth of the speed
+    (the reference has the same cliff, src/matmul.jl:121-156 and src/layout.jl:117-184).  When the columns
+    of A, B and C are 16-byte aligned it is cut up instead: ``output_regions`` of whole tiles run on the
+    fast kernels over the first K - K % 32 values of k, the ragged rims on the bounds-checked kernel (in
+    slices of K: a rim has few tiles), and one more bounds-checked launch adds the last K % 32 values of k
+    to all of C.  Every element of C is
+    still computed as alpha * op(A) * op(B) + beta * C with alpha applied to A in the compute type; only
+    the order of the fp32 additions along k differs from the single launch.  ``regions`` forces the
+    cutting on (True) or off (False); by default it is used when a rough estimate (``_estimate_us``) puts
+    the launches together clearly below the single one (from about 3000^3 on)."""
+    tA, tB = transA == 'T', transB == 'T'
+    single = _single_plan(C, tA, tB, A, B, alpha, beta, wmma)
+    conf = get_config(from_torch(A.dtype), tuple(A.shape), tuple(A.stride()), tA,
+                      from_torch(B.dtype), tuple(B.shape), tuple(B.stride()), tB,
+                      from_torch(C.dtype), tuple(C.shape), tuple(C.stride()),
+                      type(alpha), alpha == 0, type(beta), beta == 0, wmma)[0]
+    ms = conf.matmul_shape
+    M, N, K = ms.M, ms.N, ms.K
+    checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR)
+                  for l in (conf.global_a_layout, conf.global_b_layout, conf.global_c_layout, conf.global_d_layout))
+    aligned_columns = all((int(x.stride()[1]) * x.element_size()) % 16 == 0 and x.data_ptr() % 16 == 0 for x in (A, B, C))
+    Kw = K // 32 * 32        # every tile table has tiles 32 deep
+    if (regions is False or conf.operator.kind != Operator.MFMA or not aligned_columns or alpha == 0
+            or Kw == 0 or min(M, N) < _REGION_TILES[-1]):
+        return single
+    cut = output_regions(M, N)
+    if len(cut) == 1 and Kw == K:
+        return single           # whole tiles already
+    if regions is None:
+        # worth it when the launches together are clearly shorter than the one launch
+        together = sum(_estimate_us(conf.operator, m, n, Kw, whole) for _, m, _, n, whole in cut)
+        together += _estimate_us(conf.operator, M, N, K - Kw, False) if Kw < K else 0.0
+        if together > 0.8 * _estimate_us(conf.operator, M, N, K, not checked):
+            return single
+
+    def sub(X, trans, r0, r, c0, c):          # rows r0.., columns c0.. of op(X)
+        return X[c0:c0 + c, r0:r0 + r] if trans else X[r0:r0 + r, c0:c0 + c]
+    plans = []
+    for m0, m, n0, n, _ in cut:
+        plans.append(_single_plan(C[m0:m0 + m, n0:n0 + n], tA, tB, sub(A, tA, m0, m, 0, Kw), sub(B, tB, 0, Kw, n0, n),
+                                  alpha, beta, wmma))
+    if Kw < K:
+        plans.append(_single_plan(C, tA, tB, sub(A, tA, 0, M, Kw, K - Kw), sub(B, tB, Kw, K - Kw, 0, N), alpha, 1.0, wmma))
+    return PlanSequence(plans, C)
 
 
 def matmatmul_(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None):

@@ -109,3 +109,40 @@ def test_config1_benchmark_workload(gpu):
     assert oracle.rel_frobenius(d, oracle.gemm_f64(h["a"], h["b"], None)) <= 1e-5
     conf = run.conf
     assert np.array_equal(d, helpers.run_oracle(conf, h["a"], h["b"], None, (256, 256)))
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims", [(1000, 1000, 1000), (840, 328, 200), (328, 1096, 136), (264, 264, 64)])
+def test_products_cut_into_regions_of_whole_tiles(gpu, dims, ta, tb):
+    """Sizes that are not whole tiles with 16-byte aligned columns: blocks of whole tiles on the fast
+    kernels, rims and the tail of K on the bounds-checked kernel (matmatmul_plan).  Same tolerance as
+    the single launch, and the same kernels must not be all bounds-checked ones."""
+    from gemmkernels.matmul import matmatmul_plan, PlanSequence, output_regions
+    M, N, K = dims
+    a, b, c = operands(M, N, K, ta == "T", tb == "T", np.float16, 500)
+    alpha, beta = 0.75, -1.5
+    A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
+    p = matmatmul_plan(C, ta, tb, A, B, alpha, beta, regions=True)
+    assert isinstance(p, PlanSequence)
+    assert len(p.plans) == len(output_regions(M, N)) + (1 if K % 32 else 0)
+    assert any("checked" not in n for n in p.kernel_names), p.kernel_names
+    print("case", dims, ta, tb, p.kernel_names, flush=True)
+    p()
+    torch.cuda.synchronize()
+    ref = oracle.gemm_f64(a, b, c, alpha, beta, ta == "T", tb == "T")
+    assert oracle.rel_frobenius(gk.to_numpy(C), ref) <= 1e-3
+    # the single bounds-checked launch gives the same values up to the order of the fp32 sums
+    C1 = gk.colmajor(c)
+    matmatmul_plan(C1, ta, tb, A, B, alpha, beta, regions=False)()
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(gk.to_numpy(C), gk.to_numpy(C1).astype(np.float64)) <= 1e-5
+
+
+def test_region_cutting_is_left_alone_where_it_cannot_help(gpu):
+    from gemmkernels.matmul import matmatmul_plan, PlanSequence
+    # whole tiles: one fast launch; columns that are not 16-byte aligned: one bounds-checked launch; FP32: vector ALUs
+    for dims, dtype in (((1024, 1024, 1024), np.float16), ((1001, 1001, 1001), np.float16), ((1000, 1000, 1000), np.float32)):
+        M, N, K = dims
+        a, b, c = operands(M, N, K, False, False, dtype, 600)
+        p = matmatmul_plan(gk.colmajor(c), "N", "N", gk.colmajor(a), gk.colmajor(b), 1.0, 1.0, regions=True)
+        assert not isinstance(p, PlanSequence), dims

@@ -261,3 +261,22 @@ def test_complex_layout_rules_of_the_library():
         assert ei.value.status in (_lib.GK_ERR_UNSUPPORTED, _lib.GK_ERR_BLOCK_SHAPE), ei.value.message
     with pytest.raises(ConfigError):                                                            # K not a multiple of the tile
         configs.complex_planar_config(M, N, 48)
+
+
+def test_output_regions_cover_the_output_once_and_fast_regions_are_whole_tiles():
+    """The cutting used by the BLAS-level front end for sizes that are not whole tiles."""
+    from gemmkernels.matmul import output_regions
+    import numpy as np
+    for (M, N) in [(4000, 4000), (4097, 4100), (1000, 1000), (64, 64), (63, 500), (500, 63), (130, 70), (256, 257), (8200, 300), (1, 1)]:
+        cover = np.zeros((M, N), dtype=np.int32)
+        regions = output_regions(M, N)
+        for m0, m, n0, n, whole in regions:
+            assert m > 0 and n > 0 and m0 + m <= M and n0 + n <= N
+            cover[m0:m0 + m, n0:n0 + n] += 1
+            if whole:
+                assert m % 64 == 0 and n % 64 == 0 and m0 % 64 == 0 and n0 % 64 == 0
+        assert (cover == 1).all(), (M, N)
+        # what the bounds-checked kernel gets is a rim less than 64 wide (or a problem smaller than a tile)
+        slow = sum(m * n for _, m, n0, n, whole in regions if not whole)
+        assert slow <= 64 * (M + N), (M, N, slow)
+    assert output_regions(4000, 4000)[0] == (0, 3840, 0, 3840, True)
