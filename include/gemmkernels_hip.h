@@ -156,8 +156,9 @@ typedef struct gk_config {
  * into slices that run as separate workgroups; the first slice writes D = T_c(C) + its partial sum in
  * a launch of its own, the others add theirs with fp32 atomics in a second launch (when d == c and C
  * has no transform, D holds its starting value already and all slices add in one launch).  Real MFMA
- * operator, fp32 D, no transform on D and no bias; the order of the atomic adds, and so the last
- * bits of D, can differ between runs.  With enough tiles it is the pipelined kernel. */
+ * operator (aligned or bounds-checked layouts), fp32 D, no transform on D and no bias; the order of
+ * the atomic adds, and so the last bits of D, can differ between runs.  With enough tiles it is the
+ * pipelined (bounds-checked layouts: the single-stage) kernel. */
 typedef enum gk_kernel_kind {
   GK_KERNEL_SINGLESTAGE = 0,
   GK_KERNEL_PIPELINED = 1,
