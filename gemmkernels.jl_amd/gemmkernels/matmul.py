@@ -430,6 +430,22 @@ class PlanSequence:
 _REGION_TILES = (256, 128, 64)
 
 
+def overlapping_regions(M: int, N: int):
+    """For a product that does not read C (beta = 0): whole tiles only.  The part of the output whose
+    sizes are multiples of 64 is cut like ``output_regions``; the ragged right and bottom edges are covered
+    by 64-wide windows that end at the edge and reach back over cells another launch has already written
+    (which then get the same value, up to the order of the sums, a second time).  M, N >= 64."""
+    M64, N64 = M // 64 * 64, N // 64 * 64
+    out = output_regions(M64, N64)
+    if N > N64:
+        out.append((0, M64, N - 64, 64, True))
+    if M > M64:
+        out.append((M - 64, 64, 0, N64, True))
+    if N > N64 and M > M64:
+        out.append((M - 64, 64, N - 64, 64, True))
+    return out
+
+
 def output_regions(M: int, N: int):
     """Cuts an M x N output into disjoint rectangles ``(m0, m, n0, n, whole_tiles)``.  The first is the
     largest top-left block made of 256 x 256 tiles; the strip to its right (all rows) and the strip below
@@ -481,7 +497,8 @@ def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None,
     of A, B and C are 16-byte aligned it is cut up instead: ``output_regions`` of whole tiles run on the
     fast kernels over the first K - K % 32 values of k, the ragged rims on the bounds-checked kernel (in
     slices of K: a rim has few tiles), and one more bounds-checked launch adds the last K % 32 values of k
-    to all of C.  Every element of C is
+    to all of C.  With beta = 0 and M, N multiples of 8 there are no rims: ``overlapping_regions`` covers the
+    edges with whole tiles that reach back over finished cells.  Every element of C is
     still computed as alpha * op(A) * op(B) + beta * C with alpha applied to A in the compute type; only
     the order of the fp32 additions along k differs from the single launch.  ``regions`` forces the
     cutting on (True) or off (False); by default it is used when a rough estimate (``_estimate_us``) puts
@@ -501,7 +518,11 @@ def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None,
     if (regions is False or conf.operator.kind != Operator.MFMA or not aligned_columns or alpha == 0
             or Kw == 0 or min(M, N) < _REGION_TILES[-1]):
         return single
-    cut = output_regions(M, N)
+    # windows that overlap need rows M - 64 and columns N - 64 to start on 16-byte boundaries in A, B and C
+    if beta == 0 and M % 8 == 0 and N % 8 == 0:
+        cut = overlapping_regions(M, N)
+    else:
+        cut = output_regions(M, N)
     if len(cut) == 1 and Kw == K:
         return single           # whole tiles already
     if regions is None:
