@@ -165,3 +165,28 @@ def test_products_that_do_not_read_c_need_no_rims(gpu, dims, ta, tb):
     torch.cuda.synchronize()
     ref = oracle.gemm_f64(a, b, None, 1.25, 0.0, ta == "T", tb == "T")
     assert oracle.rel_frobenius(gk.to_numpy(C), ref) <= 1e-3
+
+
+@pytest.mark.parametrize("beta", [0.0, 0.25])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_cut_up_products_with_16_bit_c(gpu, beta, dtype):
+    """FP16 A, B and C, and BF16 A, B with Float32 C, through the region cutting: rims (beta != 0) and
+    overlapping windows (beta = 0)."""
+    from gemmkernels.matmul import matmatmul_plan, PlanSequence
+    M, N, K = 1000, 200, 104
+    a, b, c = operands(M, N, K, False, True, np.float16, 800)
+    if dtype == "f16":
+        A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c.astype(np.float16))
+        c_in = c.astype(np.float16).astype(np.float64)
+    else:
+        A, B = gk.colmajor(a, dtype=torch.bfloat16), gk.colmajor(b, dtype=torch.bfloat16)
+        C = gk.colmajor(c)                                                        # BF16 inputs pair with a Float32 C
+        a, b = A.float().cpu().numpy(), B.float().cpu().numpy()                  # the values after rounding to BF16
+        c_in = c.astype(np.float64)
+    p = matmatmul_plan(C, "N", "T", A, B, 0.5, beta, regions=True)
+    assert isinstance(p, PlanSequence), type(p)
+    p()
+    torch.cuda.synchronize()
+    out = C.float().cpu().numpy()
+    ref = 0.5 * a.astype(np.float64) @ b.astype(np.float64).T + beta * c_in
+    assert oracle.rel_frobenius(out, ref) <= 2e-3       # FP16 C: one rounding of D to 11 bits; BF16: alpha on A in BF16
