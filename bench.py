@@ -304,6 +304,26 @@ def main():
             del r, w, in_place
         except Exception as e:
             extras.setdefault("skinny", {})["in_place"] = {"error": f"{type(e).__name__}: {e}"}
+        # the BLAS-level front end on sizes that are not whole tiles: mul!(C, A, B) with M = N = K = 4000
+        # (whole-tile regions on the aligned kernels instead of one launch of the bounds-checked kernel)
+        try:
+            from gemmkernels import rng
+            from gemmkernels.matmul import matmatmul_plan
+            n = 4000
+            a4 = gk.colmajor(rng.matrix("upm1_f16", 9001, (n, n)))
+            b4 = gk.colmajor(rng.matrix("upm1_f16", 9002, (n, n)))
+            c4 = gk.colmajor_empty((n, n), torch.float32)
+            cut = matmatmul_plan(c4, "N", "N", a4, b4, 1.0, 0.0)
+            u, _ = time_launches(cut, 50, 10, 0.15)
+            one = matmatmul_plan(c4, "N", "N", a4, b4, 1.0, 0.0, regions=False)
+            u1, _ = time_launches(one, 20, 5, 0.15)
+            extras["mul! 4000^3 (not whole tiles)"] = {"us": round(u, 2), "TFLOP/s": round(2.0 * n ** 3 / u / 1e6, 2), "launches": len(getattr(cut, "plans", [cut])),
+                                                       "kernels": sorted(set(cut.kernel_names)),
+                                                       "single_bounds_checked_launch_us": round(u1, 2)}
+            del a4, b4, c4, cut, one
+            torch.cuda.empty_cache()
+        except Exception as e:
+            extras["mul! 4000^3 (not whole tiles)"] = {"error": f"{type(e).__name__}: {e}"}
         # the vendor library on the headline shape, for orientation only: FP16 in, FP16 out, no C read
         # (torch.mm -> hipBLASLt), so it moves 96 MiB less per launch than config 2 does
         try:
