@@ -113,7 +113,7 @@ def test_all_eight_hooks(gpu, ta, tb):
 
 ALL_TILES = [((256, 256, 64), (2, 4)), ((256, 256, 32), (2, 4)), ((256, 256, 32), (4, 2)),
              ((256, 128, 64), (2, 2)), ((128, 256, 64), (2, 2)), ((128, 128, 64), (2, 2)), ((128, 128, 64), (4, 2)), ((128, 128, 32), (2, 2)),
-             ((64, 64, 64), (2, 2)), ((64, 64, 32), (1, 1))]
+             ((64, 64, 64), (2, 2)), ((64, 64, 32), (1, 1)), ((64, 64, 32), (2, 2))]
 
 
 @pytest.mark.parametrize("block,waves", ALL_TILES)

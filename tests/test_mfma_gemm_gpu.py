@@ -23,6 +23,7 @@ TILES = [  # block shape, (waves_m, waves_n)
     ((128, 128, 32), (2, 2)),
     ((64, 64, 64), (2, 2)),
     ((64, 64, 32), (1, 1)),
+    ((64, 64, 32), (2, 2)),
 ]
 
 
