@@ -89,6 +89,34 @@ bool transforms_present(const gk_transforms* t) {
   return false;
 }
 
+// Bounds-checked layouts (Layout.ColMajor / RowMajor, reference src/layout.jl:117-184) promise nothing about
+// size or alignment.  When a product on them happens to have 16-byte aligned columns of A and B, a K that is
+// a whole number of tiles, and M (N) a multiple of 8 where that index is the contiguous one of A (B), the
+// aligned kernel runs it: the tiles that stick out over M or N clamp their loads and mask their C loads and
+// D stores.  Decided from the configuration (a leading dimension of 0 stands for a dense operand); the
+// launcher falls back to the bounds-checked kernel when the pointers themselves turn out misaligned.
+thread_local bool t_allow_ragged_fast = true;
+
+bool ragged_fast_path(const gk_config* c) {
+  if (!t_allow_ragged_fast || c->op.kind != GK_OP_MFMA) return false;
+  const gk_layout& la = c->global_a_layout; const gk_layout& lb = c->global_b_layout;
+  const gk_layout& lc = c->global_c_layout; const gk_layout& ld = c->global_d_layout;
+  auto plain = [](int k) { return k == GK_LAYOUT_COL_MAJOR || k == GK_LAYOUT_ROW_MAJOR || k == GK_LAYOUT_ALIGNED_COL_MAJOR || k == GK_LAYOUT_ALIGNED_ROW_MAJOR; };
+  if (!plain(la.kind) || !plain(lb.kind)) return false;
+  if (ld.kind != GK_LAYOUT_COL_MAJOR && ld.kind != GK_LAYOUT_ALIGNED_COL_MAJOR) return false;
+  if (lc.kind != GK_LAYOUT_ZERO && lc.kind != GK_LAYOUT_COL_MAJOR && lc.kind != GK_LAYOUT_ALIGNED_COL_MAJOR) return false;
+  if (!(is_checked_layout(la.kind) || is_checked_layout(lb.kind) || is_checked_layout(lc.kind) || is_checked_layout(ld.kind))) return false;
+  if ((la.eltype != GK_F16 && la.eltype != GK_BF16) || lb.eltype != la.eltype) return false;
+  const long long M = c->matmul_shape.M, N = c->matmul_shape.N, K = c->matmul_shape.K;
+  if (c->block_shape.K <= 0 || K % c->block_shape.K != 0) return false;
+  const bool a_row = is_row_major(la.kind), b_row = is_row_major(lb.kind);
+  const long long lda = la.ld > 0 ? la.ld : (a_row ? K : M), ldb = lb.ld > 0 ? lb.ld : (b_row ? N : K);
+  if ((lda * 2) % 16 != 0 || (ldb * 2) % 16 != 0) return false;
+  if (!a_row && M % 8 != 0) return false;      // A stored M x K: 16-byte chunks run along m
+  if (b_row && N % 8 != 0) return false;       // B stored N x K: 16-byte chunks run along n
+  return true;
+}
+
 // Builds the run-time key of the kernel instance for a configuration.
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key) {
   memset(key, 0, sizeof(*key));
@@ -100,7 +128,7 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
     case GK_OP_MFMA:
       if (ak == GK_LAYOUT_DIAGONAL) key->family = gk::FAMILY_DIAGONAL;
       else if (any_gett) key->family = gk::FAMILY_GETT;
-      else if (any_checked) key->family = gk::FAMILY_MFMA_CHECKED;
+      else if (any_checked && !ragged_fast_path(c)) key->family = gk::FAMILY_MFMA_CHECKED;
       else key->family = gk::FAMILY_MFMA;
       break;
     case GK_OP_FPU:
@@ -264,6 +292,14 @@ int find_instance(const gk_config* c, const gk_transforms* t, const gk_epilogue*
   gk::GemmArgs dummy;
   memset(&dummy, 0, sizeof(dummy));
   hipError_t err = hipSuccess;
+  if (key->family == gk::FAMILY_MFMA && t_allow_ragged_fast && ragged_fast_path(c) && (!fn || !fn(*key, dummy, dim3(1), nullptr, 0, info, &err))) {
+    // no aligned instance of this tile: the bounds-checked kernel after all
+    t_allow_ragged_fast = false;
+    rc = make_key(c, t, e, key);
+    t_allow_ragged_fast = true;
+    if (rc != GK_OK) return rc;
+    fn = family_fn(*key);
+  }
   if (!fn || !fn(*key, dummy, dim3(1), nullptr, 0, info, &err)) {
     return fail(GK_ERR_UNSUPPORTED,
                 "no compiled kernel instance for operator %d, block (%d, %d, %d), warps %d x %d, A/B layouts %d/%d, eltype %d",
@@ -628,6 +664,18 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
   gk::InstanceInfo& info = out->info;
   int rc = validate_config(conf, kernel, transforms, epilogue, &key, &info, custom);
   if (rc != GK_OK) return rc;
+  out->ragged = false;
+  if (key.family == gk::FAMILY_MFMA && ragged_fast_path(conf)) {
+    if ((((uintptr_t)a | (uintptr_t)b) & 15u) != 0) {
+      // bounds-checked layouts with misaligned operands: the kernel that takes anything
+      t_allow_ragged_fast = false;
+      rc = validate_config(conf, kernel, transforms, epilogue, &key, &info, custom);
+      t_allow_ragged_fast = true;
+      if (rc != GK_OK) return rc;
+    } else {
+      out->ragged = (conf->matmul_shape.M % conf->block_shape.M) != 0 || (conf->matmul_shape.N % conf->block_shape.N) != 0;
+    }
+  }
 
   const bool a_zero = conf->global_a_layout.kind == GK_LAYOUT_ZERO, b_zero = conf->global_b_layout.kind == GK_LAYOUT_ZERO;
   if ((!a_zero && !a) || (!b_zero && !b) || !d) return fail(GK_ERR_INVALID_ARGUMENT, "a, b and d must not be NULL");
@@ -720,7 +768,8 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
     // the bounds-checked kernel takes its K range from the launch arguments, the aligned kernels have
     // instances of their own for it
     gk::FamilyFn sk_fn = L.key.family == gk::FAMILY_MFMA_CHECKED ? fn : gk::family_mfma_splitk;
-    if (slices > 1 && sk_fn && sk_fn(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
+    // (the K-split instances of the aligned kernel have no masks for tiles over the edge)
+    if (slices > 1 && !L.ragged && sk_fn && sk_fn(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
       const int per = (kt + slices - 1) / slices;
       slices = (kt + per - 1) / per;
       if (L.args.c_mode != 0 && c == d && L.args.ldc == L.args.ldd && conf->global_c_layout.eltype == GK_F32 &&

@@ -351,6 +351,10 @@ struct MfmaGemmConfig {
   // the generic A / B hooks, and wave tiles of more than eight 32x32 blocks (256 accumulator registers),
   // need so many registers that the kernel spills: their fragment reads wait for their data inside the
   // assembly statement that issues them (see FragReader::read)
+  // plain real products may have a last tile row / column that sticks out over M / N (the host asks for it
+  // only with 16-byte aligned columns, M or N a multiple of 8 where that index is the contiguous one of A or
+  // B, and K a whole number of tiles): loads are clamped, the C load and the D store masked
+  static constexpr bool RAGGED_OK = !GETT_ && FIX_ == FIX_NONE && !SPLITK_;
   static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
   static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
@@ -452,6 +456,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         offa[i] = base + (lower ? 0u : (unsigned)(args.plane_a * 2));
         offa2[i] = base + (lower ? (unsigned)(args.plane_a * 2) : 0u);
       } else {
+        if constexpr (Cfg::RAGGED_OK) {
+          // a tile that sticks out over the last row of A: chunks beyond it re-read the last valid chunk
+          // (their products land in rows of the tile that are never stored)
+          int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
+          const int last = args.M - m0 - (Cfg::A_KIND == OPK_KMAJOR ? 1 : 8);
+          m = m > last ? last : m;
+        }
         offa[i] = (unsigned)(((long long)row * args.lda + col) * 2);
       }
     }
@@ -459,6 +470,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     for (int i = 0; i < DMA_B; ++i) {
       int row, col;
       dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
+      if constexpr (Cfg::RAGGED_OK) {
+        int& n = Cfg::B_KIND == OPK_KMAJOR ? row : col;
+        const int last = args.N - n0 - (Cfg::B_KIND == OPK_KMAJOR ? 1 : 8);
+        n = n > last ? last : n;
+      }
       offb[i] = (unsigned)(((long long)row * args.ldb + col) * 2);
     }
   } else {
@@ -649,7 +665,26 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     for (int i = 0; i < t.n; ++i) dispatch_op(t.kind[i], t.p0[i], t.p1[i], each);
 #endif
   };
-  if (args.c_mode != 0) {
+  [[maybe_unused]] const bool ragged = Cfg::RAGGED_OK && (m0 + BM > args.M || n0 + BN > args.N);   // wave-uniform
+  if (Cfg::RAGGED_OK && ragged && args.c_mode != 0) {
+    // tile over the edge: element by element, out-of-range elements start from zero
+#pragma unroll
+    for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+          const int r = mrow + MI * fi, cc = ncol + MI * fj + vcol(v);
+          acc[fi][fj][v] = (r < args.M && cc < args.N) ? load_cd(args.c, args.c_dtype, r + (long long)cc * args.ldc) : 0.0f;
+        }
+    if (Cfg::FUSED) {
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) {
+        hook_col(std::integral_constant<int, H_GL2SH_C>{}, fj);
+        hook_col(std::integral_constant<int, H_SH2RF_C>{}, fj);
+      }
+    }
+  } else if (args.c_mode != 0) {
     gett_origins();
     // column blocks outermost: with 16-row blocks the two halves of a 128-byte line of C / D belong to
     // neighbouring row blocks, which are then read (and, below, written) right after each other
@@ -938,7 +973,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       if (args.epi_kind == 1) {          // one bias value per column of D
         float bv[NV];
 #pragma unroll
-        for (int v = 0; v < NV; ++v) bv[v] = args.bias[ncol + MI * fj + vcol(v)];
+        for (int v = 0; v < NV; ++v) {
+          const int cc = ncol + MI * fj + vcol(v);
+          bv[v] = args.bias[(Cfg::RAGGED_OK && cc >= args.N) ? 0 : cc];      // columns over the edge are not stored
+        }
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
@@ -946,7 +984,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       } else if (args.epi_kind == 2) {   // one bias value per row of D
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const float bv = args.bias[mrow + MI * fi];
+          const int r = mrow + MI * fi;
+          const float bv = args.bias[(Cfg::RAGGED_OK && r >= args.M) ? 0 : r];
 #pragma unroll
           for (int v = 0; v < NV; ++v) acc[fi][fj][v] = acc[fi][fj][v] + bv;
         }
@@ -968,6 +1007,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           float* dp = (float*)args.d + off;
 #pragma unroll
           for (int v = 0; v < NV; ++v) atomicAdd(&dp[(long long)vcol(v) * ns], x[v]);
+          continue;
+        }
+      }
+      if constexpr (Cfg::RAGGED_OK) {
+        if (ragged) {       // tile over the edge: element by element, out-of-range elements are dropped
+#pragma unroll
+          for (int v = 0; v < NV; ++v) {
+            const int r = mrow + MI * fi, cc = ncol + MI * fj + vcol(v);
+            if (r < args.M && cc < args.N) store_cd(args.d, args.d_dtype, r + (long long)cc * args.ldd, x[v]);
+          }
           continue;
         }
       }

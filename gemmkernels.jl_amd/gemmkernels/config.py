@@ -179,7 +179,9 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
                 return NT(M=t[0], N=t[1], K=t[2])
         t = fitting[-1] if fitting else (64, 64, 32)
         return NT(M=t[0], N=t[1], K=t[2])
-    fitting = [t for t, _ in _MFMA_TILES if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
+    # K is always a whole number of tiles on the aligned kernels; M and N need not be when the layouts are the
+    # bounds-checked ones (the last tile row / column is then masked)
+    fitting = [t for t, _ in _MFMA_TILES if K % t[2] == 0 and (not tile_sized or (M % t[0] == 0 and N % t[1] == 0))]
     if gett:
         fitting = [t for t in fitting if t in _GETT_TILES]
     if not fitting:
@@ -217,7 +219,7 @@ def _default_waves(operator, block_shape, checked=False, planar=False, gett=Fals
         return (1, 1)
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         table = _FPU_TILES
-    elif operator.kind == Operator.MFMA and checked:
+    elif operator.kind == Operator.MFMA and checked and any(t == key for t, _ in _CHECKED_TILES):
         table = _CHECKED_TILES
     elif operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
         table = _PLANAR_TILES if planar else _COMPLEX_TILES
