@@ -1,0 +1,133 @@
+"""Products on the bounds-checked layouts (Layout.ColMajor / RowMajor, reference src/layout.jl:117-184)
+whose columns happen to be 16-byte aligned run on the aligned kernels: tiles that stick out over M or N
+clamp their loads and mask their C loads and D stores.  Parity against the oracle, bit-for-bit equality
+with the same tile on zero-padded operands, no write outside D, and the fall-back to the bounds-checked
+kernel for misaligned pointers."""
+import numpy as np
+import pytest
+import torch
+
+import gemmkernels as gk
+from gemmkernels import Epilogue, Kernel, Layout, NT, Operator, Transform, rng
+from gemmkernels.dtypes import Float16, Float32
+import helpers
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+E = Transform.Elementwise
+TILES = [((256, 256, 64), (2, 4)), ((256, 256, 32), (2, 4)), ((256, 128, 64), (2, 2)), ((128, 256, 64), (2, 2)),
+         ((128, 128, 32), (2, 2)), ((128, 128, 64), (2, 2)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2))]
+
+
+def checked_config(M, N, K, ta, tb, block, waves, zero_c=False, cd=Float32):
+    BM, BN, BK = block
+    return gk.get_config(
+        gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=BM, N=BN, K=BK),
+        warps_per_block=waves[0] * waves[1], compute_warp=NT(M=BM // waves[0], N=BN // waves[1], K=16),
+        operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+        global_a_layout=Layout.RowMajor[Float16] if ta else Layout.ColMajor[Float16],
+        global_b_layout=Layout.RowMajor[Float16] if tb else Layout.ColMajor[Float16],
+        global_c_layout=Layout.Zero[cd] if zero_c else Layout.ColMajor[cd], global_d_layout=Layout.ColMajor[cd],
+        is_a_col_major=not ta, is_b_col_major=not tb)
+
+
+def operands(M, N, K, ta, tb, seed):
+    a = rng.matrix("upm1_f16", seed + 1, (K, M) if ta else (M, K))
+    b = rng.matrix("upm1_f16", seed + 2, (N, K) if tb else (K, N))
+    c = rng.matrix("upm1_f32", seed + 3, (M, N))
+    return a, b, c
+
+
+@pytest.mark.parametrize("block,waves", TILES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_tiles_over_the_edge_against_the_oracle_and_against_padded_operands(gpu, block, waves, ta, tb):
+    BM, BN, BK = block
+    M, N, K = BM + 72, 2 * BN - 56, 3 * BK          # multiples of 8, not of any tile
+    conf = checked_config(M, N, K, ta, tb, block, waves)
+    name = gk.kernel_name(conf, Kernel.matmul_singlestage)
+    assert "checked" not in name, name
+    a, b, c = operands(M, N, K, ta, tb, 4000)
+    print("case", block, waves, ta, tb, name, flush=True)
+    d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_singlestage)
+    ref = helpers.run_oracle(conf, a, b, c, (M, N))
+    assert oracle.rel_frobenius(d, ref) <= 1e-3
+    # the same tile on operands padded with zeros to whole tiles: identical sums, identical bits
+    Mp, Np = -(-M // BM) * BM, -(-N // BN) * BN
+    ap = np.zeros((K, Mp) if ta else (Mp, K), np.float16, order="F")
+    bp = np.zeros((Np, K) if tb else (K, Np), np.float16, order="F")
+    cp = np.zeros((Mp, Np), np.float32, order="F")
+    if ta: ap[:, :M] = a
+    else: ap[:M, :] = a
+    if tb: bp[:N, :] = b
+    else: bp[:, :N] = b
+    cp[:M, :N] = c
+    import test_mfma_gemm_gpu as T
+    dp = helpers.run_gpu(T.make_config(Mp, Np, K, ta, tb, block, waves), ap, bp, cp, (Mp, Np), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d, dp[:M, :N])
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+def test_nothing_is_written_outside_d_and_hooks_bias_and_fp16_d_work_over_the_edge(gpu, ta, tb):
+    M, N, K = 328, 264, 128
+    block, waves = (256, 256, 64), (2, 4)
+    a, b, c = operands(M, N, K, ta, tb, 4100)
+    bias = rng.normal_f32(4104, N)
+    tr = dict(transform_global_to_shared_a=E(lambda x: x * 0.5), transform_shared_to_regs_c=E(lambda x: x * 3.0),
+              transform_shared_to_global_d=E(Transform.relu))
+    for cd, tdtype, tol in ((Float32, torch.float32, 1e-3), (Float16, torch.float16, 2e-3)):
+        conf = checked_config(M, N, K, ta, tb, block, waves, cd=cd)
+        A, B = gk.colmajor(a), gk.colmajor(b)
+        c_h = c if cd is Float32 else c.astype(np.float16)
+        C = gk.colmajor(c_h)
+        ld, cols = M + 24, N + 5
+        full = gk.colmajor(np.asfortranarray(np.full((ld, cols), 777.0, np.float32 if cd is Float32 else np.float16)))
+        D = full[:M, :N]                           # a window of a larger array: rows and columns around it must stay
+        gk.matmul(conf, A, B, C, D, epilogue=Epilogue.Bias(torch.from_numpy(bias).cuda()), kernel=Kernel.matmul_singlestage, **tr)
+        torch.cuda.synchronize()
+        out = full.float().cpu().numpy()
+        assert (out[M:, :] == 777.0).all() and (out[:, N:] == 777.0).all()
+        ref = helpers.run_oracle(conf, a, b, c_h, (M, N), d_dtype=np.float32 if cd is Float32 else np.float16, transforms=tr,
+                                 epilogue=Epilogue.Bias(0), bias=bias)
+        assert oracle.rel_frobenius(out[:M, :N], ref.astype(np.float32)) <= tol, cd
+
+
+def test_misaligned_pointers_fall_back_to_the_bounds_checked_kernel(gpu):
+    """Same configuration, operands that start two bytes off a 16-byte boundary: still right (the library
+    decides per launch)."""
+    M, N, K = 200, 136, 96
+    conf = checked_config(M, N, K, False, False, (64, 64, 32), (2, 2))
+    a, b, c = operands(M, N, K, False, False, 4200)
+    a_big = np.zeros((M + 8, K), np.float16, order="F"); a_big[1:M + 1, :] = a
+    b_big = np.zeros((K + 8, N), np.float16, order="F"); b_big[1:K + 1, :] = b
+    A, B, C = gk.colmajor(a_big)[1:M + 1, :], gk.colmajor(b_big)[1:K + 1, :], gk.colmajor(c)
+    assert A.data_ptr() % 16 == 2 and B.data_ptr() % 16 == 2
+    D = gk.colmajor_empty((M, N), torch.float32)
+    gk.matmul(conf, A, B, C, D, kernel=Kernel.matmul_singlestage)
+    torch.cuda.synchronize()
+    ref = helpers.run_oracle(conf, a, b, c, (M, N))
+    assert oracle.rel_frobenius(gk.to_numpy(D), ref) <= 1e-3
+    # and aligned operands of the same configuration: the aligned kernel, same values up to the order of the sums
+    D2 = gk.colmajor_empty((M, N), torch.float32)
+    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), C, D2, kernel=Kernel.matmul_singlestage)
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(gk.to_numpy(D2), ref) <= 1e-3
+
+
+def test_full_size_4000(gpu):
+    """mul!(C, A, B) at 4000^3: one launch of the 256 x 256 tile, checked through linearity and a few exact rows."""
+    from gemmkernels.matmul import matmatmul_plan, PlanSequence
+    n = 4000
+    a = rng.matrix("upm1_f16", 4301, (n, n)); b = rng.matrix("upm1_f16", 4302, (n, n))
+    A, B = gk.colmajor(a), gk.colmajor(b)
+    C = gk.colmajor_empty((n, n), torch.float32)
+    p = matmatmul_plan(C, "N", "N", A, B, 1.0, 0.0)
+    assert not isinstance(p, PlanSequence) and "checked" not in p.kernel_names[0], p.kernel_names
+    p()
+    torch.cuda.synchronize()
+    out = gk.to_numpy(C)
+    rows = [0, 1, 255, 256, 3839, 3840, 3967, 3999]
+    ref = a[rows, :].astype(np.float64) @ b.astype(np.float64)
+    assert oracle.rel_frobenius(out[rows, :], ref) <= 1e-3
+    colsel = [0, 3840, 3999]
+    refc = a.astype(np.float64) @ b[:, colsel].astype(np.float64)
+    assert oracle.rel_frobenius(out[:, colsel], refc) <= 1e-3
