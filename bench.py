@@ -38,7 +38,7 @@ def parse_args():
     p.add_argument("--steps", type=int, default=1000)
     p.add_argument("--warmup", type=int, default=2000)
     p.add_argument("--no-extras", action="store_true", help="skip the secondary configs and the CPU baseline")
-    p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4a-planar", "4b", "5", "skinny"],
+    p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4a-planar", "4b", "5", "skinny", "mul4000"],
                    help="benchmark config to time as the step (default: 2, the headline; the others are for profiling one "
                         "kernel at a time and imply --no-extras)")
     p.add_argument("--variant", default="NN", choices=["NN", "NT", "TN", "TT"], help="transposes of config 2")

@@ -374,8 +374,35 @@ def _skinny() -> Workload:
         kernel_name="mfma_gemm_splitk_nn_64x64x64_w2x2_f16")
 
 
+def _mul4000() -> Workload:
+    """Not one of the five benchmark configurations: mul!(C, A, B) at a size that is not a whole number of
+    tiles, through the BLAS-level front end (bounds-checked layouts with 16-byte aligned columns, which the
+    library runs on the aligned kernel with masked edge tiles)."""
+    M = N = K = 4000
+
+    def host():
+        return dict(a=rng.matrix("upm1_f16", 9001, (M, K)), b=rng.matrix("upm1_f16", 9002, (K, N)))
+
+    def launch(h):
+        import torch
+        from .matmul import matmatmul_plan
+        a, b = colmajor(h["a"]), colmajor(h["b"])
+        c = colmajor_empty((M, N), torch.float32)
+        launch_plan = matmatmul_plan(c, "N", "N", a, b, 1.0, 0.0)
+
+        def run():
+            launch_plan()
+        return _attach(run, a=a, b=b, c=c, d=c, conf=None)
+
+    return Workload(
+        name="mul4000",
+        description="mul!(C, A, B), M=N=K=4000 (not whole tiles), FP16 A/B, FP32 C, 'N','N', C not read",
+        flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + M * N * 4, bound="mfma", make_host=host, make_launch=launch,
+        kernel_name="mfma_gemm_nn_256x256x32_w2x4_s4__Float16")
+
+
 def benchmark_config(n, variant: Optional[str] = None) -> Workload:
-    """The benchmark workloads 1, 2 (variant NN/NT/TN/TT), 3, "4a", "4b", 5, and "skinny"."""
+    """The benchmark workloads 1, 2 (variant NN/NT/TN/TT), 3, "4a", "4b", 5, "skinny" and "mul4000"."""
     if n == 2:
         return _config2(variant or "NN")
     if n == 3:
@@ -386,4 +413,4 @@ def benchmark_config(n, variant: Optional[str] = None) -> Workload:
     raise NotImplementedError(f"benchmark config {n}")
 
 
-_LATE_BUILDERS = {1: _config1, "4a": _config4a, "4a-planar": _config4a_planar, "4b": _config4b, 5: _config5, "skinny": _skinny}
+_LATE_BUILDERS = {1: _config1, "4a": _config4a, "4a-planar": _config4a_planar, "4b": _config4b, 5: _config5, "skinny": _skinny, "mul4000": _mul4000}
