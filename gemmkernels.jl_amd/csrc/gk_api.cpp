@@ -91,9 +91,9 @@ bool transforms_present(const gk_transforms* t) {
 
 // Bounds-checked layouts (Layout.ColMajor / RowMajor, reference src/layout.jl:117-184) promise nothing about
 // size or alignment.  When a product on them happens to have 16-byte aligned columns of A and B, a K that is
-// a whole number of tiles, and M (N) a multiple of 8 where that index is the contiguous one of A (B), the
-// aligned kernel runs it: the tiles that stick out over M or N clamp their loads and mask their C loads and
-// D stores.  Decided from the configuration (a leading dimension of 0 stands for a dense operand); the
+// a multiple of 8, and M (N) a multiple of 8 where that index is the contiguous one of A (B), the aligned
+// kernel runs it: the tiles that stick out over M or N clamp their loads and mask their C loads and D
+// stores, a last partial K tile is zeroed beyond K in LDS.  Decided from the configuration (a leading dimension of 0 stands for a dense operand); the
 // launcher falls back to the bounds-checked kernel when the pointers themselves turn out misaligned.
 thread_local bool t_allow_ragged_fast = true;
 
@@ -108,7 +108,7 @@ bool ragged_fast_path(const gk_config* c) {
   if (!(is_checked_layout(la.kind) || is_checked_layout(lb.kind) || is_checked_layout(lc.kind) || is_checked_layout(ld.kind))) return false;
   if ((la.eltype != GK_F16 && la.eltype != GK_BF16) || lb.eltype != la.eltype) return false;
   const long long M = c->matmul_shape.M, N = c->matmul_shape.N, K = c->matmul_shape.K;
-  if (c->block_shape.K <= 0 || K % c->block_shape.K != 0) return false;
+  if (K % 8 != 0) return false;                // a last, partial K tile is fine; its 16-byte chunks must be whole
   const bool a_row = is_row_major(la.kind), b_row = is_row_major(lb.kind);
   const long long lda = la.ld > 0 ? la.ld : (a_row ? K : M), ldb = lb.ld > 0 ? lb.ld : (b_row ? N : K);
   if ((lda * 2) % 16 != 0 || (ldb * 2) % 16 != 0) return false;
@@ -673,7 +673,8 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
       t_allow_ragged_fast = true;
       if (rc != GK_OK) return rc;
     } else {
-      out->ragged = (conf->matmul_shape.M % conf->block_shape.M) != 0 || (conf->matmul_shape.N % conf->block_shape.N) != 0;
+      out->ragged = (conf->matmul_shape.M % conf->block_shape.M) != 0 || (conf->matmul_shape.N % conf->block_shape.N) != 0 ||
+                    (conf->matmul_shape.K % conf->block_shape.K) != 0;
     }
   }
 

@@ -351,9 +351,10 @@ struct MfmaGemmConfig {
   // the generic A / B hooks, and wave tiles of more than eight 32x32 blocks (256 accumulator registers),
   // need so many registers that the kernel spills: their fragment reads wait for their data inside the
   // assembly statement that issues them (see FragReader::read)
-  // plain real products may have a last tile row / column that sticks out over M / N (the host asks for it
-  // only with 16-byte aligned columns, M or N a multiple of 8 where that index is the contiguous one of A or
-  // B, and K a whole number of tiles): loads are clamped, the C load and the D store masked
+  // plain real products may have a last tile row / column that sticks out over M / N and a last, partial K
+  // tile (the host asks for it only with 16-byte aligned columns, M or N a multiple of 8 where that index is
+  // the contiguous one of A or B, and K a multiple of 8): loads are clamped, the C load and the D store
+  // masked, the part of the last K tile beyond K zeroed in LDS
   static constexpr bool RAGGED_OK = !GETT_ && FIX_ == FIX_NONE && !SPLITK_;
   static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
   static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
@@ -947,6 +948,81 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           if (issue) issue_part(ks_c, std::integral_constant<int, Cfg::KSTEPS>{}, (kt + STAGES - 1) % STAGES);
         }
         compute(ks_c, Whole{});
+      });
+    }
+  }
+  if constexpr (Cfg::RAGGED_OK) {
+    // --- a last, partial K tile (K not a multiple of BLOCK_K; K a multiple of 8) -----------------------
+    // Outside the pipeline: the tile is fetched with its k coordinates clamped to the valid ones, the LDS
+    // slots beyond K are set to zero by the lanes that fetched them, and the k-steps that hold valid
+    // values are multiplied.  ga / gb stand at this tile: every whole tile has been issued.
+    const int tail_k = args.K - (args.K / BK) * BK;       // wave-uniform
+    if (tail_k > 0) {
+      block_barrier();                                     // every wave is done with the stages of the loop
+      char* sa = smem;
+      char* sb = sa + GA::BYTES;
+      bool beyond_a[DMA_A], beyond_b[DMA_B];
+#pragma unroll
+      for (int i = 0; i < DMA_A; ++i) {
+        int row, col;
+        dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
+        int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
+        int& k = Cfg::A_KIND == OPK_KMAJOR ? col : row;
+        const int last_m = args.M - m0 - (Cfg::A_KIND == OPK_KMAJOR ? 1 : 8);
+        m = m > last_m ? last_m : m;
+        beyond_a[i] = k >= tail_k;
+        if (beyond_a[i]) k = tail_k - (Cfg::A_KIND == OPK_KMAJOR ? 8 : 1);
+        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + ((long long)row * args.lda + col) * 2),
+                                         GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < DMA_B; ++i) {
+        int row, col;
+        dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
+        int& n = Cfg::B_KIND == OPK_KMAJOR ? row : col;
+        int& k = Cfg::B_KIND == OPK_KMAJOR ? col : row;
+        const int last_n = args.N - n0 - (Cfg::B_KIND == OPK_KMAJOR ? 1 : 8);
+        n = n > last_n ? last_n : n;
+        beyond_b[i] = k >= tail_k;
+        if (beyond_b[i]) k = tail_k - (Cfg::B_KIND == OPK_KMAJOR ? 8 : 1);
+        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + ((long long)row * args.ldb + col) * 2),
+                                         GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      }
+      wait_vmcnt<0>();                                     // this lane's own slots have landed
+      const int4v zero = {0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < DMA_A; ++i)
+        if (beyond_a[i]) *(int4v*)(sa + (wave + i * NWAVES) * 1024 + lane * 16) = zero;
+#pragma unroll
+      for (int i = 0; i < DMA_B; ++i)
+        if (beyond_b[i]) *(int4v*)(sb + (wave + i * NWAVES) * 1024 + lane * 16) = zero;
+      __syncthreads();                                     // waits for the LDS writes as well
+      ra.set_stage(lds_base);
+      rb.set_stage(lds_base + GA::BYTES);
+      static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
+        constexpr int ks = decltype(ks_c)::value;
+        if (ks * Cfg::KSTEP_K < tail_k) {
+          if constexpr (Cfg::SPLIT_A) {
+            constexpr int HF = FM / 2;
+            static_for<0, 2>([&](auto h_c) {
+              constexpr int H = decltype(h_c)::value;
+              static_for<0, HF>([&](auto i_c) {
+                constexpr int I = decltype(i_c)::value;
+                ra.template read<H * HF + I, ks, true>(fa[H][I]);
+              });
+              if constexpr (H == 0) {
+                static_for<0, FN>([&](auto j_c) {
+                  constexpr int J = decltype(j_c)::value;
+                  rb.template read<J, ks, true>(fb[ks & 1][J]);
+                });
+              }
+              compute(ks_c, h_c);
+            });
+          } else {
+            load_frags<ks, true>(ra, rb, fa[ks & 1], fb[ks & 1]);
+            compute(ks_c, Whole{});
+          }
+        }
       });
     }
   }

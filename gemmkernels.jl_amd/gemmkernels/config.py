@@ -179,9 +179,9 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
                 return NT(M=t[0], N=t[1], K=t[2])
         t = fitting[-1] if fitting else (64, 64, 32)
         return NT(M=t[0], N=t[1], K=t[2])
-    # K is always a whole number of tiles on the aligned kernels; M and N need not be when the layouts are the
-    # bounds-checked ones (the last tile row / column is then masked)
-    fitting = [t for t, _ in _MFMA_TILES if K % t[2] == 0 and (not tile_sized or (M % t[0] == 0 and N % t[1] == 0))]
+    # sizes need not be whole tiles when the layouts are the bounds-checked ones (the aligned kernels mask the
+    # last tile row / column and zero the end of the last K tile)
+    fitting = [t for t, _ in _MFMA_TILES if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
     if gett:
         fitting = [t for t in fitting if t in _GETT_TILES]
     if not fitting:

@@ -359,10 +359,9 @@ def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stri
     if any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout)):
         # Some operand needs bounds checks.  The library runs such a product on the aligned kernels all the
         # same (tiles over the edge clamp their loads and mask their stores) when the columns of A and B are
-        # 16-byte aligned, K is a whole number of tiles and M (N) is a multiple of 8 where it is the contiguous
-        # index of A (B): then any tile that divides K will do.  Otherwise the bounds-checked kernel, which
-        # has one tile shape.
-        edge_ok = (use_mfma and a_aligned and b_aligned and k % 32 == 0 and (transA or m % 8 == 0) and (not transB or n % 8 == 0)
+        # 16-byte aligned, K is a multiple of 8 and M (N) is a multiple of 8 where it is the contiguous index
+        # of A (B): then any tile will do.  Otherwise the bounds-checked kernel, which has one tile shape.
+        edge_ok = (use_mfma and a_aligned and b_aligned and k % 8 == 0 and (transA or m % 8 == 0) and (not transB or n % 8 == 0)
                    and not zeroAlpha)
         block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=False) if edge_ok else NT(M=64, N=64, K=32)
         global_a_layout, global_b_layout, global_c_layout, global_d_layout = layouts_for(block_shape)
@@ -506,10 +505,10 @@ def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None,
     to all of C.  With beta = 0 and M, N multiples of 8 there are no rims: ``overlapping_regions`` covers the
     edges with whole tiles that reach back over finished cells.
 
-    Since the aligned kernels mask tiles that stick out over M or N themselves (when M, or N, is a multiple
-    of 8 where it is the contiguous index of A, or B), such products take one launch (two when K is not a
-    multiple of 32) and the cutting above is what remains for the others: aligned leading dimensions around
-    an M or N that is not a multiple of 8, as sub-matrices have them.  Every element of C is
+    Since the aligned kernels handle tiles that stick out over M, N or K themselves (K a multiple of 8, and
+    M, or N, where it is the contiguous index of A, or B), such products take one launch and the cutting
+    above is what remains for the others: aligned leading dimensions around an M or N that is not a multiple
+    of 8, as sub-matrices have them.  Every element of C is
     still computed as alpha * op(A) * op(B) + beta * C with alpha applied to A in the compute type; only
     the order of the fp32 additions along k differs from the single launch.  ``regions`` forces the
     cutting on (True) or off (False); by default it is used when a rough estimate (``_estimate_us``) puts
@@ -527,16 +526,8 @@ def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None,
     aligned_columns = all((int(x.stride()[1]) * x.element_size()) % 16 == 0 and x.data_ptr() % 16 == 0 for x in (A, B, C))
     Kw = K // 32 * 32        # every tile table has tiles 32 deep
     if (regions is None and checked and conf.operator.kind == Operator.MFMA and aligned_columns and alpha != 0
-            and (tA or M % 8 == 0) and (not tB or N % 8 == 0)):
-        # the aligned kernels take ragged M and N themselves (create_config has picked their tile); only a
-        # K that is not a whole number of tiles needs a second launch for its tail
-        if Kw == K:
-            return single
-        if Kw >= 256 and min(M, N) >= 64:
-            def cols(X, trans, k0, k):      # k0 .. k0 + k of the K index of op(X) given as rows (trans) or columns
-                return X[k0:k0 + k, :] if trans else X[:, k0:k0 + k]
-            return PlanSequence([_single_plan(C, tA, tB, cols(A, tA, 0, Kw), cols(B, not tB, 0, Kw), alpha, beta, wmma),
-                                 _single_plan(C, tA, tB, cols(A, tA, Kw, K - Kw), cols(B, not tB, Kw, K - Kw), alpha, 1.0, wmma)], C)
+            and K % 8 == 0 and (tA or M % 8 == 0) and (not tB or N % 8 == 0)):
+        # the aligned kernels take ragged M, N and K themselves (create_config has picked their tile)
         return single
     if (regions is False or conf.operator.kind != Operator.MFMA or not aligned_columns or alpha == 0
             or Kw == 0 or min(M, N) < _REGION_TILES[-1]):

@@ -152,7 +152,7 @@ def test_region_cutting_is_left_alone_where_it_cannot_help(gpu):
 @pytest.mark.parametrize("dims", [(1000, 1000, 1000), (840, 328, 192), (264, 72, 136)])
 def test_products_that_do_not_read_c_need_no_rims(gpu, dims, ta, tb):
     """beta = 0 and M, N multiples of 8: the ragged edges are covered by whole tiles that reach back over
-    finished cells, so only the tail of K (if any) runs on the bounds-checked kernel."""
+    finished cells; nothing runs on the bounds-checked kernel."""
     from gemmkernels.matmul import matmatmul_plan, PlanSequence
     M, N, K = dims
     a, b, c = operands(M, N, K, ta == "T", tb == "T", np.float16, 700)
@@ -160,7 +160,7 @@ def test_products_that_do_not_read_c_need_no_rims(gpu, dims, ta, tb):
     C = gk.colmajor(np.asfortranarray(np.full((M, N), np.nan, np.float32)))       # never read
     p = matmatmul_plan(C, ta, tb, A, B, 1.25, 0.0, regions=True)
     assert isinstance(p, PlanSequence)
-    assert sum("checked" in n for n in p.kernel_names) == (1 if K % 32 else 0), p.kernel_names
+    assert not any("checked" in n for n in p.kernel_names), p.kernel_names     # the tail of K is a partial tile of the aligned kernel
     p()
     torch.cuda.synchronize()
     ref = oracle.gemm_f64(a, b, None, 1.25, 0.0, ta == "T", tb == "T")

@@ -42,33 +42,38 @@ def operands(M, N, K, ta, tb, seed):
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 def test_tiles_over_the_edge_against_the_oracle_and_against_padded_operands(gpu, block, waves, ta, tb):
     BM, BN, BK = block
-    M, N, K = BM + 72, 2 * BN - 56, 3 * BK          # multiples of 8, not of any tile
+    for K in (3 * BK, 2 * BK + 24, 8):              # whole tiles; a partial last tile; less than one tile
+        _one_shape(block, waves, ta, tb, BM + 72, 2 * BN - 56, K)    # M, N: multiples of 8, not of any tile
+
+
+def _one_shape(block, waves, ta, tb, M, N, K):
+    BM, BN, BK = block
     conf = checked_config(M, N, K, ta, tb, block, waves)
     name = gk.kernel_name(conf, Kernel.matmul_singlestage)
     assert "checked" not in name, name
     a, b, c = operands(M, N, K, ta, tb, 4000)
-    print("case", block, waves, ta, tb, name, flush=True)
+    print("case", block, waves, ta, tb, (M, N, K), name, flush=True)
     d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_singlestage)
     ref = helpers.run_oracle(conf, a, b, c, (M, N))
     assert oracle.rel_frobenius(d, ref) <= 1e-3
     # the same tile on operands padded with zeros to whole tiles: identical sums, identical bits
-    Mp, Np = -(-M // BM) * BM, -(-N // BN) * BN
-    ap = np.zeros((K, Mp) if ta else (Mp, K), np.float16, order="F")
-    bp = np.zeros((Np, K) if tb else (K, Np), np.float16, order="F")
+    Mp, Np, Kp = -(-M // BM) * BM, -(-N // BN) * BN, -(-K // BK) * BK
+    ap = np.zeros((Kp, Mp) if ta else (Mp, Kp), np.float16, order="F")
+    bp = np.zeros((Np, Kp) if tb else (Kp, Np), np.float16, order="F")
     cp = np.zeros((Mp, Np), np.float32, order="F")
-    if ta: ap[:, :M] = a
-    else: ap[:M, :] = a
-    if tb: bp[:N, :] = b
-    else: bp[:, :N] = b
+    if ta: ap[:K, :M] = a
+    else: ap[:M, :K] = a
+    if tb: bp[:N, :K] = b
+    else: bp[:K, :N] = b
     cp[:M, :N] = c
     import test_mfma_gemm_gpu as T
-    dp = helpers.run_gpu(T.make_config(Mp, Np, K, ta, tb, block, waves), ap, bp, cp, (Mp, Np), kernel=Kernel.matmul_pipelined)
+    dp = helpers.run_gpu(T.make_config(Mp, Np, Kp, ta, tb, block, waves), ap, bp, cp, (Mp, Np), kernel=Kernel.matmul_pipelined)
     assert np.array_equal(d, dp[:M, :N])
 
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
 def test_nothing_is_written_outside_d_and_hooks_bias_and_fp16_d_work_over_the_edge(gpu, ta, tb):
-    M, N, K = 328, 264, 128
+    M, N, K = 328, 264, 152                      # K: two whole tiles and 24 more
     block, waves = (256, 256, 64), (2, 4)
     a, b, c = operands(M, N, K, ta, tb, 4100)
     bias = rng.normal_f32(4104, N)
