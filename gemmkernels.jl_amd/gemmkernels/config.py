@@ -191,14 +191,20 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
     # relative rate of its kernel (ties go to the tile listed first)
     def cost(t):
         tiles = -(-M // t[0]) * -(-N // t[1])
-        return -(-tiles // NUM_CUS) * t[0] * t[1] / _MFMA_TILE_RATE.get(t, 0.5)
+        rounds = -(-tiles // NUM_CUS)
+        rate = _MFMA_TILE_RATE.get(t, 0.5)
+        if isinstance(rate, tuple):
+            rate = rate[0] if rounds == 1 else rate[1]
+        return rounds * t[0] * t[1] / rate
     best = min(fitting, key=lambda t: (cost(t), fitting.index(t)))
     return NT(M=best[0], N=best[1], K=best[2])
 
 
-# throughput of a CU running each tile, relative to 256 x 256 x 64 (from 4096 x 4096 x 2048 and 4032^3 timings)
+# throughput of a CU running each tile, relative to 256 x 256 x 64; a pair: with at most one tile per CU, with
+# several in a row.  From timings of every tile at 1000^3 ... 6000^3 (4096 x 4096 x 2048 and 4032^3 for the
+# 64-wide ones): e.g. 6000^3 takes 436 us on 256 x 256 x 64, 562 us on 128 x 128 x 64, 617 us on 128 x 128 x 32.
 _MFMA_TILE_RATE = {(256, 256, 64): 1.0, (256, 256, 32): 0.95, (256, 128, 64): 0.81, (128, 256, 64): 0.82,
-                   (128, 128, 32): 0.86, (128, 128, 64): 0.86, (64, 64, 64): 0.47, (64, 64, 32): 0.42}
+                   (128, 128, 32): (0.66, 0.60), (128, 128, 64): (0.60, 0.65), (64, 64, 64): 0.47, (64, 64, 32): 0.42}
 
 
 # complex / dual tiles (complex elements) -> waves

@@ -485,7 +485,9 @@ def _estimate_us(operator, M: int, N: int, K: int, whole_tiles: bool) -> float:
     if whole_tiles:
         bs = default_block_shape(operator, NT(M=M, N=N, K=K))
         tiles = -(-M // bs.M) * -(-N // bs.N)
-        per_cu = -(-tiles // NUM_CUS) * bs.M * bs.N / _MFMA_TILE_RATE.get((bs.M, bs.N, bs.K), 0.5)
+        rate = _MFMA_TILE_RATE.get((bs.M, bs.N, bs.K), 0.5)
+        rate = rate[0 if tiles <= NUM_CUS else 1] if isinstance(rate, tuple) else rate
+        per_cu = -(-tiles // NUM_CUS) * bs.M * bs.N / rate
         return per_cu * K / (65536.0 * 4096.0) * 108.0 + 6.0
     steps = -(-M // 64) * -(-N // 64) * -(-K // 32)
     return max(-(-steps // NUM_CUS), 8) * 0.53 + 25.0
