@@ -398,7 +398,7 @@ def _mul4000() -> Workload:
         name="mul4000",
         description="mul!(C, A, B), M=N=K=4000 (not whole tiles), FP16 A/B, FP32 C, 'N','N', C not read",
         flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + M * N * 4, bound="mfma", make_host=host, make_launch=launch,
-        kernel_name="mfma_gemm_nn_256x256x32_w2x4_s4__Float16")
+        kernel_name="mfma_gemm_nn_256x256x64_w2x4_s2__Float16")
 
 
 def benchmark_config(n, variant: Optional[str] = None) -> Workload:

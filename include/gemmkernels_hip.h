@@ -81,9 +81,10 @@ typedef enum gk_layout_kind {
   GK_LAYOUT_ZERO = 0,                   /* :82-89   loads zeros, stores nothing */
   GK_LAYOUT_COL_MAJOR = 1,              /* :111-148 bounds-checked, any size and alignment.  A real MFMA product on these
                                          * layouts whose A and B happen to have 16-byte aligned columns (pointer and leading
-                                         * dimension), K a multiple of BLOCK_K, and M (N) a multiple of 8 where that is the
+                                         * dimension), K a multiple of 8, and M (N) a multiple of 8 where that is the
                                          * contiguous index of A (B), runs on the aligned kernel of its block shape: tiles
-                                         * over the edge clamp their loads and mask their stores.  Same results; decided
+                                         * over the edge clamp their loads and mask their stores, a partial last K tile is
+                                         * zeroed beyond K.  Same results; decided
                                          * per launch, everything else runs on the bounds-checked kernel (64 x 64 x 32) */
   GK_LAYOUT_ROW_MAJOR = 2,              /* :156-184 */
   GK_LAYOUT_ALIGNED_COL_MAJOR = 3,      /* :192-219 UnsafeAlignedColMajor: 16-byte vectors, tile-sized */
