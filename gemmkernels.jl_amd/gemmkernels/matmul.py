@@ -354,16 +354,19 @@ def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stri
         gd = Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C]
         return ga, gb, gc, gd
 
-    block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=True)
+    # The library runs a product on bounds-checked layouts on the aligned kernels all the same (tiles over the
+    # edge clamp their loads and mask their stores, a partial last K tile is zeroed beyond K) when the columns
+    # of A and B are 16-byte aligned, K is a multiple of 8 and M (N) is a multiple of 8 where it is the
+    # contiguous index of A (B).  Then the tile is chosen among all tiles, not only those that divide the
+    # sizes (4096 x 4096 x 4000: the 64-deep tile with a partial last step instead of the 32-deep one), and
+    # the operands it does not divide get the bounds-checked layouts, as the reference's rule says.
+    edge_ok = (use_mfma and a_aligned and b_aligned and k % 8 == 0 and (transA or m % 8 == 0) and (not transB or n % 8 == 0)
+               and not zeroAlpha)
+    block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=not edge_ok)
     global_a_layout, global_b_layout, global_c_layout, global_d_layout = layouts_for(block_shape)
-    if any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout)):
-        # Some operand needs bounds checks.  The library runs such a product on the aligned kernels all the
-        # same (tiles over the edge clamp their loads and mask their stores) when the columns of A and B are
-        # 16-byte aligned, K is a multiple of 8 and M (N) is a multiple of 8 where it is the contiguous index
-        # of A (B): then any tile will do.  Otherwise the bounds-checked kernel, which has one tile shape.
-        edge_ok = (use_mfma and a_aligned and b_aligned and k % 8 == 0 and (transA or m % 8 == 0) and (not transB or n % 8 == 0)
-                   and not zeroAlpha)
-        block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=False) if edge_ok else NT(M=64, N=64, K=32)
+    if not edge_ok and any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout)):
+        # some operand needs bounds checks: the bounds-checked kernels have one tile shape
+        block_shape = NT(M=64, N=64, K=32)
         global_a_layout, global_b_layout, global_c_layout, global_d_layout = layouts_for(block_shape)
 
     conf = _get_config(gemm_shape=NT(M=m, N=n, K=k), block_shape=block_shape, operator=operator,
