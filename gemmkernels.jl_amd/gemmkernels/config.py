@@ -151,6 +151,11 @@ _MFMA_TILES = [
     ((64, 64, 64), (2, 2)),
     ((64, 64, 32), (2, 2)),       # four stages; the one-wave instance (the tensor-contraction kernels have only that) is 1.5 - 2.7 times slower
 ]
+# Tiles with a side of 192: they fill the chip where 256 x 256 leaves CUs idle (3072^2: 192 tiles instead of 144,
+# 59 us instead of 72).  The swizzle of an LDS tile whose rows run along k needs a power of two along the other
+# index, so the 192 side must belong to an operand that is contiguous along k: B of an 'N' product (256 x 192),
+# A of a 'T' product (192 x 256).
+_MFMA_TILES_192 = [((256, 192, 64), (4, 2), "b_kmajor"), ((192, 256, 64), (2, 4), "a_kmajor")]
 NUM_CUS = 256
 
 # measured winners by problem (filled by gemmkernels.tuning.install / load, or from the JSON file
@@ -162,9 +167,11 @@ TUNED = {}
 _GETT_TILES = [(256, 256, 64), (128, 128, 64), (64, 64, 32)]
 
 
-def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: bool = False, planar: bool = False) -> NT:
+def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: bool = False, planar: bool = False,
+                        a_kmajor: bool = False, b_kmajor: bool = False) -> NT:
     """MI355X block shape: of the tiles of the table that divide the problem, the one with the shortest
-    estimated launch (tiles per CU times the cost of a tile)."""
+    estimated launch (tiles per CU times the cost of a tile).  ``a_kmajor``: A is stored K x M ('T');
+    ``b_kmajor``: B is stored K x N ('N'); they admit the tiles with a side of 192."""
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         return NT(M=64, N=64, K=32)
     M, N, K = gemm_shape["M"], gemm_shape["N"], gemm_shape["K"]
@@ -181,7 +188,8 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
         return NT(M=t[0], N=t[1], K=t[2])
     # sizes need not be whole tiles when the layouts are the bounds-checked ones (the aligned kernels mask the
     # last tile row / column and zero the end of the last K tile)
-    fitting = [t for t, _ in _MFMA_TILES if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
+    table = [t for t, _ in _MFMA_TILES] + [t for t, _, need in _MFMA_TILES_192 if (a_kmajor if need == "a_kmajor" else b_kmajor)]
+    fitting = [t for t in table if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
     if gett:
         fitting = [t for t in fitting if t in _GETT_TILES]
     if not fitting:
@@ -204,7 +212,8 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
 # several in a row.  From timings of every tile at 1000^3 ... 6000^3 (4096 x 4096 x 2048 and 4032^3 for the
 # 64-wide ones): e.g. 6000^3 takes 436 us on 256 x 256 x 64, 562 us on 128 x 128 x 64, 617 us on 128 x 128 x 32.
 _MFMA_TILE_RATE = {(256, 256, 64): 1.0, (256, 256, 32): 0.95, (256, 128, 64): 0.81, (128, 256, 64): 0.82,
-                   (128, 128, 32): (0.66, 0.60), (128, 128, 64): (0.60, 0.65), (64, 64, 64): 0.47, (64, 64, 32): 0.42}
+                   (128, 128, 32): (0.66, 0.60), (128, 128, 64): (0.60, 0.65), (64, 64, 64): 0.47, (64, 64, 32): 0.42,
+                   (256, 192, 64): 0.90, (192, 256, 64): 0.90}
 
 
 # complex / dual tiles (complex elements) -> waves
@@ -230,7 +239,7 @@ def _default_waves(operator, block_shape, checked=False, planar=False, gett=Fals
     elif operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
         table = _PLANAR_TILES if planar else _COMPLEX_TILES
     else:
-        table = _MFMA_TILES
+        table = _MFMA_TILES + [(t, w) for t, w, _ in _MFMA_TILES_192]
     for t, w in table:
         if t == key:
             return w
@@ -285,7 +294,9 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
         params.setdefault("cta_swizzle", CTASwizzle.Identity)
     is_gett = any(l.kind == Layout.GETT_KIND for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
     planar = global_a_layout.kind in (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
-    block_shape = default_block_shape(operator, gemm_shape, tile_sized, is_gett, planar) if block_shape is None else NT(block_shape)
+    block_shape = (default_block_shape(operator, gemm_shape, tile_sized, is_gett, planar, a_kmajor=global_a_layout.kind in (Layout.ROW_MAJOR, Layout.ALIGNED_ROW_MAJOR),
+                                       b_kmajor=global_b_layout.kind in (Layout.COL_MAJOR, Layout.ALIGNED_COL_MAJOR))
+                   if block_shape is None else NT(block_shape))
     op_shape = Operator.shape(operator)
 
     checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))

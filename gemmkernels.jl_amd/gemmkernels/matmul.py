@@ -362,7 +362,7 @@ def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stri
     # the operands it does not divide get the bounds-checked layouts, as the reference's rule says.
     edge_ok = (use_mfma and a_aligned and b_aligned and k % 8 == 0 and (transA or m % 8 == 0) and (not transB or n % 8 == 0)
                and not zeroAlpha)
-    block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=not edge_ok)
+    block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=not edge_ok, a_kmajor=transA, b_kmajor=not transB)
     global_a_layout, global_b_layout, global_c_layout, global_d_layout = layouts_for(block_shape)
     if not edge_ok and any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout)):
         # some operand needs bounds checks: the bounds-checked kernels have one tile shape

@@ -136,3 +136,36 @@ def test_full_size_4000(gpu):
     colsel = [0, 3840, 3999]
     refc = a.astype(np.float64) @ b[:, colsel].astype(np.float64)
     assert oracle.rel_frobenius(out[:, colsel], refc) <= 1e-3
+
+
+# tiles with a side of 192: only where the operand on that side is contiguous along k
+TILES_192 = [((256, 192, 64), (4, 2), [(False, False), (True, False)]), ((192, 256, 64), (2, 4), [(True, False), (True, True)])]
+
+
+@pytest.mark.parametrize("block,waves,transposes", TILES_192)
+def test_tiles_with_a_side_of_192(gpu, block, waves, transposes):
+    """Whole tiles (aligned layouts, C read, hooks and bias) and tiles over the edge (bounds-checked layouts,
+    partial last K tile), against the oracle; the ragged case bit for bit against zero-padded operands."""
+    import test_mfma_gemm_gpu as T
+    BM, BN, BK = block
+    for ta, tb in transposes:
+        M, N, K = 2 * BM, 3 * BN, 3 * BK
+        conf = T.make_config(M, N, K, ta, tb, block, waves)
+        a, b, c = operands(M, N, K, ta, tb, 4400)
+        name = gk.kernel_name(conf, Kernel.matmul_pipelined)
+        print("case", block, waves, ta, tb, name, flush=True)
+        d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+        assert oracle.rel_frobenius(d, helpers.run_oracle(conf, a, b, c, (M, N))) <= 1e-3
+        bias = rng.normal_f32(4404, N)
+        for tr in (dict(transform_global_to_shared_a=E(lambda x: x * 0.5), transform_shared_to_global_d=E(Transform.relu)),
+                   dict(transform_shared_to_regs_a=E(lambda x: Transform.square(x) - 0.25), transform_global_to_shared_b=E(lambda x: abs(x) * 1.5))):
+            d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=tr, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
+            ref = helpers.run_oracle(conf, a, b, c, (M, N), transforms=tr, epilogue=Epilogue.Bias(0), bias=bias)
+            assert oracle.rel_frobenius(d, ref) <= 1e-3, sorted(tr)
+        _one_shape(block, waves, ta, tb, BM + 72, 2 * BN - 56, 2 * BK + 24)
+    # the default picks them where they fill the chip and only where the kernel has them
+    from gemmkernels import default_block_shape
+    op = Operator.MFMAOp[32, 32, 16, Float16, Float32]
+    assert default_block_shape(op, NT(M=3072, N=3072, K=3072), b_kmajor=True) == NT(M=256, N=192, K=64)
+    assert default_block_shape(op, NT(M=3072, N=3072, K=3072), a_kmajor=True) == NT(M=192, N=256, K=64)
+    assert default_block_shape(op, NT(M=3072, N=3072, K=3072)) == NT(M=256, N=256, K=64)
