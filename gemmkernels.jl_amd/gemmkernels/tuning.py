@@ -32,6 +32,7 @@ MFMA_CANDIDATES = [
     ((256, 128, 64), (2, 2)), ((128, 256, 64), (2, 2)),
     ((128, 128, 64), (2, 2)), ((128, 128, 64), (4, 2)), ((128, 128, 32), (2, 2)),
     ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((64, 64, 32), (1, 1)),
+    ((256, 192, 64), (4, 2)), ((192, 256, 64), (2, 4)),     # compiled for the transposes whose 192 side is contiguous along k; skipped elsewhere
 ]
 SWIZZLE_PANELS = (1, 2, 4, 8)
 
