@@ -33,8 +33,13 @@ def test_table_round_trip_and_lookup(tmp_path):
 
 def test_every_candidate_of_the_tuner_is_a_compiled_instance():
     for block, waves in tuning.MFMA_CANDIDATES:
-        conf = tuning.mfma_config(2 * block[0], 2 * block[1], 4 * block[2], False, False, block, waves, 4)
+        # a tile with a side of 192 exists where the operand on that side is contiguous along k: 'T','N' has both
+        ta = 192 in block[:2]
+        conf = tuning.mfma_config(2 * block[0], 2 * block[1], 4 * block[2], ta, False, block, waves, 4)
         assert f"{block[0]}x{block[1]}x{block[2]}_w{waves[0]}x{waves[1]}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    # ... and nowhere else: the tuner skips it there
+    with pytest.raises(gk.ConfigError):
+        tuning.mfma_config(384, 512, 256, False, True, (192, 256, 64), (2, 4), 4)
 
 
 @pytest.mark.gpu
