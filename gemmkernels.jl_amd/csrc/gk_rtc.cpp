@@ -233,6 +233,14 @@ int gk_rtc_matmul(gk_rtc_kernel* k, const gk_config* conf, const void* a, const 
   if (bs.M != k->BM || bs.N != k->BN || bs.K != k->BK || conf->compute_warp.M * k->waves_m != bs.M || conf->compute_warp.N * k->waves_n != bs.N ||
       a_kmajor != k->a_kmajor || b_kmajor != k->b_kmajor || conf->global_a_layout.eltype != k->dtype || conf->op.kind != GK_OP_MFMA)
     return fail(GK_ERR_INVALID_ARGUMENT, "the configuration differs from the one this kernel was compiled for");
+  {
+    // the same rule as at compile time: whole tiles on aligned layouts (the bounds-checked layouts would let
+    // sizes through that this kernel cannot mask)
+    const gk_layout* ls[4] = {&conf->global_a_layout, &conf->global_b_layout, &conf->global_c_layout, &conf->global_d_layout};
+    for (const gk_layout* l : ls)
+      if (l->kind != GK_LAYOUT_ALIGNED_COL_MAJOR && l->kind != GK_LAYOUT_ALIGNED_ROW_MAJOR && l->kind != GK_LAYOUT_ZERO)
+        return fail(GK_ERR_UNSUPPORTED, "run-time specialisation needs aligned (or Zero) global layouts");
+  }
   // a bias epilogue makes the host layer choose a fused path; the hooks themselves are compiled in,
   // so no op lists travel with the launch
   gk_internal::Launch L;

@@ -134,3 +134,27 @@ def test_wave_tile_of_sixteen_blocks_runs_with_synchronous_fragment_reads(gpu):
     gk.specialize(conf, transform_shared_to_global_d="2.0f * x")(A, B, C, D)
     torch.cuda.synchronize()
     assert oracle.rel_frobenius(gk.to_numpy(D), 2.0 * oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False)) <= 1e-3
+
+
+@pytest.mark.gpu
+def test_a_specialised_kernel_refuses_bounds_checked_layouts_at_launch(gpu):
+    """Compiled for aligned layouts; a launch configuration of the same tile on bounds-checked layouts (which
+    admit sizes the specialised kernel cannot mask) is turned down before anything runs."""
+    import torch
+    from gemmkernels.matmul import Plan, _DEFAULT_EPILOGUE
+    M, N, K = 256, 256, 128
+    common = dict(operator=Operator.MFMAOp[32, 32, 16, Float16, Float32], block_shape=NT(M=128, N=128, K=64), warps_per_block=4,
+                  compute_warp=NT(M=64, N=64, K=16))
+    conf = gk.get_config(gemm_shape=NT(M=M, N=N, K=K), global_a_layout=Layout.UnsafeAlignedColMajor[Float16],
+                         global_b_layout=Layout.UnsafeAlignedColMajor[Float16], global_c_layout=Layout.Zero[Float32],
+                         global_d_layout=Layout.UnsafeAlignedColMajor[Float32], specialize=True, **common)
+    k = gk.specialize(conf, transform_shared_to_global_d="x + 1.0f")
+    loose = gk.get_config(gemm_shape=NT(M=M - 8, N=N, K=K), global_a_layout=Layout.ColMajor[Float16],
+                          global_b_layout=Layout.ColMajor[Float16], global_c_layout=Layout.Zero[Float32],
+                          global_d_layout=Layout.ColMajor[Float32], **common)
+    A = gk.colmajor(rng.matrix("upm1_f16", 31, (M, K))); B = gk.colmajor(rng.matrix("upm1_f16", 32, (K, N)))
+    D = gk.colmajor_empty((M, N), torch.float32)
+    with pytest.raises(gk.ConfigError):
+        Plan(loose, A[:M - 8, :], B, None, D[:M - 8, :], {}, _DEFAULT_EPILOGUE, Kernel.matmul_pipelined, specialized=k)()
+    k(A, B, None, D)                                  # the configuration it was compiled for still runs
+    torch.cuda.synchronize()
