@@ -54,12 +54,17 @@ struct OperandGeom {
   __device__ static __forceinline__ int swz_k(int row) { return (row / RP256) & (CPR - 1); }
   // M-major: XOR the 64-byte group index with k so that 4 consecutive k rows at one group land in
   // 4 different 64-byte slots of the 256-byte bank period.
+  // Rows of 384 bytes (192 elements): consecutive k rows are already 128 bytes apart in the bank period, so
+  // the XOR moves rows k + 2, k + 3 by one group (and stays inside the six groups of such a row).
   static constexpr int GROUPS = CPR / 4;
-  static constexpr int GMASK = (GROUPS - 1) < 3 ? (GROUPS - 1) : 3;
-  __device__ static __forceinline__ int swz_m(int k) { return (k / RP256) & GMASK; }
+  static constexpr bool ROW_384 = KIND == OPK_MMAJOR && (ROW_BYTES % 256) == 128;
+  static constexpr int GMASK = ROW_384 ? 1 : ((GROUPS - 1) < 3 ? (GROUPS - 1) : 3);
+  __device__ static __forceinline__ int swz_m(int k) { return ROW_384 ? ((k >> 1) & 1) : ((k / RP256) & GMASK); }
   // ... and the two 32-byte halves of a 64-byte group trade places on every other block of 8 k rows, so
   // that the 16-lane groups of a transposing read for 16-row fragments (k, k + 8, ...) use both halves
-  static_assert((CPR & (CPR - 1)) == 0, "chunks per row must be a power of two");
+  static_assert(KIND == OPK_MMAJOR || (CPR & (CPR - 1)) == 0, "chunks per row must be a power of two");
+  static_assert(KIND != OPK_MMAJOR || ROW_384 || (GROUPS & (GROUPS - 1)) == 0, "M-major rows: a power of two of 64-byte groups, or 384 bytes");
+  static_assert(!ROW_384 || GROUPS % 2 == 0, "the group XOR of 384-byte rows pairs groups");
   static_assert(KIND != OPK_MMAJOR || CPR >= 4, "M-major tiles need at least 32 rows");
   static_assert(BYTES % 1024 == 0, "tile must be a whole number of DMA instructions");
   static_assert(!EXPAND || KIND != OPK_MMAJOR, "complex operands are K-major or complex-row tiles");

@@ -152,10 +152,10 @@ _MFMA_TILES = [
     ((64, 64, 32), (2, 2)),       # four stages; the one-wave instance (the tensor-contraction kernels have only that) is 1.5 - 2.7 times slower
 ]
 # Tiles with a side of 192: they fill the chip where 256 x 256 leaves CUs idle (3072^2: 192 tiles instead of 144,
-# 59 us instead of 72).  The swizzle of an LDS tile whose rows run along k needs a power of two along the other
-# index, so the 192 side must belong to an operand that is contiguous along k: B of an 'N' product (256 x 192),
-# A of a 'T' product (192 x 256).
-_MFMA_TILES_192 = [((256, 192, 64), (4, 2), "b_kmajor"), ((192, 256, 64), (2, 4), "a_kmajor")]
+# 59 us instead of 72).  Compiled per transpose: 256 x 192 for 'N','N', 'T','N' and 'N','T'; 192 x 256 for
+# 'T','N' and 'T','T' (the third entry says whether a transpose (a_kmajor, b_kmajor) has the tile).
+_MFMA_TILES_192 = [((256, 192, 64), (4, 2), lambda a_kmajor, b_kmajor: b_kmajor or not a_kmajor),
+                   ((192, 256, 64), (2, 4), lambda a_kmajor, b_kmajor: a_kmajor)]
 NUM_CUS = 256
 
 # measured winners by problem (filled by gemmkernels.tuning.install / load, or from the JSON file
@@ -168,7 +168,7 @@ _GETT_TILES = [(256, 256, 64), (128, 128, 64), (64, 64, 32)]
 
 
 def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: bool = False, planar: bool = False,
-                        a_kmajor: bool = False, b_kmajor: bool = False) -> NT:
+                        a_kmajor: bool = False, b_kmajor: bool = True) -> NT:
     """MI355X block shape: of the tiles of the table that divide the problem, the one with the shortest
     estimated launch (tiles per CU times the cost of a tile).  ``a_kmajor``: A is stored K x M ('T');
     ``b_kmajor``: B is stored K x N ('N'); they admit the tiles with a side of 192."""
@@ -188,7 +188,7 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
         return NT(M=t[0], N=t[1], K=t[2])
     # sizes need not be whole tiles when the layouts are the bounds-checked ones (the aligned kernels mask the
     # last tile row / column and zero the end of the last K tile)
-    table = [t for t, _ in _MFMA_TILES] + [t for t, _, need in _MFMA_TILES_192 if (a_kmajor if need == "a_kmajor" else b_kmajor)]
+    table = [t for t, _ in _MFMA_TILES] + [t for t, _, has in _MFMA_TILES_192 if has(a_kmajor, b_kmajor)]
     fitting = [t for t in table if not tile_sized or (M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0)]
     if gett:
         fitting = [t for t in fitting if t in _GETT_TILES]
@@ -201,6 +201,8 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
         tiles = -(-M // t[0]) * -(-N // t[1])
         rounds = -(-tiles // NUM_CUS)
         rate = _MFMA_TILE_RATE.get(t, 0.5)
+        if t == (256, 192, 64) and not a_kmajor and not b_kmajor:
+            rate = 0.78      # 'N','T': the 192 side is read with transposing LDS reads (3072^3: 69.7 us, 256 x 256: 72.6 us)
         if isinstance(rate, tuple):
             rate = rate[0] if rounds == 1 else rate[1]
         return rounds * t[0] * t[1] / rate

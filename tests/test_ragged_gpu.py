@@ -138,8 +138,8 @@ def test_full_size_4000(gpu):
     assert oracle.rel_frobenius(out[:, colsel], refc) <= 1e-3
 
 
-# tiles with a side of 192: only where the operand on that side is contiguous along k
-TILES_192 = [((256, 192, 64), (4, 2), [(False, False), (True, False)]), ((192, 256, 64), (2, 4), [(True, False), (True, True)])]
+# tiles with a side of 192 are compiled per transpose
+TILES_192 = [((256, 192, 64), (4, 2), [(False, False), (True, False), (False, True)]), ((192, 256, 64), (2, 4), [(True, False), (True, True)])]
 
 
 @pytest.mark.parametrize("block,waves,transposes", TILES_192)
@@ -166,6 +166,8 @@ def test_tiles_with_a_side_of_192(gpu, block, waves, transposes):
     # the default picks them where they fill the chip and only where the kernel has them
     from gemmkernels import default_block_shape
     op = Operator.MFMAOp[32, 32, 16, Float16, Float32]
-    assert default_block_shape(op, NT(M=3072, N=3072, K=3072), b_kmajor=True) == NT(M=256, N=192, K=64)
-    assert default_block_shape(op, NT(M=3072, N=3072, K=3072), a_kmajor=True) == NT(M=192, N=256, K=64)
-    assert default_block_shape(op, NT(M=3072, N=3072, K=3072)) == NT(M=256, N=256, K=64)
+    big = NT(M=3072, N=3072, K=3072)
+    assert default_block_shape(op, big) == NT(M=256, N=192, K=64)                                        # 'N','N'
+    assert default_block_shape(op, big, a_kmajor=False, b_kmajor=False) == NT(M=256, N=192, K=64)        # 'N','T'
+    assert default_block_shape(op, big, a_kmajor=True, b_kmajor=False) == NT(M=192, N=256, K=64)         # 'T','T'
+    assert default_block_shape(op, big, a_kmajor=True, b_kmajor=True) in (NT(M=256, N=192, K=64), NT(M=192, N=256, K=64))

@@ -39,7 +39,7 @@ def test_every_candidate_of_the_tuner_is_a_compiled_instance():
         assert f"{block[0]}x{block[1]}x{block[2]}_w{waves[0]}x{waves[1]}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
     # ... and nowhere else: the tuner skips it there
     with pytest.raises(gk.ConfigError):
-        tuning.mfma_config(384, 512, 256, False, True, (192, 256, 64), (2, 4), 4)
+        tuning.mfma_config(384, 512, 256, False, True, (192, 256, 64), (2, 4), 4)      # 'N','T' has 256 x 192 instead
 
 
 @pytest.mark.gpu
