@@ -5,6 +5,14 @@
 # (get_config, create_config, matmatmul!, mul!) keeps working on the lowered objects.  Julia is not
 # available in the build image of this library, so this file has not been executed there; the
 # tested host layer is the Python package next to it, which lowers the same structs field by field.
+#
+# Sizes that are not whole tiles: the reference's create_config puts such a product on Layout.ColMajor /
+# RowMajor (src/matmul.jl:121-156).  The library runs it on the aligned kernel of the configuration's block
+# shape all the same when A and B have 16-byte aligned columns, K is a multiple of 8 and M (N) is a multiple
+# of 8 along the contiguous index of A (B); otherwise on its bounds-checked kernel, which exists for the
+# 64 x 64 x 32 block only.  A create_config that wants the fast path for ragged sizes therefore keeps the
+# reference's layout rule and picks a block shape with a compiled aligned instance (128 x 128 x 64 on 4 x 2
+# warps, which is what the reference's heuristic arrives at for FP16 x FP16 -> FP32, is one).
 module GemmKernelsHIP
 
 using Libdl
