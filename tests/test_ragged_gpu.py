@@ -16,7 +16,7 @@ from oracle import oracle
 pytestmark = pytest.mark.gpu
 E = Transform.Elementwise
 TILES = [((256, 256, 64), (2, 4)), ((256, 256, 32), (2, 4)), ((256, 128, 64), (2, 2)), ((128, 256, 64), (2, 2)),
-         ((128, 128, 32), (2, 2)), ((128, 128, 64), (2, 2)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2))]
+         ((128, 128, 32), (2, 2)), ((128, 128, 64), (2, 2)), ((128, 128, 64), (4, 2)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2))]
 
 
 def checked_config(M, N, K, ta, tb, block, waves, zero_c=False, cd=Float32):
