@@ -171,3 +171,28 @@ def test_tiles_with_a_side_of_192(gpu, block, waves, transposes):
     assert default_block_shape(op, big, a_kmajor=False, b_kmajor=False) == NT(M=256, N=192, K=64)        # 'N','T'
     assert default_block_shape(op, big, a_kmajor=True, b_kmajor=False) == NT(M=192, N=256, K=64)         # 'T','T'
     assert default_block_shape(op, big, a_kmajor=True, b_kmajor=True) in (NT(M=256, N=192, K=64), NT(M=192, N=256, K=64))
+
+
+def test_random_shapes_through_the_blas_level_front_end(gpu):
+    """Sixty seeded shapes (multiples of 8, some with an odd M, which only a K-major A lets onto the aligned
+    kernels), random transposes, alpha and beta, against the float64 product."""
+    from gemmkernels.matmul import matmatmul_plan
+    rs = np.random.RandomState(7)
+    aligned_kernel_runs = 0
+    for it in range(60):
+        M, N, K = (int(rs.randint(1, 90)) * 8 for _ in range(3))
+        if it % 5 == 0:
+            M = int(rs.randint(1, 700))
+        if it % 7 == 0:
+            K = int(rs.randint(1, 40)) * 8
+        ta, tb = bool(rs.randint(2)), bool(rs.randint(2))
+        alpha, beta = float(np.float16(rs.rand())), float(rs.choice([0.0, 1.0, -0.5]))
+        a, b, c = operands(M, N, K, ta, tb, 5000 + 10 * it)
+        C = gk.colmajor(c)
+        p = matmatmul_plan(C, "T" if ta else "N", "T" if tb else "N", gk.colmajor(a), gk.colmajor(b), alpha, beta)
+        print("case", it, (M, N, K), ta, tb, alpha, beta, p.kernel_names, flush=True)
+        p()
+        torch.cuda.synchronize()
+        aligned_kernel_runs += "checked" not in p.kernel_names[0]
+        assert oracle.rel_frobenius(gk.to_numpy(C), oracle.gemm_f64(a, b, c, alpha, beta, ta, tb)) <= 1e-3, (it, M, N, K, ta, tb)
+    assert aligned_kernel_runs >= 50
