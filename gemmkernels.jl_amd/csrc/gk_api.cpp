@@ -673,8 +673,7 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
       t_allow_ragged_fast = true;
       if (rc != GK_OK) return rc;
     } else {
-      out->ragged = (conf->matmul_shape.M % conf->block_shape.M) != 0 || (conf->matmul_shape.N % conf->block_shape.N) != 0 ||
-                    (conf->matmul_shape.K % conf->block_shape.K) != 0;
+      out->ragged = (conf->matmul_shape.K % conf->block_shape.K) != 0;
     }
   }
 
@@ -769,7 +768,7 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
     // the bounds-checked kernel takes its K range from the launch arguments, the aligned kernels have
     // instances of their own for it
     gk::FamilyFn sk_fn = L.key.family == gk::FAMILY_MFMA_CHECKED ? fn : gk::family_mfma_splitk;
-    // (the K-split instances of the aligned kernel have no masks for tiles over the edge)
+    // (the K-split instances of the aligned kernel mask tiles over M and N but take no partial K tile)
     if (slices > 1 && !L.ragged && sk_fn && sk_fn(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
       const int per = (kt + slices - 1) / slices;
       slices = (kt + per - 1) / per;

@@ -16,7 +16,7 @@ struct Launch {
   gk::InstanceInfo info;
   gk::GemmArgs args;
   int gx, gy;
-  bool ragged;      // an aligned kernel runs bounds-checked layouts and some tile sticks out over M or N
+  bool ragged;      // an aligned kernel runs bounds-checked layouts and the last K tile is a partial one
 };
 
 int prepare_launch(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,

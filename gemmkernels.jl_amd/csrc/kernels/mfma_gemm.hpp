@@ -360,7 +360,9 @@ struct MfmaGemmConfig {
   // tile (the host asks for it only with 16-byte aligned columns, M or N a multiple of 8 where that index is
   // the contiguous one of A or B, and K a multiple of 8): loads are clamped, the C load and the D store
   // masked, the part of the last K tile beyond K zeroed in LDS
-  static constexpr bool RAGGED_OK = !GETT_ && FIX_ == FIX_NONE && !SPLITK_;
+  // (the K-split instances take tiles over M and N, not a partial K tile)
+  static constexpr bool RAGGED_OK = !GETT_ && FIX_ == FIX_NONE;
+  static constexpr bool RAGGED_K_OK = RAGGED_OK && !SPLITK_;
   static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
   static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
@@ -956,7 +958,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       });
     }
   }
-  if constexpr (Cfg::RAGGED_OK) {
+  if constexpr (Cfg::RAGGED_K_OK) {
     // --- a last, partial K tile (K not a multiple of BLOCK_K; K a multiple of 8) -----------------------
     // Outside the pipeline: the tile is fetched with its k coordinates clamped to the valid ones, the LDS
     // slots beyond K are set to zero by the lanes that fetched them, and the k-steps that hold valid
@@ -1087,7 +1089,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           // last bits of the sum, is not fixed)
           float* dp = (float*)args.d + off;
 #pragma unroll
-          for (int v = 0; v < NV; ++v) atomicAdd(&dp[(long long)vcol(v) * ns], x[v]);
+          for (int v = 0; v < NV; ++v) {
+            if constexpr (Cfg::RAGGED_OK) {
+              if (ragged && (mrow + MI * fi >= args.M || ncol + MI * fj + vcol(v) >= args.N)) continue;   // over the edge
+            }
+            atomicAdd(&dp[(long long)vcol(v) * ns], x[v]);
+          }
           continue;
         }
       }

@@ -79,3 +79,27 @@ def test_blas_entry_picks_the_k_split_kernel_for_skinny_products(gpu):
     gk.matmatmul_(C, "N", "N", A, B, 0.5, 2.0)
     torch.cuda.synchronize()
     assert oracle.rel_frobenius(gk.to_numpy(C), oracle.gemm_f64(a, b, c, 0.5, 2.0)) <= TOL
+
+
+@pytest.mark.parametrize("beta", [1.0, 0.5, 0.0])
+def test_skinny_products_with_tiles_over_the_edge_are_split_too(gpu, beta):
+    """N = 100 columns of a K x N B (contiguous along k, so any N is fine), M a multiple of 8 that is not a
+    whole number of tiles, K whole tiles: the K-split instances mask the tiles over the edge; in place with
+    beta = 1 it is one launch of atomic adds."""
+    import torch
+    from gemmkernels import rng
+    from gemmkernels.matmul import matmatmul_plan
+    from oracle import oracle
+    M, N, K = 1000, 100, 4096
+    a = rng.matrix("upm1_f16", 8101, (M, K)); b = rng.matrix("upm1_f16", 8102, (K, N)); c = rng.matrix("upm1_f32", 8103, (M, N))
+    ld, cols = M + 8, N + 3
+    full = gk.colmajor(np.asfortranarray(np.full((ld, cols), 555.0, np.float32)))
+    C = full[:M, :N]
+    C.copy_(gk.colmajor(c))
+    p = matmatmul_plan(C, "N", "N", gk.colmajor(a), gk.colmajor(b), 1.0, beta)
+    assert "checked" not in p.kernel_names[0], p.kernel_names
+    p()
+    torch.cuda.synchronize()
+    out = full.cpu().numpy()
+    assert (out[M:, :] == 555.0).all() and (out[:, N:] == 555.0).all()
+    assert oracle.rel_frobenius(out[:M, :N], oracle.gemm_f64(a, b, c, 1.0, beta, False, False)) <= 1e-3
