@@ -26,7 +26,10 @@
  * brute force on tiny shapes and linearity; layouts against index-distinct prime fixtures; the
  * integer element types (Int16 / Int32 / Int64, configs/configs.jl:495-497) against exact Python
  * integers reduced modulo 2^bits with magnitudes that overflow; Float32 -> Float64 and Float64
- * against numpy float64 matmul on dyadic inputs (bit-exact) and a math.fma chain.
+ * against numpy float64 matmul on dyadic inputs (bit-exact) and a math.fma chain; every elementwise
+ * op (float and integer evaluation) against hand-typed value tables and numpy closed forms through an
+ * identity product; the bfloat16 conversions exhaustively against torch.bfloat16; the dual-number
+ * product against a0*b0 and a0*b1 + a1*b0 in float64.
  */
 #include <math.h>
 #include <stdint.h>
@@ -165,6 +168,11 @@ static void store_scalar(int dtype, void* p, int64_t idx, double v) {
 /* exported for the tests that pin the conversions */
 uint16_t gko_double_to_half(double x) { return double_to_half(x); }
 float gko_half_to_float(uint16_t h) { return half_to_float(h); }
+uint16_t gko_float_to_bf16(float f) { return float_to_bf16(f); }
+float gko_bf16_to_float(uint16_t h) { return bf16_to_float(h); }
+/* vector forms of the same two functions (the exhaustive tests convert 2^16 x several patterns) */
+void gko_float_to_bf16_n(const float* x, uint16_t* out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = float_to_bf16(x[i]); }
+void gko_bf16_to_float_n(const uint16_t* x, float* out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = bf16_to_float(x[i]); }
 
 /* ---------------- transforms ---------------- */
 /* fp32 evaluation (fp64 when wide != 0), no contraction: one rounding per op */

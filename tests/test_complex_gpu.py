@@ -80,6 +80,12 @@ def test_dual_numbers(gpu, block):
     a0, a1, b0, b1 = (x.astype(np.float64) for x in (a[0], a[1], b[0], b[1]))
     assert oracle.rel_frobenius(d[0], a0 @ b0) <= TOL
     assert oracle.rel_frobenius(d[1], a0 @ b1 + a1 @ b0) <= TOL
+    # and against the oracle's dual-number product (itself pinned against these float64 forms on the CPU)
+    ref = np.zeros((2, M, N), np.float32, order="F")
+    p = helpers.oracle_problem(conf, (M, K, M, M))
+    assert p.op_kind == oracle.OP_DUAL
+    oracle.matmul(p, a, b, None, ref)
+    assert oracle.rel_frobenius(d[0], ref[0]) <= TOL and oracle.rel_frobenius(d[1], ref[1]) <= TOL
 
 
 def test_config4a_full_size(gpu):

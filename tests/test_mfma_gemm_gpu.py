@@ -201,9 +201,16 @@ def test_bf16(gpu, ta, tb, d16):
     d = helpers.run_gpu(conf, a, b, c, (M, N), d_dtype=torch.bfloat16 if d16 else torch.float32, kernel=Kernel.matmul_pipelined)
     ref = helpers.run_oracle(conf, a, b, c, (M, N), d_dtype=np.uint16 if d16 else np.float32)
     if d16:
+        # same rounding (to nearest even, once, at the store) as the oracle: the bit patterns differ only where the
+        # two fp32 sums straddle a rounding boundary -- rarely, and then by one unit in the last place.  Truncation
+        # or round-half-up would differ in about half of the elements.
+        got_bits = gk.bf16_bits(d.astype(np.float32)).astype(np.int32)
+        ref_bits = ref.astype(np.int32)
+        diff = np.abs(got_bits - ref_bits)
+        assert diff.max() <= 1 and (diff != 0).mean() < 0.01, (diff.max(), (diff != 0).mean())
         ref = gk.bf16_values(ref)
-    tol = 4e-3 if d16 else TOL        # a BFloat16 result carries 2^-9 relative rounding per element
-    assert oracle.rel_frobenius(d, ref) <= tol
+    tol = 4e-3 if d16 else TOL        # against float64, a BFloat16 result carries 2^-9 relative rounding per element
+    assert oracle.rel_frobenius(d, ref) <= (1e-3 if d16 else tol)
     A, B = gk.bf16_values(a), gk.bf16_values(b)
     C = gk.bf16_values(c) if d16 else c
     assert oracle.rel_frobenius(d, oracle.gemm_f64(A, B, C, 1.0, 1.0, ta, tb)) <= tol

@@ -273,3 +273,206 @@ def test_float64_accumulation_of_float32_inputs():
             break
     if acc is not None:
         assert d[2, 1] == acc
+
+
+# ------------------------------------------------------------------------------------------------
+# Elementwise ops (reference src/transform.jl:20-30 applies an arbitrary f; the closed vocabulary here is
+# scale, add, relu, neg, abs, clamp, square).  Each op is pushed through oracle.matmul on a product with
+# B = I, so that D[i, j] = f(A[i, j]) exactly (every other term of the sum is f(A[i, k]) * 0), and compared
+# with values typed by hand and with numpy closed forms written from the definition of the op.
+# ------------------------------------------------------------------------------------------------
+
+def _through_identity(a32, hooks, hook_on="global_to_shared_a"):
+    n = a32.shape[0]
+    eye = np.asfortranarray(np.eye(n, dtype=np.float32))
+    d = np.zeros((n, n), np.float32, order="F")
+    p = plain(n, n, n, dt=F32, cd=F32, zero_c=True)
+    p.transforms = {hook_on: hooks}
+    if hook_on.endswith("_c"):
+        # the hook under test sits on C: D = f(C) + 0 * I
+        p = plain(n, n, n, dt=F32, cd=F32)
+        p.transforms = {hook_on: hooks}
+        oracle.matmul(p, np.zeros_like(eye), eye, np.asfortranarray(a32), d)
+    else:
+        oracle.matmul(p, np.asfortranarray(a32), eye, None, d)
+    return d
+
+
+_VALUES = np.array([[-2.0, -0.5, 0.25, 3.0],
+                    [0.75, -1.25, 0.0, 1.5],
+                    [-3.5, 2.0, 0.5, -0.125],
+                    [1.0, -1.0, 4.0, -4.0]], dtype=np.float32)
+
+
+def test_each_elementwise_op_against_hand_typed_values():
+    T = oracle
+    # add 0.75
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_ADD, 0.75, 0.0)]),
+                          np.array([[-1.25, 0.25, 1.0, 3.75], [1.5, -0.5, 0.75, 2.25], [-2.75, 2.75, 1.25, 0.625], [1.75, -0.25, 4.75, -3.25]], np.float32))
+    # neg
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_NEG, 0.0, 0.0)]),
+                          np.array([[2.0, 0.5, -0.25, -3.0], [-0.75, 1.25, -0.0, -1.5], [3.5, -2.0, -0.5, 0.125], [-1.0, 1.0, -4.0, 4.0]], np.float32))
+    # abs
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_ABS, 0.0, 0.0)]),
+                          np.array([[2.0, 0.5, 0.25, 3.0], [0.75, 1.25, 0.0, 1.5], [3.5, 2.0, 0.5, 0.125], [1.0, 1.0, 4.0, 4.0]], np.float32))
+    # clamp to [0.5, 2] (lower bound above zero; values below, inside, on and above the bounds)
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_CLAMP, 0.5, 2.0)]),
+                          np.array([[0.5, 0.5, 0.5, 2.0], [0.75, 0.5, 0.5, 1.5], [0.5, 2.0, 0.5, 0.5], [1.0, 0.5, 2.0, 0.5]], np.float32))
+    # clamp to [-1, -0.25] (both bounds negative: a swapped pair of bounds or a swapped comparison fails here)
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_CLAMP, -1.0, -0.25)]),
+                          np.array([[-1.0, -0.5, -0.25, -0.25], [-0.25, -1.0, -0.25, -0.25], [-1.0, -0.25, -0.25, -0.25], [-0.25, -1.0, -0.25, -1.0]], np.float32))
+    # square
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_SQUARE, 0.0, 0.0)]),
+                          np.array([[4.0, 0.25, 0.0625, 9.0], [0.5625, 1.5625, 0.0, 2.25], [12.25, 4.0, 0.25, 0.015625], [1.0, 1.0, 16.0, 16.0]], np.float32))
+    # relu and scale, for completeness of the table
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_RELU, 0.0, 0.0)]), np.maximum(_VALUES, 0))
+    assert np.array_equal(_through_identity(_VALUES, [(T.T_SCALE, -1.5, 0.0)]), _VALUES * np.float32(-1.5))
+
+
+@pytest.mark.parametrize("hook", ["global_to_shared_a", "shared_to_regs_a", "global_to_shared_c", "shared_to_regs_c",
+                                  "regs_to_shared_d", "shared_to_global_d"])
+def test_elementwise_ops_against_numpy_closed_forms_on_every_hook_kind(hook):
+    """Random fp32 values (not dyadic: the roundings of every op matter), one op at a time and a chain of four,
+    through hooks on A, on C and on D."""
+    T = oracle
+    rs = np.random.RandomState(7)
+    x = np.asfortranarray((rs.standard_normal((4, 4)) * 3).astype(np.float32))
+    f32 = np.float32
+    cases = [
+        ([(T.T_ADD, 0.3, 0.0)], lambda v: v + f32(0.3)),
+        ([(T.T_NEG, 0.0, 0.0)], lambda v: -v),
+        ([(T.T_ABS, 0.0, 0.0)], lambda v: np.abs(v)),
+        ([(T.T_CLAMP, 0.4, 1.7)], lambda v: np.minimum(np.maximum(v, f32(0.4)), f32(1.7))),
+        ([(T.T_SQUARE, 0.0, 0.0)], lambda v: v * v),
+        # scale by 3, subtract 1, absolute value, clamp to [0.25, 2]: one fp32 rounding after each op
+        ([(T.T_SCALE, 3.0, 0.0), (T.T_ADD, -1.0, 0.0), (T.T_ABS, 0.0, 0.0), (T.T_CLAMP, 0.25, 2.0)],
+         lambda v: np.minimum(np.maximum(np.abs((v * f32(3.0)).astype(f32) + f32(-1.0)), f32(0.25)), f32(2.0))),
+        # square, negate, add 2.5, relu
+        ([(T.T_SQUARE, 0.0, 0.0), (T.T_NEG, 0.0, 0.0), (T.T_ADD, 2.5, 0.0), (T.T_RELU, 0.0, 0.0)],
+         lambda v: np.maximum((-(v * v).astype(f32)) + f32(2.5), f32(0))),
+    ]
+    for ops, closed in cases:
+        got = _through_identity(x, ops, hook)
+        want = closed(x).astype(np.float32)
+        assert np.array_equal(got, want), (hook, ops)
+    # the clamp really cut on both sides, the chain really used all four ops
+    assert (x < 0.4).any() and (x > 1.7).any() and ((x > 0.4) & (x < 1.7)).any()
+
+
+@pytest.mark.parametrize("code,np_t,bits", [(oracle.I16, np.int16, 16), (oracle.I32, np.int32, 32), (oracle.I64, np.int64, 64)])
+def test_integer_elementwise_ops_wrap(code, np_t, bits):
+    """The integer evaluation of every op (Julia integer arithmetic wraps; abs and neg of typemin stay typemin)
+    against exact Python integers reduced modulo 2^bits, with magnitudes that overflow, through B = I."""
+    T = oracle
+    mod, half = 1 << bits, 1 << (bits - 1)
+    lo, hi = -half, half - 1
+    big = {16: 200, 32: 50000, 64: 3_100_000_000}[bits]
+    vals = [lo, hi, -big, big, -3, 0, 7, big + 1, -big - 5, 1, -1, 12, lo + 1, hi - 1, 100, -100]
+    a = np.asfortranarray(np.array(vals, dtype=object).reshape(4, 4).astype(np_t))
+    eye = np.asfortranarray(np.eye(4, dtype=np_t))
+    wrap = lambda v: (v + half) % mod - half
+    scale = {16: 300, 32: 70000, 64: 16_777_216}[bits]       # exactly representable as a binary32 parameter
+    cases = [
+        ([(T.T_SCALE, float(scale), 0.0)], lambda v: wrap(v * scale)),
+        ([(T.T_ADD, float(scale), 0.0)], lambda v: wrap(v + scale)),
+        ([(T.T_NEG, 0.0, 0.0)], lambda v: wrap(-v)),
+        ([(T.T_ABS, 0.0, 0.0)], lambda v: wrap(abs(v))),
+        ([(T.T_RELU, 0.0, 0.0)], lambda v: max(v, 0)),
+        ([(T.T_CLAMP, 5.0, 100.0)], lambda v: min(max(v, 5), 100)),
+        ([(T.T_CLAMP, -100.0, -5.0)], lambda v: min(max(v, -100), -5)),
+        ([(T.T_SQUARE, 0.0, 0.0)], lambda v: wrap(v * v)),
+        ([(T.T_SQUARE, 0.0, 0.0), (T.T_ADD, 3.0, 0.0), (T.T_NEG, 0.0, 0.0), (T.T_SCALE, float(scale), 0.0)],
+         lambda v: wrap(wrap(-wrap(wrap(v * v) + 3)) * scale)),
+    ]
+    overflowed = False
+    for ops, closed in cases:
+        for hook in ("global_to_shared_a", "shared_to_global_d"):
+            p = plain(4, 4, 4, dt=code, cd=code, zero_c=True)
+            p.transforms = {hook: ops}
+            d = np.zeros((4, 4), np_t, order="F")
+            oracle.matmul(p, a, eye, None, d)
+            for i in range(4):
+                for j in range(4):
+                    v = int(a[i, j])
+                    assert int(d[i, j]) == closed(v), (ops, hook, v)
+        overflowed |= any(not (lo <= int(v) * scale <= hi) for v in vals)
+    assert overflowed
+
+
+def test_bfloat16_conversions_match_torch_exhaustively():
+    """float -> bfloat16 is round-to-nearest-even on the upper 16 bits: every upper half with the lower-half
+    patterns just below a tie, on the tie (even and odd upper halves both occur), just above it, 0 and all ones,
+    against torch.bfloat16; bfloat16 -> float for all 2^16 patterns."""
+    import ctypes
+    import torch
+    lib = oracle.lib()
+    lib.gko_float_to_bf16_n.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    lib.gko_bf16_to_float_n.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    upper = np.arange(65536, dtype=np.uint32) << 16
+    for low in (0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF, 0x4000, 0xC000):
+        bits = (upper | np.uint32(low)).astype(np.uint32)
+        x = bits.view(np.float32).copy()
+        out = np.zeros(x.size, np.uint16)
+        lib.gko_float_to_bf16_n(x.ctypes.data, out.ctypes.data, x.size)
+        want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        nan = np.isnan(x)
+        assert np.array_equal(out[~nan], want[~nan]), hex(low)
+        # NaNs stay NaNs (payloads are not compared)
+        back = (out[nan].astype(np.uint32) << 16).view(np.float32)
+        assert np.isnan(back).all()
+    h = np.arange(65536, dtype=np.uint16)
+    f = np.zeros(65536, np.float32)
+    lib.gko_bf16_to_float_n(h.ctypes.data, f.ctypes.data, h.size)
+    want = torch.from_numpy(h.view(np.int16)).view(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(f.view(np.uint32), want.view(np.uint32))
+    # the tie cases tell round-to-nearest-even from truncation and from round-half-up
+    assert lib.gko_float_to_bf16_n is not None
+    one_tie_even = np.array([0x3F808000], np.uint32).view(np.float32)      # 1.00390625: tie, even upper half -> stays 0x3F80
+    one_tie_odd = np.array([0x3F818000], np.uint32).view(np.float32)       # tie, odd upper half -> rounds up to 0x3F82
+    o = np.zeros(1, np.uint16)
+    lib.gko_float_to_bf16_n(one_tie_even.ctypes.data, o.ctypes.data, 1); assert o[0] == 0x3F80
+    lib.gko_float_to_bf16_n(one_tie_odd.ctypes.data, o.ctypes.data, 1); assert o[0] == 0x3F82
+
+
+def test_bfloat16_gemm_rounds_its_output_once():
+    """BF16 multiplicands, BF16 D: the oracle's result equals the float64 product rounded once by torch."""
+    import torch
+    M, N, K = 6, 5, 8
+    rs = np.random.RandomState(3)
+    af = (rs.randint(-128, 128, size=(M, K)) / 64.0).astype(np.float32)      # exactly representable in bfloat16
+    bf = (rs.randint(-128, 128, size=(K, N)) / 64.0).astype(np.float32)
+    to_bits = lambda x: np.asfortranarray((x.view(np.uint32) >> 16).astype(np.uint16))
+    p = plain(M, N, K, dt=BF16, cd=F32, zero_c=True)
+    p.d = Layout(oracle.L_COL, BF16, M)
+    d = np.zeros((M, N), np.uint16, order="F")
+    oracle.matmul(p, to_bits(np.asfortranarray(af)), to_bits(np.asfortranarray(bf)), None, d)
+    exact = af.astype(np.float64) @ bf.astype(np.float64)                   # exact: small dyadic values
+    want = torch.from_numpy(exact.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(d, want)
+
+
+def test_dual_numbers_against_float64():
+    """WMMADualOp (reference src/operator.jl:359-372): (a0 + a1 e)(b0 + b1 e) = a0 b0 + (a0 b1 + a1 b0) e, no
+    a1 b1 term and no sign flip.  Against float64 matmuls of the parts; a complex product of the same data differs."""
+    M, N, K = 6, 5, 7
+    a = rand((M, K, 2), np.float16, 31)
+    b = rand((K, N, 2), np.float16, 32)
+    c = rand((M, N, 2), np.float32, 33)
+    inter = lambda x: np.ascontiguousarray(np.transpose(x, (1, 0, 2)))       # column-major interleaved pairs
+    def run(op, with_c):
+        p = Problem(M, N, K, Layout(oracle.L_ICOL, F16, M), Layout(oracle.L_ICOL, F16, K),
+                    Layout(oracle.L_ICOL, F32, M) if with_c else Layout(oracle.L_ZERO, F32), Layout(oracle.L_ICOL, F32, M),
+                    compute_dtype=F16, accum_dtype=F32, op_kind=op)
+        d = np.zeros((N, M, 2), np.float32)
+        oracle.matmul(p, inter(a), inter(b), inter(c) if with_c else None, d)
+        return np.transpose(d, (1, 0, 2))
+    a0, a1 = a[..., 0].astype(np.float64), a[..., 1].astype(np.float64)
+    b0, b1 = b[..., 0].astype(np.float64), b[..., 1].astype(np.float64)
+    for with_c in (False, True):
+        got = run(oracle.OP_DUAL, with_c)
+        c0 = c[..., 0].astype(np.float64) if with_c else 0.0
+        c1 = c[..., 1].astype(np.float64) if with_c else 0.0
+        # dyadic inputs with 11 significant bits and K = 7: every partial sum is exact in fp32
+        assert np.array_equal(got[..., 0].astype(np.float64), a0 @ b0 + c0)
+        assert np.array_equal(got[..., 1].astype(np.float64), a0 @ b1 + a1 @ b0 + c1)
+    assert not np.array_equal(run(oracle.OP_COMPLEX, False)[..., 0], run(oracle.OP_DUAL, False)[..., 0])
