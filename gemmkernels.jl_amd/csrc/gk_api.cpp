@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
@@ -95,10 +96,8 @@ bool transforms_present(const gk_transforms* t) {
 // kernel runs it: the tiles that stick out over M or N clamp their loads and mask their C loads and D
 // stores, a last partial K tile is zeroed beyond K in LDS.  Decided from the configuration (a leading dimension of 0 stands for a dense operand); the
 // launcher falls back to the bounds-checked kernel when the pointers themselves turn out misaligned.
-thread_local bool t_allow_ragged_fast = true;
-
 bool ragged_fast_path(const gk_config* c) {
-  if (!t_allow_ragged_fast || c->op.kind != GK_OP_MFMA) return false;
+  if (c->op.kind != GK_OP_MFMA) return false;
   const gk_layout& la = c->global_a_layout; const gk_layout& lb = c->global_b_layout;
   const gk_layout& lc = c->global_c_layout; const gk_layout& ld = c->global_d_layout;
   auto plain = [](int k) { return k == GK_LAYOUT_COL_MAJOR || k == GK_LAYOUT_ROW_MAJOR || k == GK_LAYOUT_ALIGNED_COL_MAJOR || k == GK_LAYOUT_ALIGNED_ROW_MAJOR; };
@@ -118,7 +117,8 @@ bool ragged_fast_path(const gk_config* c) {
 }
 
 // Builds the run-time key of the kernel instance for a configuration.
-int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key) {
+// allow_ragged_fast = false: bounds-checked layouts run on the bounds-checked kernel whatever their alignment.
+int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
   memset(key, 0, sizeof(*key));
   const int ak = c->global_a_layout.kind, bk = c->global_b_layout.kind;
   const int ck = c->global_c_layout.kind, dk = c->global_d_layout.kind;
@@ -128,7 +128,7 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
     case GK_OP_MFMA:
       if (ak == GK_LAYOUT_DIAGONAL) key->family = gk::FAMILY_DIAGONAL;
       else if (any_gett) key->family = gk::FAMILY_GETT;
-      else if (any_checked && !ragged_fast_path(c)) key->family = gk::FAMILY_MFMA_CHECKED;
+      else if (any_checked && !(allow_ragged_fast && ragged_fast_path(c))) key->family = gk::FAMILY_MFMA_CHECKED;
       else key->family = gk::FAMILY_MFMA;
       break;
     case GK_OP_FPU:
@@ -285,18 +285,17 @@ gk::FamilyFn family_fn(const gk::InstanceKey& key) {
   }
 }
 
-int find_instance(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, gk::InstanceInfo* info) {
-  int rc = make_key(c, t, e, key);
+int find_instance(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, gk::InstanceInfo* info,
+                  bool allow_ragged_fast = true) {
+  int rc = make_key(c, t, e, key, allow_ragged_fast);
   if (rc != GK_OK) return rc;
   gk::FamilyFn fn = family_fn(*key);
   gk::GemmArgs dummy;
   memset(&dummy, 0, sizeof(dummy));
   hipError_t err = hipSuccess;
-  if (key->family == gk::FAMILY_MFMA && t_allow_ragged_fast && ragged_fast_path(c) && (!fn || !fn(*key, dummy, dim3(1), nullptr, 0, info, &err))) {
+  if (key->family == gk::FAMILY_MFMA && allow_ragged_fast && ragged_fast_path(c) && (!fn || !fn(*key, dummy, dim3(1), nullptr, 0, info, &err))) {
     // no aligned instance of this tile: the bounds-checked kernel after all
-    t_allow_ragged_fast = false;
-    rc = make_key(c, t, e, key);
-    t_allow_ragged_fast = true;
+    rc = make_key(c, t, e, key, false);
     if (rc != GK_OK) return rc;
     fn = family_fn(*key);
   }
@@ -352,7 +351,7 @@ int validate_gett(const gk_config* c) {
 
 // All checks that need no pointers; reference src/config.jl:203-275 then src/matmul.jl:28-41.
 int validate_config(const gk_config* c, int kernel, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key,
-                    gk::InstanceInfo* info, const gk::InstanceInfo* custom = nullptr) {
+                    gk::InstanceInfo* info, const gk::InstanceInfo* custom = nullptr, bool allow_ragged_fast = true) {
   if (!c) return fail(GK_ERR_INVALID_ARGUMENT, "config is NULL");
   const gk_shape& g = c->matmul_shape;
   const gk_shape& b = c->block_shape;
@@ -504,10 +503,10 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   // the instance that would run; its LDS request is what Kernel.shmem_size returns
   int rc = GK_OK;
   if (custom) {      // a kernel specialised at run time: its resources are known to the caller
-    rc = make_key(c, t, e, key);
+    rc = make_key(c, t, e, key, allow_ragged_fast);
     *info = *custom;
   } else {
-    rc = find_instance(c, t, e, key, info);
+    rc = find_instance(c, t, e, key, info, allow_ragged_fast);
   }
   if (rc != GK_OK) return rc;
 
@@ -622,23 +621,42 @@ int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const
   return GK_OK;
 }
 
+}  // extern "C"
+
+namespace {
+// bytes of a rows x cols tile in a shared layout: Layout.physical_size (src/layout.jl:76, 113, 152,
+// 194, 246, 342-345, 381-383): padding goes to the leading physical dimension, planar complex
+// layouts hold two planes, interleaved ones two reals per element
+long long shared_tile_bytes(const gk_layout* l, long long rows, long long cols) {
+  const bool row = is_row_major(l->kind) || l->kind == GK_LAYOUT_SPLIT_ROW_MAJOR;
+  long long lead = row ? cols : rows, other = row ? rows : cols;
+  long long n = (lead + l->pad) * other;
+  if (l->kind == GK_LAYOUT_SPLIT_COL_MAJOR || l->kind == GK_LAYOUT_SPLIT_ROW_MAJOR ||
+      l->kind == GK_LAYOUT_INTERLEAVED_COL_MAJOR || l->kind == GK_LAYOUT_INTERLEAVED_ROW_MAJOR)
+    n *= 2;
+  return n * dtype_size(l->eltype);
+}
+}  // namespace
+
+extern "C" {
+
+int64_t gk_reference_shmem_size(const gk_config* conf) {
+  if (!conf) { fail(GK_ERR_INVALID_ARGUMENT, "config is NULL"); return -1; }
+  const gk_layout* ls[4] = {&conf->shared_a_layout, &conf->shared_b_layout, &conf->shared_c_layout, &conf->shared_d_layout};
+  for (const gk_layout* l : ls)
+    if (!valid_layout_kind(l->kind) || dtype_size(l->eltype) == 0) { fail(GK_ERR_INVALID_ARGUMENT, "unknown layout kind or element type"); return -1; }
+  const gk_shape& b = conf->block_shape;
+  const long long size_a = shared_tile_bytes(ls[0], b.M, b.K), size_b = shared_tile_bytes(ls[1], b.K, b.N);
+  const long long size_c = shared_tile_bytes(ls[2], b.M, b.N), size_d = shared_tile_bytes(ls[3], b.M, b.N);
+  return std::max(size_c, std::max(size_a + size_b, size_d));
+}
+
 int gk_heuristic_block_shape(const gk_layout* sa, const gk_layout* sb, const gk_layout* sc, const gk_layout* sd, gk_shape* out) {
   if (!sa || !sb || !sc || !sd || !out) return fail(GK_ERR_INVALID_ARGUMENT, "NULL argument");
   const gk_layout* ls[4] = {sa, sb, sc, sd};
   for (const gk_layout* l : ls)
     if (!valid_layout_kind(l->kind) || dtype_size(l->eltype) == 0) return fail(GK_ERR_INVALID_ARGUMENT, "unknown layout kind or element type");
-  // bytes of a rows x cols tile in a shared layout: Layout.physical_size (src/layout.jl:76, 113, 152,
-  // 194, 246, 342-345, 381-383): padding goes to the leading physical dimension, planar complex
-  // layouts hold two planes, interleaved ones two reals per element
-  auto nbytes = [](const gk_layout* l, long long rows, long long cols) -> long long {
-    const bool row = is_row_major(l->kind) || l->kind == GK_LAYOUT_SPLIT_ROW_MAJOR;
-    long long lead = row ? cols : rows, other = row ? rows : cols;
-    long long n = (lead + l->pad) * other;
-    if (l->kind == GK_LAYOUT_SPLIT_COL_MAJOR || l->kind == GK_LAYOUT_SPLIT_ROW_MAJOR ||
-        l->kind == GK_LAYOUT_INTERLEAVED_COL_MAJOR || l->kind == GK_LAYOUT_INTERLEAVED_ROW_MAJOR)
-      n *= 2;
-    return n * dtype_size(l->eltype);
-  };
+  auto nbytes = shared_tile_bytes;
   const long long limit = 64 * 1024;
   long long M = 1, N = 1, K = 1;
   for (;;) {     // src/config.jl:104-110
@@ -668,9 +686,7 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
   if (key.family == gk::FAMILY_MFMA && ragged_fast_path(conf)) {
     if ((((uintptr_t)a | (uintptr_t)b) & 15u) != 0) {
       // bounds-checked layouts with misaligned operands: the kernel that takes anything
-      t_allow_ragged_fast = false;
-      rc = validate_config(conf, kernel, transforms, epilogue, &key, &info, custom);
-      t_allow_ragged_fast = true;
+      rc = validate_config(conf, kernel, transforms, epilogue, &key, &info, custom, false);
       if (rc != GK_OK) return rc;
     } else {
       out->ragged = (conf->matmul_shape.K % conf->block_shape.K) != 0;

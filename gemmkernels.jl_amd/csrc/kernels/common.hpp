@@ -128,8 +128,10 @@ __host__ __device__ inline void cta_swizzle(int kind, int param, int bx, int by,
       break;
     case SWZ_XCD: {
       const int total = nbm * nbn;
-      int r = bx;
-      if (total % 8 == 0) r = (bx % 8) * (total / 8) + bx / 8;
+      // ids x, x + 8, x + 16, ... run on XCD x: XCD x holds total / 8 of them, one more when x < total % 8;
+      // the ids of one XCD become consecutive
+      const int x = bx % 8, q = total / 8, rem = total % 8;
+      const int r = x * q + (x < rem ? x : rem) + bx / 8;
       const int g = param > 0 ? param : 1;
       const int width = g * nbn;
       const int group = r / width;
@@ -270,10 +272,6 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-#ifdef GK_ABLATE_BARRIER
-__device__ __forceinline__ void block_barrier() { asm volatile("" ::: "memory"); }   // development aid (timing only, wrong results)
-#else
 __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
-#endif
 
 }  // namespace gk

@@ -270,9 +270,6 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 template <int KS, bool SYNC = false, class RA, class RB, int FM, int FN>
 __device__ __forceinline__ void load_frags(const RA& ra, const RB& rb, typename RA::Raw (&fa)[FM], typename RB::Raw (&fb)[FN]) {
-#ifdef GK_ABLATE_LDS
-  (void)ra; (void)rb; (void)fa; (void)fb; return;   // development aid (timing only, wrong results)
-#endif
   static_for<0, FM>([&](auto fi) { ra.template read<decltype(fi)::value, KS, SYNC>(fa[decltype(fi)::value]); });
   static_for<0, FN>([&](auto fj) { rb.template read<decltype(fj)::value, KS, SYNC>(fb[decltype(fj)::value]); });
 }
@@ -415,12 +412,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr int DMA_A = Cfg::DMA_A, DMA_B = Cfg::DMA_B, DPT = Cfg::DMA_PER_TILE;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-#ifdef GK_PHASE_TRACE
-  // development aid (never defined in the library build): per-block phase timestamps
-  long long trace_t[5];
-  trace_t[0] = clock64();
-  const long long trace_w0 = wall_clock64();
-#endif
 
   int ti, tj;
   cta_swizzle(args.swz_kind, args.swz_param, (int)blockIdx.x, (int)blockIdx.y, args.nbm, args.nbn, ti, tj);
@@ -511,9 +502,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   }
 
   auto issue_tile = [&](int stage) {
-#ifdef GK_ABLATE_DMA
-    (void)stage; return;
-#endif
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
     if constexpr (Cfg::PLANAR) {
@@ -550,9 +538,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   [[maybe_unused]] const char* part_b = nullptr;
   // part P of NP of the same DMA (Cfg::SPREAD); the tile pointers move on with the last part
   auto issue_part = [&](auto p_c, auto np_c, int stage) __attribute__((always_inline)) {
-#ifdef GK_ABLATE_DMA
-    (void)p_c; (void)np_c; (void)stage; return;
-#endif
     constexpr int P = decltype(p_c)::value, NP = decltype(np_c)::value;
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
@@ -752,9 +737,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   rb.init(wn * Cfg::WTN, lane);
   const unsigned lds_base = (unsigned)(uintptr_t)GK_LDS_PTR(char, smem);
 
-#ifdef GK_PHASE_TRACE
-  trace_t[1] = clock64();
-#endif
   // --- main loop ------------------------------------------------------------------------------
   // Fragments are double-buffered: the LDS reads of the next k-step are in flight while the MFMAs
   // of the current one run.  LDS reads complete in order, so "at most NEXT outstanding" means that
@@ -835,11 +817,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     for (int fi = 0; fi < NA; ++fi)
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj) {
-#ifdef GK_ABLATE_MFMA
-        acc[FI0 + fi][fj][0] += __builtin_bit_cast(float, vb[fj][0] ^ va[fi][0]);
-#else
         acc[FI0 + fi][fj] = Mfma<T, MI>::run(vb[fj], va[fi], acc[FI0 + fi][fj]);
-#endif
       }
   };
   typedef std::integral_constant<int, -1> Whole;
@@ -1044,9 +1022,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     k_loop(std::integral_constant<int, -1>{});
   }
 
-#ifdef GK_PHASE_TRACE
-  trace_t[2] = clock64();
-#endif
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   gett_origins();
 #pragma unroll
@@ -1123,15 +1098,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       }
     }
   }
-#ifdef GK_PHASE_TRACE
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  trace_t[3] = clock64();
-  if (threadIdx.x == 0) {
-    long long* out = (long long*)args.bias + (size_t)blockIdx.x * 8;
-    out[0] = trace_t[0]; out[1] = trace_t[1]; out[2] = trace_t[2]; out[3] = trace_t[3];
-    out[4] = trace_w0; out[5] = wall_clock64();
-  }
-#endif
 }
 
 }  // namespace gk

@@ -99,6 +99,7 @@ _SIGNATURES = {
     "gk_cta_swizzle": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.c_int32, ctypes.c_int32,
                                       ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]),
     "gk_shmem_size": (ctypes.c_int64, [ctypes.POINTER(gk_config), ctypes.c_int32]),
+    "gk_reference_shmem_size": (ctypes.c_int64, [ctypes.POINTER(gk_config)]),
     "gk_threads_per_block": (ctypes.c_int32, [ctypes.POINTER(gk_config)]),
     "gk_heuristic_block_shape": (ctypes.c_int, [ctypes.POINTER(gk_layout), ctypes.POINTER(gk_layout), ctypes.POINTER(gk_layout),
                                                 ctypes.POINTER(gk_layout), ctypes.POINTER(gk_shape)]),

@@ -34,3 +34,13 @@ def shmem_size(conf, kernel: KernelKind = matmul_singlestage) -> int:
     if n < 0:
         raise ConfigError(_lib.last_error(), _lib.GK_ERR_UNSUPPORTED)
     return int(n)
+
+
+def reference_shmem_size(conf) -> int:
+    """The reference's own formula (src/kernel.jl:131-145, 352-366): max(size_c, size_a + size_b, size_d)
+    over the shared layouts of ``conf`` in their physical sizes.  Host arithmetic only."""
+    c = conf.to_c()
+    n = _lib.lib().gk_reference_shmem_size(ctypes.byref(c))
+    if n < 0:
+        raise ConfigError(_lib.last_error(), _lib.GK_ERR_INVALID_ARGUMENT)
+    return int(n)

@@ -57,7 +57,9 @@ typedef enum gk_status {
 typedef enum gk_dtype { GK_F16 = 0, GK_BF16 = 1, GK_F32 = 2, GK_F64 = 3, GK_I16 = 4, GK_I32 = 5, GK_I64 = 6 } gk_dtype;
 
 /* Operators (reference src/operator.jl).  GK_OP_MFMA stands where WMMAOp stands in the reference
- * (:163-245) and runs v_mfma_f32_32x32x16_{f16,bf16}; GK_OP_MFMA_COMPLEX is WMMAComplexOp
+ * (:163-245) and runs v_mfma_f32_16x16x32_{f16,bf16} (the operator shape a configuration names --
+ * 32 x 32 x 16, or the reference's 16 x 16 x 16 WMMA shapes -- sets the granularity of the wave tiles, the
+ * instruction is the library's choice); GK_OP_MFMA_COMPLEX is WMMAComplexOp
  * (:251-314), GK_OP_MFMA_DUAL is WMMADualOp (:320-372), GK_OP_FPU is FPUOp and
  * GK_OP_FPU_TROPICAL is TropicalFPUOp (:35-153). */
 typedef enum gk_operator_kind {
@@ -241,6 +243,12 @@ int gk_cta_swizzle(const gk_config* conf, int32_t block_x, int32_t block_y, int3
 /* Kernel.shmem_size (src/kernel.jl:131-145,352-366,576-590): LDS bytes the chosen kernel
  * instance requests; negative on error. */
 int64_t gk_shmem_size(const gk_config* conf, int32_t kernel);
+
+/* The reference's own answer to Kernel.shmem_size (src/kernel.jl:131-145, 352-366), unchanged:
+ * max(size_c, size_a + size_b, size_d) over the four SHARED layouts of the configuration, each tile in
+ * its Layout.physical_size (padding on the leading dimension, two planes for Split layouts).  Host
+ * arithmetic only; the kernels of this library size their LDS differently (gk_shmem_size).  Negative on error. */
+int64_t gk_reference_shmem_size(const gk_config* conf);
 
 /* Threads per block of the launch (src/matmul.jl:24, with 64-lane wavefronts). */
 int32_t gk_threads_per_block(const gk_config* conf);

@@ -293,3 +293,33 @@ def test_overlapping_regions_cover_everything_with_whole_tiles_at_aligned_offset
             cover[m0:m0 + m, n0:n0 + n] += 1
         assert (cover >= 1).all(), (M, N)
         assert (cover[:M // 64 * 64 - 64, :N // 64 * 64 - 64] == 1).all()      # only the edges are computed twice
+
+
+def test_reference_shmem_size_known_answers():
+    """Kernel.shmem_size as the reference computes it (src/kernel.jl:131-145, 352-366):
+    max(size_c, size_a + size_b, size_d) over the shared layouts.  Answers evaluated by hand from the source:
+    the 128 x 128 x 64 WMMA configuration (Padded F16 A / B by 8, F32 C / D): A (128+8)*64*2 = 17 408,
+    B (64+8)*128*2 = 18 432, C = D = 128*128*4 = 65 536; the complex configuration of
+    configs/configs.jl:385-416 (64 x 64 x 32, padded planar F16 A / B, planar F32 C / D): A (64+8)*32*2*2 = 9 216,
+    B (32+8)*64*2*2 = 10 240, C = D = 64*64*2*4 = 32 768."""
+    from gemmkernels import configs
+    from gemmkernels.kernel import reference_shmem_size
+    conf = gk.get_config(**base_kwargs(block_shape=NT(M=128, N=128, K=64), warps_per_block=4, compute_warp=NT(M=64, N=64, K=16)))
+    assert conf.shared_a_layout == Layout.Padded[ACM[F16], 8]
+    assert reference_shmem_size(conf) == 65536
+    # with FP16 C and D the operand tiles decide: 17 408 + 18 432 against 32 768
+    conf16 = gk.get_config(**base_kwargs(block_shape=NT(M=128, N=128, K=64), warps_per_block=4, compute_warp=NT(M=64, N=64, K=16),
+                                         global_c_layout=ACM[F16], global_d_layout=ACM[F16]))
+    assert reference_shmem_size(conf16) == 17408 + 18432
+    cplx = configs.complex_config(128, 128, 128, zero_c=False, block_shape=NT(M=64, N=64, K=32))
+    assert reference_shmem_size(cplx) == 32768
+    # the operand part alone, through a configuration whose C / D tiles are smaller: B transposed keeps 10 240
+    cplx_t = configs.complex_config(128, 128, 128, tb=True, zero_c=False, block_shape=NT(M=64, N=64, K=32))
+    assert reference_shmem_size(cplx_t) == 32768
+    c = cplx.to_c()
+    from gemmkernels import _lib
+    import ctypes
+    c.shared_c_layout.kind = Layout.ZERO; c.shared_c_layout.eltype = 0; c.shared_c_layout.pad = 0
+    c.shared_d_layout.kind = Layout.ALIGNED_COL_MAJOR; c.shared_d_layout.eltype = 0
+    # C as a 64 x 64 F16 tile (8 192 B), D the same: now A + B = 9 216 + 10 240 wins
+    assert _lib.lib().gk_reference_shmem_size(ctypes.byref(c)) == 9216 + 10240

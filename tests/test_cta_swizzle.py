@@ -70,3 +70,22 @@ def test_xcd_walk_locality():
         mine = [tiles[i] for i in range(xcd, 256, 8)]
         rows, cols = {t[0] for t in mine}, {t[1] for t in mine}
         assert len(rows) == 4 and len(cols) == 8
+
+
+def test_xcd_walk_locality_when_the_tile_count_is_not_a_multiple_of_8():
+    """225 tiles (15 x 15, e.g. 3840^2 on 256 x 256 tiles): the ids of one XCD (congruent mod 8) still
+    cover consecutive positions of the panel walk, so they share rows of A and columns of B."""
+    block, shape = NT(M=256, N=256), NT(M=3840, N=3840)
+    tiles = _tiles(CTASwizzle.XCDAware[4], block, shape)
+    assert sorted(tiles) == [(i, j) for i in range(15) for j in range(15)]
+    # position of a tile in the panel walk (panels 4 tiles high, the last one 3 high)
+    def walk_pos(t):
+        i, j = t
+        first = (i // 4) * 4
+        gsz = min(4, 15 - first)
+        return first * 15 + j * gsz + (i - first)
+    for xcd in range(8):
+        pos = sorted(walk_pos(tiles[n]) for n in range(xcd, 225, 8))
+        assert pos == list(range(pos[0], pos[0] + len(pos))), xcd
+        rows = {tiles[n][0] for n in range(xcd, 225, 8)}
+        assert len(rows) <= 8
