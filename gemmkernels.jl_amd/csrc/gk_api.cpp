@@ -763,57 +763,101 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
   if (rc != GK_OK) return rc;
   gk::FamilyFn fn = family_fn(L.key);
   hipError_t err = hipSuccess;
-  if (kernel == GK_KERNEL_SPLIT_K) {
-    if (L.key.family != gk::FAMILY_MFMA && L.key.family != gk::FAMILY_MFMA_CHECKED)
-      return fail(GK_ERR_UNSUPPORTED, "the K-split kernel runs the real MFMA operator");
-    if (conf->global_d_layout.eltype != GK_F32) return fail(GK_ERR_UNSUPPORTED, "the K-split kernel adds partial sums with fp32 atomics: D must be Float32");
-    if ((epilogue && epilogue->kind != GK_EPILOGUE_DEFAULT) || L.args.t[gk::H_RF2SH_D].n > 0 || L.args.t[gk::H_SH2GL_D].n > 0)
-      return fail(GK_ERR_UNSUPPORTED, "the K-split kernel takes no transform on D and no bias (they would apply to partial sums)");
-    // K slices: enough workgroups to fill every CU as far as the LDS lets them share it (small tiles
-    // hide each other's latency, measured best at up to four per CU), each slice at least eight K tiles
-    // long so that its prologue, epilogue and atomic adds stay a small part of it
-    const int tiles = L.gx * L.gy;
-    const int kt = (conf->matmul_shape.K + conf->block_shape.K - 1) / conf->block_shape.K;   // bounds-checked layouts: the last tile may be partial
-    int per_cu = L.info.lds_bytes > 0 ? (160 * 1024) / L.info.lds_bytes : 1;
-    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
-    int slices = (per_cu * gk::kNumCUs + tiles - 1) / tiles;
-    if (slices > kt / 8) slices = kt / 8;
-    gk::InstanceInfo sk_info;
-    // K-split instances exist for the small tiles that skinny products run; anything else (a large
-    // tile, generic A / B hooks) runs unsplit below
-    // the bounds-checked kernel takes its K range from the launch arguments, the aligned kernels have
-    // instances of their own for it
-    gk::FamilyFn sk_fn = L.key.family == gk::FAMILY_MFMA_CHECKED ? fn : gk::family_mfma_splitk;
-    // (the K-split instances of the aligned kernel mask tiles over M and N but take no partial K tile)
-    if (slices > 1 && !L.ragged && sk_fn && sk_fn(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
-      const int per = (kt + slices - 1) / slices;
-      slices = (kt + per - 1) / per;
-      if (L.args.c_mode != 0 && c == d && L.args.ldc == L.args.ldd && conf->global_c_layout.eltype == GK_F32 &&
-          L.args.t[gk::H_GL2SH_C].n == 0 && L.args.t[gk::H_SH2RF_C].n == 0) {
-        // in place with an untouched C (C = A*B + C): D holds its starting value already, so every
-        // slice adds its partial sum and one launch does it all
-        gk::GemmArgs all = L.args;
-        all.k_begin = 0; all.k_steps = per; all.atomic_d = 1; all.c_mode = 0;
-        sk_fn(L.key, all, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)slices), (hipStream_t)stream, 1, &sk_info, &err);
-        if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
-        return GK_OK;
-      }
-      gk::GemmArgs first = L.args;       // slice 0: reads C, writes D
-      first.k_begin = 0; first.k_steps = per; first.atomic_d = 0;
-      sk_fn(L.key, first, dim3((unsigned)L.gx, (unsigned)L.gy, 1), (hipStream_t)stream, 1, &sk_info, &err);
-      if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
-      gk::GemmArgs rest = L.args;        // slices 1..: start from zero, add into D; stream order puts them after slice 0
-      rest.k_begin = per; rest.k_steps = per; rest.atomic_d = 1; rest.c_mode = 0;
-      rest.t[gk::H_GL2SH_C].n = 0; rest.t[gk::H_SH2RF_C].n = 0;      // the hooks of C belong to slice 0 alone
-      sk_fn(L.key, rest, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)(slices - 1)), (hipStream_t)stream, 1, &sk_info, &err);
-      if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
-      return GK_OK;
-    }
+  if (kernel == GK_KERNEL_SPLIT_K)
+    return fail(GK_ERR_INVALID_ARGUMENT, "the K-split kernel needs a workspace for the partial tiles of its slices: call gk_matmul_split_k");
+  if (!fn || !fn(L.key, L.args, dim3((unsigned)L.gx, (unsigned)L.gy), (hipStream_t)stream, 1, &L.info, &err))
+    return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance");
+  if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", L.info.name, hipGetErrorString(err));
+  return GK_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+constexpr size_t kCounterAlign = 256;
+
+// K slices of a K-split launch: enough workgroups to fill every CU as far as the LDS lets them share it
+// (small tiles hide each other's latency, measured best at up to four per CU), each slice at least eight K
+// tiles long so that its prologue and its share of the reduction stay a small part of it.
+int split_k_slices(int tiles, int k_tiles, int lds_bytes) {
+  int per_cu = lds_bytes > 0 ? (160 * 1024) / lds_bytes : 1;
+  per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+  int slices = (per_cu * gk::kNumCUs + tiles - 1) / tiles;
+  if (slices > k_tiles / 8) slices = k_tiles / 8;
+  return slices < 1 ? 1 : slices;
+}
+
+size_t split_k_counter_bytes(int tiles) { return ((size_t)tiles * sizeof(unsigned) + kCounterAlign - 1) / kCounterAlign * kCounterAlign; }
+
+}  // namespace
+
+namespace gk_internal {
+
+// Launches a K-split product whose partial tiles meet in [counters | partial tiles] at `workspace`
+// (`whose` names the workspace in the message that refuses a launch it cannot hold).
+int launch_split_k(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
+                   const gk_epilogue* epilogue, void* workspace, size_t workspace_bytes, const char* whose, void* stream) {
+  gk_internal::Launch L;
+  int rc = gk_internal::prepare_launch(conf, a, b, c, d, transforms, epilogue, GK_KERNEL_SPLIT_K, nullptr, &L);
+  if (rc != GK_OK) return rc;
+  if (L.key.family != gk::FAMILY_MFMA && L.key.family != gk::FAMILY_MFMA_CHECKED)
+    return fail(GK_ERR_UNSUPPORTED, "the K-split kernel runs the real MFMA operator");
+  gk::FamilyFn fn = family_fn(L.key);
+  hipError_t err = hipSuccess;
+  const int tiles = L.gx * L.gy;
+  const int kt = (conf->matmul_shape.K + conf->block_shape.K - 1) / conf->block_shape.K;   // bounds-checked layouts: the last tile may be partial
+  int slices = split_k_slices(tiles, kt, L.info.lds_bytes);
+  gk::InstanceInfo sk_info;
+  // K-split instances exist for the small tiles that skinny products run; anything else (a large tile,
+  // generic A / B hooks, a partial last K tile on the aligned kernel) runs unsplit.  The bounds-checked
+  // kernel takes its K range from the launch arguments, the aligned kernels have instances of their own.
+  gk::FamilyFn sk_fn = L.key.family == gk::FAMILY_MFMA_CHECKED ? fn : gk::family_mfma_splitk;
+  if (slices > 1 && !L.ragged && sk_fn && sk_fn(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
+    const int per = (kt + slices - 1) / slices;
+    slices = (kt + per - 1) / per;           // no empty slice: every slice arrives at its tile's counter
+    const size_t counters = split_k_counter_bytes(tiles);
+    const size_t need = counters + (size_t)tiles * slices * conf->block_shape.M * conf->block_shape.N * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+      return fail(GK_ERR_INVALID_ARGUMENT, "the K-split launch needs a workspace of %zu bytes (%d tiles x %d slices of %d x %d floats); %s holds %zu",
+                  need, tiles, slices, conf->block_shape.M, conf->block_shape.N, whose, workspace_bytes);
+    if (((uintptr_t)workspace & 15u) != 0) return fail(GK_ERR_ALIGNMENT, "the workspace is not aligned to 16 bytes");
+    gk::GemmArgs sk = L.args;
+    sk.k_steps = per; sk.k_slices = slices;
+    sk.ws_counters = (unsigned*)workspace;
+    sk.ws_partials = (char*)workspace + counters;
+    sk_fn(L.key, sk, dim3((unsigned)L.gx, (unsigned)L.gy, (unsigned)slices), (hipStream_t)stream, 1, &sk_info, &err);
+    if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", sk_info.name, hipGetErrorString(err));
+    return GK_OK;
   }
   if (!fn || !fn(L.key, L.args, dim3((unsigned)L.gx, (unsigned)L.gy), (hipStream_t)stream, 1, &L.info, &err))
     return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance");
   if (err != hipSuccess) return fail(GK_ERR_HIP, "HIP launch of %s failed: %s", L.info.name, hipGetErrorString(err));
   return GK_OK;
+}
+
+}  // namespace gk_internal
+
+extern "C" {
+
+int gk_split_k_workspace_size(const gk_config* conf, size_t* bytes) {
+  if (!conf || !bytes) return fail(GK_ERR_INVALID_ARGUMENT, "NULL argument");
+  const gk_shape& g = conf->matmul_shape;
+  const gk_shape& b = conf->block_shape;
+  if (g.M <= 0 || g.N <= 0 || g.K <= 0 || b.M <= 0 || b.N <= 0 || b.K <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "shapes must be positive");
+  const long long tiles = (long long)((g.M + b.M - 1) / b.M) * ((g.N + b.N - 1) / b.N);
+  const int kt = (g.K + b.K - 1) / b.K;
+  // the largest number of slices split_k_slices can pick for this grid (four workgroups per CU)
+  long long slices = (4 * gk::kNumCUs + tiles - 1) / tiles;
+  if (slices > kt / 8) slices = kt / 8;
+  if (slices < 2) { *bytes = 0; return GK_OK; }      // runs unsplit
+  *bytes = split_k_counter_bytes((int)tiles) + (size_t)tiles * (size_t)slices * b.M * b.N * sizeof(float);
+  return GK_OK;
+}
+
+int gk_matmul_split_k(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
+                      const gk_epilogue* epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+  return gk_internal::launch_split_k(conf, a, b, c, d, transforms, epilogue, workspace, workspace_bytes, "the caller's workspace", stream);
 }
 
 int gk_dev_alloc(size_t bytes, void** ptr) {

@@ -22,4 +22,9 @@ struct Launch {
 int prepare_launch(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
                    const gk_epilogue* epilogue, int32_t kernel, const gk::InstanceInfo* custom, Launch* out);
 
+// The K-split launch on a workspace of `workspace_bytes` bytes at `workspace` ([arrival counters | partial tiles]);
+// `whose` names the workspace in the message that refuses a launch it cannot hold.
+int launch_split_k(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,
+                   const gk_epilogue* epilogue, void* workspace, size_t workspace_bytes, const char* whose, void* stream);
+
 }  // namespace gk_internal

@@ -59,7 +59,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
       for (int v = 0; v < 16; ++v) {
         float c = 0.0f;
         const int r = mrow + 32 * fi, cc = ncol + 32 * fj + 8 * (v / 4) + (v % 4);
-        if (args.c_mode != 0) {
+        if (args.c_mode != 0 && blockIdx.z == 0) {       // K-split launches: the first slice starts from C
           if (r < args.M && cc < args.N) c = load_cd(args.c, args.c_dtype, r + (long long)cc * args.ldc);
           c = apply_list(args.t[H_GL2SH_C], c);
           c = apply_list(args.t[H_SH2RF_C], c);
@@ -148,7 +148,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
   // K tiles of this workgroup: all of them, or (k_steps > 0) the slice blockIdx.z of a K-split launch
   int kt_first = 0, KT = (args.K + BK - 1) / BK;
   if (args.k_steps > 0) {
-    kt_first = args.k_begin + (int)blockIdx.z * args.k_steps;
+    kt_first = (int)blockIdx.z * args.k_steps;
     KT = KT < kt_first + args.k_steps ? KT : kt_first + args.k_steps;
     if (kt_first >= KT) return;       // the whole workgroup leaves together, before any barrier
   }
@@ -191,6 +191,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
     }
   });
 
+  // K-split launches: the partial tiles of the slices meet in the workspace, the last workgroup to arrive
+  // sums them in slice order and stores D (the loop above ends with a barrier: LDS is free)
+  if (args.k_slices > 1 && !splitk_reduce<Cfg::THREADS>(acc, args, ti + tj * args.nbm, (unsigned*)smem)) return;
+
 #pragma unroll
   for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
@@ -203,9 +207,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
         else if (args.epi_kind == 2) x = x + args.bias[r < args.M ? r : 0];
         x = apply_list(args.t[H_SH2GL_D], x);
         if (r < args.M && cc < args.N) {
-          // partial result of a K slice: fp32 atomic add (the host only asks for it with a Float32 D and no hook on D)
-          if (args.atomic_d) atomicAdd((float*)args.d + r + (long long)cc * args.ldd, x);
-          else store_cd(args.d, args.d_dtype, r + (long long)cc * args.ldd, x);
+          store_cd(args.d, args.d_dtype, r + (long long)cc * args.ldd, x);
         }
       }
 }

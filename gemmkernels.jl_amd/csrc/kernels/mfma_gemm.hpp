@@ -364,8 +364,9 @@ struct MfmaGemmConfig {
   static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
-  // K-split instances: a workgroup handles one slice of K (blockIdx.z) and may add its partial result
-  // into D with atomics.  A variant of its own so that the plain kernels carry none of it.
+  // K-split instances: a workgroup handles one slice of K (blockIdx.z); the slices of a tile meet in a
+  // workspace and the last to arrive sums them in slice order and stores D (splitk_reduce).  A variant of
+  // its own so that the plain kernels carry none of it.
   static constexpr bool SPLITK = SPLITK_;
   // 16-row blocks: a k-step of 32 holds twice the fragments of a 16-wide one, so the A fragments are read
   // and consumed in two halves (rows fi < FM/2, then the rest) with the reads of one half in flight under
@@ -577,7 +578,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   [[maybe_unused]] const int KH = KT / 2;
   if constexpr (Cfg::PLANAR) to_switch = KH;
   if constexpr (Cfg::SPLITK) {
-    const int kt0 = args.k_begin + (int)blockIdx.z * args.k_steps;
+    const int kt0 = (int)blockIdx.z * args.k_steps;
     KT = (KT - kt0) < args.k_steps ? (KT - kt0) : args.k_steps;
     if (KT <= 0) return;       // the whole workgroup leaves together, before any barrier
     ga += (long long)kt0 * a_step;
@@ -659,7 +660,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #endif
   };
   [[maybe_unused]] const bool ragged = Cfg::RAGGED_OK && (m0 + BM > args.M || n0 + BN > args.N);   // wave-uniform
-  if (Cfg::RAGGED_OK && ragged && args.c_mode != 0) {
+  // K-split launches: the first slice of K starts from C, the others from zero
+  const bool load_c = args.c_mode != 0 && (!Cfg::SPLITK || blockIdx.z == 0);
+  if (Cfg::RAGGED_OK && ragged && load_c) {
     // tile over the edge: element by element, out-of-range elements start from zero
 #pragma unroll
     for (int fj = 0; fj < FN; ++fj)
@@ -677,7 +680,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         hook_col(std::integral_constant<int, H_SH2RF_C>{}, fj);
       }
     }
-  } else if (args.c_mode != 0) {
+  } else if (load_c) {
     gett_origins();
     // column blocks outermost: with 16-row blocks the two halves of a 128-byte line of C / D belong to
     // neighbouring row blocks, which are then read (and, below, written) right after each other
@@ -1022,6 +1025,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     k_loop(std::integral_constant<int, -1>{});
   }
 
+  if constexpr (Cfg::SPLITK) {
+    // every slice of K leaves its partial tile in the workspace; the last one to arrive adds them up in slice
+    // order and goes on to the epilogue, the others are done
+    if (args.k_slices > 1) {
+      block_barrier();         // every wave is done with the LDS tiles: the first word now carries the arrival count
+      if (!splitk_reduce<Cfg::THREADS>(acc, args, ti + tj * args.nbm, (unsigned*)smem)) return;
+    }
+  }
+
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   gett_origins();
 #pragma unroll
@@ -1058,21 +1070,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
       for (int v = 0; v < NV; ++v) x[v] = acc[fi][fj][v];
       // the accumulator is rounded once, to the element type of D
-      if constexpr (Cfg::SPLITK) {
-        if (args.atomic_d) {
-          // partial result of a K slice: fp32 atomic adds (the order of the slices, and with it the
-          // last bits of the sum, is not fixed)
-          float* dp = (float*)args.d + off;
-#pragma unroll
-          for (int v = 0; v < NV; ++v) {
-            if constexpr (Cfg::RAGGED_OK) {
-              if (ragged && (mrow + MI * fi >= args.M || ncol + MI * fj + vcol(v) >= args.N)) continue;   // over the edge
-            }
-            atomicAdd(&dp[(long long)vcol(v) * ns], x[v]);
-          }
-          continue;
-        }
-      }
       if constexpr (Cfg::RAGGED_OK) {
         if (ragged) {       // tile over the edge: element by element, out-of-range elements are dropped
 #pragma unroll

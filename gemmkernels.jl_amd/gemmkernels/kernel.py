@@ -23,7 +23,8 @@ matmul_singlestage = KernelKind(0, "matmul_singlestage")     # src/kernel.jl:10-
 matmul_pipelined = KernelKind(1, "matmul_pipelined")         # src/kernel.jl:147-350
 matmul_pipelined_ng = KernelKind(2, "matmul_pipelined_ng")   # src/kernel.jl:368-574
 # no counterpart in the reference: the pipelined kernel with the K range cut into slices that run as
-# separate workgroups (fp32 atomic adds into D), for problems with too few output tiles to fill the chip
+# separate workgroups of one launch, for problems with too few output tiles to fill the chip; the slices of
+# a tile meet in a workspace and are added in slice order, so results do not change from run to run
 matmul_split_k = KernelKind(3, "matmul_split_k")
 
 

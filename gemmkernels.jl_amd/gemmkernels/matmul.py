@@ -82,6 +82,30 @@ def _current_stream() -> int:
         return torch.cuda.current_stream().cuda_stream
 
 
+_workspaces = {}
+
+
+def split_k_workspace(conf_c, stream: int):
+    """Device workspace for a K-split launch of ``conf_c`` on ``stream``: (pointer, bytes).  The slices of an
+    output tile leave their partial tiles there and the last one to arrive adds them up in slice order
+    (``gk_matmul_split_k``).  One zero-initialised buffer per device and stream, grown when a launch needs
+    more: launches on one stream are ordered, so they can share it, and every launch leaves the arrival
+    counters at its head at zero.  (0, 0) when the product runs unsplit."""
+    import torch
+    need = ctypes.c_size_t()
+    rc = _lib.lib().gk_split_k_workspace_size(ctypes.byref(conf_c), ctypes.byref(need))
+    if rc != _lib.GK_OK:
+        _raise(rc)
+    if need.value == 0:
+        return 0, 0
+    key = (torch.cuda.current_device(), int(stream))
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < need.value:
+        size = max(need.value, 1 << 20)
+        buf = _workspaces[key] = torch.zeros(size, dtype=torch.uint8, device="cuda")
+    return int(buf.data_ptr()), int(buf.numel())
+
+
 _IDENTITY = Transform.Elementwise()
 _DEFAULT_EPILOGUE = Epilogue.Default()
 _lowered = {}
@@ -168,7 +192,7 @@ class Plan:
     other means while it is in use.  For loops that launch the same GEMM many times, where the
     microseconds a general ``matmul`` call spends on lowering would rival the kernel itself."""
 
-    __slots__ = ("_fn", "_conf", "_trans", "_epi", "_args", "_keep", "d", "kernel_names")
+    __slots__ = ("_fn", "_conf", "_trans", "_epi", "_args", "_keep", "_split_k", "d", "kernel_names")
 
     def __init__(self, conf: Config, a, b, c, d, transforms: dict, epilogue, kernel, specialized=None):
         if specialized is None and any(t.expr is not None for t in transforms.values()):
@@ -178,6 +202,7 @@ class Plan:
         self._conf = _lib.gk_config.from_buffer_copy(cconf)        # to_c hands out a cached, shared descriptor
         self._trans = None if specialized is not None else lower_transforms(transforms)
         self._epi = None
+        self._split_k = False
         if epilogue.kind != Epilogue.DEFAULT:
             self._epi = _lib.gk_epilogue()
             self._epi.kind = epilogue.kind
@@ -186,6 +211,11 @@ class Plan:
         if specialized is not None:
             self._fn = _lib.lib().gk_rtc_matmul
             self._args = (specialized._handle, ctypes.byref(self._conf), _ptr(a), _ptr(b), _ptr(c), _ptr(d), epi_ref)
+        elif kernel is Kernel.matmul_split_k:
+            self._fn = _lib.lib().gk_matmul_split_k
+            self._args = (ctypes.byref(self._conf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                          ctypes.byref(self._trans) if self._trans is not None else None, epi_ref)
+            self._split_k = True
         else:
             self._fn = _lib.lib().gk_matmul
             self._args = (ctypes.byref(self._conf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
@@ -195,7 +225,13 @@ class Plan:
         self.kernel_names = ()      # filled in by the BLAS-level front end
 
     def __call__(self, stream=None):
-        rc = self._fn(*self._args, _current_stream() if stream is None else int(stream))
+        stream = _current_stream() if stream is None else int(stream)
+        if self._split_k:
+            rc = self._fn(*self._args, *split_k_workspace(self._conf, stream), stream)
+            if rc != _lib.GK_OK:
+                _raise(rc)
+            return self.d
+        rc = self._fn(*self._args, stream)
         if rc != _lib.GK_OK:
             _raise(rc)
         return self.d
@@ -258,10 +294,16 @@ def matmul(conf: Config, a, b, c, d, *,
         cepi = _lib.gk_epilogue()
         cepi.kind = epilogue.kind
         cepi.bias = _ptr(epilogue.bias)
-    rc = _lib.lib().gk_matmul(ctypes.byref(cconf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
-                              ctypes.byref(ctrans) if ctrans is not None else None,
-                              ctypes.byref(cepi) if cepi is not None else None,
-                              kernel.code, _current_stream() if stream is None else int(stream))
+    stream = _current_stream() if stream is None else int(stream)
+    if kernel is Kernel.matmul_split_k:
+        rc = _lib.lib().gk_matmul_split_k(ctypes.byref(cconf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                                          ctypes.byref(ctrans) if ctrans is not None else None,
+                                          ctypes.byref(cepi) if cepi is not None else None,
+                                          *split_k_workspace(cconf, stream), stream)
+    else:
+        rc = _lib.lib().gk_matmul(ctypes.byref(cconf), _ptr(a), _ptr(b), _ptr(c), _ptr(d),
+                                  ctypes.byref(ctrans) if ctrans is not None else None,
+                                  ctypes.byref(cepi) if cepi is not None else None, kernel.code, stream)
     if rc != _lib.GK_OK:
         _raise(rc)
     return d

@@ -11,8 +11,9 @@
  * objects to the plain structs below.
  *
  * Conventions
- *  - All pointers a, b, c, d and bias are DEVICE pointers owned by the caller.  The library never
- *    allocates or frees device memory and keeps no workspace.  d may alias c.
+ *  - All pointers a, b, c, d and bias are DEVICE pointers owned by the caller.  The launchers never
+ *    allocate or free device memory; the one kind of launch that needs a workspace (K-split) takes it
+ *    from the caller.  d may alias c.
  *  - Everything is column-major like the reference: an 'N' operand A is M x K with leading
  *    dimension lda >= M (layout kinds *_COL_MAJOR), a 'T' operand is the K x M array of its
  *    transpose (layout kinds *_ROW_MAJOR), reference src/matmul.jl:79-83.
@@ -161,12 +162,14 @@ typedef struct gk_config {
 /* Kernels (reference src/kernel.jl: matmul_singlestage :10-129, matmul_pipelined :147-350,
  * matmul_pipelined_ng :368-574).  GK_KERNEL_SPLIT_K has no counterpart in the reference: for
  * problems with too few output tiles to fill the 256 CUs (skinny M or N, long K) the K range is cut
- * into slices that run as separate workgroups; the first slice writes D = T_c(C) + its partial sum in
- * a launch of its own, the others add theirs with fp32 atomics in a second launch (when d == c and C
- * has no transform, D holds its starting value already and all slices add in one launch).  Real MFMA
- * operator (aligned or bounds-checked layouts), fp32 D, no transform on D and no bias; the order of
- * the atomic adds, and so the last bits of D, can differ between runs.  With enough tiles it is the
- * pipelined (bounds-checked layouts: the single-stage) kernel. */
+ * into slices that run as separate workgroups of ONE launch.  Slice 0 starts from T_c(C), the others
+ * from zero; every slice leaves its partial tile in a workspace and counts itself at the tile's arrival
+ * counter; the last to arrive adds the partial tiles in slice order (so the bits of D do not depend on
+ * the order of arrival and do not change from run to run), applies the D hooks and the bias and
+ * stores D in its element type.  No workgroup waits for another.  It needs a workspace and therefore
+ * has its own entry point, gk_matmul_split_k; gk_matmul refuses this kind.  Real MFMA operator
+ * (aligned or bounds-checked layouts).  With enough tiles, or a tile that has no K-split instance, it
+ * is the pipelined (bounds-checked layouts: the single-stage) kernel. */
 typedef enum gk_kernel_kind {
   GK_KERNEL_SINGLESTAGE = 0,
   GK_KERNEL_PIPELINED = 1,
@@ -268,6 +271,18 @@ int gk_kernel_name(const gk_config* conf, const gk_transforms* transforms, const
  * NULL means Epilogue.Default.  Enqueues one kernel on `stream` (a hipStream_t) and returns. */
 int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
               const gk_transforms* transforms, const gk_epilogue* epilogue, int32_t kernel, void* stream);
+
+/* The K-split kind of launch (GK_KERNEL_SPLIT_K above; no counterpart in the reference, whose launcher
+ * src/matmul.jl:7-44 has one kernel per product).  gk_split_k_workspace_size gives an upper bound of
+ * the workspace a launch of `conf` needs (0: it runs unsplit); gk_matmul_split_k is gk_matmul plus the
+ * workspace: device memory owned by the caller, 16-byte aligned, ZEROED BEFORE ITS FIRST USE.  Its head
+ * holds one arrival counter per output tile, which every launch leaves at zero again, so one workspace
+ * serves any number of launches one after the other; launches that overlap in time (two streams) need
+ * a workspace each. */
+int gk_split_k_workspace_size(const gk_config* conf, size_t* bytes);
+int gk_matmul_split_k(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
+                      const gk_transforms* transforms, const gk_epilogue* epilogue, void* workspace,
+                      size_t workspace_bytes, void* stream);
 
 /* Kernels specialised at run time (hipRTC).  The reference compiles one kernel per Config type and
  * inlines arbitrary Julia functors at the eight transform hooks (src/matmul.jl:38,

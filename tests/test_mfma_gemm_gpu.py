@@ -202,12 +202,10 @@ def test_bf16(gpu, ta, tb, d16):
     ref = helpers.run_oracle(conf, a, b, c, (M, N), d_dtype=np.uint16 if d16 else np.float32)
     if d16:
         # same rounding (to nearest even, once, at the store) as the oracle: the bit patterns differ only where the
-        # two fp32 sums straddle a rounding boundary -- rarely, and then by one unit in the last place.  Truncation
-        # or round-half-up would differ in about half of the elements.
-        got_bits = gk.bf16_bits(d.astype(np.float32)).astype(np.int32)
-        ref_bits = ref.astype(np.int32)
-        diff = np.abs(got_bits - ref_bits)
-        assert diff.max() <= 1 and (diff != 0).mean() < 0.01, (diff.max(), (diff != 0).mean())
+        # two fp32 sums (different orders) straddle a rounding boundary or nearly cancel -- a few elements in a
+        # hundred thousand.  Truncation or round-half-up would differ in about half of the elements.
+        got_bits = gk.bf16_bits(d.astype(np.float32))
+        assert (got_bits != ref).mean() < 1e-3, (got_bits != ref).mean()
         ref = gk.bf16_values(ref)
     tol = 4e-3 if d16 else TOL        # against float64, a BFloat16 result carries 2^-9 relative rounding per element
     assert oracle.rel_frobenius(d, ref) <= (1e-3 if d16 else tol)
