@@ -284,6 +284,18 @@ int gk_matmul_split_k(const gk_config* conf, const void* a, const void* b, const
                       const gk_transforms* transforms, const gk_epilogue* epilogue, void* workspace,
                       size_t workspace_bytes, void* stream);
 
+/* gk_matmul_split_k for callers that cannot allocate device memory.  No counterpart in the reference; it is
+ * for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same
+ * arguments and same results, bit for bit, as gk_matmul_split_k, without the workspace: the partial tiles
+ * meet in a device array that is part of the library (gk_split_k_noalloc_capacity() bytes, 32 MiB, on every
+ * GPU the library is used on, for the life of the process).  A launch that needs more is refused with
+ * GK_ERR_INVALID_ARGUMENT and a message that names both sizes; nothing is allocated or freed by the call,
+ * on the device or through any library.  All calls on one GPU share the array: calls that overlap in time
+ * (two streams, two host threads) race on it and must be serialised by the caller. */
+size_t gk_split_k_noalloc_capacity(void);
+int gk_matmul_split_k_noalloc(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
+                              const gk_transforms* transforms, const gk_epilogue* epilogue, void* stream);
+
 /* Kernels specialised at run time (hipRTC).  The reference compiles one kernel per Config type and
  * inlines arbitrary Julia functors at the eight transform hooks (src/matmul.jl:38,
  * src/transform.jl:20-30); gk_matmul offers a closed op vocabulary and a table of tiles instead.
