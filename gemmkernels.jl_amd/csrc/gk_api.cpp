@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -116,6 +117,42 @@ bool ragged_fast_path(const gk_config* c) {
   return true;
 }
 
+// A multiplication of A (or B) by +-2^e commutes with every rounding of the sum (barring overflow and the
+// subnormal range of the operand's type, where the product on the operand would lose bits that the folded form
+// keeps): sum_k (s a) b + c = s (sum_k a b + c / s), bit for bit.  For the real matrix-core operator such a hook
+// therefore leaves the K loop: the accumulators start from T_c(C) / s and are multiplied by s before the hooks
+// of D.  Returns the transforms that remain (`storage` when something was folded) and the factor s.
+const gk_transforms* fold_pow2_scales(const gk_config* c, const gk_transforms* t, gk_transforms* storage, float* post) {
+  *post = 1.0f;
+  if (!t || c->op.kind != GK_OP_MFMA || c->global_a_layout.kind == GK_LAYOUT_DIAGONAL) return t;
+  float factor = 1.0f;
+  bool folded = false;
+  gk_transforms out = *t;
+  const int pairs[2][2] = {{GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A}, {GK_HOOK_GLOBAL_TO_SHARED_B, GK_HOOK_SHARED_TO_REGS_B}};
+  for (const auto& pr : pairs) {
+    int n = 0;
+    const gk_op* one = nullptr;
+    for (int h : pr) {
+      const gk_transform& tr = t->hook[h];
+      if (tr.n_ops < 0 || tr.n_ops > GK_MAX_OPS) return t;        // malformed: left to the checks
+      for (int i = 0; i < tr.n_ops; ++i)
+        if (tr.ops[i].kind != GK_T_IDENTITY) { ++n; one = &tr.ops[i]; }
+    }
+    if (n != 1 || one->kind != GK_T_SCALE) continue;
+    int e = 0;
+    const float m = frexpf(one->p0, &e);
+    if (!(m == 0.5f || m == -0.5f) || e < -23 || e > 24) continue;   // +-2^(e-1), a moderate exponent
+    factor *= one->p0;
+    out.hook[pr[0]].n_ops = 0;
+    out.hook[pr[1]].n_ops = 0;
+    folded = true;
+  }
+  if (!folded) return t;
+  *storage = out;
+  *post = factor;
+  return storage;
+}
+
 // Builds the run-time key of the kernel instance for a configuration.
 // allow_ragged_fast = false: bounds-checked layouts run on the bounds-checked kernel whatever their alignment.
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
@@ -160,7 +197,23 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   }
   key->dtype = c->global_a_layout.eltype;
   key->acc_dtype = c->global_d_layout.eltype;
-  key->fused = (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT)) ? 1 : 0;
+  gk_transforms folded_storage;
+  float post = 1.0f;
+  t = fold_pow2_scales(c, t, &folded_storage, &post);      // power-of-two scales of A / B do not run in the K loop
+  key->fused = (transforms_present(t) || post != 1.0f || (e && e->kind != GK_EPILOGUE_DEFAULT)) ? 1 : 0;
+  const bool mfma_family = key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT;
+  auto ab_hooks = [&]() {
+    if (!t) return false;
+    const int hooks[4] = {GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A, GK_HOOK_GLOBAL_TO_SHARED_B, GK_HOOK_SHARED_TO_REGS_B};
+    for (int h : hooks)
+      for (int i = 0; i < t->hook[h].n_ops && i < GK_MAX_OPS; ++i)
+        if (t->hook[h].ops[i].kind != GK_T_IDENTITY) return true;
+    return false;
+  };
+  if (key->fused && mfma_family && !ab_hooks()) {
+    key->fused = 3;          // hooks of C and D and the bias only: the K loop of the plain kernel
+    return GK_OK;
+  }
   if (key->fused && t && (key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT)) {
     // level 1 covers A / B hooks that are one exact 16-bit scale (or nothing); anything else needs
     // the generic per-element path of level 2
@@ -221,6 +274,11 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
   args->a_kind = c->global_a_layout.kind;
   args->b_kind = c->global_b_layout.kind;
   args->cd_gett = (c->global_d_layout.kind == GK_LAYOUT_GETT) ? 1 : 0;
+  gk_transforms folded_storage;
+  float post = 1.0f;
+  t = fold_pow2_scales(c, t, &folded_storage, &post);
+  args->acc_post_scale = post;
+  args->acc_pre_scale = 1.0f / post;       // exact: post is a power of two
   if (t) {
     for (int h = 0; h < 8; ++h) {
       const gk_transform& src = t->hook[h];

@@ -86,6 +86,10 @@ struct GemmArgs {
   // constant that is exact in the operand's 16-bit type: done as a packed 16-bit multiply
   int fast_scale_a, fast_scale_b;
   float scale_a, scale_b;
+  // a multiplication of A or B by a power of two commutes with every rounding of the sum: the host takes such
+  // a hook out of the K loop, the accumulators start from acc_pre_scale * T_c(C) and are multiplied by
+  // acc_post_scale = 1 / acc_pre_scale before the hooks of D (both 1 otherwise)
+  float acc_pre_scale, acc_post_scale;
   GettDim gm, gn, gk;
   // K-split launches (all 0 otherwise): workgroup z of k_slices handles the k_steps tiles of K that start at
   // tile z * k_steps; slice 0 starts from C.  Every slice writes its partial tile to ws_partials and counts

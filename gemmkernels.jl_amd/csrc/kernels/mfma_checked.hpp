@@ -63,6 +63,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
           if (r < args.M && cc < args.N) c = load_cd(args.c, args.c_dtype, r + (long long)cc * args.ldc);
           c = apply_list(args.t[H_GL2SH_C], c);
           c = apply_list(args.t[H_SH2RF_C], c);
+          c = c * args.acc_pre_scale;          // 1 unless the host folded a power-of-two scale of A or B
         }
         acc[fi][fj][v] = c;
       }
@@ -202,7 +203,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int r = mrow + 32 * fi, cc = ncol + 32 * fj + 8 * (v / 4) + (v % 4);
-        float x = apply_list(args.t[H_RF2SH_D], acc[fi][fj][v]);
+        float x = apply_list(args.t[H_RF2SH_D], acc[fi][fj][v] * args.acc_post_scale);
         if (args.epi_kind == 1) x = x + args.bias[cc < args.N ? cc : 0];
         else if (args.epi_kind == 2) x = x + args.bias[r < args.M ? r : 0];
         x = apply_list(args.t[H_SH2GL_D], x);

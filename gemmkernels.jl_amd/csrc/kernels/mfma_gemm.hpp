@@ -346,7 +346,8 @@ struct MfmaGemmConfig {
   static constexpr int A_KIND = A_KIND_, B_KIND = B_KIND_, FIX = FIX_;
   // 0: no transform and no bias; 1: C / D hooks, bias and at most one exact 16-bit scale on A and on B
   // (a packed multiply per fragment); 2: arbitrary op lists on A and B as well (evaluated in fp32 per
-  // element inside the K loop: complete, and markedly slower)
+  // element inside the K loop: complete, and markedly slower); 3: C / D hooks and bias only, the K loop of
+  // level 0 (also what a power-of-two scale of A or B runs on: the host folds it into the accumulators)
   static constexpr int FUSE = FUSE_;
   static constexpr bool FUSED = FUSE_ != 0;
   static constexpr bool FUSED_AB_GENERIC = FUSE_ == 2;
@@ -723,9 +724,21 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   if constexpr (Cfg::PLANAR) {
     if (args.c_mode != 0 && !lower_plane) negate_acc();   // the sign comes back between the two passes over K
   }
+  // a power-of-two scale of A or B that the host has folded into the accumulators (see GemmArgs)
+  [[maybe_unused]] auto scale_acc = [&](float f) __attribute__((always_inline)) {
+#pragma unroll
+    for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[fi][fj][v] = acc[fi][fj][v] * f;
+  };
+  if constexpr (Cfg::FUSED) {
+    if (load_c && args.acc_pre_scale != 1.0f) scale_acc(args.acc_pre_scale);
+  }
 
-  const bool xf_a = Cfg::FUSED && (hook_present<H_GL2SH_A>(args) || hook_present<H_SH2RF_A>(args));
-  const bool xf_b = Cfg::FUSED && (hook_present<H_GL2SH_B>(args) || hook_present<H_SH2RF_B>(args));
+  const bool xf_a = Cfg::FUSED && Cfg::FUSE != 3 && (hook_present<H_GL2SH_A>(args) || hook_present<H_SH2RF_A>(args));
+  const bool xf_b = Cfg::FUSED && Cfg::FUSE != 3 && (hook_present<H_GL2SH_B>(args) || hook_present<H_SH2RF_B>(args));
   // kept in registers for the whole K loop: a scalar load inside the loop would make the compiler
   // wait for lgkmcnt(0), which also drains the LDS reads that are meant to stay in flight
   const bool fast_a = std::is_same<T, _Float16>::value && args.fast_scale_a != 0;
@@ -1032,6 +1045,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       block_barrier();         // every wave is done with the LDS tiles: the first word now carries the arrival count
       if (!splitk_reduce<Cfg::THREADS>(acc, args, ti + tj * args.nbm, (unsigned*)smem)) return;
     }
+  }
+
+  if constexpr (Cfg::FUSED) {
+    if (args.acc_post_scale != 1.0f) scale_acc(args.acc_post_scale);
   }
 
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------

@@ -1,6 +1,6 @@
 // K-split instances of the MFMA GEMM (kernel kind GK_KERNEL_SPLIT_K): the small tiles that skinny
-// products run, all four transposes, FP16 with no hooks or with C hooks and one exact FP16 scale on A
-// and B (what the BLAS-style entry points produce), BF16 without hooks.
+// products run, all four transposes, FP16 with no hooks, with C / D hooks and bias, or with those and one exact
+// FP16 scale on A and B (what the BLAS-style entry points produce), BF16 with no hooks or C / D hooks and bias.
 #include "mfma_gemm.hpp"
 #include "registry.hpp"
 
@@ -23,7 +23,9 @@ int family_mfma_splitk(const InstanceKey& key, const GemmArgs& args, dim3 grid, 
 #define GK_SK_TILE(bm_, bn_, bk_, wm_, wn_, st_)                            \
   GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, _Float16, DT_F16, 0, "_f16")        \
   GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, _Float16, DT_F16, 1, "_f16_fused")  \
-  GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, __bf16, DT_BF16, 0, "_bf16")
+  GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, _Float16, DT_F16, 3, "_f16_fused_cd")  \
+  GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, __bf16, DT_BF16, 0, "_bf16")  \
+  GK_SK_T(bm_, bn_, bk_, wm_, wn_, st_, __bf16, DT_BF16, 3, "_bf16_fused_cd")
   GK_SK_TILE(128, 128, 64, 2, 2, 2)
   GK_SK_TILE(64, 64, 64, 2, 2, 4)
   GK_SK_TILE(64, 64, 32, 1, 1, 2)

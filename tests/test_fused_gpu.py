@@ -88,6 +88,33 @@ def test_fp16_scales_on_a_and_b_equal_prescaled_operands_bit_for_bit(gpu, block,
         assert np.array_equal(d, want), sorted(tr)
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+@pytest.mark.parametrize("block", [(256, 256, 64), (64, 64, 32)])
+def test_power_of_two_scales_leave_the_k_loop_and_keep_every_bit(gpu, block, ta, tb):
+    """A factor +-2^e on A or B commutes with every rounding, so the library runs the K loop of the plain kernel
+    (instances `_fused_cd`), starts the accumulators from C / s and multiplies them by s at the end.  The result
+    equals, bit for bit, the plain kernel on operands scaled beforehand (exact in FP16 for this data), with C."""
+    BM, BN, BK = block
+    M, N, K = 2 * BM, BN, 4 * BK
+    conf = configs.mfma_config(M, N, K, ta, tb, block_shape=block)
+    a = rng.matrix("upm1_f16", 74, (K, M) if ta else (M, K))
+    b = rng.matrix("upm1_f16", 75, (N, K) if tb else (K, N))
+    c = rng.matrix("upm1_f32", 76, (M, N))
+    a_s = np.asfortranarray(a * np.float16(2.0))
+    b_s = np.asfortranarray(b * np.float16(-0.25))
+    cases = [(dict(transform_shared_to_regs_a=E(lambda x: x * 2.0)), a_s, b),
+             (dict(transform_global_to_shared_b=E(lambda x: x * -0.25)), a, b_s),
+             (dict(transform_global_to_shared_a=E(lambda x: x * 2.0), transform_shared_to_regs_b=E(lambda x: x * -0.25)), a_s, b_s)]
+    for tr, a_ref, b_ref in cases:
+        name = gk.kernel_name(conf, Kernel.matmul_pipelined, tr)
+        assert name.endswith("_fused_cd"), name
+        d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=tr, kernel=Kernel.matmul_pipelined)
+        want = helpers.run_gpu(conf, a_ref, b_ref, c, (M, N), kernel=Kernel.matmul_pipelined)
+        assert np.array_equal(d, want), sorted(tr)
+        ref = helpers.run_oracle(conf, a, b, c, (M, N), transforms=tr)
+        assert oracle.rel_frobenius(d, ref) <= TOL
+
+
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
 def test_all_eight_hooks(gpu, ta, tb):
     """Every hook carries a different op list; the oracle applies them at the same points with the
@@ -117,11 +144,12 @@ ALL_TILES = [((256, 256, 64), (2, 4)), ((256, 256, 32), (2, 4)), ((256, 256, 32)
 
 
 @pytest.mark.parametrize("block,waves", ALL_TILES)
-@pytest.mark.parametrize("level", [1, 2])
-def test_every_tile_at_both_fuse_levels(gpu, block, waves, level):
-    """Level 1: C / D hooks, bias and one exact FP16 scale on A; level 2: arbitrary op lists on A and B
-    evaluated per element inside the K loop (the large-code kernels).  'T','N' puts both operands on
-    the direct-read path, 'N','T' on the transposing reads."""
+@pytest.mark.parametrize("level", [1, 2, 3])
+def test_every_tile_at_every_fuse_level(gpu, block, waves, level):
+    """Level 1: C / D hooks, bias and one exact FP16 scale on A (0.75: not a power of two); level 2: arbitrary op
+    lists on A and B evaluated per element inside the K loop (the large-code kernels); level 3: C / D hooks and
+    bias, with a power-of-two scale of A folded into the accumulators.  'T','N' puts both operands on the
+    direct-read path, 'N','T' on the transposing reads."""
     from gemmkernels import NT
     BM, BN, BK = block
     M, N, K = 2 * BM, BN, 3 * BK
@@ -132,13 +160,14 @@ def test_every_tile_at_both_fuse_levels(gpu, block, waves, level):
         b = rng.matrix("upm1_f16", 62, (N, K) if tb else (K, N))
         c = rng.matrix("upm1_f32", 63, (M, N))
         bias = rng.normal_f32(64, N)
-        tr = dict(transform_global_to_shared_a=E(lambda x: x * 0.5), transform_shared_to_global_d=E(Transform.relu),
-                  transform_shared_to_regs_c=E(lambda x: x * 3.0))
+        tr = dict(transform_global_to_shared_a=E((lambda x: x * 0.5) if level == 3 else (lambda x: x * 0.75)),
+                  transform_shared_to_global_d=E(Transform.relu), transform_shared_to_regs_c=E(lambda x: x * 3.0))
         if level == 2:
             tr["transform_shared_to_regs_a"] = E(lambda x: Transform.square(x) - 0.25)
             tr["transform_global_to_shared_b"] = E(lambda x: abs(x) * 1.5)
         name = gk.kernel_name(conf, Kernel.matmul_pipelined, tr, Epilogue.Bias(0))
         print("case", block, waves, level, ta, tb, name, flush=True)
+        assert name.endswith({1: "_fused", 2: "_fused_ab", 3: "_fused_cd"}[level]), name
         d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=tr, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
         ref = helpers.run_oracle(conf, a, b, c, (M, N), transforms=tr, epilogue=Epilogue.Bias(0), bias=bias)
         assert oracle.rel_frobenius(d, ref) <= TOL, (ta, tb)
