@@ -319,9 +319,20 @@ def main():
             c4 = gk.colmajor_empty((n, n), torch.float32)
             cut = matmatmul_plan(c4, "N", "N", a4, b4, 1.0, 0.0)
             u, _ = time_launches(cut, 50, 10, 0.15)
-            extras["mul! 4000^3 (not whole tiles)"] = {"us": round(u, 2), "TFLOP/s": round(2.0 * n ** 3 / u / 1e6, 2), "launches": len(getattr(cut, "plans", [cut])),
+            extras["mul! 4000^3 (not whole tiles)"] = {"us": round(u, 2), "TFLOP/s": round(2.0 * n ** 3 / u / 1e6, 2), "launches": 1,
                                                        "kernels": sorted(set(cut.kernel_names))}
             del a4, b4, c4, cut
+            torch.cuda.empty_cache()
+            # sizes that are not multiples of 8 either: odd leading dimensions, every column at another offset from
+            # a 16-byte boundary, 16-byte chunks that straddle the last row of A and the last column of B
+            m5, n5, k5 = 4001, 4003, 4005
+            a5 = gk.colmajor(rng.matrix("upm1_f16", 9003, (m5, k5)))
+            b5 = gk.colmajor(rng.matrix("upm1_f16", 9004, (k5, n5)))
+            c5 = gk.colmajor_empty((m5, n5), torch.float32)
+            odd = matmatmul_plan(c5, "N", "N", a5, b5, 1.0, 0.0)
+            u, _ = time_launches(odd, 50, 10, 0.15)
+            extras["mul! 4001x4003x4005 (odd sizes)"] = {"us": round(u, 2), "TFLOP/s": round(2.0 * m5 * n5 * k5 / u / 1e6, 2), "kernels": sorted(set(odd.kernel_names))}
+            del a5, b5, c5, odd
             torch.cuda.empty_cache()
         except Exception as e:
             extras["mul! 4000^3 (not whole tiles)"] = {"error": f"{type(e).__name__}: {e}"}

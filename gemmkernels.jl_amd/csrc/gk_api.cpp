@@ -92,11 +92,12 @@ bool transforms_present(const gk_transforms* t) {
 }
 
 // Bounds-checked layouts (Layout.ColMajor / RowMajor, reference src/layout.jl:117-184) promise nothing about
-// size or alignment.  When a product on them happens to have 16-byte aligned columns of A and B, a K that is
-// a multiple of 8, and M (N) a multiple of 8 where that index is the contiguous one of A (B), the aligned
-// kernel runs it: the tiles that stick out over M or N clamp their loads and mask their C loads and D
-// stores, a last partial K tile is zeroed beyond K in LDS.  Decided from the configuration (a leading dimension of 0 stands for a dense operand); the
-// launcher falls back to the bounds-checked kernel when the pointers themselves turn out misaligned.
+// size or alignment, and the aligned kernel of the configuration's block shape runs them all the same: its
+// 16-byte global -> LDS transfers take any 2-byte aligned address; tiles that stick out over M or N clamp
+// their loads and mask their C loads and D stores; the last K tile, when it is partial or has a 16-byte chunk
+// that reaches over the last row of an operand (M, N or K not a multiple of 8), is fetched outside the
+// pipeline and repaired in LDS.  What it needs is at least one whole chunk along the contiguous index of A
+// and of B (else the bounds-checked kernel runs).  Decided from the configuration alone.
 bool ragged_fast_path(const gk_config* c) {
   if (c->op.kind != GK_OP_MFMA) return false;
   const gk_layout& la = c->global_a_layout; const gk_layout& lb = c->global_b_layout;
@@ -108,13 +109,17 @@ bool ragged_fast_path(const gk_config* c) {
   if (!(is_checked_layout(la.kind) || is_checked_layout(lb.kind) || is_checked_layout(lc.kind) || is_checked_layout(ld.kind))) return false;
   if ((la.eltype != GK_F16 && la.eltype != GK_BF16) || lb.eltype != la.eltype) return false;
   const long long M = c->matmul_shape.M, N = c->matmul_shape.N, K = c->matmul_shape.K;
-  if (K % 8 != 0) return false;                // a last, partial K tile is fine; its 16-byte chunks must be whole
   const bool a_row = is_row_major(la.kind), b_row = is_row_major(lb.kind);
-  const long long lda = la.ld > 0 ? la.ld : (a_row ? K : M), ldb = lb.ld > 0 ? lb.ld : (b_row ? N : K);
-  if ((lda * 2) % 16 != 0 || (ldb * 2) % 16 != 0) return false;
-  if (!a_row && M % 8 != 0) return false;      // A stored M x K: 16-byte chunks run along m
-  if (b_row && N % 8 != 0) return false;       // B stored N x K: 16-byte chunks run along n
+  // a chunk is 8 elements along the contiguous index: k for a row-major ('T') A and a column-major ('N') B
+  if ((a_row ? K : M) < 8 || (b_row ? N : K) < 8) return false;
   return true;
+}
+
+// The aligned kernel has to take the last K tile out of its pipeline (see ragged_fast_path): the instances that
+// cannot (K-split) must not run such a product.
+bool needs_tail_tile(const gk_config* c) {
+  const bool a_row = is_row_major(c->global_a_layout.kind), b_row = is_row_major(c->global_b_layout.kind);
+  return (c->matmul_shape.K % c->block_shape.K) != 0 || (!a_row && (c->matmul_shape.M % 8) != 0) || (b_row && (c->matmul_shape.N % 8) != 0);
 }
 
 // A multiplication of A (or B) by +-2^e commutes with every rounding of the sum (barring overflow and the
@@ -742,13 +747,8 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
   if (rc != GK_OK) return rc;
   out->ragged = false;
   if (key.family == gk::FAMILY_MFMA && ragged_fast_path(conf)) {
-    if ((((uintptr_t)a | (uintptr_t)b) & 15u) != 0) {
-      // bounds-checked layouts with misaligned operands: the kernel that takes anything
-      rc = validate_config(conf, kernel, transforms, epilogue, &key, &info, custom, false);
-      if (rc != GK_OK) return rc;
-    } else {
-      out->ragged = (conf->matmul_shape.K % conf->block_shape.K) != 0;
-    }
+    if ((((uintptr_t)a | (uintptr_t)b) & 1u) != 0) return fail(GK_ERR_ALIGNMENT, "A and B must be aligned to their 2-byte elements");
+    out->ragged = needs_tail_tile(conf);
   }
 
   const bool a_zero = conf->global_a_layout.kind == GK_LAYOUT_ZERO, b_zero = conf->global_b_layout.kind == GK_LAYOUT_ZERO;
@@ -835,14 +835,15 @@ namespace {
 
 constexpr size_t kCounterAlign = 256;
 
-// K slices of a K-split launch: enough workgroups to fill every CU as far as the LDS lets them share it
-// (small tiles hide each other's latency, measured best at up to four per CU), each slice at least eight K
-// tiles long so that its prologue and its share of the reduction stay a small part of it.
-int split_k_slices(int tiles, int k_tiles, int lds_bytes) {
-  int per_cu = lds_bytes > 0 ? (160 * 1024) / lds_bytes : 1;
-  per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
-  int slices = (per_cu * gk::kNumCUs + tiles - 1) / tiles;
-  if (slices > k_tiles / 8) slices = k_tiles / 8;
+// K slices of a K-split launch, from a sweep of slice counts on 4096 x 64 x 4096, 256 x 256 x 16384 and
+// 8192 x 128 x 8192: about two workgroups per CU, and slices at least 1024 deep in K -- a slice pays for its
+// prologue, for the trip of its partial tile to memory and for the arrival counter (about 3 us on the last
+// workgroup's path), which shorter slices do not earn back (4096 x 64 x 4096: 4 slices 12.4 us, 8 slices 14.1 us,
+// 16 slices 19.4 us).
+int split_k_slices(int tiles, int k_tiles, int block_k) {
+  int slices = (2 * gk::kNumCUs + tiles - 1) / tiles;
+  const int min_tiles = (1024 + block_k - 1) / block_k;
+  if (slices > k_tiles / min_tiles) slices = k_tiles / min_tiles;
   return slices < 1 ? 1 : slices;
 }
 
@@ -865,7 +866,7 @@ int launch_split_k(const gk_config* conf, const void* a, const void* b, const vo
   hipError_t err = hipSuccess;
   const int tiles = L.gx * L.gy;
   const int kt = (conf->matmul_shape.K + conf->block_shape.K - 1) / conf->block_shape.K;   // bounds-checked layouts: the last tile may be partial
-  int slices = split_k_slices(tiles, kt, L.info.lds_bytes);
+  int slices = split_k_slices(tiles, kt, conf->block_shape.K);
   gk::InstanceInfo sk_info;
   // K-split instances exist for the small tiles that skinny products run; anything else (a large tile,
   // generic A / B hooks, a partial last K tile on the aligned kernel) runs unsplit.  The bounds-checked
@@ -905,9 +906,7 @@ int gk_split_k_workspace_size(const gk_config* conf, size_t* bytes) {
   if (g.M <= 0 || g.N <= 0 || g.K <= 0 || b.M <= 0 || b.N <= 0 || b.K <= 0) return fail(GK_ERR_INVALID_ARGUMENT, "shapes must be positive");
   const long long tiles = (long long)((g.M + b.M - 1) / b.M) * ((g.N + b.N - 1) / b.N);
   const int kt = (g.K + b.K - 1) / b.K;
-  // the largest number of slices split_k_slices can pick for this grid (four workgroups per CU)
-  long long slices = (4 * gk::kNumCUs + tiles - 1) / tiles;
-  if (slices > kt / 8) slices = kt / 8;
+  const long long slices = split_k_slices((int)(tiles > (1 << 30) ? (1 << 30) : tiles), kt, b.K);
   if (slices < 2) { *bytes = 0; return GK_OK; }      // runs unsplit
   *bytes = split_k_counter_bytes((int)tiles) + (size_t)tiles * (size_t)slices * b.M * b.N * sizeof(float);
   return GK_OK;

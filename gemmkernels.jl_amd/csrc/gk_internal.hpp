@@ -16,7 +16,7 @@ struct Launch {
   gk::InstanceInfo info;
   gk::GemmArgs args;
   int gx, gy;
-  bool ragged;      // an aligned kernel runs bounds-checked layouts and the last K tile is a partial one
+  bool ragged;      // an aligned kernel runs bounds-checked layouts and has to take the last K tile out of its pipeline
 };
 
 int prepare_launch(const gk_config* conf, const void* a, const void* b, const void* c, void* d, const gk_transforms* transforms,

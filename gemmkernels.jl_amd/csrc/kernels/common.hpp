@@ -315,16 +315,28 @@ __device__ __forceinline__ bool splitk_reduce(V (&acc2)[ROWS][COLS], const GemmA
   for (int i = 0; i < COUNT; ++i)
 #pragma unroll
     for (int e = 0; e < NV; ++e) blk(i)[e] = 0.0f;
-  for (int s = 0; s < S; ++s) {
-    const float* part = tile_ws + (size_t)s * TILE_FLOATS;
-    float x[COUNT * NV];
+  // The partial tiles of U slices travel together (one slice at a time the loop would pay the latency of the
+  // memory behind the L2 once per slice); they are added in slice order all the same.
+  constexpr int PER = COUNT * NV;                            // floats per lane and slice
+  constexpr int U = PER >= 32 ? 1 : (PER >= 16 ? 3 : 4);     // at most 63 loads can be outstanding per wave
+  for (int s0 = 0; s0 < S; s0 += U) {
+    float x[U][PER];
 #pragma unroll
-    for (int q = 0; q < COUNT * NV; ++q)
-      x[q] = __hip_atomic_load(&part[(size_t)q * THREADS + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int u = 0; u < U; ++u) {
+      // a slice beyond the last one re-reads the last (its values are not added)
+      const float* part = tile_ws + (size_t)(s0 + u < S ? s0 + u : S - 1) * TILE_FLOATS;
 #pragma unroll
-    for (int i = 0; i < COUNT; ++i)
+      for (int q = 0; q < PER; ++q)
+        x[u][q] = __hip_atomic_load(&part[(size_t)q * THREADS + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 #pragma unroll
-      for (int e = 0; e < NV; ++e) blk(i)[e] += x[i * NV + e];
+    for (int u = 0; u < U; ++u)
+      if (s0 + u < S) {
+#pragma unroll
+        for (int i = 0; i < COUNT; ++i)
+#pragma unroll
+          for (int e = 0; e < NV; ++e) blk(i)[e] += x[u][i * NV + e];
+      }
   }
   // the next launch on this workspace finds the counter at zero
   if (tid == 0) __hip_atomic_store(&args.ws_counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

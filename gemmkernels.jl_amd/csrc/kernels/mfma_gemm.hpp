@@ -461,7 +461,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           // a tile that sticks out over the last row of A: chunks beyond it re-read the last valid chunk
           // (their products land in rows of the tile that are never stored)
           int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
-          const int last = args.M - m0 - (Cfg::A_KIND == OPK_KMAJOR ? 1 : 8);
+          const int last = Cfg::A_KIND == OPK_KMAJOR ? args.M - m0 - 1 : ((args.M - m0 - 1) >> 3) << 3;   // the row, or the chunk, of the last valid row
           m = m > last ? last : m;
         }
         offa[i] = (unsigned)(((long long)row * args.lda + col) * 2);
@@ -473,7 +473,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
       if constexpr (Cfg::RAGGED_OK) {
         int& n = Cfg::B_KIND == OPK_KMAJOR ? row : col;
-        const int last = args.N - n0 - (Cfg::B_KIND == OPK_KMAJOR ? 1 : 8);
+        const int last = Cfg::B_KIND == OPK_KMAJOR ? args.N - n0 - 1 : ((args.N - n0 - 1) >> 3) << 3;
         n = n > last ? last : n;
       }
       offb[i] = (unsigned)(((long long)row * args.ldb + col) * 2);
@@ -577,6 +577,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // K tiles of this workgroup: all of them, or one slice of a K-split launch
   int KT = args.K / BK;       // planar complex: args.K counts both passes
   [[maybe_unused]] const int KH = KT / 2;
+  // The last K tile runs outside the pipeline (after the loop) when it is a partial one, and also when it is whole
+  // but a 16-byte chunk of this workgroup's tiles straddles the last row of an operand whose rows are contiguous in
+  // memory (M, or N, not a multiple of 8): in the last k such a chunk would read past the end of the operand.
+  [[maybe_unused]] int tail_k = 0;
+  if constexpr (Cfg::RAGGED_K_OK) {
+    tail_k = args.K - KT * BK;
+    const bool straddle = (Cfg::A_KIND == OPK_MMAJOR && (args.M & 7) != 0 && m0 + BM > args.M) ||
+                          (Cfg::B_KIND == OPK_MMAJOR && (args.N & 7) != 0 && n0 + BN > args.N);
+    if (tail_k == 0 && straddle && KT > 0) { KT -= 1; tail_k = BK; }
+  }
   if constexpr (Cfg::PLANAR) to_switch = KH;
   if constexpr (Cfg::SPLITK) {
     const int kt0 = (int)blockIdx.z * args.k_steps;
@@ -953,50 +963,62 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     }
   }
   if constexpr (Cfg::RAGGED_K_OK) {
-    // --- a last, partial K tile (K not a multiple of BLOCK_K; K a multiple of 8) -----------------------
-    // Outside the pipeline: the tile is fetched with its k coordinates clamped to the valid ones, the LDS
-    // slots beyond K are set to zero by the lanes that fetched them, and the k-steps that hold valid
-    // values are multiplied.  ga / gb stand at this tile: every whole tile has been issued.
-    const int tail_k = args.K - (args.K / BK) * BK;       // wave-uniform
+    // --- the last K tile, when it is partial or has a chunk over the end of an operand (see tail_k above) ---------
+    // Outside the pipeline: every lane fetches its 16-byte chunks with coordinates clamped to valid ones -- a chunk
+    // that would reach past the last element of the operand is fetched from 1 .. 7 elements further back -- and
+    // then repairs its own chunks in LDS: shifted into place, values whose k is beyond K set to zero.  Then the
+    // k-steps that hold valid values are multiplied.  ga / gb stand at this tile: every earlier tile has been issued.
     if (tail_k > 0) {
       block_barrier();                                     // every wave is done with the stages of the loop
       char* sa = smem;
       char* sb = sa + GA::BYTES;
-      bool beyond_a[DMA_A], beyond_b[DMA_B];
-#pragma unroll
-      for (int i = 0; i < DMA_A; ++i) {
+      // per chunk: elements it was fetched too far back (0 .. 7), leading elements that keep their value (0 .. 8)
+      int shift_a[DMA_A], keep_a[DMA_A], shift_b[DMA_B], keep_b[DMA_B];
+      auto fetch = [&](auto kind_c, auto geom, int q, const char* g, long long ld, int rows_valid, char* dst, int& shift, int& keep)
+          __attribute__((always_inline)) {
+        constexpr int KIND = decltype(kind_c)::value;
+        typedef decltype(geom) G;
         int row, col;
-        dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
-        int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
-        int& k = Cfg::A_KIND == OPK_KMAJOR ? col : row;
-        const int last_m = args.M - m0 - (Cfg::A_KIND == OPK_KMAJOR ? 1 : 8);
-        m = m > last_m ? last_m : m;
-        beyond_a[i] = k >= tail_k;
-        if (beyond_a[i]) k = tail_k - (Cfg::A_KIND == OPK_KMAJOR ? 8 : 1);
-        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + ((long long)row * args.lda + col) * 2),
-                                         GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < DMA_B; ++i) {
-        int row, col;
-        dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
-        int& n = Cfg::B_KIND == OPK_KMAJOR ? row : col;
-        int& k = Cfg::B_KIND == OPK_KMAJOR ? col : row;
-        const int last_n = args.N - n0 - (Cfg::B_KIND == OPK_KMAJOR ? 1 : 8);
-        n = n > last_n ? last_n : n;
-        beyond_b[i] = k >= tail_k;
-        if (beyond_b[i]) k = tail_k - (Cfg::B_KIND == OPK_KMAJOR ? 8 : 1);
-        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + ((long long)row * args.ldb + col) * 2),
-                                         GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
-      }
-      wait_vmcnt<0>();                                     // this lane's own slots have landed
-      const int4v zero = {0, 0, 0, 0};
+        dma_lane_coords<G, KIND>(q, lane, row, col);
+        int& r = KIND == OPK_KMAJOR ? row : col;           // index along M (A) or N (B), from the tile origin
+        int& k = KIND == OPK_KMAJOR ? col : row;
+        const int last_r = KIND == OPK_KMAJOR ? rows_valid - 1 : ((rows_valid - 1) >> 3) << 3;
+        r = r > last_r ? last_r : r;
+        keep = 8;
+        if (KIND == OPK_KMAJOR) {                          // the chunk runs along k
+          if (k >= tail_k) { keep = 0; k = ((tail_k - 1) >> 3) << 3; }
+          else if (k + 8 > tail_k) keep = tail_k - k;
+        } else if (k >= tail_k) { keep = 0; k = tail_k - 1; }
+        long long e = (long long)row * ld + col;
+        // one past the last element of the operand, counted from the tile origin
+        const long long end = KIND == OPK_KMAJOR ? (long long)(rows_valid - 1) * ld + tail_k : (long long)(tail_k - 1) * ld + rows_valid;
+        shift = 0;
+        if (e + 8 > end) { shift = (int)(e + 8 - end); e -= shift; }
+        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(g + e * 2), GK_LDS_PTR(void, dst + q * 1024), 16, 0, 0);
+      };
 #pragma unroll
       for (int i = 0; i < DMA_A; ++i)
-        if (beyond_a[i]) *(int4v*)(sa + (wave + i * NWAVES) * 1024 + lane * 16) = zero;
+        fetch(std::integral_constant<int, Cfg::A_KIND>{}, GA{}, wave + i * NWAVES, ga, args.lda, args.M - m0, sa, shift_a[i], keep_a[i]);
 #pragma unroll
       for (int i = 0; i < DMA_B; ++i)
-        if (beyond_b[i]) *(int4v*)(sb + (wave + i * NWAVES) * 1024 + lane * 16) = zero;
+        fetch(std::integral_constant<int, Cfg::B_KIND>{}, GB{}, wave + i * NWAVES, gb, args.ldb, args.N - n0, sb, shift_b[i], keep_b[i]);
+      wait_vmcnt<0>();                                     // this lane's own slots have landed
+      auto repair = [&](char* slot, int shift, int keep) __attribute__((always_inline)) {
+        if (shift == 0 && keep == 8) return;
+        short8v v = *(const short8v*)slot, out;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          short x = 0;
+#pragma unroll
+          for (int f = 0; f < 8; ++f) x = (f == e + shift) ? v[f] : x;      // element e was fetched into place e + shift
+          out[e] = e < keep ? x : (short)0;
+        }
+        *(short8v*)slot = out;
+      };
+#pragma unroll
+      for (int i = 0; i < DMA_A; ++i) repair(sa + (wave + i * NWAVES) * 1024 + lane * 16, shift_a[i], keep_a[i]);
+#pragma unroll
+      for (int i = 0; i < DMA_B; ++i) repair(sb + (wave + i * NWAVES) * 1024 + lane * 16, shift_b[i], keep_b[i]);
       __syncthreads();                                     // waits for the LDS writes as well
       ra.set_stage(lds_base);
       rb.set_stage(lds_base + GA::BYTES);

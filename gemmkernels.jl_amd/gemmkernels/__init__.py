@@ -14,7 +14,7 @@ from . import cta_swizzle as CTASwizzle
 from .config import Config, get_config, heuristic_block_shape, adjacent_elements, default_block_shape, check_config
 from .dtypes import Float16, BFloat16, Float32, Float64, Int16, Int32, Int64, ComplexF16, ComplexF32, DType
 from .errors import ConfigError, DimensionMismatch
-from .matmul import matmul, plan, Plan, PlanSequence, output_regions, overlapping_regions, specialize, SpecializedKernel, matmatmul_plan, matmatmul_, mul_, create_config, Transpose, Adjoint, kernel_name
+from .matmul import matmul, plan, Plan, specialize, SpecializedKernel, matmatmul_plan, matmatmul_, mul_, create_config, Transpose, Adjoint, kernel_name
 from .arrays import colmajor, colmajor_empty, to_numpy, bf16_bits, bf16_values
 from .tiling import NT
 from . import contraction
@@ -22,6 +22,6 @@ from .contraction import contract
 
 __all__ = ["Tiling", "Layout", "Operator", "Transform", "Epilogue", "Kernel", "CTASwizzle", "Config", "get_config",
            "heuristic_block_shape", "adjacent_elements", "default_block_shape", "check_config", "ConfigError",
-           "DimensionMismatch", "matmul", "plan", "Plan", "PlanSequence", "output_regions", "overlapping_regions", "specialize", "SpecializedKernel", "matmatmul_plan", "matmatmul_", "mul_", "create_config", "Transpose", "Adjoint", "kernel_name",
+           "DimensionMismatch", "matmul", "plan", "Plan", "specialize", "SpecializedKernel", "matmatmul_plan", "matmatmul_", "mul_", "create_config", "Transpose", "Adjoint", "kernel_name",
            "colmajor", "colmajor_empty", "to_numpy", "bf16_bits", "bf16_values", "NT", "Float16", "BFloat16", "Float32", "Float64", "Int16", "Int32", "Int64", "ComplexF16",
            "ComplexF32", "DType", "contraction", "contract"]

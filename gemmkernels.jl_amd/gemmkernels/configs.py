@@ -369,7 +369,7 @@ def _skinny() -> Workload:
 
     return Workload(
         name="skinny",
-        description="skinny product C = A*B + C, M=4096, N=64, K=4096, FP16 A/B, FP32 C/D, 'N','N', K-split kernel (64 tiles x 8 K slices)",
+        description="skinny product C = A*B + C, M=4096, N=64, K=4096, FP16 A/B, FP32 C/D, 'N','N', K-split kernel (64 tiles x 4 K slices, ordered reduction)",
         flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + 2 * M * N * 4, bound="hbm", make_host=host, make_launch=launch,
         kernel_name="mfma_gemm_splitk_nn_64x64x64_w2x2_f16")
 

@@ -351,8 +351,12 @@ def get_config(*args):
 
 
 def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stridesB, transB: bool,
-                  C: DType, sizeC, stridesC, alpha: type, zeroAlpha: bool, beta: type, zeroBeta: bool, wmma=None):
-    """reference src/matmul.jl:66-183, with the MI355X operator and block-shape choices."""
+                  C: DType, sizeC, stridesC, alpha: type, zeroAlpha: bool, beta: type, zeroBeta: bool, wmma=None,
+                  aligned_pointers=(True, True, True)):
+    """reference src/matmul.jl:66-183, with the MI355X operator and block-shape choices.  ``aligned_pointers``
+    says whether A, B and C start on 16-byte boundaries: the reference decides on the aligned layouts from the
+    strides alone (a misaligned view then traps on the device, src/layout.jl:22-25); here such an operand gets
+    the bounds-checked layout, which takes any address."""
     m = sizeA[1 if transA else 0]
     k = sizeA[0 if transA else 1]
     n = sizeB[0 if transB else 1]
@@ -378,9 +382,9 @@ def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stri
         operator = Operator.MFMAOp[32, 32, 16, compute_type, Float32 if C == Float16 else C]
     else:
         operator = Operator.FPUOp[8, 8, 1, 8, 8, 1, compute_type, C]
-    a_aligned = (stridesA[1] * A.size) % 16 == 0
-    b_aligned = (stridesB[1] * B.size) % 16 == 0
-    c_aligned = (stridesC[1] * C.size) % 16 == 0
+    a_aligned = (stridesA[1] * A.size) % 16 == 0 and aligned_pointers[0]
+    b_aligned = (stridesB[1] * B.size) % 16 == 0 and aligned_pointers[1]
+    c_aligned = (stridesC[1] * C.size) % 16 == 0 and aligned_pointers[2]
 
     def layouts_for(block_shape):
         # src/matmul.jl:121-156: vector loads and stores need 16-byte aligned columns and whole tiles
@@ -396,14 +400,13 @@ def create_config(A: DType, sizeA, stridesA, transA: bool, B: DType, sizeB, stri
         gd = Layout.UnsafeAlignedColMajor[C] if cd_aligned else Layout.ColMajor[C]
         return ga, gb, gc, gd
 
-    # The library runs a product on bounds-checked layouts on the aligned kernels all the same (tiles over the
-    # edge clamp their loads and mask their stores, a partial last K tile is zeroed beyond K) when the columns
-    # of A and B are 16-byte aligned, K is a multiple of 8 and M (N) is a multiple of 8 where it is the
-    # contiguous index of A (B).  Then the tile is chosen among all tiles, not only those that divide the
-    # sizes (4096 x 4096 x 4000: the 64-deep tile with a partial last step instead of the 32-deep one), and
-    # the operands it does not divide get the bounds-checked layouts, as the reference's rule says.
-    edge_ok = (use_mfma and a_aligned and b_aligned and k % 8 == 0 and (transA or m % 8 == 0) and (not transB or n % 8 == 0)
-               and not zeroAlpha)
+    # The library runs a 16-bit product on bounds-checked layouts on the aligned kernels all the same (any address
+    # and leading dimension; tiles over the edge clamp their loads and mask their stores; the last K tile is
+    # repaired in LDS when a 16-byte chunk reaches over the end of an operand) as long as A and B hold one whole
+    # chunk of 8 elements along their contiguous index.  Then the tile is chosen among all tiles, not only those
+    # that divide the sizes (4096 x 4096 x 4000: the 64-deep tile with a partial last step instead of the 32-deep
+    # one), and the operands it does not divide get the bounds-checked layouts, as the reference's rule says.
+    edge_ok = use_mfma and not zeroAlpha and (k if transA else m) >= 8 and (n if transB else k) >= 8
     block_shape = default_block_shape(operator, NT(M=m, N=n, K=k), tile_sized=not edge_ok, a_kmajor=transA, b_kmajor=not transB)
     global_a_layout, global_b_layout, global_c_layout, global_d_layout = layouts_for(block_shape)
     if not edge_ok and any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout)):
@@ -437,7 +440,7 @@ def _single_plan(C, tA: bool, tB: bool, A, B, alpha, beta, wmma=None) -> Plan:
         from_torch(A.dtype), tuple(A.shape), tuple(A.stride()), tA,
         from_torch(B.dtype), tuple(B.shape), tuple(B.stride()), tB,
         from_torch(C.dtype), tuple(C.shape), tuple(C.stride()),
-        type(alpha), alpha == 0, type(beta), beta == 0, wmma)
+        type(alpha), alpha == 0, type(beta), beta == 0, wmma, tuple(x.data_ptr() % 16 == 0 for x in (A, B, C)))
     alpha_c = _round_to(compute_type, float(alpha))          # convert(compute_type, alpha), :196
     beta_c = _round_to(from_torch(C.dtype), float(beta))     # convert(eltype(C), beta), :197
     for name, value in (("alpha", alpha_c), ("beta", beta_c)):
@@ -448,160 +451,27 @@ def _single_plan(C, tA: bool, tB: bool, A, B, alpha, beta, wmma=None) -> Plan:
     # beta = 0 has already turned C into a Zero layout: nothing is loaded, nothing to scale
     ta = Transform.Elementwise(ops=[] if alpha_c == 1.0 else [(Transform.SCALE, alpha_c, 0.0)])
     tc = Transform.Elementwise(ops=[] if beta_c == 1.0 or beta == 0 else [(Transform.SCALE, beta_c, 0.0)])
-    if conf.operator.kind == Operator.MFMA and from_torch(C.dtype) == Float32:
-        # few output tiles and a long K loop (skinny products, the rims of a cut-up product): cut K into
-        # slices so that every CU gets work
+    if conf.operator.kind == Operator.MFMA:
+        # few output tiles and a long K loop (skinny products, the rims of a cut-up product): the K-split kind
+        # cuts K into slices so that every CU gets work (the library decides how many, and runs the product
+        # unsplit when slices would be shorter than 1024 or the tile has no K-split instance).  Its sum is
+        # ordered, so the result is the same on every run, like the reference's mul!.
         bs, ms = conf.block_shape, conf.matmul_shape
         tiles = -(-ms.M // bs.M) * -(-ms.N // bs.N)
-        if kernel is Kernel.matmul_pipelined and tiles <= 128 and ms.K // bs.K >= 4:
+        if tiles <= 256 and ms.K >= 2048:
             kernel = Kernel.matmul_split_k
-        elif kernel is Kernel.matmul_singlestage and tiles <= 128 and ms.K // bs.K >= 16:
-            kernel = Kernel.matmul_split_k          # the bounds-checked kernel: slices of at least eight K tiles
     p = plan(conf, A, B, C, C, transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc, kernel=kernel)
     p.kernel_names = (kernel_name(conf, kernel, dict(transform_shared_to_regs_a=ta, transform_shared_to_regs_c=tc)),)
     return p
 
 
-class PlanSequence:
-    """Several launches on one stream that together compute one product (``matmatmul_plan`` for sizes
-    that are not whole tiles).  Called like a ``Plan``."""
-
-    def __init__(self, plans, d):
-        self.plans = list(plans)
-        self.d = d
-        self.kernel_names = tuple(n for p in self.plans for n in p.kernel_names)
-
-    def __call__(self, stream=None):
-        for p in self.plans:
-            p(stream)
-        return self.d
-
-
-_REGION_TILES = (256, 128, 64)
-
-
-def overlapping_regions(M: int, N: int):
-    """For a product that does not read C (beta = 0): whole tiles only.  The part of the output whose
-    sizes are multiples of 64 is cut like ``output_regions``; the ragged right and bottom edges are covered
-    by 64-wide windows that end at the edge and reach back over cells another launch has already written
-    (which then get the same value, up to the order of the sums, a second time).  M, N >= 64."""
-    M64, N64 = M // 64 * 64, N // 64 * 64
-    out = output_regions(M64, N64)
-    if N > N64:
-        out.append((0, M64, N - 64, 64, True))
-    if M > M64:
-        out.append((M - 64, 64, 0, N64, True))
-    if N > N64 and M > M64:
-        out.append((M - 64, 64, N - 64, 64, True))
-    return out
-
-
-def output_regions(M: int, N: int):
-    """Cuts an M x N output into disjoint rectangles ``(m0, m, n0, n, whole_tiles)``.  The first is the
-    largest top-left block made of 256 x 256 tiles; the strip to its right (all rows) and the strip below
-    it are cut the same way with 128 and then 64; what is left over, or narrower than 64, is marked
-    ``whole_tiles = False`` and goes to the bounds-checked kernel.  Offsets of rectangles with whole tiles
-    are multiples of 64 elements, so 16-byte aligned columns stay 16-byte aligned."""
-    out = []
-
-    def cut(m0, m, n0, n, level):
-        if m <= 0 or n <= 0:
-            return
-        while level < len(_REGION_TILES) and (m < _REGION_TILES[level] or n < _REGION_TILES[level]):
-            level += 1
-        if level == len(_REGION_TILES):
-            out.append((m0, m, n0, n, False))
-            return
-        t = _REGION_TILES[level]
-        mi, ni = m // t * t, n // t * t
-        out.append((m0, mi, n0, ni, True))
-        cut(m0, m, n0 + ni, n - ni, level + 1)       # right of the block: every row
-        cut(m0 + mi, m - mi, n0, ni, level + 1)      # below the block
-    cut(0, M, 0, N, 0)
-    return out
-
-
-def _estimate_us(operator, M: int, N: int, K: int, whole_tiles: bool) -> float:
-    """Rough duration of one launch, from two measured rates: a CU multiplies a 256 x 256 x 64 tile over
-    K = 4096 in 108 us (other tiles by ``config._MFMA_TILE_RATE``), and the bounds-checked kernel spends
-    0.53 us per CU on a 64 x 64 x 32 step; a launch costs a few microseconds whatever it does, a K-split
-    rim two launches and the atomic adds."""
-    from .config import _MFMA_TILE_RATE, NUM_CUS, default_block_shape
-    if whole_tiles:
-        bs = default_block_shape(operator, NT(M=M, N=N, K=K))
-        tiles = -(-M // bs.M) * -(-N // bs.N)
-        rate = _MFMA_TILE_RATE.get((bs.M, bs.N, bs.K), 0.5)
-        rate = rate[0 if tiles <= NUM_CUS else 1] if isinstance(rate, tuple) else rate
-        per_cu = -(-tiles // NUM_CUS) * bs.M * bs.N / rate
-        return per_cu * K / (65536.0 * 4096.0) * 108.0 + 6.0
-    steps = -(-M // 64) * -(-N // 64) * -(-K // 32)
-    return max(-(-steps // NUM_CUS), 8) * 0.53 + 25.0
-
-
-def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None, regions=None):
-    """The launches ``matmatmul_`` would make, as a ``Plan`` (or a ``PlanSequence``) to call any number of
-    times.
-
-    Sizes that are whole tiles, and everything the matrix cores do not run, take one launch of the
-    configuration ``create_config`` picks (reference src/matmul.jl:185-204).  A large 16-bit product whose
-    sizes are *not* whole tiles would run entirely on the bounds-checked kernel, at a tenth of the speed
-    (the reference has the same cliff, src/matmul.jl:121-156 and src/layout.jl:117-184).  When the columns
-    of A, B and C are 16-byte aligned it is cut up instead: ``output_regions`` of whole tiles run on the
-    fast kernels over the first K - K % 32 values of k, the ragged rims on the bounds-checked kernel (in
-    slices of K: a rim has few tiles), and one more bounds-checked launch adds the last K % 32 values of k
-    to all of C.  With beta = 0 and M, N multiples of 8 there are no rims: ``overlapping_regions`` covers the
-    edges with whole tiles that reach back over finished cells.
-
-    Since the aligned kernels handle tiles that stick out over M, N or K themselves (K a multiple of 8, and
-    M, or N, where it is the contiguous index of A, or B), such products take one launch and the cutting
-    above is what remains for the others: aligned leading dimensions around an M or N that is not a multiple
-    of 8, as sub-matrices have them.  Every element of C is
-    still computed as alpha * op(A) * op(B) + beta * C with alpha applied to A in the compute type; only
-    the order of the fp32 additions along k differs from the single launch.  ``regions`` forces the
-    cutting on (True) or off (False); by default it is used when a rough estimate (``_estimate_us``) puts
-    the launches together clearly below the single one (from about 3000^3 on)."""
-    tA, tB = transA == 'T', transB == 'T'
-    single = _single_plan(C, tA, tB, A, B, alpha, beta, wmma)
-    conf = get_config(from_torch(A.dtype), tuple(A.shape), tuple(A.stride()), tA,
-                      from_torch(B.dtype), tuple(B.shape), tuple(B.stride()), tB,
-                      from_torch(C.dtype), tuple(C.shape), tuple(C.stride()),
-                      type(alpha), alpha == 0, type(beta), beta == 0, wmma)[0]
-    ms = conf.matmul_shape
-    M, N, K = ms.M, ms.N, ms.K
-    checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR)
-                  for l in (conf.global_a_layout, conf.global_b_layout, conf.global_c_layout, conf.global_d_layout))
-    aligned_columns = all((int(x.stride()[1]) * x.element_size()) % 16 == 0 and x.data_ptr() % 16 == 0 for x in (A, B, C))
-    Kw = K // 32 * 32        # every tile table has tiles 32 deep
-    if (regions is None and checked and conf.operator.kind == Operator.MFMA and aligned_columns and alpha != 0
-            and K % 8 == 0 and (tA or M % 8 == 0) and (not tB or N % 8 == 0)):
-        # the aligned kernels take ragged M, N and K themselves (create_config has picked their tile)
-        return single
-    if (regions is False or conf.operator.kind != Operator.MFMA or not aligned_columns or alpha == 0
-            or Kw == 0 or min(M, N) < _REGION_TILES[-1]):
-        return single
-    # windows that overlap need rows M - 64 and columns N - 64 to start on 16-byte boundaries in A, B and C
-    if beta == 0 and M % 8 == 0 and N % 8 == 0:
-        cut = overlapping_regions(M, N)
-    else:
-        cut = output_regions(M, N)
-    if len(cut) == 1 and Kw == K:
-        return single           # whole tiles already
-    if regions is None:
-        # worth it when the launches together are clearly shorter than the one launch
-        together = sum(_estimate_us(conf.operator, m, n, Kw, whole) for _, m, _, n, whole in cut)
-        together += _estimate_us(conf.operator, M, N, K - Kw, False) if Kw < K else 0.0
-        if together > 0.8 * _estimate_us(conf.operator, M, N, K, not checked):
-            return single
-
-    def sub(X, trans, r0, r, c0, c):          # rows r0.., columns c0.. of op(X)
-        return X[c0:c0 + c, r0:r0 + r] if trans else X[r0:r0 + r, c0:c0 + c]
-    plans = []
-    for m0, m, n0, n, _ in cut:
-        plans.append(_single_plan(C[m0:m0 + m, n0:n0 + n], tA, tB, sub(A, tA, m0, m, 0, Kw), sub(B, tB, 0, Kw, n0, n),
-                                  alpha, beta, wmma))
-    if Kw < K:
-        plans.append(_single_plan(C, tA, tB, sub(A, tA, 0, M, Kw, K - Kw), sub(B, tB, Kw, K - Kw, 0, N), alpha, 1.0, wmma))
-    return PlanSequence(plans, C)
+def matmatmul_plan(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None):
+    """The launch ``matmatmul_`` would make, as a ``Plan`` to call any number of times: one launch of the
+    configuration ``create_config`` picks (reference src/matmul.jl:185-204), whatever the sizes.  A 16-bit
+    product whose sizes are not whole tiles, whose leading dimensions are odd or whose operands start off a
+    16-byte boundary still runs on the aligned kernels (``create_config``); the bounds-checked kernel is left
+    with operands that have fewer than 8 elements along their contiguous index."""
+    return _single_plan(C, transA == 'T', transB == 'T', A, B, alpha, beta, wmma)
 
 
 def matmatmul_(C, transA: str, transB: str, A, B, alpha, beta, *, wmma=None):

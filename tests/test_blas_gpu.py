@@ -42,6 +42,37 @@ def test_matmatmul(gpu, dims, ta, tb, dtype):
     assert err <= (1e-3 if dtype == np.float16 else 1e-5), err
 
 
+# (A / B type, C type, min_dimension, tolerance) -- the three type rows of reference test/blas.jl:15 and :43; the
+# reference's own tolerance is the norm-wise sqrt(eps(AB_type)) (0.031 for Float16, 3.5e-4 for Float32)
+_CUBE_ROWS = {"f16_f16": (np.float16, np.float16, 256, 2e-3), "f16_f32": (np.float16, np.float32, 128, 1e-3),
+              "f32_f32": (np.float32, np.float32, 128, 1e-5)}
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("row", sorted(_CUBE_ROWS))
+def test_the_reference_cube_of_sizes(gpu, row, ta, tb):
+    """reference test/blas.jl:11-67 in full: M, N, K each from {10, min_dimension, 1000} (27 shapes) for every
+    transpose pair and type row, A and B ~ U[0,1) / sqrt(K), random alpha (in the A / B type) and beta (in the C
+    type), through matmatmul_ with wmma = true for the Float16 rows and false for the Float32 row."""
+    ab_t, c_t, min_dim, tol = _CUBE_ROWS[row]
+    rs = np.random.RandomState(hash((row, ta, tb)) % (2 ** 31))
+    worst = 0.0
+    for M in (10, min_dim, 1000):
+        for N in (10, min_dim, 1000):
+            for K in (10, min_dim, 1000):
+                a = np.asfortranarray((rs.rand(*((K, M) if ta == "T" else (M, K))) / np.sqrt(K)).astype(ab_t))
+                b = np.asfortranarray((rs.rand(*((N, K) if tb == "T" else (K, N))) / np.sqrt(K)).astype(ab_t))
+                c = np.asfortranarray(rs.rand(M, N).astype(c_t))
+                alpha, beta = float(ab_t(rs.rand())), float(c_t(rs.rand()))
+                C = gk.colmajor(c)
+                gk.matmatmul_(C, ta, tb, gk.colmajor(a), gk.colmajor(b), alpha, beta, wmma=(ab_t == np.float16))
+                torch.cuda.synchronize()
+                err = oracle.rel_frobenius(gk.to_numpy(C), oracle.gemm_f64(a, b, c, alpha, beta, ta == "T", tb == "T"))
+                worst = max(worst, err)
+                assert err <= tol, (row, ta, tb, (M, N, K), err)
+    print("cube", row, ta, tb, "worst relative error", worst, flush=True)
+
+
 @pytest.mark.parametrize("dims", [(256, 256, 256), (1000, 200, 72)])
 def test_matmatmul_f16_output(gpu, dims):
     """FP16 A, B and C (reference test/blas.jl:15, the (Float16, Float16, Float16) row): FP32
@@ -112,68 +143,62 @@ def test_config1_benchmark_workload(gpu):
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
-@pytest.mark.parametrize("dims", [(1000, 1000, 1000), (840, 328, 200), (328, 1096, 136), (264, 264, 64)])
-def test_products_cut_into_regions_of_whole_tiles(gpu, dims, ta, tb):
-    """Sizes that are not whole tiles with 16-byte aligned columns: blocks of whole tiles on the fast
-    kernels, rims and the tail of K on the bounds-checked kernel (matmatmul_plan).  Same tolerance as
-    the single launch, and the same kernels must not be all bounds-checked ones."""
-    from gemmkernels.matmul import matmatmul_plan, PlanSequence, output_regions
+@pytest.mark.parametrize("dims", [(1000, 1000, 1000), (1001, 1001, 1001), (841, 329, 203), (327, 1097, 139), (265, 263, 65), (9, 8, 8)])
+def test_any_size_is_one_launch_of_an_aligned_kernel(gpu, dims, ta, tb):
+    """Sizes that are not whole tiles, not multiples of 8, with odd leading dimensions: still one launch of the
+    aligned kernels (the reference would run them on its bounds-checked layouts, src/matmul.jl:121-156)."""
+    from gemmkernels.matmul import matmatmul_plan
     M, N, K = dims
     a, b, c = operands(M, N, K, ta == "T", tb == "T", np.float16, 500)
     alpha, beta = 0.75, -1.5
     A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
-    p = matmatmul_plan(C, ta, tb, A, B, alpha, beta, regions=True)
-    assert isinstance(p, PlanSequence)
-    assert len(p.plans) == len(output_regions(M, N)) + (1 if K % 32 else 0)
-    assert any("checked" not in n for n in p.kernel_names), p.kernel_names
+    p = matmatmul_plan(C, ta, tb, A, B, alpha, beta)
+    assert len(p.kernel_names) == 1 and "checked" not in p.kernel_names[0], p.kernel_names
     print("case", dims, ta, tb, p.kernel_names, flush=True)
     p()
     torch.cuda.synchronize()
     ref = oracle.gemm_f64(a, b, c, alpha, beta, ta == "T", tb == "T")
     assert oracle.rel_frobenius(gk.to_numpy(C), ref) <= 1e-3
-    # the single bounds-checked launch gives the same values up to the order of the fp32 sums
-    C1 = gk.colmajor(c)
-    matmatmul_plan(C1, ta, tb, A, B, alpha, beta, regions=False)()
-    torch.cuda.synchronize()
-    assert oracle.rel_frobenius(gk.to_numpy(C), gk.to_numpy(C1).astype(np.float64)) <= 1e-5
 
 
-def test_region_cutting_is_left_alone_where_it_cannot_help(gpu):
-    from gemmkernels.matmul import matmatmul_plan, PlanSequence
-    # whole tiles: one fast launch; columns that are not 16-byte aligned: one bounds-checked launch; FP32: vector ALUs
-    for dims, dtype in (((1024, 1024, 1024), np.float16), ((1001, 1001, 1001), np.float16), ((1000, 1000, 1000), np.float32)):
-        M, N, K = dims
-        a, b, c = operands(M, N, K, False, False, dtype, 600)
-        p = matmatmul_plan(gk.colmajor(c), "N", "N", gk.colmajor(a), gk.colmajor(b), 1.0, 1.0, regions=True)
-        assert not isinstance(p, PlanSequence), dims
+def test_operands_with_less_than_a_chunk_along_their_contiguous_index_run_bounds_checked(gpu):
+    from gemmkernels.matmul import matmatmul_plan
+    for M, N, K, ta, tb in ((5, 40, 64, "N", "N"), (40, 40, 4, "N", "N"), (40, 3, 64, "N", "T")):
+        a, b, c = operands(M, N, K, ta == "T", tb == "T", np.float16, 600)
+        C = gk.colmajor(c)
+        p = matmatmul_plan(C, ta, tb, gk.colmajor(a), gk.colmajor(b), 1.0, 1.0)
+        assert "checked" in p.kernel_names[0], p.kernel_names
+        p()
+        torch.cuda.synchronize()
+        assert oracle.rel_frobenius(gk.to_numpy(C), oracle.gemm_f64(a, b, c, 1.0, 1.0, ta == "T", tb == "T")) <= 1e-3
 
 
-@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
-@pytest.mark.parametrize("dims", [(1000, 1000, 1000), (840, 328, 192), (264, 72, 136)])
-def test_products_that_do_not_read_c_need_no_rims(gpu, dims, ta, tb):
-    """beta = 0 and M, N multiples of 8: the ragged edges are covered by whole tiles that reach back over
-    finished cells; nothing runs on the bounds-checked kernel."""
-    from gemmkernels.matmul import matmatmul_plan, PlanSequence
-    M, N, K = dims
-    a, b, c = operands(M, N, K, ta == "T", tb == "T", np.float16, 700)
-    A, B = gk.colmajor(a), gk.colmajor(b)
-    C = gk.colmajor(np.asfortranarray(np.full((M, N), np.nan, np.float32)))       # never read
-    p = matmatmul_plan(C, ta, tb, A, B, 1.25, 0.0, regions=True)
-    assert isinstance(p, PlanSequence)
-    assert not any("checked" in n for n in p.kernel_names), p.kernel_names     # the tail of K is a partial tile of the aligned kernel
-    p()
-    torch.cuda.synchronize()
-    ref = oracle.gemm_f64(a, b, None, 1.25, 0.0, ta == "T", tb == "T")
-    assert oracle.rel_frobenius(gk.to_numpy(C), ref) <= 1e-3
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "T")])
+def test_views_that_start_off_a_16_byte_boundary(gpu, ta, tb):
+    """A[1:M+1, :] of a larger array has aligned strides and a misaligned first element: the operand gets the
+    bounds-checked layout and the product still runs on the aligned kernel (1000^3 and a small one)."""
+    from gemmkernels.matmul import matmatmul_plan
+    for M, N, K in ((1000, 1000, 1000), (200, 136, 96)):
+        a, b, c = operands(M, N, K, ta == "T", tb == "T", np.float16, 650)
+        big_a = np.zeros((a.shape[0] + 8, a.shape[1]), np.float16, order="F"); big_a[1:a.shape[0] + 1, :] = a
+        big_b = np.zeros((b.shape[0] + 8, b.shape[1]), np.float16, order="F"); big_b[1:b.shape[0] + 1, :] = b
+        A = gk.colmajor(big_a)[1:a.shape[0] + 1, :]
+        B = gk.colmajor(big_b)[1:b.shape[0] + 1, :]
+        assert A.data_ptr() % 16 == 2 and B.data_ptr() % 16 == 2
+        C = gk.colmajor(c)
+        p = matmatmul_plan(C, ta, tb, A, B, 1.0, 0.5)
+        assert "checked" not in p.kernel_names[0], p.kernel_names
+        p()
+        torch.cuda.synchronize()
+        assert oracle.rel_frobenius(gk.to_numpy(C), oracle.gemm_f64(a, b, c, 1.0, 0.5, ta == "T", tb == "T")) <= 1e-3
 
 
 @pytest.mark.parametrize("beta", [0.0, 0.25])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_cut_up_products_with_16_bit_c(gpu, beta, dtype):
-    """FP16 A, B and C, and BF16 A, B with Float32 C, through the region cutting: rims (beta != 0) and
-    overlapping windows (beta = 0)."""
-    from gemmkernels.matmul import matmatmul_plan, PlanSequence
-    M, N, K = 1000, 200, 104
+def test_odd_sizes_with_16_bit_c(gpu, beta, dtype):
+    """FP16 A, B and C, and BF16 A, B with Float32 C, on sizes that are not multiples of 8."""
+    from gemmkernels.matmul import matmatmul_plan
+    M, N, K = 1001, 203, 107
     a, b, c = operands(M, N, K, False, True, np.float16, 800)
     if dtype == "f16":
         A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c.astype(np.float16))
@@ -183,8 +208,8 @@ def test_cut_up_products_with_16_bit_c(gpu, beta, dtype):
         C = gk.colmajor(c)                                                        # BF16 inputs pair with a Float32 C
         a, b = A.float().cpu().numpy(), B.float().cpu().numpy()                  # the values after rounding to BF16
         c_in = c.astype(np.float64)
-    p = matmatmul_plan(C, "N", "T", A, B, 0.5, beta, regions=True)
-    assert isinstance(p, PlanSequence), type(p)
+    p = matmatmul_plan(C, "N", "T", A, B, 0.5, beta)
+    assert "checked" not in p.kernel_names[0], p.kernel_names
     p()
     torch.cuda.synchronize()
     out = C.float().cpu().numpy()

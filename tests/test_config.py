@@ -263,38 +263,6 @@ def test_complex_layout_rules_of_the_library():
         configs.complex_planar_config(M, N, 48)
 
 
-def test_output_regions_cover_the_output_once_and_fast_regions_are_whole_tiles():
-    """The cutting used by the BLAS-level front end for sizes that are not whole tiles."""
-    from gemmkernels.matmul import output_regions
-    import numpy as np
-    for (M, N) in [(4000, 4000), (4097, 4100), (1000, 1000), (64, 64), (63, 500), (500, 63), (130, 70), (256, 257), (8200, 300), (1, 1)]:
-        cover = np.zeros((M, N), dtype=np.int32)
-        regions = output_regions(M, N)
-        for m0, m, n0, n, whole in regions:
-            assert m > 0 and n > 0 and m0 + m <= M and n0 + n <= N
-            cover[m0:m0 + m, n0:n0 + n] += 1
-            if whole:
-                assert m % 64 == 0 and n % 64 == 0 and m0 % 64 == 0 and n0 % 64 == 0
-        assert (cover == 1).all(), (M, N)
-        # what the bounds-checked kernel gets is a rim less than 64 wide (or a problem smaller than a tile)
-        slow = sum(m * n for _, m, n0, n, whole in regions if not whole)
-        assert slow <= 64 * (M + N), (M, N, slow)
-    assert output_regions(4000, 4000)[0] == (0, 3840, 0, 3840, True)
-
-
-def test_overlapping_regions_cover_everything_with_whole_tiles_at_aligned_offsets():
-    from gemmkernels.matmul import overlapping_regions
-    import numpy as np
-    for (M, N) in [(4000, 4000), (4104, 4096), (1000, 1000), (64, 72), (72, 64), (264, 72), (8200, 328)]:
-        cover = np.zeros((M, N), dtype=np.int32)
-        for m0, m, n0, n, whole in overlapping_regions(M, N):
-            assert whole and m % 64 == 0 and n % 64 == 0 and m > 0 and n > 0
-            assert m0 % 8 == 0 and n0 % 8 == 0 and m0 >= 0 and n0 >= 0 and m0 + m <= M and n0 + n <= N
-            cover[m0:m0 + m, n0:n0 + n] += 1
-        assert (cover >= 1).all(), (M, N)
-        assert (cover[:M // 64 * 64 - 64, :N // 64 * 64 - 64] == 1).all()      # only the edges are computed twice
-
-
 def test_reference_shmem_size_known_answers():
     """Kernel.shmem_size as the reference computes it (src/kernel.jl:131-145, 352-366):
     max(size_c, size_a + size_b, size_d) over the shared layouts.  Answers evaluated by hand from the source:

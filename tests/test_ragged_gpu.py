@@ -1,8 +1,8 @@
-"""Products on the bounds-checked layouts (Layout.ColMajor / RowMajor, reference src/layout.jl:117-184)
-whose columns happen to be 16-byte aligned run on the aligned kernels: tiles that stick out over M or N
-clamp their loads and mask their C loads and D stores.  Parity against the oracle, bit-for-bit equality
-with the same tile on zero-padded operands, no write outside D, and the fall-back to the bounds-checked
-kernel for misaligned pointers."""
+"""Products on the bounds-checked layouts (Layout.ColMajor / RowMajor, reference src/layout.jl:117-184) run on
+the aligned kernels: tiles that stick out over M or N clamp their loads and mask their C loads and D stores, the
+last K tile is repaired in LDS when it is partial or a 16-byte chunk reaches over the end of an operand.  Parity
+against the oracle, bit-for-bit equality with the same tile on zero-padded operands, no write outside D, odd
+sizes, odd leading dimensions and misaligned pointers."""
 import numpy as np
 import pytest
 import torch
@@ -44,6 +44,18 @@ def test_tiles_over_the_edge_against_the_oracle_and_against_padded_operands(gpu,
     BM, BN, BK = block
     for K in (3 * BK, 2 * BK + 24, 8):              # whole tiles; a partial last tile; less than one tile
         _one_shape(block, waves, ta, tb, BM + 72, 2 * BN - 56, K)    # M, N: multiples of 8, not of any tile
+
+
+@pytest.mark.parametrize("block,waves", TILES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_sizes_that_are_not_multiples_of_8(gpu, block, waves, ta, tb):
+    """M, N and K odd: 16-byte chunks straddle the last row of A / column of B / value of k, and every column
+    starts at a different offset from a 16-byte boundary.  Same bits as the tile on zero-padded operands."""
+    BM, BN, BK = block
+    for K in (3 * BK, 2 * BK + 27, 2 * BK + 1, 13):     # whole tiles (the last one leaves the pipeline at the edges); partial tiles; less than a tile
+        _one_shape(block, waves, ta, tb, BM + 73, 2 * BN - 59, K)
+    _one_shape(block, waves, ta, tb, 2 * BM, BN, 2 * BK + 3)             # only K is odd
+    _one_shape(block, waves, ta, tb, 9, 11, 8)                           # a corner of one tile
 
 
 def _one_shape(block, waves, ta, tb, M, N, K):
@@ -96,37 +108,70 @@ def test_nothing_is_written_outside_d_and_hooks_bias_and_fp16_d_work_over_the_ed
         assert oracle.rel_frobenius(out[:M, :N], ref.astype(np.float32)) <= tol, cd
 
 
-def test_misaligned_pointers_fall_back_to_the_bounds_checked_kernel(gpu):
-    """Same configuration, operands that start two bytes off a 16-byte boundary: still right (the library
-    decides per launch)."""
+def test_misaligned_pointers_and_odd_leading_dimensions(gpu):
+    """Operands that start two bytes off a 16-byte boundary inside arrays with odd leading dimensions: the same
+    aligned kernel, the same bits as with aligned copies of the operands."""
     M, N, K = 200, 136, 96
-    conf = checked_config(M, N, K, False, False, (64, 64, 32), (2, 2))
-    a, b, c = operands(M, N, K, False, False, 4200)
-    a_big = np.zeros((M + 8, K), np.float16, order="F"); a_big[1:M + 1, :] = a
-    b_big = np.zeros((K + 8, N), np.float16, order="F"); b_big[1:K + 1, :] = b
-    A, B, C = gk.colmajor(a_big)[1:M + 1, :], gk.colmajor(b_big)[1:K + 1, :], gk.colmajor(c)
-    assert A.data_ptr() % 16 == 2 and B.data_ptr() % 16 == 2
-    D = gk.colmajor_empty((M, N), torch.float32)
-    gk.matmul(conf, A, B, C, D, kernel=Kernel.matmul_singlestage)
-    torch.cuda.synchronize()
-    ref = helpers.run_oracle(conf, a, b, c, (M, N))
-    assert oracle.rel_frobenius(gk.to_numpy(D), ref) <= 1e-3
-    # and aligned operands of the same configuration: the aligned kernel, same values up to the order of the sums
-    D2 = gk.colmajor_empty((M, N), torch.float32)
-    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), C, D2, kernel=Kernel.matmul_singlestage)
-    torch.cuda.synchronize()
-    assert oracle.rel_frobenius(gk.to_numpy(D2), ref) <= 1e-3
+    for ta, tb in ((False, False), (True, True), (False, True), (True, False)):
+        conf = checked_config(M, N, K, ta, tb, (64, 64, 32), (2, 2))
+        assert "checked" not in gk.kernel_name(conf, Kernel.matmul_singlestage)
+        a, b, c = operands(M, N, K, ta, tb, 4200)
+        a_big = np.zeros((a.shape[0] + 9, a.shape[1]), np.float16, order="F"); a_big[1:a.shape[0] + 1, :] = a
+        b_big = np.zeros((b.shape[0] + 11, b.shape[1]), np.float16, order="F"); b_big[1:b.shape[0] + 1, :] = b
+        A, B, C = gk.colmajor(a_big)[1:a.shape[0] + 1, :], gk.colmajor(b_big)[1:b.shape[0] + 1, :], gk.colmajor(c)
+        assert A.data_ptr() % 16 == 2 and B.data_ptr() % 16 == 2 and A.stride(1) % 2 == 1 and B.stride(1) % 2 == 1
+        D = gk.colmajor_empty((M, N), torch.float32)
+        gk.matmul(conf, A, B, C, D, kernel=Kernel.matmul_singlestage)
+        torch.cuda.synchronize()
+        ref = helpers.run_oracle(conf, a, b, c, (M, N))
+        assert oracle.rel_frobenius(gk.to_numpy(D), ref) <= 1e-3
+        D2 = gk.colmajor_empty((M, N), torch.float32)
+        gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), C, D2, kernel=Kernel.matmul_singlestage)
+        torch.cuda.synchronize()
+        assert np.array_equal(gk.to_numpy(D2), gk.to_numpy(D)), (ta, tb)
+
+
+def test_the_last_element_of_an_operand_may_be_the_last_of_its_allocation(gpu):
+    """The chunk that straddles the last row of A in the last k must not be read past the end of A: here A and B
+    end exactly where their device allocations end (the library's own allocator, sizes rounded to nothing)."""
+    import ctypes
+    from gemmkernels import _lib
+    lib = _lib.lib()
+    M, N, K = 2 * 256 - 3, 256 + 5, 64 + 7
+    for ta, tb in ((False, False), (True, True)):
+        conf = checked_config(M, N, K, ta, tb, (256, 256, 64), (2, 4), zero_c=True)
+        a, b, _ = operands(M, N, K, ta, tb, 4250)
+        # place the operands at the very end of 2 MiB allocations
+        size = 2 << 20
+        pa, pb = ctypes.c_void_p(), ctypes.c_void_p()
+        assert lib.gk_dev_alloc(size, ctypes.byref(pa)) == 0 and lib.gk_dev_alloc(size, ctypes.byref(pb)) == 0
+        try:
+            a_addr = pa.value + size - a.nbytes
+            b_addr = pb.value + size - b.nbytes
+            assert lib.gk_copy_to_device(a_addr, a.ctypes.data, a.nbytes) == 0
+            assert lib.gk_copy_to_device(b_addr, b.ctypes.data, b.nbytes) == 0
+            D = gk.colmajor_empty((M, N), torch.float32)
+            cconf = conf.to_c(a.shape[0], b.shape[0], M, M)
+            print("case end of allocation", ta, tb, hex(a_addr), hex(b_addr), flush=True)
+            rc = lib.gk_matmul(ctypes.byref(cconf), a_addr, b_addr, None, D.data_ptr(), None, None, Kernel.matmul_singlestage.code, None)
+            assert rc == 0, _lib.last_error()
+            torch.cuda.synchronize()
+            ref = helpers.run_oracle(conf, a, b, None, (M, N))
+            assert oracle.rel_frobenius(gk.to_numpy(D), ref) <= 1e-3
+        finally:
+            lib.gk_dev_free(pa)
+            lib.gk_dev_free(pb)
 
 
 def test_full_size_4000(gpu):
     """mul!(C, A, B) at 4000^3: one launch of the 256 x 256 tile, checked through linearity and a few exact rows."""
-    from gemmkernels.matmul import matmatmul_plan, PlanSequence
+    from gemmkernels.matmul import matmatmul_plan
     n = 4000
     a = rng.matrix("upm1_f16", 4301, (n, n)); b = rng.matrix("upm1_f16", 4302, (n, n))
     A, B = gk.colmajor(a), gk.colmajor(b)
     C = gk.colmajor_empty((n, n), torch.float32)
     p = matmatmul_plan(C, "N", "N", A, B, 1.0, 0.0)
-    assert not isinstance(p, PlanSequence) and "checked" not in p.kernel_names[0], p.kernel_names
+    assert "checked" not in p.kernel_names[0], p.kernel_names
     p()
     torch.cuda.synchronize()
     out = gk.to_numpy(C)

@@ -53,8 +53,8 @@ def test_two_calls_in_a_row_the_second_smaller(gpu):
     _both_ways(128, 192, 2048, (64, 64, 64), 7200)
     print("no-alloc K-split: 256 x 256 x 8192 on 128 x 128 x 64 tiles", flush=True)
     _both_ways(256, 256, 8192, (128, 128, 64), 7300)
-    print("no-alloc K-split: 64 x 64 x 1024", flush=True)
-    _both_ways(64, 64, 1024, (64, 64, 64), 7400)
+    print("no-alloc K-split: 64 x 64 x 4096", flush=True)
+    _both_ways(64, 64, 4096, (64, 64, 64), 7400)
 
 
 def test_a_product_beyond_the_static_workspace_is_refused(gpu):
