@@ -462,6 +462,13 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
       return fail(GK_ERR_OP_SHAPE, "The base FPU operator shape should adhere to the following constraint: OPERATOR_K_BASE = 1.");
     if (op.M % op.mb != 0 || op.N % op.nb != 0 || op.K % op.kb != 0)
       return fail(GK_ERR_OP_SHAPE, "The operator shape should adhere to the following constraint: OPERATOR_M, OPERATOR_N, OPERATOR_K are multiples of OPERATOR_M_BASE, OPERATOR_N_BASE, OPERATOR_K_BASE, respectively.");
+    // The base shape says how the lanes of a wave are laid over a block of outputs; the operator shape, how many
+    // outputs a lane owns.  Neither changes a result (every output is one fma chain in ascending k).  The
+    // vector-ALU kernels are compiled for the square 8 x 8 lane grid and own their outputs in 4-wide chunks
+    // whatever the operator shape says; another lane grid is refused rather than silently replaced.
+    if (op.mb != 8 || op.nb != 8)
+      return fail(GK_ERR_OP_SHAPE, "The vector-ALU kernels of this library are compiled for the base shape OPERATOR_M_BASE = OPERATOR_N_BASE = 8 "
+                                   "(a wave as an 8 x 8 grid of lanes), got %d x %d.", op.mb, op.nb);
   } else if (is_mfma_kind(op.kind)) {
     const bool native = (op.M == 32 && op.N == 32 && op.K == 16);
     const bool wmma_compat = (op.K == 16) && ((op.M == 16 && op.N == 16) || (op.M == 8 && op.N == 32) || (op.M == 32 && op.N == 8));

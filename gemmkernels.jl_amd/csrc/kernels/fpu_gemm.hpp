@@ -68,10 +68,31 @@ __device__ __forceinline__ X apply_op_t(int kind, float p0, float p1, X x) {
   }
 }
 
-template <typename X>
-__device__ __forceinline__ X apply_list_t(const OpList& t, X x) {
-  for (int i = 0; i < t.n; ++i) x = apply_op_t<X>(t.kind[i], t.p0[i], t.p1[i], x);
-  return x;
+// A list applied to COUNT values at once.  The loop over the slots of the list is unrolled (with constant indices
+// the launch arguments stay in the kernel-argument segment; a run-time index makes the compiler copy the whole
+// argument block to scratch memory once the kernel is large, and every later access to it then goes to memory)
+// and the switch on the op is paid once per slot, not once per value.
+template <typename X, int COUNT>
+__device__ __forceinline__ void apply_list_regs_t(const OpList& t, X (&x)[COUNT]) {
+#pragma unroll
+  for (int i = 0; i < kMaxOps; ++i)
+    if (i < t.n) {
+      const float p0 = t.p0[i], p1 = t.p1[i];
+      auto each = [&](auto kind_c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < COUNT; ++e) x[e] = apply_op_t<X>(decltype(kind_c)::value, p0, p1, x[e]);
+      };
+      switch (t.kind[i]) {
+        case T_SCALE: each(std::integral_constant<int, T_SCALE>{}); break;
+        case T_ADD: each(std::integral_constant<int, T_ADD>{}); break;
+        case T_RELU: each(std::integral_constant<int, T_RELU>{}); break;
+        case T_NEG: each(std::integral_constant<int, T_NEG>{}); break;
+        case T_ABS: each(std::integral_constant<int, T_ABS>{}); break;
+        case T_CLAMP: each(std::integral_constant<int, T_CLAMP>{}); break;
+        case T_SQUARE: each(std::integral_constant<int, T_SQUARE>{}); break;
+        default: break;
+      }
+    }
 }
 
 // acc <- a * b + acc with one rounding (floats) or wrap-around (integers): operator_fma of FPUOp
@@ -86,8 +107,10 @@ __device__ __forceinline__ TACC fpu_fma(TACC a, TACC b, TACC c) {
 }
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, typename TIN_, bool A_KMAJOR_, bool B_KMAJOR_, bool CHECKED_,
-          bool TROPICAL_, typename TACC_ = float>
+          bool TROPICAL_, typename TACC_ = float, bool FUSED_ = true>
 struct FpuGemmConfig {
+  // FUSED: the kernel carries the eight transform hooks and the bias; without, none of that code exists
+  static constexpr bool FUSED = FUSED_;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, CHECKED = CHECKED_, TROPICAL = TROPICAL_;
   typedef TIN_ TIN;
@@ -101,6 +124,12 @@ struct FpuGemmConfig {
   static constexpr int LDS_BYTES = (BK * LDA_S + BK * LDB_S) * (int)sizeof(TACC);
   static constexpr int A_CHUNKS = BM * BK / 4, B_CHUNKS = BN * BK / 4;
   static constexpr int A_PER_THREAD = A_CHUNKS / THREADS, B_PER_THREAD = B_CHUNKS / THREADS;
+  // K tiles whose global loads are in flight (in registers) while the current one is multiplied: the fma chain
+  // of a tile is shorter than the memory latency, so one tile ahead left every tile waiting for its loads
+  // (256^3 on 16 workgroups: 19.4 us with one tile in flight)
+  // -- four tiles without hooks, two with; the bounds-checked and the 64-bit kernels stay with one (their
+  // per-element loads and wide registers make deeper buffers expensive to compile and to hold)
+  static constexpr int DEPTH = (CHECKED_ || sizeof(TIN_) > 4) ? 1 : (FUSED_ ? 2 : 4);
   static_assert(TM % 4 == 0 && TN % 4 == 0, "a lane owns whole 4-wide chunks");
   static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "tile loads divide evenly over the threads");
   static_assert(!TROPICAL || std::is_same<TACC, float>::value, "the max-plus product is compiled for fp32");
@@ -147,6 +176,14 @@ __device__ __forceinline__ void load_chunk(const typename Cfg::TIN* __restrict__
   }
 }
 
+template <int I, int N, class F>
+__device__ __forceinline__ void fpu_static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    fpu_static_for<I + 1, N>(f);
+  }
+}
+
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs args) {
   typedef typename Cfg::TIN TIN;
@@ -169,8 +206,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
   const TIN* B = (const TIN*)args.b;
   const TACC* C = (const TACC*)args.c;
   const bool zero_ab = (args.a_kind == 0 /* Layout.Zero */);
-  const bool xf_a = args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0;
-  const bool xf_b = args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0;
+  const bool xf_a = Cfg::FUSED && (args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0);
+  const bool xf_b = Cfg::FUSED && (args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0);
 
   // accumulators: acc[i][j] is row wm*WTM + (i/4)*32 + 4*ly + i%4, column wn*WTN + (j/4)*32 + 4*lx + j%4
   TACC acc[TM][TN];
@@ -184,48 +221,77 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
       if (args.c_mode != 0) {
         const int r = row_of(i), cc = col_of(j);
         if (!Cfg::CHECKED || (r < args.M && cc < args.N)) c = C[r + (long long)cc * args.ldc];
-        c = apply_list_t<TACC>(args.t[H_GL2SH_C], c);
-        c = apply_list_t<TACC>(args.t[H_SH2RF_C], c);
       }
       acc[i][j] = c;
     }
+  // one hook over all accumulators of the lane
+  [[maybe_unused]] auto hook_acc = [&](const OpList& t) __attribute__((always_inline)) {
+    TACC flat[TM * TN];
+#pragma unroll
+    for (int q = 0; q < TM * TN; ++q) flat[q] = acc[q % TM][q / TM];
+    apply_list_regs_t<TACC, TM * TN>(t, flat);
+#pragma unroll
+    for (int q = 0; q < TM * TN; ++q) acc[q % TM][q / TM] = flat[q];
+  };
+  if constexpr (Cfg::FUSED) {
+    if (args.c_mode != 0) {
+      hook_acc(args.t[H_GL2SH_C]);
+      hook_acc(args.t[H_SH2RF_C]);
+    }
+  }
 
-  TIN ra[Cfg::A_PER_THREAD][4], rb[Cfg::B_PER_THREAD][4];
-  bool pa[Cfg::A_PER_THREAD][4], pb[Cfg::B_PER_THREAD][4];
-  int ar[Cfg::A_PER_THREAD], ak[Cfg::A_PER_THREAD], br[Cfg::B_PER_THREAD], bk[Cfg::B_PER_THREAD];
+  constexpr int DEPTH = Cfg::DEPTH;
+  TIN ra[DEPTH][Cfg::A_PER_THREAD][4], rb[DEPTH][Cfg::B_PER_THREAD][4];
+  bool pa[DEPTH][Cfg::A_PER_THREAD][4], pb[DEPTH][Cfg::B_PER_THREAD][4];
+  int ar[Cfg::A_PER_THREAD], ak[Cfg::A_PER_THREAD], br[Cfg::B_PER_THREAD], bk[Cfg::B_PER_THREAD];   // the same for every tile
 
-  auto fetch = [&](int k0) {
+  auto fetch = [&](int k0, auto slot_c) __attribute__((always_inline)) {
+    constexpr int S = decltype(slot_c)::value;
 #pragma unroll
     for (int i = 0; i < Cfg::A_PER_THREAD; ++i) {
-      load_chunk<Cfg, BM, Cfg::A_KMAJOR>(A, args.lda, m0, k0, tid + i * Cfg::THREADS, args.M, args.K, zero_ab, ra[i], pa[i], ar[i], ak[i]);
+      load_chunk<Cfg, BM, Cfg::A_KMAJOR>(A, args.lda, m0, k0, tid + i * Cfg::THREADS, args.M, args.K, zero_ab, ra[S][i], pa[S][i], ar[i], ak[i]);
     }
 #pragma unroll
     for (int i = 0; i < Cfg::B_PER_THREAD; ++i) {
-      load_chunk<Cfg, BN, Cfg::B_KMAJOR>(B, args.ldb, n0, k0, tid + i * Cfg::THREADS, args.N, args.K, zero_ab, rb[i], pb[i], br[i], bk[i]);
+      load_chunk<Cfg, BN, Cfg::B_KMAJOR>(B, args.ldb, n0, k0, tid + i * Cfg::THREADS, args.N, args.K, zero_ab, rb[S][i], pb[S][i], br[i], bk[i]);
     }
   };
   // the two load hooks, each rounded to the element type of its destination (the operand's own
   // type), then the conversion to the accumulator type for the fma
   auto prepare = [&](const TIN (&v)[4], const bool (&pad)[4], bool xf, const OpList& t0, const OpList& t1, TACC (&out)[4]) {
+    TIN x[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] = v[e];
+    if constexpr (Cfg::FUSED) {
+      if (xf) {
+        TAR y[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = (TAR)x[e];
+        if (t0.n > 0) {
+          apply_list_regs_t<TAR, 4>(t0, y);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] = (TAR)(TIN)y[e];       // rounded to the operand's type between the hooks
+        }
+        if (t1.n > 0) apply_list_regs_t<TAR, 4>(t1, y);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = (TIN)y[e];
+      }
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      TIN x = v[e];
-      if (xf) {
-        if (t0.n > 0) x = (TIN)apply_list_t<TAR>(t0, (TAR)x);
-        if (t1.n > 0) x = (TIN)apply_list_t<TAR>(t1, (TAR)x);
-      }
-      TACC y = (TACC)x;
+      TACC y = (TACC)x[e];
       if constexpr (Cfg::TROPICAL && Cfg::CHECKED) {
         if (pad[e]) y = -__builtin_inff();
       }
       out[e] = y;
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](auto slot_c) __attribute__((always_inline)) {
+    constexpr int S = decltype(slot_c)::value;
 #pragma unroll
     for (int i = 0; i < Cfg::A_PER_THREAD; ++i) {
       TACC v[4];
-      prepare(ra[i], pa[i], xf_a, args.t[H_GL2SH_A], args.t[H_SH2RF_A], v);
+      prepare(ra[S][i], pa[S][i], xf_a, args.t[H_GL2SH_A], args.t[H_SH2RF_A], v);
       if (Cfg::A_KMAJOR) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) As[(ak[i] + e) * Cfg::LDA_S + ar[i]] = v[e];
@@ -236,7 +302,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
 #pragma unroll
     for (int i = 0; i < Cfg::B_PER_THREAD; ++i) {
       TACC v[4];
-      prepare(rb[i], pb[i], xf_b, args.t[H_GL2SH_B], args.t[H_SH2RF_B], v);
+      prepare(rb[S][i], pb[S][i], xf_b, args.t[H_GL2SH_B], args.t[H_SH2RF_B], v);
       if (Cfg::B_KMAJOR) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) Bs[(bk[i] + e) * Cfg::LDB_S + br[i]] = v[e];
@@ -247,12 +313,19 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
   };
 
   const int KT = (args.K + BK - 1) / BK;
-  fetch(0);
-  for (int kt = 0; kt < KT; ++kt) {
+  fpu_static_for<0, DEPTH>([&](auto slot_c) __attribute__((always_inline)) {
+    constexpr int S = decltype(slot_c)::value;
+    if (S < KT) fetch(S * BK, slot_c);
+  });
+  for (int kt0 = 0; kt0 < KT; kt0 += DEPTH)
+  fpu_static_for<0, DEPTH>([&](auto slot_c) __attribute__((always_inline)) {
+    constexpr int S = decltype(slot_c)::value;       // register buffer of tile kt
+    const int kt = kt0 + S;
+    if (kt < KT) {
     __syncthreads();          // everyone is done reading the previous tile
-    stash();
+    stash(slot_c);
     __syncthreads();
-    if (kt + 1 < KT) fetch((kt + 1) * BK);
+    if (kt + DEPTH < KT) fetch((kt + DEPTH) * BK, slot_c);      // its buffer is free again
     const TACC* ap = As + wm * Cfg::WTM + 4 * ly;
     const TACC* bp = Bs + wn * Cfg::WTN + 4 * lx;
 #pragma unroll 4
@@ -280,33 +353,47 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
           }
         }
     }
-  }
+    }
+  });
 
   // epilogue: transform, bias, transform, store (4 consecutive rows per vector store); the bias of
   // Epilogue.Bias is fp32 (reference src/epilogue.jl:44-52) and only offered with fp32 accumulators
   TACC* D = (TACC*)args.d;
+  if constexpr (Cfg::FUSED) {
+    hook_acc(args.t[H_RF2SH_D]);
+    if constexpr (std::is_same<TACC, float>::value) {
+      if (args.epi_kind == 1) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int cc = col_of(j);
+          const float bv = args.bias[Cfg::CHECKED ? (cc < args.N ? cc : 0) : cc];
+#pragma unroll
+          for (int i = 0; i < TM; ++i) acc[i][j] = acc[i][j] + bv;
+        }
+      } else if (args.epi_kind == 2) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int r = row_of(i);
+          const float bv = args.bias[Cfg::CHECKED ? (r < args.M ? r : 0) : r];
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = acc[i][j] + bv;
+        }
+      }
+    }
+    hook_acc(args.t[H_SH2GL_D]);
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int cc = col_of(j);
 #pragma unroll
     for (int c = 0; c < Cfg::CM; ++c) {
-      TACC x[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        TACC v = apply_list_t<TACC>(args.t[H_RF2SH_D], acc[4 * c + e][j]);
-        if constexpr (std::is_same<TACC, float>::value) {
-          if (args.epi_kind == 1) v = v + args.bias[Cfg::CHECKED ? (cc < args.N ? cc : 0) : cc];
-          else if (args.epi_kind == 2) { const int r = row_of(4 * c + e); v = v + args.bias[Cfg::CHECKED ? (r < args.M ? r : 0) : r]; }
-        }
-        x[e] = apply_list_t<TACC>(args.t[H_SH2GL_D], v);
-      }
       const int r = row_of(4 * c);
       if (!Cfg::CHECKED) {
-        *(acc4*)&D[r + (long long)cc * args.ldd] = (acc4){x[0], x[1], x[2], x[3]};
+        *(acc4*)&D[r + (long long)cc * args.ldd] = (acc4){acc[4 * c][j], acc[4 * c + 1][j], acc[4 * c + 2][j], acc[4 * c + 3][j]};
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (r + e < args.M && cc < args.N) D[r + e + (long long)cc * args.ldd] = x[e];
+          if (r + e < args.M && cc < args.N) D[r + e + (long long)cc * args.ldd] = acc[4 * c + e][j];
       }
     }
   }

@@ -172,9 +172,14 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
     """MI355X block shape: of the tiles of the table that divide the problem, the one with the shortest
     estimated launch (tiles per CU times the cost of a tile).  ``a_kmajor``: A is stored K x M ('T');
     ``b_kmajor``: B is stored K x N ('N'); they admit the tiles with a side of 192."""
-    if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
-        return NT(M=64, N=64, K=32)
     M, N, K = gemm_shape["M"], gemm_shape["N"], gemm_shape["K"]
+    if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
+        # a small Float32 product in whole 32 x 32 x 32 tiles: one wave per workgroup, four times the workgroups
+        # of the 64 x 64 tile (256^3: 64 workgroups instead of 16; every output is still one fma chain in k)
+        if (operator.kind == Operator.FPU and operator.CT.name == "Float32" and operator.AT.name == "Float32" and tile_sized
+                and M % 32 == 0 and N % 32 == 0 and K % 32 == 0 and -(-M // 64) * -(-N // 64) < NUM_CUS // 2):
+            return NT(M=32, N=32, K=32)
+        return NT(M=64, N=64, K=32)
     if operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
         # complex tiles, in complex elements; every MFMA row pair is one complex row
         table = _PLANAR_TILES if planar else _COMPLEX_TILES
@@ -226,7 +231,7 @@ _COMPLEX_TILES = [((128, 256, 32), (2, 4)), ((64, 128, 32), (2, 2)), ((128, 128,
 _PLANAR_TILES = [((128, 256, 64), (2, 4)), ((64, 128, 64), (2, 2)), ((128, 128, 64), (2, 2)), ((64, 128, 32), (2, 2)), ((64, 64, 32), (2, 2))]
 
 # tiles of the vector-ALU kernel and of the bounds-checked MFMA kernel
-_FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2))]
+_FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (1, 1))]
 _CHECKED_TILES = [((64, 64, 32), (2, 2))]
 
 

@@ -215,3 +215,38 @@ def test_odd_sizes_with_16_bit_c(gpu, beta, dtype):
     out = C.float().cpu().numpy()
     ref = 0.5 * a.astype(np.float64) @ b.astype(np.float64).T + beta * c_in
     assert oracle.rel_frobenius(out, ref) <= 2e-3       # FP16 C: one rounding of D to 11 bits; BF16: alpha on A in BF16
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+def test_fpu_operator_shapes(gpu, ta, tb):
+    """The operator-shape sweep of the reference (configs/configs.jl:521-551) on 64-lane waves: operator shapes that
+    are multiples of the 8 x 8 lane grid run and give, bit for bit, the sequential fma chain (the shape only says
+    which lane owns which output); other lane grids are refused with the operator-shape error, not replaced."""
+    from gemmkernels import Kernel, Layout, NT, Operator
+    M = N = K = 128
+    a, b, c = operands(M, N, K, ta, tb, np.float32, 900)
+    la = Layout.UnsafeAlignedRowMajor[Float32] if ta else Layout.UnsafeAlignedColMajor[Float32]
+    lb = Layout.UnsafeAlignedRowMajor[Float32] if tb else Layout.UnsafeAlignedColMajor[Float32]
+    def conf_for(shape, block):
+        return gk.get_config(gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=block[0], N=block[1], K=block[2]),
+                             operator=Operator.FPUOp[(*shape, Float32, Float32)], global_a_layout=la, global_b_layout=lb,
+                             global_c_layout=Layout.UnsafeAlignedColMajor[Float32], global_d_layout=Layout.UnsafeAlignedColMajor[Float32],
+                             is_a_col_major=not ta, is_b_col_major=not tb)
+    ref = None
+    for shape in [(8, 8, 1, 8, 8, 1), (16, 8, 1, 8, 8, 1), (8, 16, 1, 8, 8, 1), (8, 8, 2, 8, 8, 1), (16, 16, 2, 8, 8, 1)]:
+        for block in ((64, 64, 32), (32, 32, 32)):
+            conf = conf_for(shape, block)
+            d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+            if ref is None:
+                ref = helpers.run_oracle(conf, a, b, c, (M, N))
+            assert np.array_equal(d, ref), (shape, block)
+    for shape in [(4, 64, 1, 1, 64, 1), (4, 32, 1, 2, 32, 1), (16, 16, 1, 4, 16, 1), (16, 16, 1, 16, 4, 1), (32, 4, 1, 32, 2, 1), (64, 4, 1, 64, 1, 1)]:
+        with pytest.raises(gk.ConfigError) as ei:
+            conf = conf_for(shape, (128, 128, 32))
+            helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+        assert ei.value.status == _lib_status_op_shape(), shape
+
+
+def _lib_status_op_shape():
+    from gemmkernels import _lib
+    return _lib.GK_ERR_OP_SHAPE

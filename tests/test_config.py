@@ -112,6 +112,7 @@ ERROR_CASES = [
     ("block < 2 x operator (src/config.jl:209-212)", dict(block_shape=NT(M=32, N=128, K=64), compute_warp=NT(M=32, N=32, K=16), warps_per_block=4), _lib.GK_ERR_BLOCK_SHAPE),
     ("unsupported matrix-core shape (src/config.jl:159-169)", dict(operator=Operator.MFMAOp[16, 16, 4, F16, F32]), _lib.GK_ERR_OP_SHAPE),
     ("FPU base shape is not one wave (src/config.jl:147-149)", dict(operator=Operator.FPUOp[8, 8, 1, 4, 8, 1, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
+    ("FPU lane grid other than 8 x 8 (one wave, but not the grid the kernels are compiled for)", dict(operator=Operator.FPUOp[16, 4, 1, 16, 4, 1, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
     ("FPU kb != 1 (src/config.jl:151-153)", dict(operator=Operator.FPUOp[8, 8, 2, 8, 8, 2, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
     ("FPU operator smaller than a wave (src/config.jl:142-145)", dict(operator=Operator.FPUOp[4, 8, 1, 4, 8, 1, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
     ("FPU shape not a multiple of its base (src/config.jl:155-157)", dict(operator=Operator.FPUOp[12, 8, 1, 8, 8, 1, F32, F32], block_shape=NT(M=64, N=64, K=32)), _lib.GK_ERR_OP_SHAPE),
