@@ -206,7 +206,7 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   float post = 1.0f;
   t = fold_pow2_scales(c, t, &folded_storage, &post);      // power-of-two scales of A / B do not run in the K loop
   key->fused = (transforms_present(t) || post != 1.0f || (e && e->kind != GK_EPILOGUE_DEFAULT)) ? 1 : 0;
-  const bool mfma_family = key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT;
+  const bool mfma_family = key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT || key->family == gk::FAMILY_COMPLEX;
   auto ab_hooks = [&]() {
     if (!t) return false;
     const int hooks[4] = {GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A, GK_HOOK_GLOBAL_TO_SHARED_B, GK_HOOK_SHARED_TO_REGS_B};
@@ -258,7 +258,10 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
   if (c->op.kind == GK_OP_MFMA_COMPLEX || c->op.kind == GK_OP_MFMA_DUAL) {
     // interleaved complex operands seen as real matrices: M and K double, and so does every
     // leading dimension (counted in real elements)
-    args->M *= 2; args->K *= 2;
+    // (unless both A and B are contiguous along k, the real views of A and B meet in one real product of 2M x 2N x K)
+    const bool pair = !is_split_layout(c->global_a_layout.kind) && !(is_row_major(c->global_a_layout.kind) && !is_row_major(c->global_b_layout.kind));
+    args->M *= 2;
+    if (pair) args->N *= 2; else args->K *= 2;
     if (is_split_layout(c->global_a_layout.kind)) {
       // planar operands: a matrix is the real array (rows, cols, 2) in column-major order, so the
       // imaginary plane starts ld * cols elements after the real one; the kernel walks K twice
@@ -518,8 +521,23 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
     if (!all_inter && !all_split)
       return fail(GK_ERR_UNSUPPORTED, "complex and dual operators need Interleaved layouts for A and B and InterleavedColMajor for C and D "
                                       "(the complex operator also takes Split layouts for all of them)");
-    if (transforms_present(t) || (e && e->kind != GK_EPILOGUE_DEFAULT))
-      return fail(GK_ERR_UNSUPPORTED, "transforms and bias are not available with the complex and dual operators");
+    // Hooks see complex numbers (src/kernel.jl:167-187, 337-347 hand tiles of the layout's element type to the
+    // transform).  The hooks of C and D take the ops whose result on a complex number is the op on its two parts,
+    // x * p0 and -x, and x + p0, which acts on the real part; max / abs / clamp have no complex counterpart of the
+    // same type.  A bias value is real and goes to the real part.
+    if (t) {
+      const int ab_hooks[4] = {GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A, GK_HOOK_GLOBAL_TO_SHARED_B, GK_HOOK_SHARED_TO_REGS_B};
+      for (int h : ab_hooks)
+        for (int i = 0; i < t->hook[h].n_ops && i < GK_MAX_OPS; ++i)
+          if (t->hook[h].ops[i].kind != GK_T_IDENTITY)
+            return fail(GK_ERR_UNSUPPORTED, "the complex and dual operators take transforms on C and D only");
+      for (int h = 0; h < 8; ++h)
+        for (int i = 0; i < t->hook[h].n_ops && i < GK_MAX_OPS; ++i) {
+          const int k = t->hook[h].ops[i].kind;
+          if (k != GK_T_IDENTITY && k != GK_T_SCALE && k != GK_T_ADD && k != GK_T_NEG)
+            return fail(GK_ERR_UNSUPPORTED, "transform op %d is not defined on complex numbers (scale, add and neg are)", k);
+        }
+    }
   }
   if (c->global_a_layout.kind == GK_LAYOUT_DIAGONAL) {
     if (g.M != g.K) return fail(GK_ERR_DIMENSION_MISMATCH, "Diagonal only supports a square A matrix (M == K)");
@@ -557,7 +575,7 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
     if (op.kind == GK_OP_FPU_TROPICAL && cd != GK_F32) return fail(GK_ERR_UNSUPPORTED, "the max-plus operator is compiled for fp32");
     if (e && e->kind != GK_EPILOGUE_DEFAULT && cd != GK_F32) return fail(GK_ERR_UNSUPPORTED, "the bias epilogue is fp32 (src/epilogue.jl:44-52)");
   } else {
-    const bool cd16_ok = op.kind == GK_OP_MFMA && c->global_a_layout.kind != GK_LAYOUT_DIAGONAL;
+    const bool cd16_ok = c->global_a_layout.kind != GK_LAYOUT_DIAGONAL;
     auto cd_ok = [&](int dt) { return dt == GK_F32 || (cd16_ok && (dt == GK_F16 || dt == GK_BF16)); };
     if (!cd_ok(c->global_d_layout.eltype))
       return fail(GK_ERR_UNSUPPORTED, "element type %d of D is not available with this operator", c->global_d_layout.eltype);
@@ -792,7 +810,9 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
     // extents in the unit the leading dimensions count: real elements (two per complex number of an
     // interleaved matrix, one per complex number of a plane)
     const bool planar = is_split_layout(conf->global_a_layout.kind);
-    const long long em = planar ? conf->matmul_shape.M : args.M, ek = planar ? conf->matmul_shape.K : args.K;
+    const bool cplx = conf->op.kind == GK_OP_MFMA_COMPLEX || conf->op.kind == GK_OP_MFMA_DUAL;
+    const long long em = planar ? conf->matmul_shape.M : args.M;
+    const long long ek = (cplx && !planar) ? 2ll * conf->matmul_shape.K : conf->matmul_shape.K;
     if (!a_zero && conf->global_a_layout.kind != GK_LAYOUT_DIAGONAL && conf->global_a_layout.kind != GK_LAYOUT_GETT &&
         args.lda < (a_row ? ek : em))
       return fail(GK_ERR_DIMENSION_MISMATCH, "lda = %lld is smaller than the leading extent of A", args.lda);

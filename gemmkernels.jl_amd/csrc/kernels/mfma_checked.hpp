@@ -180,9 +180,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
       wait_lgkmcnt<0>();
       int4v va[FM], vb[FN];
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi) { RA::pin_raw(fa[fi]); va[fi] = RA::finish(fa[fi]); }
+      for (int fi = 0; fi < FM; ++fi) { RA::pin_raw(fa[fi]); va[fi] = RA::finish(fa[fi], lane); }
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[fj]); vb[fj] = RB::finish(fb[fj]); }
+      for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[fj]); vb[fj] = RB::finish(fb[fj], lane); }
 #pragma unroll
       for (int fi = 0; fi < FM; ++fi)
 #pragma unroll

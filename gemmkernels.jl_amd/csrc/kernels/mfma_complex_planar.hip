@@ -8,6 +8,7 @@
 // so it runs on the real MFMA kernel with a real tile of 2*BM rows and two passes over K; only the
 // tile addressing and one sign flip of the upper accumulators differ (FIX_PLANAR).  Every element
 // of A and B is staged through LDS exactly as in the real kernel; nothing is expanded in registers.
+// Every instance carries the hooks of C and D and the bias (they cost nothing when absent).
 // Tile shapes below are in complex elements.
 #include "mfma_gemm.hpp"
 #include "registry.hpp"
@@ -16,12 +17,12 @@ namespace gk {
 
 int family_complex_planar(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode, InstanceInfo* info,
                           hipError_t* err) {
-  if (key.dtype != DT_F16 || key.fused != 0 || key.variant != 2) return 0;
+  if (key.dtype != DT_F16 || (key.fused != 0 && key.fused != 3) || key.variant != 2) return 0;
 #define GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, akm_, bkm_, NAME)                                                          \
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
       key.a_kmajor == akm_ && key.b_kmajor == bkm_) {                                                                     \
     typedef MfmaGemmConfig<2 * bm_, bn_, bk_, wm_, wn_, st_, (akm_ ? OPK_KMAJOR : OPK_MMAJOR),                             \
-                           (bkm_ ? OPK_KMAJOR : OPK_MMAJOR), _Float16, 0, false, FIX_PLANAR, false, 16> Cfg;                          \
+                           (bkm_ ? OPK_KMAJOR : OPK_MMAJOR), _Float16, 3, false, FIX_PLANAR, false, 16> Cfg;                          \
     return run_instance<Cfg>(mfma_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
 #define GK_PLANAR_T(bm_, bn_, bk_, wm_, wn_, st_)                                                               \

@@ -28,23 +28,31 @@ namespace gk {
 // dimension (m or n), BK the number of 16-bit k-values per K step.
 //   OPK_KMAJOR: LDS row = tile row, 16-byte chunk c = k / 8            (memory contiguous along k)
 //   OPK_MMAJOR: LDS row = k,        16-byte chunk c = row / 8          (memory contiguous along m / n)
-//   OPK_CROWK : interleaved complex data contiguous along m / n: LDS row = complex k, one 32-bit
-//               (re, im) element per complex row index
+//   OPK_KPAIR : interleaved complex data contiguous along k, for the FIX_PAIR products: LDS row = complex
+//               row index (R/2 of them), 16-byte chunk c = complex k / 4; the two MFMA rows of a complex row
+//               read the same 32 bytes (8 complex k) and keep the real or the imaginary halves
 // EXPAND marks the A operand of a complex (or dual-number) product: one complex row feeds two MFMA
 // rows, so the tile holds R/2 complex rows.
 // ----------------------------------------------------------------------------------------------
-enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_CROWK = 2 };
+enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_KPAIR = 3 };
 // FIX_PLANAR: complex product on planar (split re / im) matrices.  Nothing is expanded in registers:
 // a workgroup owns BM/2 complex rows, the upper half of its real tile is the real plane of D and the
 // lower half the imaginary plane, and K runs twice: first over B_im with [A_im; A_re] as the A tile,
 // then over B_re with [A_re; A_im].  The upper half starts from -C_re and flips the sign of its
 // accumulators between the two passes, which gives C_re - A_im B_im + A_re B_re.
-enum : int { FIX_NONE = 0, FIX_COMPLEX = 1, FIX_DUAL = 2, FIX_PLANAR = 3 };
+// FIX_PAIR / FIX_PAIR_DUAL: complex (dual-number) product on interleaved matrices as ONE real product of the
+// matrices seen as real ones.  An interleaved matrix whose contiguous index is m (or n) is a real matrix with
+// twice the rows, row 2m the real and row 2m+1 the imaginary part, and the K loop of the real kernel runs on it
+// unchanged (K counts complex k); one whose contiguous index is k is read as OPK_KPAIR.  The 2M x 2N real
+// product holds the four real products re*re, re*im, im*re, im*im of every complex element of D in the lanes
+// 2i, 2i+1 (the two parts of a row of A) and the accumulator values 2j, 2j+1 (the two parts of a column of B);
+// they are combined once, before the epilogue (pair_combine).
+enum : int { FIX_NONE = 0, FIX_COMPLEX = 1, FIX_DUAL = 2, FIX_PLANAR = 3, FIX_PAIR = 4, FIX_PAIR_DUAL = 5 };
 
 template <int R, int BK, int KIND, bool EXPAND>
 struct OperandGeom {
-  static constexpr int LDS_ROWS = KIND == OPK_KMAJOR ? (EXPAND ? R / 2 : R) : (KIND == OPK_MMAJOR ? BK : BK / 2);
-  static constexpr int ROW_BYTES = KIND == OPK_KMAJOR ? BK * 2 : (KIND == OPK_MMAJOR ? R * 2 : (EXPAND ? R * 2 : R * 4));
+  static constexpr int LDS_ROWS = KIND == OPK_KMAJOR ? (EXPAND ? R / 2 : R) : (KIND == OPK_KPAIR ? R / 2 : BK);
+  static constexpr int ROW_BYTES = KIND == OPK_KMAJOR ? BK * 2 : (KIND == OPK_KPAIR ? BK * 4 : R * 2);
   static constexpr int CPR = ROW_BYTES / 16;                   // 16-byte chunks per LDS row
   static constexpr int BYTES = LDS_ROWS * ROW_BYTES;
   static constexpr int NDMA = BYTES / 1024;                    // wave-wide 16 B/lane DMA instructions per tile
@@ -52,6 +60,9 @@ struct OperandGeom {
   // K-major: XOR the chunk index with the row (per 256 B) so that 32 consecutive rows at one chunk
   // index spread evenly over the 16 chunk slots of the 64 banks.
   __device__ static __forceinline__ int swz_k(int row) { return (row / RP256) & (CPR - 1); }
+  // OPK_KPAIR: the same with pairs of chunks (a lane reads two neighbouring chunks from one address), so that
+  // the 8 complex rows of a 16-lane group spread over the 8 32-byte slots of the bank period
+  __device__ static __forceinline__ int swz_kp(int row) { return ((row / RP256) & (CPR / 2 - 1)) << 1; }
   // M-major: XOR the 64-byte group index with k so that 4 consecutive k rows at one group land in
   // 4 different 64-byte slots of the 256-byte bank period.
   // Rows of 384 bytes (192 elements): consecutive k rows are already 128 bytes apart in the bank period, so
@@ -67,7 +78,7 @@ struct OperandGeom {
   static_assert(!ROW_384 || GROUPS % 2 == 0, "the group XOR of 384-byte rows pairs groups");
   static_assert(KIND != OPK_MMAJOR || CPR >= 4, "M-major tiles need at least 32 rows");
   static_assert(BYTES % 1024 == 0, "tile must be a whole number of DMA instructions");
-  static_assert(!EXPAND || KIND != OPK_MMAJOR, "complex operands are K-major or complex-row tiles");
+  static_assert(!EXPAND || KIND == OPK_KMAJOR, "an operand that is expanded in registers is K-major");
 };
 
 // Where lane `lane` of DMA instruction q reads: LDS row `row` of the tile and the first of its 8
@@ -79,8 +90,8 @@ __device__ __forceinline__ void dma_lane_coords(int q, int lane, int& row, int& 
   row = p / G::CPR;
   const int cs = p % G::CPR;
   if (KIND == OPK_KMAJOR) col = (cs ^ G::swz_k(row)) * 8;
-  else if (KIND == OPK_MMAJOR) col = (((cs >> 2) ^ G::swz_m(row)) * 4 + ((cs & 3) ^ (((row >> 3) & 1) << 1))) * 8;
-  else col = cs * 8;
+  else if (KIND == OPK_KPAIR) col = (cs ^ G::swz_kp(row)) * 8;
+  else col = (((cs >> 2) ^ G::swz_m(row)) * 4 + ((cs & 3) ^ (((row >> 3) & 1) << 1))) * 8;
 }
 
 // Tensor-contraction index maps: walks the K index of a contraction tile by tile.  The first K
@@ -140,13 +151,13 @@ struct FragReader {
   // M-major, 16-row fragments: fragments 2j and 2j+1 are the two 32-byte halves of one 64-byte group, so one
   // address serves both (the odd one is the even one with bit 5 flipped)
   static constexpr bool PAIRED = KIND == OPK_MMAJOR && MI == 16 && F % 2 == 0;
-  static constexpr int NBASE = KIND == OPK_KMAJOR ? KSTEPS : (KIND == OPK_MMAJOR ? (PAIRED ? F / 2 : F) : 1);
-  static constexpr int OPS = KIND == OPK_KMAJOR ? 1 : (KIND == OPK_MMAJOR ? 2 : 4);   // LDS instructions per fragment
-  static constexpr int FRAG_ROWS = EXPAND ? MI / 2 : MI;       // tile rows (complex rows when EXPAND) per fragment
+  static constexpr int NBASE = (KIND == OPK_KMAJOR || KIND == OPK_KPAIR) ? KSTEPS : (PAIRED ? F / 2 : F);
+  static constexpr int OPS = KIND == OPK_KMAJOR ? 1 : 2;   // LDS instructions per fragment
+  static constexpr int FRAG_ROWS = (EXPAND || KIND == OPK_KPAIR) ? MI / 2 : MI;       // tile rows (complex rows when EXPAND / OPK_KPAIR) per fragment
   struct Raw {
-    int4v q;          // OPK_KMAJOR
+    int4v q;          // OPK_KMAJOR; OPK_KPAIR: complex k 0..3 of the lane's eight
+    int4v q1;         // OPK_KPAIR: complex k 4..7
     int2v lo, hi;     // OPK_MMAJOR
-    int x0, x1, x2, x3;   // OPK_CROWK
   };
   unsigned cur[NBASE];                          // lane-dependent byte addresses inside the tile of the current stage
   unsigned stage_addr;                          // LDS address of that tile (wave-uniform)
@@ -160,7 +171,16 @@ struct FragReader {
         const int c = ks * (KSTEP_K / 8) + (lane / MI);
         cur[ks < NBASE ? ks : 0] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_k(row)));
       }
-    } else if (KIND == OPK_MMAJOR) {
+    } else if (KIND == OPK_KPAIR) {
+      // MFMA row r of the block tile is part r & 1 of complex row r >> 1; the lane's eight k-slots of a k-step
+      // are the complex k 8*(lane/MI) .. +7 of it: chunks 2*(lane/MI) and the next one (the swizzle is even)
+      const int row = (row0 + (lane % MI)) >> 1;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int c = ks * (KSTEP_K / 4) + 2 * (lane / MI);
+        cur[ks < NBASE ? ks : 0] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_kp(row)));
+      }
+    } else {
       const int i = lane & 15;
       const int k = 8 * (lane / MI) + (i >> 2);
       const int m = (MI == 32 ? (lane & 16) : 0) + 4 * (i & 3);          // offset inside the fragment
@@ -172,9 +192,6 @@ struct FragReader {
         const int c = ((mm >> 3) & 3) ^ (((k >> 3) & 1) << 1);
         cur[(PAIRED ? fi / 2 : fi) < NBASE ? (PAIRED ? fi / 2 : fi) : 0] = (unsigned)(k * G::ROW_BYTES + g * 64 + c * 16 + (mm & 4) * 2);
       }
-    } else {
-      const int elem = EXPAND ? ((row0 + (lane % MI)) >> 1) : (row0 + (lane % MI));
-      cur[0] = (unsigned)(4 * (lane / MI) * G::ROW_BYTES + elem * 4);
     }
     stage_addr = 0;
   }
@@ -192,6 +209,11 @@ struct FragReader {
     if constexpr (SYNC && KIND == OPK_KMAJOR) {
       asm volatile("ds_read_b128 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
       return;
+    } else if constexpr (SYNC && KIND == OPK_KPAIR) {
+      asm volatile("ds_read_b128 %0, %2 offset:%3\n\tds_read_b128 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
+                   : "=&v"(r.q), "=&v"(r.q1)
+                   : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES), "n"(FI * FRAG_ROWS * G::ROW_BYTES + 16) : "memory");
+      return;
     } else if constexpr (SYNC && KIND == OPK_MMAJOR) {
       asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
                    : "=&v"(r.lo), "=&v"(r.hi)
@@ -200,14 +222,12 @@ struct FragReader {
     }
     if (KIND == OPK_KMAJOR) {
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
-    } else if (KIND == OPK_MMAJOR) {
+    } else if (KIND == OPK_KPAIR) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q1) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES + 16) : "memory");
+    } else {
       asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.lo) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K) * G::ROW_BYTES) : "memory");
       asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.hi) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K + 4) * G::ROW_BYTES) : "memory");
-    } else {
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x0) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 0) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x1) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 1) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x2) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 2) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r.x3) : "v"(cur[0]), "n"((KS * (KSTEP_K / 2) + 3) * G::ROW_BYTES + FI * FRAG_ROWS * 4) : "memory");
     }
   }
   template <int FI>
@@ -217,25 +237,32 @@ struct FragReader {
   }
   __device__ static __forceinline__ void pin_raw(Raw& r) {
     if (KIND == OPK_KMAJOR) pin(r.q);
-    else if (KIND == OPK_MMAJOR) { pin(r.lo); pin(r.hi); }
-    else { pin(r.x0); pin(r.x1); pin(r.x2); pin(r.x3); }
+    else if (KIND == OPK_KPAIR) { pin(r.q); pin(r.q1); }
+    else { pin(r.lo); pin(r.hi); }
   }
-  __device__ static __forceinline__ int4v finish(const Raw& r) {
+  __device__ static __forceinline__ int4v finish(const Raw& r, [[maybe_unused]] int lane) {
     if (KIND == OPK_KMAJOR) return r.q;
     int4v v;
-    if (KIND == OPK_MMAJOR) { v[0] = r.lo[0]; v[1] = r.lo[1]; v[2] = r.hi[0]; v[3] = r.hi[1]; }
-    else { v[0] = r.x0; v[1] = r.x1; v[2] = r.x2; v[3] = r.x3; }
+    if (KIND == OPK_KPAIR) {
+      // the lane's part of its eight complex k: the low (real) or the high (imaginary) halves of the eight words
+      const unsigned sel = (lane & 1) ? 0x07060302u : 0x05040100u;
+      v[0] = (int)__builtin_amdgcn_perm((unsigned)r.q[1], (unsigned)r.q[0], sel);
+      v[1] = (int)__builtin_amdgcn_perm((unsigned)r.q[3], (unsigned)r.q[2], sel);
+      v[2] = (int)__builtin_amdgcn_perm((unsigned)r.q1[1], (unsigned)r.q1[0], sel);
+      v[3] = (int)__builtin_amdgcn_perm((unsigned)r.q1[3], (unsigned)r.q1[2], sel);
+      return v;
+    }
+    v[0] = r.lo[0]; v[1] = r.lo[1]; v[2] = r.hi[0]; v[3] = r.hi[1];
     return v;
   }
   // puts a (transformed) operand back into the registers of its fragment
   __device__ static __forceinline__ void store(Raw& r, int4v v) {
     if (KIND == OPK_KMAJOR) r.q = v;
-    else if (KIND == OPK_MMAJOR) { r.lo[0] = v[0]; r.lo[1] = v[1]; r.hi[0] = v[2]; r.hi[1] = v[3]; }
-    else { r.x0 = v[0]; r.x1 = v[1]; r.x2 = v[2]; r.x3 = v[3]; }
+    else { r.lo[0] = v[0]; r.lo[1] = v[1]; r.hi[0] = v[2]; r.hi[1] = v[3]; }
   }
   static_assert(KIND != OPK_MMAJOR || (KSTEPS * KSTEP_K + 4) * G::ROW_BYTES < 65536, "LDS immediate offset is 16 bits");
-  static_assert(KIND != OPK_KMAJOR || F * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
-  static_assert(KIND != OPK_CROWK || (KSTEPS * (KSTEP_K / 2)) * G::ROW_BYTES + F * FRAG_ROWS * 4 <= 65536, "LDS immediate offset is 16 bits");
+  static_assert((KIND != OPK_KMAJOR && KIND != OPK_KPAIR) || F * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
+  static_assert(KIND != OPK_KPAIR || (MI == 16 && (8 % G::RP256) == 0), "complex-pair fragments: 16-row blocks, whose 8 complex rows keep the swizzle of the first");
   static_assert(MI == 32 || MI == 16, "fragments of 32 or 16 rows");
   static_assert(!(EXPAND && KIND == OPK_KMAJOR && MI == 16), "expanded K-major fragments of 8 tile rows break the swizzle invariance of the read offsets");
 };
@@ -247,7 +274,7 @@ struct FragReader {
 // (reference src/operator.jl:307-311 and :366-369).
 template <int FIX>
 __device__ __forceinline__ int4v expand_fixup(int4v x, int lane) {
-  if (FIX == FIX_NONE || FIX == FIX_PLANAR) return x;
+  if (FIX != FIX_COMPLEX && FIX != FIX_DUAL) return x;
   const bool odd = (lane & 1) != 0;
   const unsigned sel = odd ? 0x01000302u : 0x03020100u;                       // swap halves on odd rows
   const unsigned flip = (FIX == FIX_COMPLEX && !odd) ? 0x80000000u : 0u;       // negate the imaginary half
@@ -364,6 +391,8 @@ struct MfmaGemmConfig {
   static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
   static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
+  static constexpr bool PAIR = (FIX_ == FIX_PAIR || FIX_ == FIX_PAIR_DUAL);     // complex / dual product as one real product (see FIX_PAIR)
+  static constexpr bool COMPLEX = FIX_ != FIX_NONE;                             // C / D hold complex numbers
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
   // K-split instances: a workgroup handles one slice of K (blockIdx.z); the slices of a tile meet in a
   // workspace and the last to arrive sums them in slice order and stores D (splitk_reduce).  A variant of
@@ -399,9 +428,13 @@ struct MfmaGemmConfig {
   static_assert(STAGES >= 2, "at least two LDS stages");
   static_assert((STAGES - 2) * DMA_PER_TILE <= 63, "vmcnt is a 6-bit counter");
   static_assert(FM * FN > 0, "empty wave tile");
-  static_assert(!GETT || (A_KIND != OPK_CROWK && B_KIND != OPK_CROWK && FIX == FIX_NONE), "contractions are real");
+  static_assert(!GETT || FIX == FIX_NONE, "contractions are real");
   static_assert(!SPLITK || (!GETT && FIX == FIX_NONE), "K-split instances are plain real GEMMs");
-  static_assert(!PLANAR || (WAVES_M_ % 2 == 0 && FUSE_ == 0), "planar complex: a wave's rows lie in one plane of D; no hooks");
+  static_assert(!PLANAR || (WAVES_M_ % 2 == 0 && (FUSE_ == 0 || FUSE_ == 3)), "planar complex: a wave's rows lie in one plane of D; hooks on C and D only");
+  static_assert(!COMPLEX || FUSE_ == 0 || FUSE_ == 3, "complex products take hooks on C and D only");
+  static_assert(!PAIR || (MI_ == 16 && (A_KIND_ == OPK_MMAJOR || A_KIND_ == OPK_KPAIR) && (B_KIND_ == OPK_MMAJOR || B_KIND_ == OPK_KPAIR)),
+                "complex-pair products: 16-row blocks on the real view of the operands");
+  static_assert(PAIR || (A_KIND_ != OPK_KPAIR && B_KIND_ != OPK_KPAIR), "OPK_KPAIR belongs to the complex-pair products");
 };
 
 template <class Cfg>
@@ -437,13 +470,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // tile origin and K step in 16-bit elements (lda / ldb are in 16-bit elements as well; an
     // interleaved complex matrix counts two per complex number)
     const int m0g = Cfg::EXPAND_A ? m0 / 2 : (Cfg::PLANAR ? m0 / 2 : m0);   // first row of the tile in the stored matrix
-    const long long a_org = Cfg::A_KIND == OPK_KMAJOR ? (long long)m0g * args.lda : (long long)(Cfg::PLANAR ? m0g : m0);
-    const long long b_org = Cfg::B_KIND == OPK_KMAJOR ? (long long)n0 * args.ldb : (Cfg::B_KIND == OPK_MMAJOR ? (long long)n0 : 2ll * n0);
+    const long long a_org = Cfg::A_KIND == OPK_KMAJOR ? (long long)m0g * args.lda
+                          : (Cfg::A_KIND == OPK_KPAIR ? (long long)(m0 / 2) * args.lda : (long long)(Cfg::PLANAR ? m0g : m0));
+    const long long b_org = Cfg::B_KIND == OPK_KMAJOR ? (long long)n0 * args.ldb
+                          : (Cfg::B_KIND == OPK_KPAIR ? (long long)(n0 / 2) * args.ldb : (long long)n0);
     ga = (const char*)args.a + a_org * 2;
     gb = (const char*)args.b + b_org * 2;
     if constexpr (Cfg::PLANAR) gb += args.plane_b * 2;   // the first pass over K reads B_im
-    a_step = (Cfg::A_KIND == OPK_KMAJOR ? (long long)BK : (long long)GA::LDS_ROWS * args.lda) * 2;
-    b_step = (Cfg::B_KIND == OPK_KMAJOR ? (long long)BK : (long long)GB::LDS_ROWS * args.ldb) * 2;
+    a_step = (Cfg::A_KIND == OPK_KMAJOR ? (long long)BK : (Cfg::A_KIND == OPK_KPAIR ? 2ll * BK : (long long)GA::LDS_ROWS * args.lda)) * 2;
+    b_step = (Cfg::B_KIND == OPK_KMAJOR ? (long long)BK : (Cfg::B_KIND == OPK_KPAIR ? 2ll * BK : (long long)GB::LDS_ROWS * args.ldb)) * 2;
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i) {
       int row, col;
@@ -608,11 +643,18 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr int NV = MI == 32 ? 16 : 4;                       // accumulator values per lane and block
   typedef typename Mfma<T, MI>::Acc AccV;
   auto vcol = [](int v) { return MI == 32 ? 8 * (v / 4) + (v % 4) : v; };   // column of value v inside a block, from the lane's first
+  // complex-pair products: a lane's four values of a block are two complex columns x the two parts of B; C is
+  // loaded into, and D stored from, the values 0 and 2 (one per complex column), see pair_combine
+  constexpr int NVO = Cfg::PAIR ? 2 : NV;                     // values per lane and block that C / D see
+  constexpr int CB = Cfg::PAIR ? MI / 2 : MI;                 // columns of C / D per block
+  auto slot = [](int v) { return Cfg::PAIR ? 2 * v : v; };
   AccV acc[FM][FN];
   // planar complex: the wave's rows lie in the real (upper) or the imaginary (lower) plane of C / D
   [[maybe_unused]] const bool lower_plane = Cfg::PLANAR && (wm * Cfg::WTM >= BM / 2);
   const int mrow = Cfg::PLANAR ? m0 / 2 + wm * Cfg::WTM - (lower_plane ? BM / 2 : 0) + (lane % MI) : m0 + wm * Cfg::WTM + (lane % MI);
-  const int ncol = n0 + wn * Cfg::WTN + 4 * (lane / MI);
+  const int ncol = Cfg::PAIR ? (n0 + wn * Cfg::WTN) / 2 + 2 * (lane / MI) : n0 + wn * Cfg::WTN + 4 * (lane / MI);
+  // complex C / D: this lane's row is the imaginary part of its complex row
+  [[maybe_unused]] const bool im_lane = Cfg::PLANAR ? lower_plane : (Cfg::COMPLEX && (lane & 1) != 0);
   // element offset of the lane's first element of accumulator block (fi, fj) in C / D, and the
   // stride between its consecutive columns.  With a tensor-contraction map the first M mode and
   // the first N mode cover whole 32-wide blocks, so only the block origin needs the digit walk.
@@ -638,7 +680,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if constexpr (Cfg::PLANAR) {
       return (long long)(mrow + MI * fi) + (long long)(ncol + MI * fj) * ld + (lower_plane ? plane : 0ll);
     } else if constexpr (!Cfg::GETT) {
-      return (long long)(mrow + MI * fi) + (long long)(ncol + MI * fj) * ld;
+      return (long long)(mrow + MI * fi) + (long long)(ncol + CB * fj) * ld;
     } else {
       return gett_om[fi] + (long long)(lane % MI) * args.gm.stride1[0] + gett_on[fj] + (long long)(4 * (lane / MI)) * args.gn.stride1[0];
     }
@@ -661,13 +703,24 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
       for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
-        for (int v = 0; v < NV; ++v) acc[fi][fj][v] = f(acc[fi][fj][v]);
+        for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = f(acc[fi][fj][slot(v)]);
     };
 #ifdef GK_USER_HOOKS
     if constexpr (UserHooks::present[H]) each([](float x) { return UserHooks::template apply<H>(x); });
 #else
     const OpList& t = args.t[H];
-    for (int i = 0; i < t.n; ++i) dispatch_op(t.kind[i], t.p0[i], t.p1[i], each);
+    for (int i = 0; i < t.n; ++i) {
+      if constexpr (Cfg::COMPLEX) {
+        // z + p0 with a real p0 leaves the imaginary part as it is (the host admits the ops that act on the
+        // two parts independently, and this one)
+        if (t.kind[i] == T_ADD) {
+          const float p0 = t.p0[i];
+          each([=](float x) { return im_lane ? x : x + p0; });
+          continue;
+        }
+      }
+      dispatch_op(t.kind[i], t.p0[i], t.p1[i], each);
+    }
 #endif
   };
   [[maybe_unused]] const bool ragged = Cfg::RAGGED_OK && (m0 + BM > args.M || n0 + BN > args.N);   // wave-uniform
@@ -701,18 +754,19 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fi = 0; fi < FM; ++fi) {
         const long long off = cd_offset(fi, fj, args.ldc, args.plane_c);
         const long long ns = cd_nstride(args.ldc);
+        if constexpr (Cfg::PAIR) acc[fi][fj] = AccV{};      // the values between the complex columns start from zero
         if (args.c_dtype == DT_F32) {
           const float* cp = (const float*)args.c + off;
 #pragma unroll
-          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = cp[(long long)vcol(v) * ns];
+          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = cp[(long long)vcol(v) * ns];
         } else if (args.c_dtype == DT_F16) {
           const _Float16* cp = (const _Float16*)args.c + off;
 #pragma unroll
-          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = (float)cp[(long long)vcol(v) * ns];
+          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = (float)cp[(long long)vcol(v) * ns];
         } else {
           const __bf16* cp = (const __bf16*)args.c + off;
 #pragma unroll
-          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = (float)cp[(long long)vcol(v) * ns];
+          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = (float)cp[(long long)vcol(v) * ns];
         }
       }
     if (Cfg::FUSED) {
@@ -790,12 +844,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
     for (int fi = 0; fi < NA; ++fi) {
       RA::pin_raw(fa[ABUF][fi]);
-      va[fi] = expand_fixup<Cfg::FIX>(RA::finish(fa[ABUF][fi]), lane);
+      va[fi] = expand_fixup<Cfg::FIX>(RA::finish(fa[ABUF][fi], lane), lane);
     }
 #pragma unroll
     for (int fj = 0; fj < FN; ++fj) {
       RB::pin_raw(fb[ks & 1][fj]);
-      vb[fj] = RB::finish(fb[ks & 1][fj]);
+      vb[fj] = RB::finish(fb[ks & 1][fj], lane);
     }
     if constexpr (MODE >= 0) {
       // A is scaled one fragment ahead of the MFMAs that use it: in this order the compiler lets part of
@@ -1073,6 +1127,28 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if (args.acc_post_scale != 1.0f) scale_acc(args.acc_post_scale);
   }
 
+  if constexpr (Cfg::PAIR) {
+    // The four real products of a complex element of D = (re A + i im A)(re B + i im B): lane 2i holds, for
+    // each of its two complex columns, re A * re B (value 0 / 2) and re A * im B (value 1 / 3), lane 2i+1
+    // im A * re B and im A * im B.  The neighbours trade their odd values: lane 2i becomes the real part
+    // re*re - im*im, lane 2i+1 the imaginary part im*re + re*im (dual numbers: re*re, and du*re + re*du), left in
+    // the values 0 and 2 -- the row of the real view of D that the lane already stands for.  C came in through
+    // the same values.
+#pragma unroll
+    for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+          const float own = acc[fi][fj][2 * v];
+          // (the value goes through a scalar first: a bit cast applied to the vector element itself is
+          // compiled as a cast of the whole vector, of which element 0 is then taken)
+          const float mine = acc[fi][fj][2 * v + 1];
+          const float other = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mine), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+          acc[fi][fj][2 * v] = im_lane ? own + other : (Cfg::FIX == FIX_PAIR_DUAL ? own : own - other);
+        }
+  }
+
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   gett_origins();
 #pragma unroll
@@ -1080,23 +1156,24 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if (Cfg::FUSED) {
       hook_col(std::integral_constant<int, H_RF2SH_D>{}, fj);
       if (args.epi_kind == 1) {          // one bias value per column of D
-        float bv[NV];
+        // (a real bias value goes to the real part of a complex D)
+        float bv[NVO];
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-          const int cc = ncol + MI * fj + vcol(v);
+        for (int v = 0; v < NVO; ++v) {
+          const int cc = ncol + CB * fj + vcol(v);
           bv[v] = args.bias[(Cfg::RAGGED_OK && cc >= args.N) ? 0 : cc];      // columns over the edge are not stored
         }
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
-          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = acc[fi][fj][v] + bv[v];
+          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = (Cfg::COMPLEX && im_lane) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + bv[v];
       } else if (args.epi_kind == 2) {   // one bias value per row of D
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const int r = mrow + MI * fi;
+          const int r = (Cfg::COMPLEX && !Cfg::PLANAR) ? (mrow + MI * fi) >> 1 : mrow + MI * fi;
           const float bv = args.bias[(Cfg::RAGGED_OK && r >= args.M) ? 0 : r];
 #pragma unroll
-          for (int v = 0; v < NV; ++v) acc[fi][fj][v] = acc[fi][fj][v] + bv;
+          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = (Cfg::COMPLEX && im_lane) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + bv;
         }
       }
       hook_col(std::integral_constant<int, H_SH2GL_D>{}, fj);
@@ -1107,7 +1184,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       const long long ns = cd_nstride(args.ldd);
       float x[NV];
 #pragma unroll
-      for (int v = 0; v < NV; ++v) x[v] = acc[fi][fj][v];
+      for (int v = 0; v < NVO; ++v) x[v] = acc[fi][fj][slot(v)];
       // the accumulator is rounded once, to the element type of D
       if constexpr (Cfg::RAGGED_OK) {
         if (ragged) {       // tile over the edge: element by element, out-of-range elements are dropped
@@ -1122,15 +1199,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       if (args.d_dtype == DT_F32) {
         float* dp = (float*)args.d + off;
 #pragma unroll
-        for (int v = 0; v < NV; ++v) dp[(long long)vcol(v) * ns] = x[v];
+        for (int v = 0; v < NVO; ++v) dp[(long long)vcol(v) * ns] = x[v];
       } else if (args.d_dtype == DT_F16) {
         _Float16* dp = (_Float16*)args.d + off;
 #pragma unroll
-        for (int v = 0; v < NV; ++v) dp[(long long)vcol(v) * ns] = (_Float16)x[v];
+        for (int v = 0; v < NVO; ++v) dp[(long long)vcol(v) * ns] = (_Float16)x[v];
       } else {
         __bf16* dp = (__bf16*)args.d + off;
 #pragma unroll
-        for (int v = 0; v < NV; ++v) dp[(long long)vcol(v) * ns] = (__bf16)x[v];
+        for (int v = 0; v < NVO; ++v) dp[(long long)vcol(v) * ns] = (__bf16)x[v];
       }
     }
   }

@@ -69,6 +69,7 @@ int family_fpu_types(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int
 int family_fpu_more(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_splitk(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_complex(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+int family_complex_pair(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_complex_planar(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_diagonal(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_checked(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);

@@ -181,11 +181,9 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
             return NT(M=32, N=32, K=32)
         return NT(M=64, N=64, K=32)
     if operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
-        # complex tiles, in complex elements; every MFMA row pair is one complex row
-        table = _PLANAR_TILES if planar else _COMPLEX_TILES
+        # complex tiles, in complex elements
+        table = _complex_tiles(operator, planar, a_kmajor, b_kmajor)
         fitting = [t for t, _ in table if M % t[0] == 0 and N % t[1] == 0 and K % t[2] == 0]
-        if operator.kind == Operator.MFMA_DUAL:
-            fitting = [t for t in fitting if t in ((64, 128, 32), (64, 64, 32))]
         for t in fitting:
             if (M // t[0]) * (N // t[1]) >= NUM_CUS:
                 return NT(M=t[0], N=t[1], K=t[2])
@@ -223,8 +221,13 @@ _MFMA_TILE_RATE = {(256, 256, 64): 1.0, (256, 256, 32): 0.95, (256, 128, 64): 0.
                    (256, 192, 64): 0.90, (192, 256, 64): 0.90}
 
 
-# complex / dual tiles (complex elements) -> waves
-_COMPLEX_TILES = [((128, 256, 32), (2, 4)), ((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
+# complex / dual tiles (complex elements) -> waves, for interleaved A and B of which at least one is contiguous
+# along m or n: one real product of the real views of A and B, whose real tile has twice the rows and columns.
+# ('T','T' runs the first tile with the wave grid transposed, see _complex_tiles.)
+_COMPLEX_PAIR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
+# ... and for 'T','N' (both contiguous along k): the A fragments are expanded to [re -im; im re] in registers
+_COMPLEX_TN_TILES = [((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
+_DUAL_TN_TILES = [((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 
 # complex tiles (complex elements) of the kernel for planar global matrices -> waves; a workgroup's real
 # tile has twice as many rows (both planes of D)
@@ -235,7 +238,18 @@ _FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (
 _CHECKED_TILES = [((64, 64, 32), (2, 2))]
 
 
-def _default_waves(operator, block_shape, checked=False, planar=False, gett=False):
+def _complex_tiles(operator, planar, a_kmajor, b_kmajor):
+    """(tile, waves) of the complex / dual instances for these layouts, in order of preference."""
+    if planar:
+        return _PLANAR_TILES
+    if a_kmajor and b_kmajor:
+        return _DUAL_TN_TILES if operator.kind == Operator.MFMA_DUAL else _COMPLEX_TN_TILES
+    if a_kmajor:      # 'T','T': A is the operand that is read twice from LDS, so the waves line up along m
+        return [(t, (w[1], w[0])) for t, w in _COMPLEX_PAIR_TILES]
+    return _COMPLEX_PAIR_TILES
+
+
+def _default_waves(operator, block_shape, checked=False, planar=False, gett=False, a_kmajor=False, b_kmajor=True):
     key = (block_shape["M"], block_shape["N"], block_shape["K"])
     if gett and key == (64, 64, 32):
         return (1, 1)
@@ -244,7 +258,7 @@ def _default_waves(operator, block_shape, checked=False, planar=False, gett=Fals
     elif operator.kind == Operator.MFMA and checked and any(t == key for t, _ in _CHECKED_TILES):
         table = _CHECKED_TILES
     elif operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL):
-        table = _PLANAR_TILES if planar else _COMPLEX_TILES
+        table = _complex_tiles(operator, planar, a_kmajor, b_kmajor)
     else:
         table = _MFMA_TILES + [(t, w) for t, w, _ in _MFMA_TILES_192]
     for t, w in table:
@@ -301,13 +315,14 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
         params.setdefault("cta_swizzle", CTASwizzle.Identity)
     is_gett = any(l.kind == Layout.GETT_KIND for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
     planar = global_a_layout.kind in (Layout.SPLIT_COL_MAJOR, Layout.SPLIT_ROW_MAJOR)
-    block_shape = (default_block_shape(operator, gemm_shape, tile_sized, is_gett, planar, a_kmajor=global_a_layout.kind in (Layout.ROW_MAJOR, Layout.ALIGNED_ROW_MAJOR),
-                                       b_kmajor=global_b_layout.kind in (Layout.COL_MAJOR, Layout.ALIGNED_COL_MAJOR))
+    a_kmajor = global_a_layout.kind in (Layout.ROW_MAJOR, Layout.ALIGNED_ROW_MAJOR, Layout.INTERLEAVED_ROW_MAJOR, Layout.SPLIT_ROW_MAJOR)
+    b_kmajor = global_b_layout.kind in (Layout.COL_MAJOR, Layout.ALIGNED_COL_MAJOR, Layout.INTERLEAVED_COL_MAJOR, Layout.SPLIT_COL_MAJOR)
+    block_shape = (default_block_shape(operator, gemm_shape, tile_sized, is_gett, planar, a_kmajor=a_kmajor, b_kmajor=b_kmajor)
                    if block_shape is None else NT(block_shape))
     op_shape = Operator.shape(operator)
 
     checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
-    waves = _default_waves(operator, block_shape, checked, planar, is_gett)
+    waves = _default_waves(operator, block_shape, checked, planar, is_gett, a_kmajor, b_kmajor)
     if waves is not None:
         warps_default = waves[0] * waves[1]
         compute_warp_default = NT(M=block_shape.M // waves[0], N=block_shape.N // waves[1], K=op_shape.K)

@@ -227,16 +227,17 @@ def _config4b() -> Workload:
         kernel_name=kernel_name(conf, Kernel.matmul_singlestage))
 
 
-def complex_config(M, N, K, ta=False, tb=False, zero_c=True, dual=False, **kw):
+def complex_config(M, N, K, ta=False, tb=False, zero_c=True, dual=False, cd_type=Float32, **kw):
     """@get_wmma_complex_config / @get_wmma_dual_config of the reference (configs/configs.jl:385-490):
-    interleaved Complex{Float16} in global memory, planar in shared memory, Complex{Float32} out."""
+    interleaved Complex{Float16} in global memory, planar in shared memory, Complex{Float32} out
+    (``cd_type``: the real type of the complex elements of C and D)."""
     il = lambda t: Layout.InterleavedRowMajor[Float16] if t else Layout.InterleavedColMajor[Float16]
     sp = lambda t: Layout.Padded[Layout.SplitRowMajor[Float16], 8] if t else Layout.Padded[Layout.SplitColMajor[Float16], 8]
     op = (Operator.MFMADualOp if dual else Operator.MFMAComplexOp)[16, 16, 16, Float16, Float32]
     params = dict(gemm_shape=NT(M=M, N=N, K=K), operator=op,
                   global_a_layout=il(ta), global_b_layout=il(tb),
-                  global_c_layout=Layout.Zero[Float32] if zero_c else Layout.InterleavedColMajor[Float32],
-                  global_d_layout=Layout.InterleavedColMajor[Float32],
+                  global_c_layout=Layout.Zero[cd_type] if zero_c else Layout.InterleavedColMajor[cd_type],
+                  global_d_layout=Layout.InterleavedColMajor[cd_type],
                   shared_a_layout=sp(ta), shared_b_layout=sp(tb),
                   shared_c_layout=Layout.Zero[Float32] if zero_c else Layout.SplitColMajor[Float32],
                   shared_d_layout=Layout.SplitColMajor[Float32],

@@ -341,7 +341,15 @@ const MFMA_TILES = [((256, 256, 64), (2, 4)), ((256, 256, 32), (2, 4)), ((256, 1
 # relative throughput of a CU running each tile (256 x 256 x 64 = 1), measured
 const MFMA_TILE_RATE = Dict((256, 256, 64) => 1.0, (256, 256, 32) => 0.95, (256, 128, 64) => 0.81, (128, 256, 64) => 0.82,
                             (128, 128, 32) => 0.63, (128, 128, 64) => 0.62, (64, 64, 64) => 0.47, (64, 64, 32) => 0.42)
-const COMPLEX_TILES = [((128, 256, 32), (2, 4)), ((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
+# complex / dual tiles (complex elements): interleaved A and B of which at least one is contiguous along m or n run as
+# one real product of their real views ('T','T' with the wave grid transposed); 'T','N' expands A in registers
+const COMPLEX_PAIR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
+const COMPLEX_TN_TILES = [((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
+const DUAL_TN_TILES = [((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
+function complex_tiles(operator::Type, a_kmajor::Bool, b_kmajor::Bool)
+    a_kmajor && b_kmajor && return nameof(operator) in (:WMMADualOp, :MFMADualOp) ? DUAL_TN_TILES : COMPLEX_TN_TILES
+    a_kmajor ? [(t, (w[2], w[1])) for (t, w) in COMPLEX_PAIR_TILES] : COMPLEX_PAIR_TILES
+end
 const FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (1, 1))]
 
 "reference src/config.jl:84-120, unchanged (the reference-compatible answer; the launch uses the tile table)"
@@ -361,14 +369,14 @@ function adjacent_elements(num, parent_size, is_col_major)
 end
 
 "MI355X block shape: of the tiles of the table that fit, the one with the shortest estimated launch"
-function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true)
+function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true, a_kmajor::Bool = false, b_kmajor::Bool = true)
     M, N, K = gemm_shape.M, gemm_shape.N, gemm_shape.K
     if Operator.is_fpu(operator)
         small = nameof(operator) == :FPUOp && Operator.compute_type(operator) == Float32 && Operator.accum_type(operator) == Float32 &&
                 tile_sized && M % 32 == 0 && N % 32 == 0 && K % 32 == 0 && cld(M, 64) * cld(N, 64) < NUM_CUS ÷ 2
         return small ? (M = 32, N = 32, K = 32) : (M = 64, N = 64, K = 32)
     elseif !Operator.is_mfma(operator)
-        fitting = [t for (t, _) in COMPLEX_TILES if M % t[1] == 0 && N % t[2] == 0 && K % t[3] == 0]
+        fitting = [t for (t, _) in complex_tiles(operator, a_kmajor, b_kmajor) if M % t[1] == 0 && N % t[2] == 0 && K % t[3] == 0]
         for t in fitting
             (M ÷ t[1]) * (N ÷ t[2]) >= NUM_CUS && return (M = t[1], N = t[2], K = t[3])
         end
@@ -382,9 +390,9 @@ function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true
     (M = best[1], N = best[2], K = best[3])
 end
 
-function default_waves(operator::Type, block_shape)
+function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_kmajor::Bool = true)
     key = (block_shape.M, block_shape.N, block_shape.K)
-    table = Operator.is_fpu(operator) ? FPU_TILES : (Operator.is_mfma(operator) ? MFMA_TILES : COMPLEX_TILES)
+    table = Operator.is_fpu(operator) ? FPU_TILES : (Operator.is_mfma(operator) ? MFMA_TILES : complex_tiles(operator, a_kmajor, b_kmajor))
     for (t, w) in table
         t == key && return w
     end
@@ -411,10 +419,12 @@ function get_config(; gemm_shape, operator, global_a_layout, global_c_layout, kw
 
     globals = (global_a_layout, global_b_layout, global_c_layout, global_d_layout)
     tile_sized = any(require_tile_sized_global, globals)
-    block_shape = get(params, :block_shape, default_block_shape(operator, gemm_shape; tile_sized = tile_sized))
+    a_kmajor = Layout.is_row_major(global_a_layout)             # 'T' A: stored K x M, k contiguous
+    b_kmajor = !Layout.is_row_major(global_b_layout)            # 'N' B: stored K x N, k contiguous
+    block_shape = get(params, :block_shape, default_block_shape(operator, gemm_shape; tile_sized = tile_sized, a_kmajor = a_kmajor, b_kmajor = b_kmajor))
     op_shape = Operator.shape(operator)
 
-    waves = default_waves(operator, block_shape)
+    waves = default_waves(operator, block_shape; a_kmajor = a_kmajor, b_kmajor = b_kmajor)
     if waves !== nothing
         warps_default = waves[1] * waves[2]
         compute_warp_default = (M = block_shape.M ÷ waves[1], N = block_shape.N ÷ waves[2], K = op_shape.K)

@@ -210,6 +210,29 @@ static double apply_transform(const gko_transform* t, double x, int wide) {
   return x;
 }
 
+/* One part (0: real, 1: imaginary) of a hook applied to a complex number.  The reference hands tiles of the
+ * layout's element type to the transform (src/kernel.jl:167-187, 337-347, src/transform.jl:20-30), so a hook of a
+ * complex product sees Complex values: z * p0 and -z act on both parts, z + p0 (p0 real) on the real part only.
+ * The other ops have no complex method of the same type (max / clamp) or change the type (abs): not defined here,
+ * complex_transform_ok() says so. */
+static double apply_transform_part(const gko_transform* t, double x, int part, int wide) {
+  for (int i = 0; i < t->n; ++i) {
+    gko_transform one;
+    one.n = 1;
+    one.ops[0] = t->ops[i];
+    if (one.ops[0].kind == GKO_T_ADD && part == 1) continue;
+    x = apply_transform(&one, x, wide);
+  }
+  return x;
+}
+static int complex_transform_ok(const gko_transform* t) {
+  for (int i = 0; i < t->n; ++i) {
+    const int k = t->ops[i].kind;
+    if (k != GKO_T_SCALE && k != GKO_T_ADD && k != GKO_T_NEG && k != 0) return 0;
+  }
+  return 1;
+}
+
 /* ---------------- layouts ---------------- */
 static int64_t gett_offset(const gko_layout* L, int which, int64_t idx) {
   int64_t off = 0;
@@ -354,6 +377,9 @@ int gko_matmul(const gko_problem* P, const void* a, const void* b, const void* c
   const int wide_t = (P->compute_dtype == GKO_F64);   /* transforms of A/B in fp64 only for fp64 data */
   const int wide_cd = (P->accum_dtype == GKO_F64);
   if (two == 2 && !(is_complex_layout(&P->a) && is_complex_layout(&P->b))) return 1;
+  if (two == 2)
+    for (int h = 0; h < 8; ++h)
+      if (!complex_transform_ok(&P->t[h])) return 3;
 
   /* transformed operands, k-contiguous: At[i*K + k], Bt[j*K + k]; planes for complex/dual */
   double* At = (double*)malloc(sizeof(double) * (size_t)M * (size_t)K * two);
@@ -368,8 +394,8 @@ int gko_matmul(const gko_problem* P, const void* a, const void* b, const void* c
       if (two == 2) layout_load_complex(&P->a, a, i, k, &v[0], &v[1]);
       else v[0] = layout_load(&P->a, a, i, k);
       for (int q = 0; q < two; ++q) {
-        double x = round_to(P->shared_a_dtype, apply_transform(&P->t[0], v[q], wide_t));
-        x = round_to(P->compute_dtype, apply_transform(&P->t[4], x, wide_t));
+        double x = round_to(P->shared_a_dtype, apply_transform_part(&P->t[0], v[q], q, wide_t));
+        x = round_to(P->compute_dtype, apply_transform_part(&P->t[4], x, q, wide_t));
         At[q * planeA + (size_t)i * K + k] = x;
       }
     }
@@ -380,8 +406,8 @@ int gko_matmul(const gko_problem* P, const void* a, const void* b, const void* c
       if (two == 2) layout_load_complex(&P->b, b, k, j, &v[0], &v[1]);
       else v[0] = layout_load(&P->b, b, k, j);
       for (int q = 0; q < two; ++q) {
-        double x = round_to(P->shared_b_dtype, apply_transform(&P->t[1], v[q], wide_t));
-        x = round_to(P->compute_dtype, apply_transform(&P->t[5], x, wide_t));
+        double x = round_to(P->shared_b_dtype, apply_transform_part(&P->t[1], v[q], q, wide_t));
+        x = round_to(P->compute_dtype, apply_transform_part(&P->t[5], x, q, wide_t));
         Bt[q * planeB + (size_t)j * K + k] = x;
       }
     }
@@ -401,8 +427,8 @@ int gko_matmul(const gko_problem* P, const void* a, const void* b, const void* c
         if (two == 2) layout_load_complex(&P->c, c, i, j, &c0[0], &c0[1]);
         else c0[0] = layout_load(&P->c, c, i, j);
         for (int q = 0; q < two; ++q) {
-          double x = round_to(P->shared_c_dtype, apply_transform(&P->t[2], c0[q], wide_cd));
-          c0[q] = round_to(P->accum_dtype, apply_transform(&P->t[6], x, wide_cd));
+          double x = round_to(P->shared_c_dtype, apply_transform_part(&P->t[2], c0[q], q, wide_cd));
+          c0[q] = round_to(P->accum_dtype, apply_transform_part(&P->t[6], x, q, wide_cd));
         }
       }
       const double* ar = At + (size_t)i * K;
@@ -455,10 +481,12 @@ int gko_matmul(const gko_problem* P, const void* a, const void* b, const void* c
         }
       }
       for (int q = 0; q < two; ++q) {
-        double x = round_to(P->shared_d_dtype, apply_transform(&P->t[7], res[q], wide_cd));
-        if (P->epilogue == 1 && P->bias) { volatile float s = (float)x + P->bias[j]; x = (double)s; }
-        else if (P->epilogue == 2 && P->bias) { volatile float s = (float)x + P->bias[i]; x = (double)s; }
-        x = apply_transform(&P->t[3], x, wide_cd);
+        double x = round_to(P->shared_d_dtype, apply_transform_part(&P->t[7], res[q], q, wide_cd));
+        /* a bias value is real: on a complex D it goes to the real part (the reference's apply_bias,
+         * src/epilogue.jl:45-53, takes Float32 tiles only and has no complex method) */
+        if (P->epilogue == 1 && P->bias && q == 0) { volatile float s = (float)x + P->bias[j]; x = (double)s; }
+        else if (P->epilogue == 2 && P->bias && q == 0) { volatile float s = (float)x + P->bias[i]; x = (double)s; }
+        x = apply_transform_part(&P->t[3], x, q, wide_cd);
         out[q * planeD + (size_t)j * M + i] = x;
       }
     }

@@ -28,25 +28,131 @@ def run(conf, a, b, c, M, N):
     return gk.to_numpy(td)
 
 
-@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("dims,block", [((128, 128, 64), (32, 64, 32)), ((128, 128, 128), (64, 64, 32)), ((128, 256, 96), (64, 128, 32)),
-                                        ((256, 256, 160), (128, 128, 32)),
-                                        ((256, 512, 64), (128, 256, 32))])
-def test_complex_all_transposes(gpu, dims, block, ta, tb):
-    M, N, K = dims
-    conf = configs.complex_config(M, N, K, ta, tb, block_shape=gk.NT(M=block[0], N=block[1], K=block[2]))
+def _tiles(ta, tb, dual=False):
+    from gemmkernels import config as cfg, Operator, Float16, Float32
+    op = (Operator.MFMADualOp if dual else Operator.MFMAComplexOp)[16, 16, 16, Float16, Float32]
+    return [t for t, _ in cfg._complex_tiles(op, False, ta, not tb)]
+
+
+TRANSPOSES = [(False, False), (False, True), (True, False), (True, True)]
+CASES = [(ta, tb, block) for ta, tb in TRANSPOSES for block in _tiles(ta, tb)]
+
+
+@pytest.mark.parametrize("ta,tb,block", CASES)
+@pytest.mark.parametrize("zero_c", [True, False])
+def test_complex_all_transposes(gpu, ta, tb, block, zero_c):
+    """Every compiled tile of every transpose (one real product of the real views for 'N','N' / 'N','T' / 'T','T',
+    the register-expanded A for 'T','N'), with and without C."""
+    M, N, K = 2 * block[0], 3 * block[1], 5 * block[2]
+    conf = configs.complex_config(M, N, K, ta, tb, zero_c=zero_c, block_shape=gk.NT(M=block[0], N=block[1], K=block[2]))
     a = configs.complex_matrix(61, K if ta else M, M if ta else K)
     b = configs.complex_matrix(62, N if tb else K, K if tb else N)
-    print("case", dims, block, ta, tb, gk.kernel_name(conf, Kernel.matmul_pipelined), flush=True)
-    d = run(conf, a, b, None, M, N)
+    c = None if zero_c else rng.matrix("upm1_f32", 63, (2, M, N))
+    name = gk.kernel_name(conf, Kernel.matmul_pipelined)
+    print("case", block, ta, tb, zero_c, name, flush=True)
+    assert ("pair" in name) == (not (ta and not tb))
+    d = run(conf, a, b, c, M, N)
     A = to_c128(a).T if ta else to_c128(a)          # 'T' is a plain transpose, no conjugation (src/matmul.jl:211-213)
     B = to_c128(b).T if tb else to_c128(b)
-    assert oracle.rel_frobenius(to_c128(d), A @ B) <= TOL
+    want = A @ B + (0 if zero_c else to_c128(c))
+    assert oracle.rel_frobenius(d[0], want.real) <= TOL and oracle.rel_frobenius(d[1], want.imag) <= TOL
     # the CPU oracle restates WMMAComplexOp.mma (src/operator.jl:307-311)
     ref = np.zeros((2, M, N), np.float32, order="F")
     p = helpers.oracle_problem(conf, (a.shape[1], b.shape[1], M, M))
-    oracle.matmul(p, a, b, None, ref)
+    oracle.matmul(p, a, b, c, ref)
     assert oracle.rel_frobenius(to_c128(d), to_c128(ref)) <= TOL
+
+
+@pytest.mark.parametrize("ta,tb", TRANSPOSES)
+def test_complex_default_tile_and_odd_k(gpu, ta, tb):
+    """The tile the defaults pick, for a K that only the 32-deep tiles divide and for a large product."""
+    for M, N, K in [(128, 192, 96), (512, 256, 320)]:
+        conf = configs.complex_config(M, N, K, ta, tb)
+        a = configs.complex_matrix(64, K if ta else M, M if ta else K)
+        b = configs.complex_matrix(65, N if tb else K, K if tb else N)
+        print("case", (M, N, K), ta, tb, gk.kernel_name(conf, Kernel.matmul_pipelined), flush=True)
+        d = run(conf, a, b, None, M, N)
+        A = to_c128(a).T if ta else to_c128(a)
+        B = to_c128(b).T if tb else to_c128(b)
+        assert oracle.rel_frobenius(to_c128(d), A @ B) <= TOL
+
+
+def _hooked(conf, a, b, c, M, N, transforms, bias, cd_np=np.float32):
+    """(GPU result, oracle result) of a complex product with hooks on C / D and a bias."""
+    import torch
+    from gemmkernels import Epilogue
+    ta_, tb_ = gk.colmajor(a), gk.colmajor(b)
+    tc = None if c is None else gk.colmajor(c)
+    td = gk.colmajor_empty((2, M, N), torch.float16 if cd_np == np.float16 else torch.float32)
+    td.fill_(float("nan"))
+    tbias = None if bias is None else torch.from_numpy(bias).cuda()
+    epi = None if bias is None else Epilogue.Bias(tbias)
+    gk.matmul(conf, ta_, tb_, tc, td, epilogue=epi, kernel=Kernel.matmul_pipelined, **transforms)
+    torch.cuda.synchronize()
+    ref = np.zeros((2, M, N), cd_np, order="F")
+    p = helpers.oracle_problem(conf, (a.shape[1], b.shape[1], M, M), transforms, epi, bias)
+    oracle.matmul(p, a, b, c, ref)
+    return gk.to_numpy(td), ref
+
+
+@pytest.mark.parametrize("ta,tb", TRANSPOSES)
+@pytest.mark.parametrize("dual", [False, True])
+def test_hooks_and_bias_on_complex(gpu, ta, tb, dual):
+    """Hooks of C and D and the bias on the complex and dual operators (the eight hooks of the reference are
+    operator-agnostic, src/kernel.jl:167-187, 337-347): z * s and -z act on both parts, z + c and the (real) bias on
+    the real part.  Checked against the oracle, and the oracle's complex hooks against numpy in tests/test_oracle.py."""
+    from gemmkernels import Transform
+    M, N, K = 128, 192, 128
+    conf = configs.complex_config(M, N, K, ta, tb, zero_c=False, dual=dual)
+    a = configs.complex_matrix(66, K if ta else M, M if ta else K)
+    b = configs.complex_matrix(67, N if tb else K, K if tb else N)
+    c = rng.matrix("upm1_f32", 68, (2, M, N))
+    bias = rng.normal_f32(69, N)
+    transforms = dict(transform_global_to_shared_c=Transform.Elementwise(lambda x: x * 2.0),
+                      transform_shared_to_regs_c=Transform.Elementwise(lambda x: x + 0.75),
+                      transform_regs_to_shared_d=Transform.Elementwise(lambda x: -(x * 0.5)),
+                      transform_shared_to_global_d=Transform.Elementwise(lambda x: x + 0.25))
+    print("case", ta, tb, dual, gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=transforms), flush=True)
+    d, ref = _hooked(conf, a, b, c, M, N, transforms, bias)
+    assert np.isfinite(d).all()
+    assert oracle.rel_frobenius(d[0], ref[0]) <= TOL and oracle.rel_frobenius(d[1], ref[1]) <= TOL
+    if not dual:
+        A = to_c128(a).T if ta else to_c128(a)
+        B = to_c128(b).T if tb else to_c128(b)
+        want = -((A @ B + (2.0 * to_c128(c) + 0.75)) * 0.5) + bias[None, :].astype(np.float64) + 0.25
+        assert oracle.rel_frobenius(d[0], want.real) <= TOL and oracle.rel_frobenius(d[1], want.imag) <= TOL
+
+
+def test_complex_fp16_c_and_d(gpu):
+    """Complex{Float16} C and D: fp32 accumulation, one rounding at the store."""
+    from gemmkernels import Float16
+    M, N, K = 128, 128, 192
+    for ta, tb in TRANSPOSES:
+        conf = configs.complex_config(M, N, K, ta, tb, zero_c=False, cd_type=Float16)
+        a = configs.complex_matrix(70, K if ta else M, M if ta else K)
+        b = configs.complex_matrix(71, N if tb else K, K if tb else N)
+        c = rng.matrix("upm1_f16", 72, (2, M, N))
+        d, ref = _hooked(conf, a, b, c, M, N, {}, None, np.float16)
+        assert d.dtype == np.float16 and np.isfinite(d).all()
+        A = to_c128(a).T if ta else to_c128(a)
+        B = to_c128(b).T if tb else to_c128(b)
+        assert oracle.rel_frobenius(to_c128(d), A @ B + to_c128(c)) <= 2e-3      # half an ulp of FP16 on top
+        assert np.mean(d.view(np.uint16) != ref.view(np.uint16)) < 2e-3          # same rounding as the oracle's single one
+
+
+def test_complex_hooks_that_are_not_defined_are_refused(gpu):
+    from gemmkernels import Transform, ConfigError, _lib
+    M = N = K = 128
+    conf = configs.complex_config(M, N, K)
+    a = gk.colmajor(configs.complex_matrix(73, M, K))
+    b = gk.colmajor(configs.complex_matrix(74, K, N))
+    d = gk.colmajor_empty((2, M, N), torch.float32)
+    for kw in (dict(transform_shared_to_global_d=Transform.Elementwise(Transform.relu)),          # max(z, 0) has no complex method
+               dict(transform_regs_to_shared_d=Transform.Elementwise(lambda x: abs(x))),         # abs(z) is real
+               dict(transform_global_to_shared_a=Transform.Elementwise(lambda x: x * 2.0))):     # A / B hooks: C and D only
+        with pytest.raises(ConfigError) as ei:
+            gk.matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined, **kw)
+        assert ei.value.status == _lib.GK_ERR_UNSUPPORTED, ei.value.message
 
 
 def test_complex_identities_and_c(gpu):
@@ -69,20 +175,22 @@ def test_complex_identities_and_c(gpu):
     assert oracle.rel_frobenius(to_c128(d), to_c128(a) @ to_c128(b) + to_c128(c)) <= TOL
 
 
-@pytest.mark.parametrize("block", [(64, 64, 32), (64, 128, 32)])
-def test_dual_numbers(gpu, block):
+@pytest.mark.parametrize("ta,tb,block", [(ta, tb, block) for ta, tb in TRANSPOSES for block in _tiles(ta, tb, dual=True)])
+def test_dual_numbers(gpu, ta, tb, block):
     """(re, du): re = a_re b_re, du = a_re b_du + a_du b_re (reference src/operator.jl:366-369)."""
-    M, N, K = 128, 256, 64
-    conf = configs.complex_config(M, N, K, dual=True, block_shape=gk.NT(M=block[0], N=block[1], K=block[2]))
-    a = configs.complex_matrix(81, M, K)
-    b = configs.complex_matrix(82, K, N)
+    M, N, K = 2 * block[0], 2 * block[1], 3 * block[2]
+    conf = configs.complex_config(M, N, K, ta, tb, dual=True, block_shape=gk.NT(M=block[0], N=block[1], K=block[2]))
+    a = configs.complex_matrix(81, K if ta else M, M if ta else K)
+    b = configs.complex_matrix(82, N if tb else K, K if tb else N)
+    print("case", block, ta, tb, gk.kernel_name(conf, Kernel.matmul_pipelined), flush=True)
     d = run(conf, a, b, None, M, N)
-    a0, a1, b0, b1 = (x.astype(np.float64) for x in (a[0], a[1], b[0], b[1]))
+    a0, a1 = (x.astype(np.float64).T if ta else x.astype(np.float64) for x in (a[0], a[1]))
+    b0, b1 = (x.astype(np.float64).T if tb else x.astype(np.float64) for x in (b[0], b[1]))
     assert oracle.rel_frobenius(d[0], a0 @ b0) <= TOL
     assert oracle.rel_frobenius(d[1], a0 @ b1 + a1 @ b0) <= TOL
     # and against the oracle's dual-number product (itself pinned against these float64 forms on the CPU)
     ref = np.zeros((2, M, N), np.float32, order="F")
-    p = helpers.oracle_problem(conf, (M, K, M, M))
+    p = helpers.oracle_problem(conf, (a.shape[1], b.shape[1], M, M))
     assert p.op_kind == oracle.OP_DUAL
     oracle.matmul(p, a, b, None, ref)
     assert oracle.rel_frobenius(d[0], ref[0]) <= TOL and oracle.rel_frobenius(d[1], ref[1]) <= TOL
@@ -166,6 +274,33 @@ def test_planar_kernel_every_tile(gpu, block, ta, tb):
     conf, err, err_re, err_im = _run_planar(M, N, K, ta, tb, False, block)
     assert "planar" in gk.kernel_name(conf, Kernel.matmul_pipelined)
     assert err <= TOL and err_re <= TOL and err_im <= TOL
+
+
+@pytest.mark.parametrize("ta,tb", TRANSPOSES)
+def test_planar_hooks_and_bias(gpu, ta, tb):
+    """Hooks of C and D and the bias on planar matrices: the same rules as on interleaved ones (a plane is a part)."""
+    from gemmkernels import Transform, Epilogue
+    M, N, K = 128, 256, 128
+    conf = configs.complex_planar_config(M, N, K, ta, tb, zero_c=False)
+    a = planar(111, K if ta else M, M if ta else K)
+    b = planar(112, N if tb else K, K if tb else N)
+    c = planar(113, M, N, np.float32)
+    bias = rng.normal_f32(114, N)
+    tbias = torch.from_numpy(bias).cuda()
+    transforms = dict(transform_global_to_shared_c=Transform.Elementwise(lambda x: x * 2.0),
+                      transform_shared_to_regs_c=Transform.Elementwise(lambda x: x + 0.75),
+                      transform_regs_to_shared_d=Transform.Elementwise(lambda x: -(x * 0.5)),
+                      transform_shared_to_global_d=Transform.Elementwise(lambda x: x + 0.25))
+    td = gk.colmajor_empty((M, N, 2), torch.float32)
+    td.fill_(float("nan"))
+    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), gk.colmajor(c), td, epilogue=Epilogue.Bias(tbias), kernel=Kernel.matmul_pipelined, **transforms)
+    torch.cuda.synchronize()
+    A = planar_to_c128(a).T if ta else planar_to_c128(a)
+    B = planar_to_c128(b).T if tb else planar_to_c128(b)
+    want = -((A @ B + (2.0 * planar_to_c128(c) + 0.75)) * 0.5) + bias[None, :].astype(np.float64) + 0.25
+    d = planar_to_c128(gk.to_numpy(td))
+    assert np.isfinite(d).all()
+    assert oracle.rel_frobenius(d.real, want.real) <= TOL and oracle.rel_frobenius(d.imag, want.imag) <= TOL
 
 
 @pytest.mark.parametrize("ktiles", [1, 2, 3])

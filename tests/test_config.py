@@ -212,8 +212,17 @@ def test_every_tile_of_the_python_tables_has_a_compiled_instance():
         conf = gk.get_config(gemm_shape=NT(M=2 * bm, N=2 * bn, K=2 * bk), block_shape=NT(M=bm, N=bn, K=bk),
                              operator=Operator.FPUOp[8, 8, 1, 8, 8, 1, F32, F32], global_a_layout=ACM[F32], global_c_layout=ACM[F32])
         assert f"{bm}x{bn}x{bk}_w{wm}x{wn}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
-    for (bm, bn, bk), (wm, wn) in cfg._COMPLEX_TILES:
-        conf = configs.complex_config(2 * bm, 2 * bn, 4 * bk, block_shape=NT(M=bm, N=bn, K=bk))
+    for dual in (False, True):
+        for ta in (False, True):
+            for tb in (False, True):
+                op = Operator.MFMADualOp if dual else Operator.MFMAComplexOp
+                for (bm, bn, bk), (wm, wn) in cfg._complex_tiles(op[16, 16, 16, F16, F32], False, ta, not tb):
+                    conf = configs.complex_config(2 * bm, 2 * bn, 4 * bk, ta, tb, dual=dual, block_shape=NT(M=bm, N=bn, K=bk))
+                    name = gk.kernel_name(conf, Kernel.matmul_pipelined)
+                    assert f"_{'nt'[ta]}{'nt'[tb]}_{bm}x{bn}x{bk}_w{wm}x{wn}" in name, name
+                    assert ("pair" in name) == (not (ta and not tb)), name
+    for (bm, bn, bk), (wm, wn) in cfg._PLANAR_TILES:
+        conf = configs.complex_planar_config(2 * bm, 2 * bn, 4 * bk, block_shape=NT(M=bm, N=bn, K=bk))
         assert f"{bm}x{bn}x{bk}_w{wm}x{wn}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
 
 
@@ -249,7 +258,8 @@ def test_complex_layout_rules_of_the_library():
     M, N, K = 256, 256, 128
     conf = configs.complex_planar_config(M, N, K)
     assert "mfma_complex_planar_nn_" in gk.kernel_name(conf, Kernel.matmul_pipelined)
-    assert "mfma_complex_nn_" in gk.kernel_name(configs.complex_config(M, N, K), Kernel.matmul_pipelined)
+    assert "mfma_complex_pair_nn_" in gk.kernel_name(configs.complex_config(M, N, K), Kernel.matmul_pipelined)
+    assert "mfma_complex_tn_" in gk.kernel_name(configs.complex_config(M, N, K, True, False), Kernel.matmul_pipelined)
     cases = [
         dict(global_b_layout=Layout.InterleavedColMajor[F16]),                                   # planar A, interleaved B
         dict(global_d_layout=Layout.InterleavedColMajor[F32]),                                   # planar inputs, interleaved D

@@ -476,3 +476,42 @@ def test_dual_numbers_against_float64():
         assert np.array_equal(got[..., 0].astype(np.float64), a0 @ b0 + c0)
         assert np.array_equal(got[..., 1].astype(np.float64), a0 @ b1 + a1 @ b0 + c1)
     assert not np.array_equal(run(oracle.OP_COMPLEX, False)[..., 0], run(oracle.OP_DUAL, False)[..., 0])
+
+
+def test_hooks_on_complex_numbers_against_numpy_complex():
+    """Hooks of a complex product see complex numbers (the reference hands tiles of the layout's element type to the
+    transform, src/kernel.jl:167-187, 337-347): z * s and -z act on both parts, z + c (c real) and the real bias on
+    the real part only.  Checked against numpy's own complex arithmetic on dyadic data (every step exact), on every
+    hook, and the ops without a complex method of the same type are refused."""
+    M, N, K = 5, 4, 6
+    a = rand((M, K, 2), np.float16, 41)
+    b = rand((K, N, 2), np.float16, 42)
+    c = rand((M, N, 2), np.float32, 43)
+    bias = np.array([0.5, -1.25, 2.0, -0.75, 1.5], np.float32)        # N values per column, M per row
+    inter = lambda x: np.ascontiguousarray(np.transpose(x, (1, 0, 2)))
+    z = lambda x: x[..., 0].astype(np.complex128) + 1j * x[..., 1].astype(np.complex128)
+    def run(transforms, epilogue=0):
+        p = Problem(M, N, K, Layout(oracle.L_ICOL, F16, M), Layout(oracle.L_ICOL, F16, K), Layout(oracle.L_ICOL, F32, M),
+                    Layout(oracle.L_ICOL, F32, M), compute_dtype=F16, accum_dtype=F32, op_kind=oracle.OP_COMPLEX,
+                    transforms=transforms, epilogue=epilogue, bias=bias if epilogue else None)
+        d = np.zeros((N, M, 2), np.float32)
+        oracle.matmul(p, inter(a), inter(b), inter(c), d)
+        return z(np.transpose(d, (1, 0, 2)))
+    A, B, C = z(a), z(b), z(c)
+    assert np.array_equal(run({}), A @ B + C)
+    # A and B hooks: (2 A + 0.5) and (-B), both hooks of each operand in turn
+    for ha, hb in (("global_to_shared_a", "global_to_shared_b"), ("shared_to_regs_a", "shared_to_regs_b")):
+        got = run({ha: [(oracle.T_SCALE, 2.0, 0.0), (oracle.T_ADD, 0.5, 0.0)], hb: [(oracle.T_NEG, 0.0, 0.0)]})
+        assert np.array_equal(got, (2.0 * A + 0.5) @ (-B) + C)
+    # C hooks, D hooks and the bias in the reference's order: regs_to_shared_d, bias, shared_to_global_d
+    got = run({"global_to_shared_c": [(oracle.T_SCALE, 2.0, 0.0)], "shared_to_regs_c": [(oracle.T_ADD, 0.75, 0.0)],
+               "regs_to_shared_d": [(oracle.T_SCALE, 0.5, 0.0), (oracle.T_NEG, 0.0, 0.0)],
+               "shared_to_global_d": [(oracle.T_ADD, 0.25, 0.0)]}, epilogue=oracle.EPI_BIAS_COL)
+    want = -((A @ B + (2.0 * C + 0.75)) * 0.5) + bias[None, :N].astype(np.complex128) + 0.25
+    assert np.array_equal(got, want)
+    assert np.array_equal(got.imag, (-((A @ B + 2.0 * C) * 0.5)).imag)          # nothing was added to the imaginary part
+    got = run({}, epilogue=oracle.EPI_BIAS_ROW)
+    assert np.array_equal(got, A @ B + C + bias[:M, None].astype(np.complex128))
+    for kind in (oracle.T_RELU, oracle.T_ABS, oracle.T_CLAMP, oracle.T_SQUARE):
+        with pytest.raises(Exception):
+            run({"shared_to_global_d": [(kind, 0.0, 1.0)]})
