@@ -242,6 +242,8 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   return GK_OK;
 }
 
+bool gett_k_tiling(const gk_gett_dim& k, int bk, int* mode, int* prod, int* step);
+
 void make_args(const gk_config* c, const void* a, const void* b, const void* cc, void* d, const gk_transforms* t,
                const gk_epilogue* e, gk::GemmArgs* args) {
   memset(args, 0, sizeof(*args));
@@ -261,10 +263,10 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
     // (unless both A and B are contiguous along k, the real views of A and B meet in one real product of 2M x 2N x K)
     const bool pair = !is_split_layout(c->global_a_layout.kind) && !(is_row_major(c->global_a_layout.kind) && !is_row_major(c->global_b_layout.kind));
     args->M *= 2;
-    if (pair) args->N *= 2; else args->K *= 2;
+    if (pair || is_split_layout(c->global_a_layout.kind)) args->N *= 2; else args->K *= 2;
     if (is_split_layout(c->global_a_layout.kind)) {
       // planar operands: a matrix is the real array (rows, cols, 2) in column-major order, so the
-      // imaginary plane starts ld * cols elements after the real one; the kernel walks K twice
+      // imaginary plane starts ld * cols elements after the real one
       args->plane_a = args->lda * (a_row ? c->matmul_shape.M : c->matmul_shape.K);
       args->plane_b = args->ldb * (b_row ? c->matmul_shape.K : c->matmul_shape.N);
       args->plane_c = args->ldc * c->matmul_shape.N;
@@ -330,6 +332,15 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
   copy_dim(c->gett.m, args->gm);
   copy_dim(c->gett.n, args->gn);
   copy_dim(c->gett.k, args->gk);
+  gk::gett_fill_division(args->gm);
+  gk::gett_fill_division(args->gn);
+  gk::gett_fill_division(args->gk);
+  args->gk_mode = 0; args->gk_step = c->block_shape.K;
+  if (c->global_a_layout.kind == GK_LAYOUT_GETT) {
+    int prod = 1;
+    gett_k_tiling(c->gett.k, c->block_shape.K, &args->gk_mode, &prod, &args->gk_step);     // validated before
+    args->gett_fast = (c->gett.m.extent[0] % 32 == 0 && c->gett.n.extent[0] % 32 == 0) ? 1 : 0;
+  }
 }
 
 gk::FamilyFn family_fn(const gk::InstanceKey& key) {
@@ -375,6 +386,36 @@ int find_instance(const gk_config* c, const gk_transforms* t, const gk_epilogue*
 }
 
 // Tensor-contraction index maps: what the GETT loader assumes about the mode tables.
+// How a K tile of bk indices lies in the K modes: it covers modes 0 .. *mode - 1 whole (extents multiplying to *prod)
+// and *step indices of mode *mode.  False when no such split exists (bk does not divide evenly into the modes).
+bool gett_k_tiling(const gk_gett_dim& k, int bk, int* mode, int* prod, int* step) {
+  long long p = 1;
+  for (int j = 0; j < k.nmodes && j < GK_MAX_MODES; ++j) {
+    if (p <= 0 || bk % p != 0) return false;
+    const long long need = bk / p;            // indices of mode j that a tile takes
+    if (need <= k.extent[j]) {
+      if (k.extent[j] % need != 0) return false;
+      *mode = j; *prod = (int)p; *step = (int)need;
+      return true;
+    }
+    p *= k.extent[j];                         // mode j lies inside the tile whole
+  }
+  return false;
+}
+
+// Number of leading modes of `d` (strides `stride`) that are packed densely and whose extents multiply to a multiple
+// of 8, so that 8 consecutive indices of the GEMM dimension are 8 consecutive elements in memory (a 16-byte vector);
+// 0 when there is no such prefix.
+int gett_dense_prefix(const gk_gett_dim& d, const int64_t* stride) {
+  long long p = 1;
+  for (int i = 0; i < d.nmodes && i < GK_MAX_MODES; ++i) {
+    if (stride[i] != p) return 0;
+    p *= d.extent[i];
+    if (p % 8 == 0) return i + 1;
+  }
+  return 0;
+}
+
 int validate_gett(const gk_config* c) {
   const gk_gett& g = c->gett;
   if (c->op.kind != GK_OP_MFMA) return fail(GK_ERR_UNSUPPORTED, "tensor-contraction layouts need the MFMA operator");
@@ -400,18 +441,27 @@ int validate_gett(const gk_config* c) {
     if (prod != want[d]) return fail(GK_ERR_DIMENSION_MISMATCH, "the extents of the %s modes multiply to %lld, matmul_shape.%s is %d", names[d], prod, names[d], want[d]);
   }
   if (span[0] * 2 >= (1ll << 31) || span[1] * 2 >= (1ll << 31)) return fail(GK_ERR_UNSUPPORTED, "tensor too large for 32-bit tile offsets");
-  if (g.k.extent[0] % c->block_shape.K != 0)
-    return fail(GK_ERR_TILE_MULTIPLE, "BLOCK_K = %d must divide the extent %d of the first K mode", c->block_shape.K, g.k.extent[0]);
-  if (g.m.extent[0] % 32 != 0 || g.n.extent[0] % 32 != 0)
-    return fail(GK_ERR_TILE_MULTIPLE, "the first M mode and the first N mode must have extents that are multiples of 32");
-  // 16-byte vectors: one mode of each operand is contiguous and every other stride keeps the alignment
+  // a K tile is a whole number of leading K modes times a slab of the next one (BLOCK_K dividing the first K mode is
+  // the simplest case)
+  int kmode = 0, kprod = 1, kstep = 0;
+  if (!gett_k_tiling(g.k, c->block_shape.K, &kmode, &kprod, &kstep))
+    return fail(GK_ERR_TILE_MULTIPLE, "BLOCK_K = %d does not tile the K modes: it must divide the extent %d of the first K mode, or be a whole number "
+                                      "of leading K modes times a divisor of the next one", c->block_shape.K, g.k.extent[0]);
+  // a lane's four columns of C / D follow each other with the stride of the first N mode
+  if (g.n.extent[0] % 4 != 0)
+    return fail(GK_ERR_TILE_MULTIPLE, "the first N mode must have an extent that is a multiple of 4, got %d", g.n.extent[0]);
+  // 16-byte vectors: each operand has 8 consecutive elements along its leading M (N) modes or along its leading K
+  // modes (modes packed densely, extents multiplying to a multiple of 8), and every stride outside that run keeps the
+  // alignment
   const bool a_k = g.k.stride0[0] == 1, b_k = g.k.stride1[0] == 1;
-  if (!a_k && g.m.stride0[0] != 1) return fail(GK_ERR_ALIGNMENT, "A must be contiguous along its first M mode or its first K mode");
-  if (!b_k && g.n.stride0[0] != 1) return fail(GK_ERR_ALIGNMENT, "B must be contiguous along its first N mode or its first K mode");
-  for (int i = 0; i < g.m.nmodes; ++i) if (!(i == 0 && !a_k) && g.m.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of M mode %d of A is not a multiple of 16 bytes", i);
-  for (int i = 0; i < g.k.nmodes; ++i) if (!(i == 0 && a_k) && g.k.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of K mode %d of A is not a multiple of 16 bytes", i);
-  for (int i = 0; i < g.n.nmodes; ++i) if (!(i == 0 && !b_k) && g.n.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of N mode %d of B is not a multiple of 16 bytes", i);
-  for (int i = 0; i < g.k.nmodes; ++i) if (!(i == 0 && b_k) && g.k.stride1[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of K mode %d of B is not a multiple of 16 bytes", i);
+  const int a_run = a_k ? gett_dense_prefix(g.k, g.k.stride0) : gett_dense_prefix(g.m, g.m.stride0);
+  const int b_run = b_k ? gett_dense_prefix(g.k, g.k.stride1) : gett_dense_prefix(g.n, g.n.stride0);
+  if (a_run == 0) return fail(GK_ERR_ALIGNMENT, "A needs 8 consecutive elements along its leading M modes or its leading K modes (densely packed modes whose extents multiply to a multiple of 8)");
+  if (b_run == 0) return fail(GK_ERR_ALIGNMENT, "B needs 8 consecutive elements along its leading N modes or its leading K modes (densely packed modes whose extents multiply to a multiple of 8)");
+  for (int i = 0; i < g.m.nmodes; ++i) if (!(!a_k && i < a_run) && g.m.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of M mode %d of A is not a multiple of 16 bytes", i);
+  for (int i = 0; i < g.k.nmodes; ++i) if (!(a_k && i < a_run) && g.k.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of K mode %d of A is not a multiple of 16 bytes", i);
+  for (int i = 0; i < g.n.nmodes; ++i) if (!(!b_k && i < b_run) && g.n.stride0[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of N mode %d of B is not a multiple of 16 bytes", i);
+  for (int i = 0; i < g.k.nmodes; ++i) if (!(b_k && i < b_run) && g.k.stride1[i] % 8 != 0) return fail(GK_ERR_ALIGNMENT, "stride of K mode %d of B is not a multiple of 16 bytes", i);
   return GK_OK;
 }
 
@@ -811,12 +861,12 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
     // interleaved matrix, one per complex number of a plane)
     const bool planar = is_split_layout(conf->global_a_layout.kind);
     const bool cplx = conf->op.kind == GK_OP_MFMA_COMPLEX || conf->op.kind == GK_OP_MFMA_DUAL;
-    const long long em = planar ? conf->matmul_shape.M : args.M;
+    const long long em = planar ? conf->matmul_shape.M : args.M, en = planar ? conf->matmul_shape.N : args.N;
     const long long ek = (cplx && !planar) ? 2ll * conf->matmul_shape.K : conf->matmul_shape.K;
     if (!a_zero && conf->global_a_layout.kind != GK_LAYOUT_DIAGONAL && conf->global_a_layout.kind != GK_LAYOUT_GETT &&
         args.lda < (a_row ? ek : em))
       return fail(GK_ERR_DIMENSION_MISMATCH, "lda = %lld is smaller than the leading extent of A", args.lda);
-    if (!b_zero && conf->global_b_layout.kind != GK_LAYOUT_GETT && args.ldb < (b_row ? args.N : ek))
+    if (!b_zero && conf->global_b_layout.kind != GK_LAYOUT_GETT && args.ldb < (b_row ? en : ek))
       return fail(GK_ERR_DIMENSION_MISMATCH, "ldb = %lld is smaller than the leading extent of B", args.ldb);
     if (conf->global_d_layout.kind != GK_LAYOUT_GETT && (args.ldd < em || (args.c_mode && args.ldc < em)))
       return fail(GK_ERR_DIMENSION_MISMATCH, "ldc/ldd is smaller than M");

@@ -52,7 +52,41 @@ struct GettDim {
   int extent[kMaxModes];
   long long stride0[kMaxModes];
   long long stride1[kMaxModes];
+  // division by extent[i] as a multiplication (see gett_div), filled by the host with gett_fill_division()
+  unsigned magic[kMaxModes];
+  int shift[kMaxModes];
 };
+
+// n / e for 0 <= n < 2^31 and a divisor known on the host: with s = ceil(log2 e), magic = floor(2^(31+s) / e) + 1
+// fits in 32 bits and floor(n * magic / 2^(31+s)) is the quotient exactly (the error of the reciprocal, at most
+// e / 2^(31+s) relative, stays below 1/e for every n < 2^31).  e = 1 is marked by magic = 0.
+__host__ __device__ inline void gett_fill_division(GettDim& d) {
+  for (int i = 0; i < kMaxModes; ++i) {
+    d.magic[i] = 0;
+    d.shift[i] = 0;
+    const unsigned e = i < d.nmodes ? (unsigned)d.extent[i] : 1u;
+    if (e <= 1) continue;
+    int s = 0;
+    while ((1ull << s) < e) ++s;
+    d.magic[i] = (unsigned)(((1ull << (31 + s)) / e) + 1ull);
+    d.shift[i] = s - 1;
+  }
+}
+__host__ __device__ inline int gett_div(int n, unsigned magic, int shift) {
+  if (magic == 0) return n;
+  return (int)((unsigned)(((unsigned long long)(unsigned)n * magic) >> 32) >> shift);
+}
+// the two element offsets of index idx (< 2^31) of a GEMM dimension: a mixed-radix walk over its modes
+__host__ __device__ inline void gett_offsets32(const GettDim& d, int idx, long long& off0, long long& off1) {
+  off0 = 0; off1 = 0;
+  for (int i = 0; i < d.nmodes; ++i) {
+    const int q = gett_div(idx, d.magic[i], d.shift[i]);
+    const int digit = idx - q * d.extent[i];
+    idx = q;
+    off0 += (long long)digit * d.stride0[i];
+    off1 += (long long)digit * d.stride1[i];
+  }
+}
 
 __host__ __device__ inline void gett_offsets(const GettDim& d, long long idx, long long& off0, long long& off1) {
   off0 = 0; off1 = 0;
@@ -91,6 +125,13 @@ struct GemmArgs {
   // acc_post_scale = 1 / acc_pre_scale before the hooks of D (both 1 otherwise)
   float acc_pre_scale, acc_post_scale;
   GettDim gm, gn, gk;
+  // How a K tile lies in the K modes of a contraction: it covers the modes below gk_mode whole (their extents
+  // multiply to a divisor of BLOCK_K) and gk_step indices of mode gk_mode, whose extent gk_step divides.
+  // (BLOCK_K divides the first K mode: gk_mode 0, gk_step BLOCK_K.)
+  int gk_mode, gk_step;
+  // 1: the first M mode and the first N mode are multiples of 32, so the 16 rows and the 4 columns of an accumulator
+  // block follow each other in C / D with one stride and block origins need one walk per wave; 0: every lane walks
+  int gett_fast;
   // K-split launches (all 0 otherwise): workgroup z of k_slices handles the k_steps tiles of K that start at
   // tile z * k_steps; slice 0 starts from C.  Every slice writes its partial tile to ws_partials and counts
   // itself in ws_counters[tile]; the last one to arrive adds the partial tiles in slice order, runs the

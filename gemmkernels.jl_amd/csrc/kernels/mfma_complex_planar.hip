@@ -1,15 +1,15 @@
 // Complex GEMM on planar (split re / im) global matrices in one launch (the global-memory
 // counterpart of the reference's SplitColMajor / SplitRowMajor layouts, src/layout.jl:340-411, with
-// the sign pattern of WMMAComplexOp.mma, src/operator.jl:307-311).
+// the products of WMMAComplexOp.mma, src/operator.jl:307-311).
 //
-// With D = [D_re; D_im] stacked along M, the product is the real GEMM
-//     [D_re]   [C_re]   [-A_im]          [A_re]
-//     [D_im] = [C_im] + [ A_re] B_im  +  [A_im] B_re
-// so it runs on the real MFMA kernel with a real tile of 2*BM rows and two passes over K; only the
-// tile addressing and one sign flip of the upper accumulators differ (FIX_PLANAR).  Every element
-// of A and B is staged through LDS exactly as in the real kernel; nothing is expanded in registers.
+// The planes of a planar matrix are plain real matrices, so the product is ONE real product of the real views
+// [A_re; A_im] (2M x K) and [B_re, B_im] (K x 2N), like the interleaved form (mfma_complex_pair.hip), on the K loop
+// of the real kernel.  Only the tile addressing differs: the rows and columns of a tile are dealt out so that every
+// wave holds both parts of its complex rows and columns, and the four real products of an element of D are combined
+// inside a lane before the epilogue (FIX_PLANAR in mfma_gemm.hpp).  All four transposes read their operands the way
+// the real kernel does: nothing is expanded or read twice.
 // Every instance carries the hooks of C and D and the bias (they cost nothing when absent).
-// Tile shapes below are in complex elements.
+// Tile shapes below are in complex elements; the real tile has twice the rows and columns.
 #include "mfma_gemm.hpp"
 #include "registry.hpp"
 
@@ -21,7 +21,7 @@ int family_complex_planar(const InstanceKey& key, const GemmArgs& args, dim3 gri
 #define GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, akm_, bkm_, NAME)                                                          \
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
       key.a_kmajor == akm_ && key.b_kmajor == bkm_) {                                                                     \
-    typedef MfmaGemmConfig<2 * bm_, bn_, bk_, wm_, wn_, st_, (akm_ ? OPK_KMAJOR : OPK_MMAJOR),                             \
+    typedef MfmaGemmConfig<2 * bm_, 2 * bn_, bk_, wm_, wn_, st_, (akm_ ? OPK_KMAJOR : OPK_MMAJOR),                             \
                            (bkm_ ? OPK_KMAJOR : OPK_MMAJOR), _Float16, 3, false, FIX_PLANAR, false, 16> Cfg;                          \
     return run_instance<Cfg>(mfma_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
@@ -30,11 +30,10 @@ int family_complex_planar(const InstanceKey& key, const GemmArgs& args, dim3 gri
   GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, 0, 0, "mfma_complex_planar_nt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, 1, 1, "mfma_complex_planar_tn_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, 1, 0, "mfma_complex_planar_tt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)
-  GK_PLANAR_T(128, 256, 64, 2, 4, 2)
-  GK_PLANAR_T(128, 128, 64, 2, 2, 2)
-  GK_PLANAR_T(64, 128, 64, 2, 2, 2)
-  GK_PLANAR_T(64, 128, 32, 2, 2, 4)
-  GK_PLANAR_T(64, 64, 32, 2, 2, 2)
+  GK_PLANAR_T(128, 128, 64, 2, 4, 2)
+  GK_PLANAR_T(64, 64, 64, 2, 2, 2)
+  GK_PLANAR_T(64, 64, 32, 2, 2, 4)
+  GK_PLANAR_T(32, 32, 32, 2, 2, 4)
 #undef GK_PLANAR_T
 #undef GK_PLANAR
   (void)args; (void)grid; (void)stream; (void)mode; (void)info; (void)err;

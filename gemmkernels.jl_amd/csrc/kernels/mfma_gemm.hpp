@@ -35,11 +35,6 @@ namespace gk {
 // rows, so the tile holds R/2 complex rows.
 // ----------------------------------------------------------------------------------------------
 enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_KPAIR = 3 };
-// FIX_PLANAR: complex product on planar (split re / im) matrices.  Nothing is expanded in registers:
-// a workgroup owns BM/2 complex rows, the upper half of its real tile is the real plane of D and the
-// lower half the imaginary plane, and K runs twice: first over B_im with [A_im; A_re] as the A tile,
-// then over B_re with [A_re; A_im].  The upper half starts from -C_re and flips the sign of its
-// accumulators between the two passes, which gives C_re - A_im B_im + A_re B_re.
 // FIX_PAIR / FIX_PAIR_DUAL: complex (dual-number) product on interleaved matrices as ONE real product of the
 // matrices seen as real ones.  An interleaved matrix whose contiguous index is m (or n) is a real matrix with
 // twice the rows, row 2m the real and row 2m+1 the imaginary part, and the K loop of the real kernel runs on it
@@ -47,6 +42,12 @@ enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_KPAIR = 3 };
 // product holds the four real products re*re, re*im, im*re, im*im of every complex element of D in the lanes
 // 2i, 2i+1 (the two parts of a row of A) and the accumulator values 2j, 2j+1 (the two parts of a column of B);
 // they are combined once, before the epilogue (pair_combine).
+// FIX_PLANAR: the same for planar (split re / im) matrices, whose planes are plain real matrices: the real view of A
+// is [A_re; A_im] stacked along m and that of B [B_re, B_im] side by side along n.  The tile rows (columns) are
+// dealt out so that every wave holds both parts of its complex rows (columns): the upper half of the row blocks of
+// a wave tile comes from A_re, the lower half from the same rows of A_im, the left half of the column blocks from
+// B_re and the right half from B_im.  The four real products of an element of D then lie in four accumulator
+// blocks of one lane and are combined without any exchange.
 enum : int { FIX_NONE = 0, FIX_COMPLEX = 1, FIX_DUAL = 2, FIX_PLANAR = 3, FIX_PAIR = 4, FIX_PAIR_DUAL = 5 };
 
 template <int R, int BK, int KIND, bool EXPAND>
@@ -94,33 +95,62 @@ __device__ __forceinline__ void dma_lane_coords(int q, int lane, int& row, int& 
   else col = (((cs >> 2) ^ G::swz_m(row)) * 4 + ((cs & 3) ^ (((row >> 3) & 1) << 1))) * 8;
 }
 
-// Tensor-contraction index maps: walks the K index of a contraction tile by tile.  The first K
-// mode is consumed BK at a time (BK divides its extent), the others are the digits of a counter.
+// Tensor-contraction index maps: walks the K index of a contraction tile by tile.  A tile covers the K modes below
+// `mode` whole and `step` indices of mode `mode` (see GemmArgs::gk_mode); the modes above are the digits of a counter.
 struct KWalker {
-  int kf, d1, d2, d3;
-  __device__ __forceinline__ void reset() { kf = d1 = d2 = d3 = 0; }
-  __device__ __forceinline__ void advance(const GettDim& gk, int bk) {
-    kf += bk;
-    if (kf >= gk.extent[0]) {
-      kf = 0;
-      if (gk.nmodes > 1 && ++d1 >= gk.extent[1]) {
-        d1 = 0;
-        if (gk.nmodes > 2 && ++d2 >= gk.extent[2]) {
-          d2 = 0;
-          if (gk.nmodes > 3) ++d3;
-        }
-      }
-    }
+  int d0, d1, d2;           // digits of the K modes 0 .. 2 at the first k of the tile (modes below `mode` stay 0)
+  long long oa, ob;         // element offsets of the tile's first k in A and in B, kept up to date by advance()
+  // copies of the mode table, held in scalar registers for the whole K loop: read from the kernel arguments inside the
+  // loop they would be scalar loads, and the wait for a scalar load also waits for every LDS read in flight.  Only
+  // additions are left in the loop: step_a / step_b move the offsets by one tile along `mode`, wrap_a[i] / wrap_b[i]
+  // are what a carry out of mode i adds (one stride of mode i + 1 minus the whole extent of mode i).
+  int nmodes, mode, step, e0, e1, e2;
+  long long step_a, step_b, wa0, wa1, wa2, wb0, wb1, wb2;
+  // (the values are the same in every lane; readfirstlane says so to the compiler where it has loaded the kernel
+  // arguments with vector instructions)
+  __device__ __forceinline__ static void keep(int& x) { x = __builtin_amdgcn_readfirstlane(x); asm volatile("" : "+s"(x)); }
+  __device__ __forceinline__ static void keep(long long& x) {
+    int lo = __builtin_amdgcn_readfirstlane((int)(unsigned)(unsigned long long)x), hi = __builtin_amdgcn_readfirstlane((int)((unsigned long long)x >> 32));
+    asm volatile("" : "+s"(lo), "+s"(hi));
+    x = (long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
   }
-  // element offset of the tile's first k in the tensor whose K strides are `stride`
-  __device__ __forceinline__ long long offset(const GettDim& gk, const long long* stride) const {
-    long long o = (long long)kf * stride[0];
-    if (gk.nmodes > 1) o += (long long)d1 * stride[1];
-    if (gk.nmodes > 2) o += (long long)d2 * stride[2];
-    if (gk.nmodes > 3) o += (long long)d3 * stride[3];
-    return o;
+  __device__ __forceinline__ void init(const GettDim& gk, int mode_, int step_) {
+    d0 = d1 = d2 = 0;
+    oa = ob = 0;
+    nmodes = gk.nmodes; mode = mode_; step = step_;
+    e0 = gk.extent[0]; e1 = gk.extent[1]; e2 = gk.extent[2];
+    step_a = (long long)step_ * gk.stride0[mode_];
+    step_b = (long long)step_ * gk.stride1[mode_];
+    wa0 = gk.stride0[1] - (long long)e0 * gk.stride0[0]; wb0 = gk.stride1[1] - (long long)e0 * gk.stride1[0];
+    wa1 = gk.stride0[2] - (long long)e1 * gk.stride0[1]; wb1 = gk.stride1[2] - (long long)e1 * gk.stride1[1];
+    wa2 = gk.stride0[3] - (long long)e2 * gk.stride0[2]; wb2 = gk.stride1[3] - (long long)e2 * gk.stride1[2];
+    keep(nmodes); keep(mode); keep(step); keep(e0); keep(e1); keep(e2);
+    keep(step_a); keep(step_b); keep(wa0); keep(wa1); keep(wa2); keep(wb0); keep(wb1); keep(wb2);
   }
+  __device__ __forceinline__ void advance() {
+    // the digit of `mode` moves on by step; a digit that reaches its extent goes back to 0 and carries (the digit
+    // of the last mode never wraps inside K and is not kept)
+    if (mode == 0) d0 += step; else if (mode == 1) d1 += step; else if (mode == 2) d2 += step;
+    oa += step_a; ob += step_b;
+    if (nmodes > 1 && d0 >= e0) { d0 = 0; ++d1; oa += wa0; ob += wb0; }
+    if (nmodes > 2 && d1 >= e1) { d1 = 0; ++d2; oa += wa1; ob += wb1; }
+    if (nmodes > 3 && d2 >= e2) { d2 = 0; oa += wa2; ob += wb2; }
+  }
+  // element offsets of the tile's first k in A and in B
+  __device__ __forceinline__ long long offset_a() const { return oa; }
+  __device__ __forceinline__ long long offset_b() const { return ob; }
 };
+// element offset of k-value k (< BLOCK_K) of a tile from the tile's first k: digits of the modes the tile covers whole,
+// the rest along mode `mode`
+__device__ __forceinline__ long long gett_k_local(const GettDim& gk, int mode, int k, const long long* stride) {
+  long long o = 0;
+  for (int i = 0; i < mode; ++i) {
+    const int q = gett_div(k, gk.magic[i], gk.shift[i]);
+    o += (long long)(k - q * gk.extent[i]) * stride[i];
+    k = q;
+  }
+  return o + (long long)k * stride[mode];
+}
 
 // Makes every later use of x depend on the point where pin() stands (no instruction is emitted).
 __device__ __forceinline__ void pin(int4v& x) { asm volatile("" : "+v"(x)); }
@@ -430,7 +460,7 @@ struct MfmaGemmConfig {
   static_assert(FM * FN > 0, "empty wave tile");
   static_assert(!GETT || FIX == FIX_NONE, "contractions are real");
   static_assert(!SPLITK || (!GETT && FIX == FIX_NONE), "K-split instances are plain real GEMMs");
-  static_assert(!PLANAR || (WAVES_M_ % 2 == 0 && (FUSE_ == 0 || FUSE_ == 3)), "planar complex: a wave's rows lie in one plane of D; hooks on C and D only");
+  static_assert(!PLANAR || (MI_ == 16 && A_KIND_ != OPK_KPAIR && B_KIND_ != OPK_KPAIR), "planar complex: 16-row blocks on plain real planes");
   static_assert(!COMPLEX || FUSE_ == 0 || FUSE_ == 3, "complex products take hooks on C and D only");
   static_assert(!PAIR || (MI_ == 16 && (A_KIND_ == OPK_MMAJOR || A_KIND_ == OPK_KPAIR) && (B_KIND_ == OPK_MMAJOR || B_KIND_ == OPK_KPAIR)),
                 "complex-pair products: 16-row blocks on the real view of the operands");
@@ -462,21 +492,26 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const char* gb;
   long long a_step = 0, b_step = 0;
   unsigned offa[DMA_A], offb[DMA_B];
-  unsigned offa2[Cfg::PLANAR ? DMA_A : 1];   // planar complex: the A offsets of the second pass over K
-  int to_switch = 0;                         // planar complex: tiles left to issue in the first pass
-  KWalker walk;
-  walk.reset();
+  [[maybe_unused]] KWalker walk;
+  if constexpr (Cfg::GETT) walk.init(args.gk, args.gk_mode, args.gk_step);
   if constexpr (!Cfg::GETT) {
     // tile origin and K step in 16-bit elements (lda / ldb are in 16-bit elements as well; an
     // interleaved complex matrix counts two per complex number)
-    const int m0g = Cfg::EXPAND_A ? m0 / 2 : (Cfg::PLANAR ? m0 / 2 : m0);   // first row of the tile in the stored matrix
+    const int m0g = (Cfg::EXPAND_A || Cfg::PLANAR) ? m0 / 2 : m0;   // first row of the tile in the stored matrix
+    const int n0g = Cfg::PLANAR ? n0 / 2 : n0;
     const long long a_org = Cfg::A_KIND == OPK_KMAJOR ? (long long)m0g * args.lda
-                          : (Cfg::A_KIND == OPK_KPAIR ? (long long)(m0 / 2) * args.lda : (long long)(Cfg::PLANAR ? m0g : m0));
-    const long long b_org = Cfg::B_KIND == OPK_KMAJOR ? (long long)n0 * args.ldb
-                          : (Cfg::B_KIND == OPK_KPAIR ? (long long)(n0 / 2) * args.ldb : (long long)n0);
+                          : (Cfg::A_KIND == OPK_KPAIR ? (long long)(m0 / 2) * args.lda : (long long)m0g);
+    const long long b_org = Cfg::B_KIND == OPK_KMAJOR ? (long long)n0g * args.ldb
+                          : (Cfg::B_KIND == OPK_KPAIR ? (long long)(n0 / 2) * args.ldb : (long long)n0g);
     ga = (const char*)args.a + a_org * 2;
     gb = (const char*)args.b + b_org * 2;
-    if constexpr (Cfg::PLANAR) gb += args.plane_b * 2;   // the first pass over K reads B_im
+    // planar complex: tile row (column) r belongs to wave row r / WT; the first half of a wave's rows are complex rows
+    // of the real plane, the second half the same complex rows of the imaginary plane
+    [[maybe_unused]] auto planar_index = [](int r, int wt, bool& imag) {
+      const int w = r / wt, in = r % wt;
+      imag = in >= wt / 2;
+      return w * (wt / 2) + (in % (wt / 2));
+    };
     a_step = (Cfg::A_KIND == OPK_KMAJOR ? (long long)BK : (Cfg::A_KIND == OPK_KPAIR ? 2ll * BK : (long long)GA::LDS_ROWS * args.lda)) * 2;
     b_step = (Cfg::B_KIND == OPK_KMAJOR ? (long long)BK : (Cfg::B_KIND == OPK_KPAIR ? 2ll * BK : (long long)GB::LDS_ROWS * args.ldb)) * 2;
 #pragma unroll
@@ -484,13 +519,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       int row, col;
       dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
       if constexpr (Cfg::PLANAR) {
-        // rows [0, BM/2) of the tile come from one plane of A, rows [BM/2, BM) from the other
         int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
-        const bool lower = m >= BM / 2;
-        if (lower) m -= BM / 2;
-        const unsigned base = (unsigned)(((long long)row * args.lda + col) * 2);
-        offa[i] = base + (lower ? 0u : (unsigned)(args.plane_a * 2));
-        offa2[i] = base + (lower ? (unsigned)(args.plane_a * 2) : 0u);
+        bool imag;
+        m = planar_index(m, Cfg::WTM, imag);
+        offa[i] = (unsigned)(((long long)row * args.lda + col + (imag ? args.plane_a : 0ll)) * 2);
       } else {
         if constexpr (Cfg::RAGGED_OK) {
           // a tile that sticks out over the last row of A: chunks beyond it re-read the last valid chunk
@@ -511,7 +543,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         const int last = Cfg::B_KIND == OPK_KMAJOR ? args.N - n0 - 1 : ((args.N - n0 - 1) >> 3) << 3;
         n = n > last ? last : n;
       }
-      offb[i] = (unsigned)(((long long)row * args.ldb + col) * 2);
+      [[maybe_unused]] bool imag = false;
+      if constexpr (Cfg::PLANAR) {
+        int& n = Cfg::B_KIND == OPK_KMAJOR ? row : col;
+        n = planar_index(n, Cfg::WTN, imag);
+      }
+      offb[i] = (unsigned)(((long long)row * args.ldb + col + ((Cfg::PLANAR && imag) ? args.plane_b : 0ll)) * 2);
     }
   } else {
     // element (m, k) of A lives at offM(m) + offK(k): the row part is a mixed-radix walk over the M
@@ -524,8 +561,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
       const int r = Cfg::A_KIND == OPK_KMAJOR ? row : col, k = Cfg::A_KIND == OPK_KMAJOR ? col : row;
       long long o0, o1;
-      gett_offsets(args.gm, m0 + r, o0, o1);
-      offa[i] = (unsigned)((o0 + (long long)k * args.gk.stride0[0]) * 2);
+      gett_offsets32(args.gm, m0 + r, o0, o1);
+      offa[i] = (unsigned)((o0 + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride0)) * 2);
     }
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i) {
@@ -533,31 +570,20 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
       const int r = Cfg::B_KIND == OPK_KMAJOR ? row : col, k = Cfg::B_KIND == OPK_KMAJOR ? col : row;
       long long o0, o1;
-      gett_offsets(args.gn, n0 + r, o0, o1);
-      offb[i] = (unsigned)((o0 + (long long)k * args.gk.stride1[0]) * 2);
+      gett_offsets32(args.gn, n0 + r, o0, o1);
+      offb[i] = (unsigned)((o0 + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride1)) * 2);
     }
   }
 
   auto issue_tile = [&](int stage) {
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
-    if constexpr (Cfg::PLANAR) {
-      if (to_switch == 0) {
-        // second pass: back to k = 0, B_re instead of B_im, the planes of A trade places
-        const long long kh = (args.K / BK) / 2;
-        ga -= kh * a_step;
-        gb -= kh * b_step + args.plane_b * 2;
-#pragma unroll
-        for (int i = 0; i < DMA_A; ++i) offa[i] = offa2[i];
-      }
-      --to_switch;
-    }
     const char* pa = ga;
     const char* pb = gb;
     if constexpr (Cfg::GETT) {
-      pa = ga + walk.offset(args.gk, args.gk.stride0) * 2;
-      pb = gb + walk.offset(args.gk, args.gk.stride1) * 2;
-      walk.advance(args.gk, BK);
+      pa = ga + walk.offset_a() * 2;
+      pb = gb + walk.offset_b() * 2;
+      walk.advance();
     }
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i)
@@ -578,22 +604,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     constexpr int P = decltype(p_c)::value, NP = decltype(np_c)::value;
     char* sa = smem + stage * Cfg::STAGE_BYTES;
     char* sb = sa + GA::BYTES;
-    if constexpr (Cfg::PLANAR && P == 0) {
-      if (to_switch == 0) {
-        // second pass: back to k = 0, B_re instead of B_im, the planes of A trade places
-        const long long kh = (args.K / BK) / 2;
-        ga -= kh * a_step;
-        gb -= kh * b_step + args.plane_b * 2;
-#pragma unroll
-        for (int i = 0; i < DMA_A; ++i) offa[i] = offa2[i];
-      }
-      --to_switch;
-    }
     if constexpr (Cfg::GETT && P == 0) {
       // tile base of the tensor walk, the same for every part of this tile
-      part_a = ga + walk.offset(args.gk, args.gk.stride0) * 2;
-      part_b = gb + walk.offset(args.gk, args.gk.stride1) * 2;
-      walk.advance(args.gk, BK);
+      part_a = ga + walk.offset_a() * 2;
+      part_b = gb + walk.offset_b() * 2;
+      walk.advance();
     }
     const char* pa = Cfg::GETT ? part_a : ga;
     const char* pb = Cfg::GETT ? part_b : gb;
@@ -610,8 +625,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   };
 
   // K tiles of this workgroup: all of them, or one slice of a K-split launch
-  int KT = args.K / BK;       // planar complex: args.K counts both passes
-  [[maybe_unused]] const int KH = KT / 2;
+  int KT = args.K / BK;
   // The last K tile runs outside the pipeline (after the loop) when it is a partial one, and also when it is whole
   // but a 16-byte chunk of this workgroup's tiles straddles the last row of an operand whose rows are contiguous in
   // memory (M, or N, not a multiple of 8): in the last k such a chunk would read past the end of the operand.
@@ -622,7 +636,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
                           (Cfg::B_KIND == OPK_MMAJOR && (args.N & 7) != 0 && n0 + BN > args.N);
     if (tail_k == 0 && straddle && KT > 0) { KT -= 1; tail_k = BK; }
   }
-  if constexpr (Cfg::PLANAR) to_switch = KH;
   if constexpr (Cfg::SPLITK) {
     const int kt0 = (int)blockIdx.z * args.k_steps;
     KT = (KT - kt0) < args.k_steps ? (KT - kt0) : args.k_steps;
@@ -648,51 +661,61 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr int NVO = Cfg::PAIR ? 2 : NV;                     // values per lane and block that C / D see
   constexpr int CB = Cfg::PAIR ? MI / 2 : MI;                 // columns of C / D per block
   auto slot = [](int v) { return Cfg::PAIR ? 2 * v : v; };
+  // planar complex: C / D see the left half of the column blocks (the right half holds the products with B_im until
+  // they are combined); row block fi is complex rows of the real plane for fi < FM / 2, of the imaginary plane above
+  constexpr int FNO = Cfg::PLANAR ? FN / 2 : FN;
+  constexpr int FMH = Cfg::PLANAR ? FM / 2 : FM;
   AccV acc[FM][FN];
-  // planar complex: the wave's rows lie in the real (upper) or the imaginary (lower) plane of C / D
-  [[maybe_unused]] const bool lower_plane = Cfg::PLANAR && (wm * Cfg::WTM >= BM / 2);
-  const int mrow = Cfg::PLANAR ? m0 / 2 + wm * Cfg::WTM - (lower_plane ? BM / 2 : 0) + (lane % MI) : m0 + wm * Cfg::WTM + (lane % MI);
-  const int ncol = Cfg::PAIR ? (n0 + wn * Cfg::WTN) / 2 + 2 * (lane / MI) : n0 + wn * Cfg::WTN + 4 * (lane / MI);
-  // complex C / D: this lane's row is the imaginary part of its complex row
-  [[maybe_unused]] const bool im_lane = Cfg::PLANAR ? lower_plane : (Cfg::COMPLEX && (lane & 1) != 0);
+  const int mrow = Cfg::PLANAR ? (m0 + wm * Cfg::WTM) / 2 + (lane % MI) : m0 + wm * Cfg::WTM + (lane % MI);
+  const int ncol = Cfg::PAIR ? (n0 + wn * Cfg::WTN) / 2 + 2 * (lane / MI)
+                 : (Cfg::PLANAR ? (n0 + wn * Cfg::WTN) / 2 + 4 * (lane / MI) : n0 + wn * Cfg::WTN + 4 * (lane / MI));
+  // complex C / D: row block fi of this lane holds imaginary parts (interleaved: the odd lanes, whatever fi; planar:
+  // the lower half of the row blocks)
+  [[maybe_unused]] auto imag_rows = [&](int fi) { return Cfg::PLANAR ? fi >= FMH : (Cfg::COMPLEX && (lane & 1) != 0); };
   // element offset of the lane's first element of accumulator block (fi, fj) in C / D, and the
-  // stride between its consecutive columns.  With a tensor-contraction map the first M mode and
-  // the first N mode cover whole 32-wide blocks, so only the block origin needs the digit walk.
-  // contractions: origins of the blocks of the wave tile in C / D, one digit walk per 32 rows (columns);
-  // filled before the C load and again before the D store (not kept across the K loop)
+  // stride between its consecutive columns.
+  // contractions: offset of the lane's row of row block fi (gett_om) and of the first of its four columns of
+  // column block fj (gett_on) in C / D; filled before the C load and again before the D store (not kept across
+  // the K loop)
   [[maybe_unused]] long long gett_om[Cfg::GETT ? FM : 1], gett_on[Cfg::GETT ? FN : 1];
   [[maybe_unused]] auto gett_origins = [&]() __attribute__((always_inline)) {
     if constexpr (Cfg::GETT) {
       long long t0;
+      if (args.gett_fast) {
+        // whole 32-wide blocks inside the first M mode and the first N mode: one walk per block origin (the same
+        // for every lane of the wave), the lane's own row and first column follow with the strides of those modes
+        const long long lane_m = (long long)(lane % MI) * args.gm.stride1[0], lane_n = (long long)(4 * (lane / MI)) * args.gn.stride1[0];
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi) {
-        if (MI == 16 && (fi & 1)) gett_om[fi] = gett_om[fi - 1] + 16 * args.gm.stride1[0];
-        else gett_offsets(args.gm, m0 + wm * Cfg::WTM + MI * fi, t0, gett_om[fi]);
-      }
+        for (int fi = 0; fi < FM; ++fi) {
+          if (MI == 16 && (fi & 1)) gett_om[fi] = gett_om[fi - 1] + 16 * args.gm.stride1[0];
+          else { gett_offsets32(args.gm, m0 + wm * Cfg::WTM + MI * fi, t0, gett_om[fi]); gett_om[fi] += lane_m; }
+        }
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) {
-        if (MI == 16 && (fj & 1)) gett_on[fj] = gett_on[fj - 1] + 16 * args.gn.stride1[0];
-        else gett_offsets(args.gn, n0 + wn * Cfg::WTN + MI * fj, t0, gett_on[fj]);
+        for (int fj = 0; fj < FN; ++fj) {
+          if (MI == 16 && (fj & 1)) gett_on[fj] = gett_on[fj - 1] + 16 * args.gn.stride1[0];
+          else { gett_offsets32(args.gn, n0 + wn * Cfg::WTN + MI * fj, t0, gett_on[fj]); gett_on[fj] += lane_n; }
+        }
+      } else {
+        // any extents: every lane walks the modes for its own row of each block and for the first of its four
+        // columns (which lie inside the first N mode: its extent is a multiple of 4)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) gett_offsets32(args.gm, m0 + wm * Cfg::WTM + MI * fi + (lane % MI), t0, gett_om[fi]);
+#pragma unroll
+        for (int fj = 0; fj < FN; ++fj) gett_offsets32(args.gn, n0 + wn * Cfg::WTN + MI * fj + 4 * (lane / MI), t0, gett_on[fj]);
       }
     }
   };
   auto cd_offset = [&](int fi, int fj, long long ld, [[maybe_unused]] long long plane) -> long long {
     if constexpr (Cfg::PLANAR) {
-      return (long long)(mrow + MI * fi) + (long long)(ncol + MI * fj) * ld + (lower_plane ? plane : 0ll);
+      return (long long)(mrow + MI * (fi % FMH)) + (long long)(ncol + MI * fj) * ld + (fi >= FMH ? plane : 0ll);
     } else if constexpr (!Cfg::GETT) {
       return (long long)(mrow + MI * fi) + (long long)(ncol + CB * fj) * ld;
     } else {
-      return gett_om[fi] + (long long)(lane % MI) * args.gm.stride1[0] + gett_on[fj] + (long long)(4 * (lane / MI)) * args.gn.stride1[0];
+      return gett_om[fi] + gett_on[fj];
     }
   };
   auto cd_nstride = [&](long long ld) -> long long {
     if constexpr (!Cfg::GETT) return ld; else return args.gn.stride1[0];
-  };
-  auto negate_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int fi = 0; fi < FM; ++fi)
-#pragma unroll
-      for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = -acc[fi][fj];
   };
   // One hook over the accumulators of column block fj (FM blocks): the dispatch on the op is paid once per
   // op and column block, not once per 16x16 block.  (Over all accumulators at once the cases of the
@@ -715,7 +738,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         // two parts independently, and this one)
         if (t.kind[i] == T_ADD) {
           const float p0 = t.p0[i];
-          each([=](float x) { return im_lane ? x : x + p0; });
+#pragma unroll
+          for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+            for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = imag_rows(fi) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + p0;
           continue;
         }
       }
@@ -748,8 +774,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     gett_origins();
     // column blocks outermost: with 16-row blocks the two halves of a 128-byte line of C / D belong to
     // neighbouring row blocks, which are then read (and, below, written) right after each other
+    if constexpr (Cfg::PLANAR) {
 #pragma unroll
-    for (int fj = 0; fj < FN; ++fj)
+      for (int fj = FNO; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) acc[fi][fj] = AccV{};     // the products with B_im start from zero
+    }
+#pragma unroll
+    for (int fj = 0; fj < FNO; ++fj)
 #pragma unroll
       for (int fi = 0; fi < FM; ++fi) {
         const long long off = cd_offset(fi, fj, args.ldc, args.plane_c);
@@ -771,7 +803,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       }
     if (Cfg::FUSED) {
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) {
+      for (int fj = 0; fj < FNO; ++fj) {
         hook_col(std::integral_constant<int, H_GL2SH_C>{}, fj);
         hook_col(std::integral_constant<int, H_SH2RF_C>{}, fj);
       }
@@ -785,9 +817,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         for (int v = 0; v < NV; ++v) acc[fi][fj][v] = 0.0f;
   }
 
-  if constexpr (Cfg::PLANAR) {
-    if (args.c_mode != 0 && !lower_plane) negate_acc();   // the sign comes back between the two passes over K
-  }
   // a power-of-two scale of A or B that the host has folded into the accumulators (see GemmArgs)
   [[maybe_unused]] auto scale_acc = [&](float f) __attribute__((always_inline)) {
 #pragma unroll
@@ -909,9 +938,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       // tile kt has landed once at most the DMA of the STAGES-2 younger tiles is outstanding
       if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 2) * DPT>(); else wait_vmcnt<0>();
       block_barrier();   // every wave's share of tile kt is in LDS; every wave is done with tile kt-1
-      if constexpr (Cfg::PLANAR) {
-        if (kt == KH && !lower_plane) negate_acc();
-      }
       const unsigned stage_addr = lds_base + (unsigned)(kt % STAGES) * Cfg::STAGE_BYTES;
       ra.set_stage(stage_addr);
       rb.set_stage(stage_addr + GA::BYTES);
@@ -985,9 +1011,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       // tiles <= kt+1 have landed once at most the STAGES-3 younger tiles are outstanding
       if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 3) * DPT>(); else wait_vmcnt<0>();
       block_barrier();   // tile kt+1 is visible; every wave is done reading tile kt-1
-      if constexpr (Cfg::PLANAR) {
-        if (kt == KH && !lower_plane) negate_acc();
-      }
       const bool issue = (kt + STAGES - 1 < KT);
       const bool last = (kt + 1 >= KT);
       static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
@@ -1145,14 +1168,27 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           // compiled as a cast of the whole vector, of which element 0 is then taken)
           const float mine = acc[fi][fj][2 * v + 1];
           const float other = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mine), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-          acc[fi][fj][2 * v] = im_lane ? own + other : (Cfg::FIX == FIX_PAIR_DUAL ? own : own - other);
+          acc[fi][fj][2 * v] = (lane & 1) ? own + other : (Cfg::FIX == FIX_PAIR_DUAL ? own : own - other);
         }
+  }
+
+  if constexpr (Cfg::PLANAR) {
+    // The four real products of the elements of D lie in four blocks of the lane: (row blocks of A_re | A_im) x
+    // (column blocks of B_re | B_im).  Real part re*re - im*im into the upper left block, imaginary part
+    // im*re + re*im into the lower left one; C came in through the same two.
+#pragma unroll
+    for (int fi = 0; fi < FMH; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FNO; ++fj) {
+        acc[fi][fj] = acc[fi][fj] - acc[fi + FMH][fj + FNO];
+        acc[fi + FMH][fj] = acc[fi + FMH][fj] + acc[fi][fj + FNO];
+      }
   }
 
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   gett_origins();
 #pragma unroll
-  for (int fj = 0; fj < FN; ++fj) {
+  for (int fj = 0; fj < FNO; ++fj) {
     if (Cfg::FUSED) {
       hook_col(std::integral_constant<int, H_RF2SH_D>{}, fj);
       if (args.epi_kind == 1) {          // one bias value per column of D
@@ -1166,14 +1202,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
-          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = (Cfg::COMPLEX && im_lane) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + bv[v];
+          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = imag_rows(fi) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + bv[v];
       } else if (args.epi_kind == 2) {   // one bias value per row of D
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const int r = (Cfg::COMPLEX && !Cfg::PLANAR) ? (mrow + MI * fi) >> 1 : mrow + MI * fi;
+          const int r = Cfg::PLANAR ? mrow + MI * (fi % FMH) : (Cfg::COMPLEX ? (mrow + MI * fi) >> 1 : mrow + MI * fi);
           const float bv = args.bias[(Cfg::RAGGED_OK && r >= args.M) ? 0 : r];
 #pragma unroll
-          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = (Cfg::COMPLEX && im_lane) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + bv;
+          for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = imag_rows(fi) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + bv;
         }
       }
       hook_col(std::integral_constant<int, H_SH2GL_D>{}, fj);

@@ -229,9 +229,9 @@ _COMPLEX_PAIR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 6
 _COMPLEX_TN_TILES = [((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 _DUAL_TN_TILES = [((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 
-# complex tiles (complex elements) of the kernel for planar global matrices -> waves; a workgroup's real
-# tile has twice as many rows (both planes of D)
-_PLANAR_TILES = [((128, 256, 64), (2, 4)), ((64, 128, 64), (2, 2)), ((128, 128, 64), (2, 2)), ((64, 128, 32), (2, 2)), ((64, 64, 32), (2, 2))]
+# complex tiles (complex elements) of the kernel for planar global matrices -> waves; the real tile has twice
+# the rows and columns (both planes of A, B and D)
+_PLANAR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
 
 # tiles of the vector-ALU kernel and of the bounds-checked MFMA kernel
 _FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (1, 1))]

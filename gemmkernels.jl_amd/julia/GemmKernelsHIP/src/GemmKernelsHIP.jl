@@ -346,7 +346,8 @@ const MFMA_TILE_RATE = Dict((256, 256, 64) => 1.0, (256, 256, 32) => 0.95, (256,
 const COMPLEX_PAIR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
 const COMPLEX_TN_TILES = [((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 const DUAL_TN_TILES = [((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
-function complex_tiles(operator::Type, a_kmajor::Bool, b_kmajor::Bool)
+function complex_tiles(operator::Type, a_kmajor::Bool, b_kmajor::Bool; planar::Bool = false)
+    planar && return COMPLEX_PAIR_TILES            # planar global matrices: the planes are plain real matrices, one table for all transposes
     a_kmajor && b_kmajor && return nameof(operator) in (:WMMADualOp, :MFMADualOp) ? DUAL_TN_TILES : COMPLEX_TN_TILES
     a_kmajor ? [(t, (w[2], w[1])) for (t, w) in COMPLEX_PAIR_TILES] : COMPLEX_PAIR_TILES
 end
@@ -369,14 +370,14 @@ function adjacent_elements(num, parent_size, is_col_major)
 end
 
 "MI355X block shape: of the tiles of the table that fit, the one with the shortest estimated launch"
-function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true, a_kmajor::Bool = false, b_kmajor::Bool = true)
+function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true, a_kmajor::Bool = false, b_kmajor::Bool = true, planar::Bool = false)
     M, N, K = gemm_shape.M, gemm_shape.N, gemm_shape.K
     if Operator.is_fpu(operator)
         small = nameof(operator) == :FPUOp && Operator.compute_type(operator) == Float32 && Operator.accum_type(operator) == Float32 &&
                 tile_sized && M % 32 == 0 && N % 32 == 0 && K % 32 == 0 && cld(M, 64) * cld(N, 64) < NUM_CUS ÷ 2
         return small ? (M = 32, N = 32, K = 32) : (M = 64, N = 64, K = 32)
     elseif !Operator.is_mfma(operator)
-        fitting = [t for (t, _) in complex_tiles(operator, a_kmajor, b_kmajor) if M % t[1] == 0 && N % t[2] == 0 && K % t[3] == 0]
+        fitting = [t for (t, _) in complex_tiles(operator, a_kmajor, b_kmajor; planar = planar) if M % t[1] == 0 && N % t[2] == 0 && K % t[3] == 0]
         for t in fitting
             (M ÷ t[1]) * (N ÷ t[2]) >= NUM_CUS && return (M = t[1], N = t[2], K = t[3])
         end
@@ -390,9 +391,9 @@ function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true
     (M = best[1], N = best[2], K = best[3])
 end
 
-function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_kmajor::Bool = true)
+function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_kmajor::Bool = true, planar::Bool = false)
     key = (block_shape.M, block_shape.N, block_shape.K)
-    table = Operator.is_fpu(operator) ? FPU_TILES : (Operator.is_mfma(operator) ? MFMA_TILES : complex_tiles(operator, a_kmajor, b_kmajor))
+    table = Operator.is_fpu(operator) ? FPU_TILES : (Operator.is_mfma(operator) ? MFMA_TILES : complex_tiles(operator, a_kmajor, b_kmajor; planar = planar))
     for (t, w) in table
         t == key && return w
     end
@@ -421,10 +422,11 @@ function get_config(; gemm_shape, operator, global_a_layout, global_c_layout, kw
     tile_sized = any(require_tile_sized_global, globals)
     a_kmajor = Layout.is_row_major(global_a_layout)             # 'T' A: stored K x M, k contiguous
     b_kmajor = !Layout.is_row_major(global_b_layout)            # 'N' B: stored K x N, k contiguous
-    block_shape = get(params, :block_shape, default_block_shape(operator, gemm_shape; tile_sized = tile_sized, a_kmajor = a_kmajor, b_kmajor = b_kmajor))
+    planar = Layout.kind_name(global_a_layout) in (:SplitColMajor, :SplitRowMajor)      # planar complex global matrices
+    block_shape = get(params, :block_shape, default_block_shape(operator, gemm_shape; tile_sized = tile_sized, a_kmajor = a_kmajor, b_kmajor = b_kmajor, planar = planar))
     op_shape = Operator.shape(operator)
 
-    waves = default_waves(operator, block_shape; a_kmajor = a_kmajor, b_kmajor = b_kmajor)
+    waves = default_waves(operator, block_shape; a_kmajor = a_kmajor, b_kmajor = b_kmajor, planar = planar)
     if waves !== nothing
         warps_default = waves[1] * waves[2]
         compute_warp_default = (M = block_shape.M ÷ waves[1], N = block_shape.N ÷ waves[2], K = op_shape.K)

@@ -15,12 +15,13 @@ TCCG = [
     ("ab-ac-cb", dict(a=128, b=64, c=96)),                                 # a plain GEMM, A 'N', B 'N'
     ("ab-ca-cb", dict(a=64, b=128, c=64)),                                 # A transposed
     ("abcdef-dega-gfbc", dict(a=2, b=2, c=2, d=32, e=2, f=32, g=64)),
-    ("abcd-dbea-ec", dict(a=64, b=4, c=64, d=2, e=64)),                    # refused: see REFUSED
+    ("abcd-dbea-ec", dict(a=64, b=4, c=64, d=2, e=64)),                    # A's leading M modes d (2) and b (4) make one run of 8
+    ("abcd-dbea-ec", dict(a=64, b=3, c=64, d=2, e=64)),                    # refused: see REFUSED
 ]
 
 
-# contractions whose leading mode in A is too short for 16-byte vectors and 32-wide blocks: refused, not mis-run
-REFUSED = {("abcd-dbea-ec", 64)}
+# contractions whose operand has no run of 8 consecutive elements (here d x b = 2 x 3) for 16-byte vectors: refused, not mis-run
+REFUSED = {("abcd-dbea-ec", 3)}
 
 
 def test_parse_classify_and_refusals():
@@ -50,10 +51,10 @@ def test_fusion_of_neighbouring_modes():
     assert contraction.fuse("abc", "bda", "dc", dict(a=4, b=64, c=128, d=64))[:3] == ("abc", "bda", "dc")
 
 
-@pytest.mark.parametrize("spec,ext", TCCG, ids=[f"{t[0]}/{t[1]['a']}" for t in TCCG])
+@pytest.mark.parametrize("spec,ext", TCCG, ids=[f"{t[0]}/{t[1]['a']}/{t[1]['b']}" for t in TCCG])
 def test_every_benchmark_shape_maps_onto_a_compiled_kernel(spec, ext):
     found = [(swapped, info) for swapped, _, conf, info in contraction.candidates(spec, ext) if conf is not None]
-    if (spec, ext["a"]) in REFUSED:
+    if (spec, ext["b"]) in REFUSED:
         assert not found
         return
     assert found, list(contraction.candidates(spec, ext))
@@ -72,10 +73,10 @@ def test_operands_are_swapped_when_only_that_assignment_fits():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("spec,ext", TCCG, ids=[f"{t[0]}/{t[1]['a']}" for t in TCCG])
+@pytest.mark.parametrize("spec,ext", TCCG, ids=[f"{t[0]}/{t[1]['a']}/{t[1]['b']}" for t in TCCG])
 def test_contractions_against_einsum(gpu, spec, ext):
     import torch
-    if (spec, ext["a"]) in REFUSED:
+    if (spec, ext["b"]) in REFUSED:
         pytest.skip("refused by the planner (covered on the CPU)")
     dm, am, bm = contraction.parse(spec)
     rs = np.random.RandomState(len(spec))
@@ -107,3 +108,23 @@ def test_refused_contraction_names_the_reasons(gpu):
     assert "does not map onto the GEMM kernel" in ei.value.message
     with pytest.raises(gk.ConfigError):                   # extent of c differs between A and B
         contraction.plan("ab-ac-cb", a, gk.colmajor(np.zeros((32, 64), np.float16, order="F")), d)
+
+
+def test_division_by_multiplication_is_exact():
+    """The kernels divide mode indices by the extents through a multiplication by a 32-bit reciprocal (s = ceil(log2 e),
+    magic = floor(2^(31+s) / e) + 1, quotient = (n * magic) >> (31 + s)): exact for every n < 2^31.  Checked here on the
+    arithmetic itself, at the places where a too small or too large reciprocal would first fail."""
+    rs = np.random.RandomState(5)
+    extents = list(range(2, 130)) + [255, 256, 257, 1000, 4095, 4096, 4097, 65535, 65536, 65537, 2**20 + 7, 2**30 - 1, 2**30 + 1, 2**31 - 1]
+    for e in extents:
+        s = (e - 1).bit_length()
+        magic = (1 << (31 + s)) // e + 1
+        assert magic < 2**32
+        span = min(4 * e + 2, 3000)                 # around 0, around the multiples of e, around 2^31
+        mult = np.arange(1, 500, dtype=np.int64) * e
+        ns = np.concatenate([np.arange(0, span, dtype=np.int64), (2**31 - 1) - np.arange(0, span, dtype=np.int64), mult - 1, mult,
+                             ((2**31 - 1) // e - np.arange(0, 50, dtype=np.int64)) * e - 1, ((2**31 - 1) // e - np.arange(0, 50, dtype=np.int64)) * e,
+                             rs.randint(0, 2**31 - 1, size=2000).astype(np.int64)])
+        ns = ns[(ns >= 0) & (ns < 2**31)]
+        q = [(int(n) * magic) >> (31 + s) for n in ns]
+        assert q == [int(n) // e for n in ns], e

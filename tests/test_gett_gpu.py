@@ -130,7 +130,48 @@ def test_bit_exact_against_the_plain_kernel_on_materialised_matrices(gpu, extent
 
 def test_gett_config_errors():
     from gemmkernels import ConfigError
-    with pytest.raises(ConfigError):      # BLOCK_K must divide the first K mode
-        configs.gett_config("aebf", "dfce", "abcd", dict(a=32, b=2, c=2, d=32, e=16, f=4), block_shape=(64, 64, 32))
-    with pytest.raises(ConfigError):      # first M mode not a multiple of 32
-        configs.gett_config("aebf", "dfce", "abcd", dict(a=16, b=4, c=2, d=32, e=32, f=2), block_shape=(64, 64, 32))
+    with pytest.raises(ConfigError):      # BLOCK_K = 32 neither divides the first K mode (24) nor is a multiple of it
+        configs.gett_config("aebf", "dfce", "abcd", dict(a=32, b=2, c=2, d=32, e=24, f=4), block_shape=(64, 64, 32))
+    with pytest.raises(ConfigError):      # the tile would cover e (16) whole and 2 of f, but f = 3 is not a multiple of 2
+        configs.gett_config("aebf", "dfce", "abcd", dict(a=32, b=2, c=2, d=32, e=16, f=3), block_shape=(64, 64, 32))
+    with pytest.raises(ConfigError):      # A has only 4 consecutive elements (a = 4, the next M mode b is not adjacent to it)
+        configs.gett_config("aebf", "dfce", "abcd", dict(a=4, b=16, c=2, d=32, e=32, f=2), block_shape=(64, 64, 32))
+    with pytest.raises(ConfigError):      # first N mode (d = 2) is not a multiple of 4
+        configs.gett_config("aebf", "dfce", "abcd", dict(a=32, b=2, c=32, d=2, e=32, f=2), block_shape=(64, 64, 32))
+
+
+# modes that the 32-wide fast path does not cover: (extents, block, what is special)
+GENERAL = [
+    (dict(a=32, b=2, c=2, d=32, e=16, f=4), (64, 64, 32), "a K tile = the whole first K mode (16) x 2 of the second"),
+    (dict(a=32, b=4, c=4, d=32, e=16, f=4), (128, 128, 64), "a K tile = the whole first K mode x the whole second"),
+    (dict(a=16, b=4, c=2, d=32, e=32, f=2), (64, 64, 32), "first M mode 16: rows of a 32-row block in two runs of D"),
+    (dict(a=8, b=16, c=8, d=8, e=64, f=1), (128, 64, 32), "first M and N modes 8"),
+    (dict(a=24, b=16, c=4, d=48, e=8, f=8), (128, 64, 64), "extents that are not powers of two; K tile = 8 x 8"),
+]
+
+
+@pytest.mark.parametrize("ext,block,what", GENERAL, ids=[g[2] for g in GENERAL])
+def test_general_mode_extents_are_exact_against_einsum(gpu, ext, block, what):
+    """Contractions whose modes do not come in multiples of 32 and whose K tile spans several K modes: every lane
+    walks the mode tables for its own rows and columns of D, the K walker steps through the second K mode."""
+    if block not in [(64, 64, 32), (128, 128, 64), (256, 256, 64)]:
+        # only those tiles are compiled with contraction addressing: take the largest that divides
+        M, N = ext["a"] * ext["b"], ext["c"] * ext["d"]
+        block = (128, 128, 64) if (M % 128 == 0 and N % 128 == 0 and (ext["e"] * ext["f"]) % 64 == 0) else (64, 64, 32)
+    conf, gmap = configs.gett_config("aebf", "dfce", "abcd", ext, block_shape=block)
+    print("case", what, ext, block, gk.kernel_name(conf, Kernel.matmul_pipelined), flush=True)
+    A = small_ints(tuple(ext[ch] for ch in "aebf"), 11)
+    B = small_ints(tuple(ext[ch] for ch in "dfce"), 12)
+    D = run_gett(conf, A, B, tuple(ext[ch] for ch in "abcd"))
+    want = np.einsum("aebf,dfce->abcd", A.astype(np.float64), B.astype(np.float64))
+    assert np.array_equal(D.astype(np.float64), want)
+    # with C read through the same index map, and D hooks: D = 2 * (A*B + C)
+    from gemmkernels import Transform, Float32
+    conf_c, _ = configs.gett_config("aebf", "dfce", "abcd", ext, block_shape=block, zero_c=False)
+    C = np.asfortranarray(np.random.RandomState(13).randint(-9, 10, size=D.shape).astype(np.float32))
+    d = gk.colmajor_empty(D.shape, torch.float32)
+    d.fill_(float("nan"))
+    gk.matmul(conf_c, gk.colmajor(A), gk.colmajor(B), gk.colmajor(C), d, kernel=Kernel.matmul_pipelined,
+              transform_shared_to_global_d=Transform.Elementwise(lambda x: x * 2.0))
+    torch.cuda.synchronize()
+    assert np.array_equal(gk.to_numpy(d).astype(np.float64), 2.0 * (want + C))

@@ -205,3 +205,20 @@ def test_get_config_keywords_are_the_reference_keywords():
                "mem_cd_warp", "mem_a_thread", "mem_b_thread", "mem_cd_thread", "cta_swizzle"):
         assert re.search(r"get\(params, :%s," % kw, CODE), kw
     assert re.search(r"function get_config\(; gemm_shape, operator, global_a_layout, global_c_layout, kwargs\.\.\.\)", CODE)
+
+
+def test_tile_tables_match_the_python_tables():
+    """The tables from which both host layers draw their default block shapes and wave grids."""
+    from gemmkernels import config as cfg
+
+    def jl_table(name):
+        m = re.search(r"const " + name + r" = \[(.*?)\]\n", SRC, flags=re.S)
+        assert m, name
+        return [((int(a), int(b), int(c)), (int(d), int(e)))
+                for a, b, c, d, e in re.findall(r"\(\((\d+), (\d+), (\d+)\), \((\d+), (\d+)\)\)", m.group(1))]
+
+    assert jl_table("MFMA_TILES") == [(t, w) for t, w in cfg._MFMA_TILES]
+    assert jl_table("COMPLEX_PAIR_TILES") == cfg._COMPLEX_PAIR_TILES == cfg._PLANAR_TILES
+    assert jl_table("COMPLEX_TN_TILES") == cfg._COMPLEX_TN_TILES
+    assert jl_table("DUAL_TN_TILES") == cfg._DUAL_TN_TILES
+    assert jl_table("FPU_TILES") == cfg._FPU_TILES
