@@ -258,12 +258,11 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
   args->nbm = (args->M + c->block_shape.M - 1) / c->block_shape.M;
   args->nbn = (args->N + c->block_shape.N - 1) / c->block_shape.N;
   if (c->op.kind == GK_OP_MFMA_COMPLEX || c->op.kind == GK_OP_MFMA_DUAL) {
-    // interleaved complex operands seen as real matrices: M and K double, and so does every
-    // leading dimension (counted in real elements)
-    // (unless both A and B are contiguous along k, the real views of A and B meet in one real product of 2M x 2N x K)
-    const bool pair = !is_split_layout(c->global_a_layout.kind) && !(is_row_major(c->global_a_layout.kind) && !is_row_major(c->global_b_layout.kind));
+    // complex operands seen as real matrices: the real views of A (both parts of every row) and of B (both parts of
+    // every column) meet in one real product of 2M x 2N x K; the leading dimensions of interleaved matrices count
+    // real elements
     args->M *= 2;
-    if (pair || is_split_layout(c->global_a_layout.kind)) args->N *= 2; else args->K *= 2;
+    args->N *= 2;
     if (is_split_layout(c->global_a_layout.kind)) {
       // planar operands: a matrix is the real array (rows, cols, 2) in column-major order, so the
       // imaginary plane starts ld * cols elements after the real one

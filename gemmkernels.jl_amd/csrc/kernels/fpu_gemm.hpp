@@ -118,7 +118,9 @@ struct FpuGemmConfig {
   static constexpr int THREADS = WAVES_M * WAVES_N * kWaveSize;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   static constexpr int TM = WTM / 8, TN = WTN / 8;          // outputs per lane
-  static constexpr int CM = TM / 4, CN = TN / 4;            // 4-wide chunks per lane
+  // a lane's outputs come in chunks of consecutive rows (columns), 4 wide, or 2 wide for the smallest wave tile
+  static constexpr int CWM = TM < 4 ? TM : 4, CWN = TN < 4 ? TN : 4;
+  static constexpr int CM = TM / CWM, CN = TN / CWN;        // chunks per lane
   static constexpr int PAD = 4;
   static constexpr int LDA_S = BM + PAD, LDB_S = BN + PAD;  // LDS row pitch (elements of TACC), rows are k
   static constexpr int LDS_BYTES = (BK * LDA_S + BK * LDB_S) * (int)sizeof(TACC);
@@ -130,7 +132,7 @@ struct FpuGemmConfig {
   // -- four tiles without hooks, two with; the bounds-checked and the 64-bit kernels stay with one (their
   // per-element loads and wide registers make deeper buffers expensive to compile and to hold)
   static constexpr int DEPTH = (CHECKED_ || sizeof(TIN_) > 4) ? 1 : (FUSED_ ? 2 : 4);
-  static_assert(TM % 4 == 0 && TN % 4 == 0, "a lane owns whole 4-wide chunks");
+  static_assert(TM >= 2 && TN >= 2 && TM % CWM == 0 && TN % CWN == 0, "a lane owns whole chunks of 2 or 4 outputs");
   static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "tile loads divide evenly over the threads");
   static_assert(!TROPICAL || std::is_same<TACC, float>::value, "the max-plus product is compiled for fp32");
 };
@@ -209,10 +211,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
   const bool xf_a = Cfg::FUSED && (args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0);
   const bool xf_b = Cfg::FUSED && (args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0);
 
-  // accumulators: acc[i][j] is row wm*WTM + (i/4)*32 + 4*ly + i%4, column wn*WTN + (j/4)*32 + 4*lx + j%4
+  // accumulators: acc[i][j] is row wm*WTM + (i/CW)*8*CW + CW*ly + i%CW (CW = 4, or 2), columns likewise with lx
+  constexpr int CWM = Cfg::CWM, CWN = Cfg::CWN;
+  typedef TACC accm __attribute__((ext_vector_type(CWM)));
+  typedef TACC accn __attribute__((ext_vector_type(CWN)));
   TACC acc[TM][TN];
-  auto row_of = [&](int i) { return m0 + wm * Cfg::WTM + (i / 4) * 32 + 4 * ly + (i % 4); };
-  auto col_of = [&](int j) { return n0 + wn * Cfg::WTN + (j / 4) * 32 + 4 * lx + (j % 4); };
+  auto row_of = [&](int i) { return m0 + wm * Cfg::WTM + (i / CWM) * 8 * CWM + CWM * ly + (i % CWM); };
+  auto col_of = [&](int j) { return n0 + wn * Cfg::WTN + (j / CWN) * 8 * CWN + CWN * lx + (j % CWN); };
 #pragma unroll
   for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -326,20 +331,22 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
     stash(slot_c);
     __syncthreads();
     if (kt + DEPTH < KT) fetch((kt + DEPTH) * BK, slot_c);      // its buffer is free again
-    const TACC* ap = As + wm * Cfg::WTM + 4 * ly;
-    const TACC* bp = Bs + wn * Cfg::WTN + 4 * lx;
+    const TACC* ap = As + wm * Cfg::WTM + CWM * ly;
+    const TACC* bp = Bs + wn * Cfg::WTN + CWN * lx;
 #pragma unroll 4
     for (int k = 0; k < BK; ++k) {
       TACC a[TM], b[TN];
 #pragma unroll
       for (int c = 0; c < Cfg::CM; ++c) {
-        const acc4 v = *(const acc4*)&ap[k * Cfg::LDA_S + c * 32];
-        a[4 * c] = v[0]; a[4 * c + 1] = v[1]; a[4 * c + 2] = v[2]; a[4 * c + 3] = v[3];
+        const accm v = *(const accm*)&ap[k * Cfg::LDA_S + c * 8 * CWM];
+#pragma unroll
+        for (int e = 0; e < CWM; ++e) a[CWM * c + e] = v[e];
       }
 #pragma unroll
       for (int c = 0; c < Cfg::CN; ++c) {
-        const acc4 v = *(const acc4*)&bp[k * Cfg::LDB_S + c * 32];
-        b[4 * c] = v[0]; b[4 * c + 1] = v[1]; b[4 * c + 2] = v[2]; b[4 * c + 3] = v[3];
+        const accn v = *(const accn*)&bp[k * Cfg::LDB_S + c * 8 * CWN];
+#pragma unroll
+        for (int e = 0; e < CWN; ++e) b[CWN * c + e] = v[e];
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j)
@@ -356,7 +363,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
     }
   });
 
-  // epilogue: transform, bias, transform, store (4 consecutive rows per vector store); the bias of
+  // epilogue: transform, bias, transform, store (a chunk of consecutive rows per vector store); the bias of
   // Epilogue.Bias is fp32 (reference src/epilogue.jl:44-52) and only offered with fp32 accumulators
   TACC* D = (TACC*)args.d;
   if constexpr (Cfg::FUSED) {
@@ -387,13 +394,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
     const int cc = col_of(j);
 #pragma unroll
     for (int c = 0; c < Cfg::CM; ++c) {
-      const int r = row_of(4 * c);
+      const int r = row_of(CWM * c);
       if (!Cfg::CHECKED) {
-        *(acc4*)&D[r + (long long)cc * args.ldd] = (acc4){acc[4 * c][j], acc[4 * c + 1][j], acc[4 * c + 2][j], acc[4 * c + 3][j]};
+        accm v;
+#pragma unroll
+        for (int e = 0; e < CWM; ++e) v[e] = acc[CWM * c + e][j];
+        *(accm*)&D[r + (long long)cc * args.ldd] = v;
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (r + e < args.M && cc < args.N) D[r + e + (long long)cc * args.ldd] = acc[4 * c + e][j];
+        for (int e = 0; e < CWM; ++e)
+          if (r + e < args.M && cc < args.N) D[r + e + (long long)cc * args.ldd] = acc[CWM * c + e][j];
       }
     }
   }

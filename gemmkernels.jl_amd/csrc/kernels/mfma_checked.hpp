@@ -18,8 +18,8 @@ struct MfmaCheckedConfig {
   typedef T_ T;
   static constexpr int NWAVES = WAVES_M * WAVES_N, THREADS = NWAVES * kWaveSize;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, FM = WTM / 32, FN = WTN / 32, KSTEPS = BK / 16;
-  typedef OperandGeom<BM, BK, OPK_KMAJOR, false> GA;     // both LDS tiles are K-major whatever the memory order
-  typedef OperandGeom<BN, BK, OPK_KMAJOR, false> GB;
+  typedef OperandGeom<BM, BK, OPK_KMAJOR> GA;     // both LDS tiles are K-major whatever the memory order
+  typedef OperandGeom<BN, BK, OPK_KMAJOR> GB;
   static constexpr int LDS_BYTES = GA::BYTES + GB::BYTES;
   static constexpr int A_PER_THREAD = BM * BK / THREADS, B_PER_THREAD = BN * BK / THREADS;
   static_assert((BM * BK) % THREADS == 0 && (BN * BK) % THREADS == 0, "tile loads divide evenly over the threads");
@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
       const T x = vals[i];
       constexpr int CPR = BK / 8;
       const int c = k >> 3;
-      const int swz = (r / OperandGeom<64, BK, OPK_KMAJOR, false>::RP256) & (CPR - 1);
+      const int swz = (r / OperandGeom<64, BK, OPK_KMAJOR>::RP256) & (CPR - 1);
       *(T*)(dst + 16 * (r * CPR + (c ^ swz)) + (k & 7) * 2) = x;
     }
   };
@@ -136,8 +136,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_checked_kernel(const G
   constexpr int DEPTH = 4;
   T ga[DEPTH][Cfg::A_PER_THREAD], gb[DEPTH][Cfg::B_PER_THREAD];
 
-  typedef FragReader<BM, BK, OPK_KMAJOR, false, FM> RA;
-  typedef FragReader<BN, BK, OPK_KMAJOR, false, FN> RB;
+  typedef FragReader<BM, BK, OPK_KMAJOR, FM> RA;
+  typedef FragReader<BN, BK, OPK_KMAJOR, FN> RB;
   RA ra;
   RB rb;
   ra.init(wm * Cfg::WTM, lane);

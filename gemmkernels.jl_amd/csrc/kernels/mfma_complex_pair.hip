@@ -4,36 +4,33 @@
 //
 // An interleaved Complex{Float16} matrix that is contiguous along m (A of an 'N' product, B of a 'T' one) IS a
 // real FP16 matrix with twice the rows, row 2m the real and row 2m+1 the imaginary parts: the real kernel
-// stages and reads it like any other matrix.  The 2M x 2N real product of the two views holds
-// re*re, re*im, im*re and im*im of every element of D; the epilogue combines them (FIX_PAIR in mfma_gemm.hpp).
-// Nothing happens to a fragment on its way to the matrix cores, which is what the older instances of
-// mfma_complex.hip pay for (a byte permute and a sign flip per register of every A fragment, and four
-// 4-byte LDS reads where these issue one transposing read).  A matrix that is contiguous along k is staged
-// as it lies (OPK_KPAIR) and each of the two lanes of a complex row keeps its half of the words it reads.
+// stages and reads it like any other matrix.  One that is contiguous along k is staged as it lies (OPK_KSPLIT) and
+// a lane makes a fragment of real parts and a fragment of imaginary parts out of the 32 bytes it reads.  Either way
+// the 2M x 2N real product of the two views holds re*re, re*im, im*re and im*im of every element of D, and they are
+// combined once, before the epilogue (FIX_PAIR in mfma_gemm.hpp): nothing else happens on the way to the matrix
+// cores, and the K loop is the one of the real kernel on a 256 x 256 x 64 real tile.
 // Tile shapes below are in complex elements; the real tile has twice the rows and columns.
 #include "mfma_gemm.hpp"
 #include "registry.hpp"
 
 namespace gk {
 
-// 'T','N' products (both operands contiguous along k) stay with the instances of mfma_complex.hip: staged as
-// OPK_KPAIR both operands would be read twice from LDS, which is what bounds this kernel.
 int family_complex_pair(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode, InstanceInfo* info,
                         hipError_t* err) {
-  if (key.dtype != DT_F16 || (key.fused != 0 && key.fused != 3) || key.variant > 1 || (key.a_kmajor && key.b_kmajor)) return 0;
+  if (key.dtype != DT_F16 || (key.fused != 0 && key.fused != 3) || key.variant > 1) return 0;
   // every instance carries the hooks of C and D and the bias (FUSE level 3: they cost nothing when absent)
 #define GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, akm_, bkm_, dual_, NAME)                                                     \
   if (key.BM == bm_ && key.BN == bn_ && key.BK == bk_ && key.waves_m == wm_ && key.waves_n == wn_ &&                      \
       key.a_kmajor == akm_ && key.b_kmajor == bkm_ && key.variant == dual_) {                                             \
-    typedef MfmaGemmConfig<2 * bm_, 2 * bn_, bk_, wm_, wn_, st_, (akm_ ? OPK_KPAIR : OPK_MMAJOR),                          \
-                           (bkm_ ? OPK_KPAIR : OPK_MMAJOR), _Float16, 3, false, (dual_ ? FIX_PAIR_DUAL : FIX_PAIR), false, 16> Cfg; \
+    typedef MfmaGemmConfig<2 * bm_, 2 * bn_, bk_, wm_, wn_, st_, (akm_ ? OPK_KSPLIT : OPK_MMAJOR),                         \
+                           (bkm_ ? OPK_KSPLIT : OPK_MMAJOR), _Float16, 3, false, (dual_ ? FIX_PAIR_DUAL : FIX_PAIR), false, 16> Cfg; \
     return run_instance<Cfg>(mfma_gemm_kernel<Cfg>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
   }
-  // the wave grid puts the operand that is read twice (OPK_KPAIR) on the side with fewer fragments per wave
 #define GK_PAIR_T(bm_, bn_, bk_, wm_, wn_, st_, dual_, TAG)                                                         \
   GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, 0, 1, dual_, "mfma_" TAG "_nn_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, 0, 0, dual_, "mfma_" TAG "_nt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
-  GK_PAIR(bm_, bn_, bk_, wn_, wm_, st_, 1, 0, dual_, "mfma_" TAG "_tt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wn_ "x" #wm_)
+  GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, 1, 1, dual_, "mfma_" TAG "_tn_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
+  GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, 1, 0, dual_, "mfma_" TAG "_tt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)
   GK_PAIR_T(128, 128, 64, 2, 4, 2, 0, "complex_pair")
   GK_PAIR_T(64, 64, 64, 2, 2, 2, 0, "complex_pair")
   GK_PAIR_T(64, 64, 32, 2, 2, 4, 0, "complex_pair")

@@ -28,32 +28,33 @@ namespace gk {
 // dimension (m or n), BK the number of 16-bit k-values per K step.
 //   OPK_KMAJOR: LDS row = tile row, 16-byte chunk c = k / 8            (memory contiguous along k)
 //   OPK_MMAJOR: LDS row = k,        16-byte chunk c = row / 8          (memory contiguous along m / n)
-//   OPK_KPAIR : interleaved complex data contiguous along k, for the FIX_PAIR products: LDS row = complex
-//               row index (R/2 of them), 16-byte chunk c = complex k / 4; the two MFMA rows of a complex row
-//               read the same 32 bytes (8 complex k) and keep the real or the imaginary halves
-// EXPAND marks the A operand of a complex (or dual-number) product: one complex row feeds two MFMA
-// rows, so the tile holds R/2 complex rows.
+//   OPK_KSPLIT: interleaved complex data contiguous along k, for the FIX_PAIR products: LDS row = complex row index
+//               (R/2 of them), 16-byte chunk c = complex k / 4.  A lane reads the 32 bytes (8 complex k) of its
+//               complex row once and makes two fragments of them, the real parts for fragment f and the imaginary
+//               parts for fragment f + F/2
 // ----------------------------------------------------------------------------------------------
-enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_KPAIR = 3 };
+enum : int { OPK_KMAJOR = 0, OPK_MMAJOR = 1, OPK_KSPLIT = 4 };
+constexpr bool opk_complex_k(int kind) { return kind == OPK_KSPLIT; }
 // FIX_PAIR / FIX_PAIR_DUAL: complex (dual-number) product on interleaved matrices as ONE real product of the
-// matrices seen as real ones.  An interleaved matrix whose contiguous index is m (or n) is a real matrix with
-// twice the rows, row 2m the real and row 2m+1 the imaginary part, and the K loop of the real kernel runs on it
-// unchanged (K counts complex k); one whose contiguous index is k is read as OPK_KPAIR.  The 2M x 2N real
-// product holds the four real products re*re, re*im, im*re, im*im of every complex element of D in the lanes
-// 2i, 2i+1 (the two parts of a row of A) and the accumulator values 2j, 2j+1 (the two parts of a column of B);
-// they are combined once, before the epilogue (pair_combine).
+// matrices seen as real ones (2M x 2N x K: it holds re*re, re*im, im*re, im*im of every element of D, the four
+// products of WMMAComplexOp.mma, reference src/operator.jl:307-311; dual numbers :366-369 use three of them).
+// An interleaved matrix whose contiguous index is m (or n) is a real matrix with twice the rows, row 2m the real and
+// row 2m+1 the imaginary parts, and the K loop of the real kernel runs on it unchanged (K counts complex k): the two
+// parts of a row of A then sit in the lanes 2i, 2i+1, those of a column of B in the accumulator values 2j, 2j+1.
+// One whose contiguous index is k is read as OPK_KSPLIT: the two parts sit in the row (column) blocks f and f + F/2.
+// The four products are combined once, before the epilogue.
 // FIX_PLANAR: the same for planar (split re / im) matrices, whose planes are plain real matrices: the real view of A
 // is [A_re; A_im] stacked along m and that of B [B_re, B_im] side by side along n.  The tile rows (columns) are
 // dealt out so that every wave holds both parts of its complex rows (columns): the upper half of the row blocks of
 // a wave tile comes from A_re, the lower half from the same rows of A_im, the left half of the column blocks from
 // B_re and the right half from B_im.  The four real products of an element of D then lie in four accumulator
 // blocks of one lane and are combined without any exchange.
-enum : int { FIX_NONE = 0, FIX_COMPLEX = 1, FIX_DUAL = 2, FIX_PLANAR = 3, FIX_PAIR = 4, FIX_PAIR_DUAL = 5 };
+enum : int { FIX_NONE = 0, FIX_PLANAR = 3, FIX_PAIR = 4, FIX_PAIR_DUAL = 5 };
 
-template <int R, int BK, int KIND, bool EXPAND>
+template <int R, int BK, int KIND>
 struct OperandGeom {
-  static constexpr int LDS_ROWS = KIND == OPK_KMAJOR ? (EXPAND ? R / 2 : R) : (KIND == OPK_KPAIR ? R / 2 : BK);
-  static constexpr int ROW_BYTES = KIND == OPK_KMAJOR ? BK * 2 : (KIND == OPK_KPAIR ? BK * 4 : R * 2);
+  static constexpr int LDS_ROWS = KIND == OPK_KMAJOR ? R : (opk_complex_k(KIND) ? R / 2 : BK);
+  static constexpr int ROW_BYTES = KIND == OPK_KMAJOR ? BK * 2 : (opk_complex_k(KIND) ? BK * 4 : R * 2);
   static constexpr int CPR = ROW_BYTES / 16;                   // 16-byte chunks per LDS row
   static constexpr int BYTES = LDS_ROWS * ROW_BYTES;
   static constexpr int NDMA = BYTES / 1024;                    // wave-wide 16 B/lane DMA instructions per tile
@@ -61,9 +62,14 @@ struct OperandGeom {
   // K-major: XOR the chunk index with the row (per 256 B) so that 32 consecutive rows at one chunk
   // index spread evenly over the 16 chunk slots of the 64 banks.
   __device__ static __forceinline__ int swz_k(int row) { return (row / RP256) & (CPR - 1); }
-  // OPK_KPAIR: the same with pairs of chunks (a lane reads two neighbouring chunks from one address), so that
-  // the 8 complex rows of a 16-lane group spread over the 8 32-byte slots of the bank period
-  __device__ static __forceinline__ int swz_kp(int row) { return ((row / RP256) & (CPR / 2 - 1)) << 1; }
+  // OPK_KSPLIT: the 16 lanes of a read take one 16-byte chunk each from 16 consecutive complex rows, first the
+  // chunk 2g of every row, then the chunk 2g + 1.  The XOR below sends the 16 rows to the 16 chunk slots of the
+  // bank period for either chunk: eight rows in a row differ in the upper bits, a row and the one eight rows
+  // further trade the two chunks of a pair.
+  __device__ static __forceinline__ int swz_kp(int row) {
+    const int q = row / RP256;
+    return ((q & (CPR / 2 - 1)) << 1) | ((q / (CPR / 2)) & 1);
+  }
   // M-major: XOR the 64-byte group index with k so that 4 consecutive k rows at one group land in
   // 4 different 64-byte slots of the 256-byte bank period.
   // Rows of 384 bytes (192 elements): consecutive k rows are already 128 bytes apart in the bank period, so
@@ -79,7 +85,6 @@ struct OperandGeom {
   static_assert(!ROW_384 || GROUPS % 2 == 0, "the group XOR of 384-byte rows pairs groups");
   static_assert(KIND != OPK_MMAJOR || CPR >= 4, "M-major tiles need at least 32 rows");
   static_assert(BYTES % 1024 == 0, "tile must be a whole number of DMA instructions");
-  static_assert(!EXPAND || KIND == OPK_KMAJOR, "an operand that is expanded in registers is K-major");
 };
 
 // Where lane `lane` of DMA instruction q reads: LDS row `row` of the tile and the first of its 8
@@ -91,7 +96,7 @@ __device__ __forceinline__ void dma_lane_coords(int q, int lane, int& row, int& 
   row = p / G::CPR;
   const int cs = p % G::CPR;
   if (KIND == OPK_KMAJOR) col = (cs ^ G::swz_k(row)) * 8;
-  else if (KIND == OPK_KPAIR) col = (cs ^ G::swz_kp(row)) * 8;
+  else if (opk_complex_k(KIND)) col = (cs ^ G::swz_kp(row)) * 8;
   else col = (((cs >> 2) ^ G::swz_m(row)) * 4 + ((cs & 3) ^ (((row >> 3) & 1) << 1))) * 8;
 }
 
@@ -171,9 +176,9 @@ __device__ __forceinline__ void wait_lgkmcnt() {
 // apart), which serialises the pipeline.  Their completion is therefore tracked by hand:
 // read() only issues, the registers it names (Raw) must not be looked at before
 // wait_lgkmcnt<N>() + pin_raw(), and finish() turns them into the MFMA operand afterwards.
-template <int R, int BK, int KIND, bool EXPAND, int F, int MI = 32>
+template <int R, int BK, int KIND, int F, int MI = 32>
 struct FragReader {
-  typedef OperandGeom<R, BK, KIND, EXPAND> G;
+  typedef OperandGeom<R, BK, KIND> G;
   // MI = 32: fragments of 32 rows x 16 k (v_mfma_f32_32x32x16); MI = 16: 16 rows x 32 k (v_mfma_f32_16x16x32),
   // lane l holds the 8 k-values 8*(l/MI)..+7 of row l%MI in both cases
   static constexpr int KSTEP_K = MI == 32 ? 16 : 32;
@@ -181,12 +186,13 @@ struct FragReader {
   // M-major, 16-row fragments: fragments 2j and 2j+1 are the two 32-byte halves of one 64-byte group, so one
   // address serves both (the odd one is the even one with bit 5 flipped)
   static constexpr bool PAIRED = KIND == OPK_MMAJOR && MI == 16 && F % 2 == 0;
-  static constexpr int NBASE = (KIND == OPK_KMAJOR || KIND == OPK_KPAIR) ? KSTEPS : (PAIRED ? F / 2 : F);
-  static constexpr int OPS = KIND == OPK_KMAJOR ? 1 : 2;   // LDS instructions per fragment
-  static constexpr int FRAG_ROWS = (EXPAND || KIND == OPK_KPAIR) ? MI / 2 : MI;       // tile rows (complex rows when EXPAND / OPK_KPAIR) per fragment
+  static constexpr int NBASE = KIND == OPK_KMAJOR ? KSTEPS : (opk_complex_k(KIND) ? 2 * KSTEPS : (PAIRED ? F / 2 : F));
+  static constexpr int OPS = KIND == OPK_KMAJOR ? 1 : 2;   // LDS instructions per fragment that is read
+  static constexpr int NREAD = KIND == OPK_KSPLIT ? F / 2 : F;   // fragments that are read (OPK_KSPLIT: each read serves two)
+  static constexpr int FRAG_ROWS = MI;       // tile rows (complex rows for OPK_KSPLIT) per fragment
   struct Raw {
-    int4v q;          // OPK_KMAJOR; OPK_KPAIR: complex k 0..3 of the lane's eight
-    int4v q1;         // OPK_KPAIR: complex k 4..7
+    int4v q;          // OPK_KMAJOR; OPK_KSPLIT: complex k 0..3 of the lane's eight
+    int4v q1;         // OPK_KSPLIT: complex k 4..7
     int2v lo, hi;     // OPK_MMAJOR
   };
   unsigned cur[NBASE];                          // lane-dependent byte addresses inside the tile of the current stage
@@ -195,20 +201,22 @@ struct FragReader {
   // row0: first MFMA row of the wave inside the block tile (multiple of 32)
   __device__ __forceinline__ void init(int row0, int lane) {
     if (KIND == OPK_KMAJOR) {
-      const int row = EXPAND ? ((row0 + (lane % MI)) >> 1) : (row0 + (lane % MI));
+      const int row = row0 + (lane % MI);
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
         const int c = ks * (KSTEP_K / 8) + (lane / MI);
         cur[ks < NBASE ? ks : 0] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_k(row)));
       }
-    } else if (KIND == OPK_KPAIR) {
-      // MFMA row r of the block tile is part r & 1 of complex row r >> 1; the lane's eight k-slots of a k-step
-      // are the complex k 8*(lane/MI) .. +7 of it: chunks 2*(lane/MI) and the next one (the swizzle is even)
-      const int row = (row0 + (lane % MI)) >> 1;
+    } else if (opk_complex_k(KIND)) {
+      // the wave's rows are complex rows row0 / 2 ..., 16 per fragment, for both parts.  The lane's eight k-slots of a
+      // k-step are the complex k 8*(lane/MI) .. +7 of its row: chunks 2*(lane/MI) and the next one, each with an
+      // address of its own (the swizzle may have traded their places)
+      const int row = (row0 >> 1) + (lane % MI);
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
         const int c = ks * (KSTEP_K / 4) + 2 * (lane / MI);
-        cur[ks < NBASE ? ks : 0] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_kp(row)));
+        cur[2 * ks] = 16u * (unsigned)(row * G::CPR + (c ^ G::swz_kp(row)));
+        cur[2 * ks + 1] = 16u * (unsigned)(row * G::CPR + ((c + 1) ^ G::swz_kp(row)));
       }
     } else {
       const int i = lane & 15;
@@ -239,10 +247,10 @@ struct FragReader {
     if constexpr (SYNC && KIND == OPK_KMAJOR) {
       asm volatile("ds_read_b128 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
       return;
-    } else if constexpr (SYNC && KIND == OPK_KPAIR) {
-      asm volatile("ds_read_b128 %0, %2 offset:%3\n\tds_read_b128 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
+    } else if constexpr (SYNC && opk_complex_k(KIND)) {
+      asm volatile("ds_read_b128 %0, %2 offset:%4\n\tds_read_b128 %1, %3 offset:%4\n\ts_waitcnt lgkmcnt(0)"
                    : "=&v"(r.q), "=&v"(r.q1)
-                   : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES), "n"(FI * FRAG_ROWS * G::ROW_BYTES + 16) : "memory");
+                   : "v"(cur[2 * KS]), "v"(cur[2 * KS + 1]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
       return;
     } else if constexpr (SYNC && KIND == OPK_MMAJOR) {
       asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
@@ -252,9 +260,9 @@ struct FragReader {
     }
     if (KIND == OPK_KMAJOR) {
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
-    } else if (KIND == OPK_KPAIR) {
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q1) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES + 16) : "memory");
+    } else if (opk_complex_k(KIND)) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[2 * KS]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q1) : "v"(cur[2 * KS + 1]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
     } else {
       asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.lo) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K) * G::ROW_BYTES) : "memory");
       asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.hi) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K + 4) * G::ROW_BYTES) : "memory");
@@ -267,15 +275,16 @@ struct FragReader {
   }
   __device__ static __forceinline__ void pin_raw(Raw& r) {
     if (KIND == OPK_KMAJOR) pin(r.q);
-    else if (KIND == OPK_KPAIR) { pin(r.q); pin(r.q1); }
+    else if (opk_complex_k(KIND)) { pin(r.q); pin(r.q1); }
     else { pin(r.lo); pin(r.hi); }
   }
-  __device__ static __forceinline__ int4v finish(const Raw& r, [[maybe_unused]] int lane) {
+  // imag: OPK_KSPLIT, the fragment of imaginary parts is asked for
+  __device__ static __forceinline__ int4v finish(const Raw& r, [[maybe_unused]] int lane, [[maybe_unused]] bool imag = false) {
     if (KIND == OPK_KMAJOR) return r.q;
     int4v v;
-    if (KIND == OPK_KPAIR) {
-      // the lane's part of its eight complex k: the low (real) or the high (imaginary) halves of the eight words
-      const unsigned sel = (lane & 1) ? 0x07060302u : 0x05040100u;
+    if (opk_complex_k(KIND)) {
+      // one part of the lane's eight complex k: the low (real) or the high (imaginary) halves of the eight words
+      const unsigned sel = imag ? 0x07060302u : 0x05040100u;
       v[0] = (int)__builtin_amdgcn_perm((unsigned)r.q[1], (unsigned)r.q[0], sel);
       v[1] = (int)__builtin_amdgcn_perm((unsigned)r.q[3], (unsigned)r.q[2], sel);
       v[2] = (int)__builtin_amdgcn_perm((unsigned)r.q1[1], (unsigned)r.q1[0], sel);
@@ -291,31 +300,11 @@ struct FragReader {
     else { r.lo[0] = v[0]; r.lo[1] = v[1]; r.hi[0] = v[2]; r.hi[1] = v[3]; }
   }
   static_assert(KIND != OPK_MMAJOR || (KSTEPS * KSTEP_K + 4) * G::ROW_BYTES < 65536, "LDS immediate offset is 16 bits");
-  static_assert((KIND != OPK_KMAJOR && KIND != OPK_KPAIR) || F * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
-  static_assert(KIND != OPK_KPAIR || (MI == 16 && (8 % G::RP256) == 0), "complex-pair fragments: 16-row blocks, whose 8 complex rows keep the swizzle of the first");
+  static_assert((KIND != OPK_KMAJOR && !opk_complex_k(KIND)) || NREAD * FRAG_ROWS * G::ROW_BYTES <= 65536, "LDS immediate offset is 16 bits");
+  static_assert(!opk_complex_k(KIND) || (MI == 16 && G::RP256 * G::CPR == 16), "complex fragments: 16-row blocks; the swizzle has a period of 16 rows, so every fragment of a wave shares the addresses of the first");
+  static_assert(KIND != OPK_KSPLIT || F % 2 == 0, "the fragments of real and of imaginary parts come in pairs");
   static_assert(MI == 32 || MI == 16, "fragments of 32 or 16 rows");
-  static_assert(!(EXPAND && KIND == OPK_KMAJOR && MI == 16), "expanded K-major fragments of 8 tile rows break the swizzle invariance of the read offsets");
 };
-
-// The A operand of a complex product D = A * B computed as the real product of the expanded
-// matrix [re -im; im re] with the interleaved B: every register of the fragment holds one complex
-// value (re in the low half, im in the high half); the even MFMA row of a pair needs (re, -im),
-// the odd one (im, re).  Dual numbers (re, du) need (re, 0) and (du, re)
-// (reference src/operator.jl:307-311 and :366-369).
-template <int FIX>
-__device__ __forceinline__ int4v expand_fixup(int4v x, int lane) {
-  if (FIX != FIX_COMPLEX && FIX != FIX_DUAL) return x;
-  const bool odd = (lane & 1) != 0;
-  const unsigned sel = odd ? 0x01000302u : 0x03020100u;                       // swap halves on odd rows
-  const unsigned flip = (FIX == FIX_COMPLEX && !odd) ? 0x80000000u : 0u;       // negate the imaginary half
-  const unsigned keep = (FIX == FIX_DUAL && !odd) ? 0x0000FFFFu : 0xFFFFFFFFu; // drop the dual half
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    unsigned v = __builtin_amdgcn_perm((unsigned)x[i], (unsigned)x[i], sel);
-    x[i] = (int)((v ^ flip) & keep);
-  }
-  return x;
-}
 
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -327,8 +316,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 template <int KS, bool SYNC = false, class RA, class RB, int FM, int FN>
 __device__ __forceinline__ void load_frags(const RA& ra, const RB& rb, typename RA::Raw (&fa)[FM], typename RB::Raw (&fb)[FN]) {
-  static_for<0, FM>([&](auto fi) { ra.template read<decltype(fi)::value, KS, SYNC>(fa[decltype(fi)::value]); });
-  static_for<0, FN>([&](auto fj) { rb.template read<decltype(fj)::value, KS, SYNC>(fb[decltype(fj)::value]); });
+  static_for<0, RA::NREAD>([&](auto fi) { ra.template read<decltype(fi)::value, KS, SYNC>(fa[decltype(fi)::value]); });
+  static_for<0, RB::NREAD>([&](auto fj) { rb.template read<decltype(fj)::value, KS, SYNC>(fb[decltype(fj)::value]); });
 }
 
 template <typename T, int MI = 32> struct Mfma;
@@ -419,10 +408,18 @@ struct MfmaGemmConfig {
   static constexpr bool RAGGED_OK = !GETT_ && FIX_ == FIX_NONE;
   static constexpr bool RAGGED_K_OK = RAGGED_OK && !SPLITK_;
   static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
-  static constexpr bool EXPAND_A = (FIX_ == FIX_COMPLEX || FIX_ == FIX_DUAL);   // interleaved complex / dual A: one complex row feeds two MFMA rows
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
   static constexpr bool PAIR = (FIX_ == FIX_PAIR || FIX_ == FIX_PAIR_DUAL);     // complex / dual product as one real product (see FIX_PAIR)
   static constexpr bool COMPLEX = FIX_ != FIX_NONE;                             // C / D hold complex numbers
+  // where the two parts of a complex column of B meet in the accumulators: in neighbouring values of a lane
+  // (COLS_LANE: B seen as a real matrix with twice the columns) or in the column blocks fj and fj + FN / 2
+  // (COLS_FRAG: planar B, or interleaved B contiguous along k read as OPK_KSPLIT)
+  static constexpr bool COLS_FRAG = PLANAR || (PAIR && B_KIND_ == OPK_KSPLIT);
+  static constexpr bool COLS_LANE = PAIR && !COLS_FRAG;
+  // ... and the two parts of a complex row of A: in neighbouring lanes (ROWS_LANE: A seen as a real matrix with twice
+  // the rows) or in the row blocks fi and fi + FM / 2 (ROWS_FRAG: planar A, or interleaved A contiguous along k)
+  static constexpr bool ROWS_FRAG = PLANAR || (PAIR && A_KIND_ == OPK_KSPLIT);
+  static constexpr bool ROWS_LANE = PAIR && !ROWS_FRAG;
   static constexpr bool GETT = GETT_;   // operands addressed through tensor-contraction index maps
   // K-split instances: a workgroup handles one slice of K (blockIdx.z); the slices of a tile meet in a
   // workspace and the last to arrive sums them in slice order and stores D (splitk_reduce).  A variant of
@@ -445,8 +442,8 @@ struct MfmaGemmConfig {
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;   // wave tile
   static constexpr int FM = WTM / MI, FN = WTN / MI;             // MI x MI accumulator blocks per wave
   static constexpr int KSTEPS = BK / KSTEP_K;
-  typedef OperandGeom<BM, BK, A_KIND, EXPAND_A> GA;
-  typedef OperandGeom<BN, BK, B_KIND, false> GB;
+  typedef OperandGeom<BM, BK, A_KIND> GA;
+  typedef OperandGeom<BN, BK, B_KIND> GB;
   static constexpr int STAGE_BYTES = GA::BYTES + GB::BYTES;
   static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
   static constexpr int DMA_A = (GA::NDMA + NWAVES - 1) / NWAVES;   // per wave, per tile
@@ -460,11 +457,12 @@ struct MfmaGemmConfig {
   static_assert(FM * FN > 0, "empty wave tile");
   static_assert(!GETT || FIX == FIX_NONE, "contractions are real");
   static_assert(!SPLITK || (!GETT && FIX == FIX_NONE), "K-split instances are plain real GEMMs");
-  static_assert(!PLANAR || (MI_ == 16 && A_KIND_ != OPK_KPAIR && B_KIND_ != OPK_KPAIR), "planar complex: 16-row blocks on plain real planes");
+  static_assert(!PLANAR || (MI_ == 16 && !opk_complex_k(A_KIND_) && !opk_complex_k(B_KIND_)), "planar complex: 16-row blocks on plain real planes");
   static_assert(!COMPLEX || FUSE_ == 0 || FUSE_ == 3, "complex products take hooks on C and D only");
-  static_assert(!PAIR || (MI_ == 16 && (A_KIND_ == OPK_MMAJOR || A_KIND_ == OPK_KPAIR) && (B_KIND_ == OPK_MMAJOR || B_KIND_ == OPK_KPAIR)),
+  static_assert(!PAIR || (MI_ == 16 && A_KIND_ != OPK_KMAJOR && B_KIND_ != OPK_KMAJOR),
                 "complex-pair products: 16-row blocks on the real view of the operands");
-  static_assert(PAIR || (A_KIND_ != OPK_KPAIR && B_KIND_ != OPK_KPAIR), "OPK_KPAIR belongs to the complex-pair products");
+  static_assert(A_KIND_ != OPK_KSPLIT || SPLIT_A, "the real and the imaginary fragments of A are the two halves in which A is consumed");
+  static_assert(PAIR || (!opk_complex_k(A_KIND_) && !opk_complex_k(B_KIND_)), "OPK_KSPLIT belongs to the complex-pair products");
 };
 
 template <class Cfg>
@@ -497,12 +495,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   if constexpr (!Cfg::GETT) {
     // tile origin and K step in 16-bit elements (lda / ldb are in 16-bit elements as well; an
     // interleaved complex matrix counts two per complex number)
-    const int m0g = (Cfg::EXPAND_A || Cfg::PLANAR) ? m0 / 2 : m0;   // first row of the tile in the stored matrix
+    const int m0g = Cfg::PLANAR ? m0 / 2 : m0;   // first row of the tile in the stored matrix
     const int n0g = Cfg::PLANAR ? n0 / 2 : n0;
     const long long a_org = Cfg::A_KIND == OPK_KMAJOR ? (long long)m0g * args.lda
-                          : (Cfg::A_KIND == OPK_KPAIR ? (long long)(m0 / 2) * args.lda : (long long)m0g);
+                          : (opk_complex_k(Cfg::A_KIND) ? (long long)(m0 / 2) * args.lda : (long long)m0g);
     const long long b_org = Cfg::B_KIND == OPK_KMAJOR ? (long long)n0g * args.ldb
-                          : (Cfg::B_KIND == OPK_KPAIR ? (long long)(n0 / 2) * args.ldb : (long long)n0g);
+                          : (opk_complex_k(Cfg::B_KIND) ? (long long)(n0 / 2) * args.ldb : (long long)n0g);
     ga = (const char*)args.a + a_org * 2;
     gb = (const char*)args.b + b_org * 2;
     // planar complex: tile row (column) r belongs to wave row r / WT; the first half of a wave's rows are complex rows
@@ -512,8 +510,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       imag = in >= wt / 2;
       return w * (wt / 2) + (in % (wt / 2));
     };
-    a_step = (Cfg::A_KIND == OPK_KMAJOR ? (long long)BK : (Cfg::A_KIND == OPK_KPAIR ? 2ll * BK : (long long)GA::LDS_ROWS * args.lda)) * 2;
-    b_step = (Cfg::B_KIND == OPK_KMAJOR ? (long long)BK : (Cfg::B_KIND == OPK_KPAIR ? 2ll * BK : (long long)GB::LDS_ROWS * args.ldb)) * 2;
+    a_step = (Cfg::A_KIND == OPK_KMAJOR ? (long long)BK : (opk_complex_k(Cfg::A_KIND) ? 2ll * BK : (long long)GA::LDS_ROWS * args.lda)) * 2;
+    b_step = (Cfg::B_KIND == OPK_KMAJOR ? (long long)BK : (opk_complex_k(Cfg::B_KIND) ? 2ll * BK : (long long)GB::LDS_ROWS * args.ldb)) * 2;
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i) {
       int row, col;
@@ -658,20 +656,21 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   auto vcol = [](int v) { return MI == 32 ? 8 * (v / 4) + (v % 4) : v; };   // column of value v inside a block, from the lane's first
   // complex-pair products: a lane's four values of a block are two complex columns x the two parts of B; C is
   // loaded into, and D stored from, the values 0 and 2 (one per complex column), see pair_combine
-  constexpr int NVO = Cfg::PAIR ? 2 : NV;                     // values per lane and block that C / D see
-  constexpr int CB = Cfg::PAIR ? MI / 2 : MI;                 // columns of C / D per block
-  auto slot = [](int v) { return Cfg::PAIR ? 2 * v : v; };
-  // planar complex: C / D see the left half of the column blocks (the right half holds the products with B_im until
-  // they are combined); row block fi is complex rows of the real plane for fi < FM / 2, of the imaginary plane above
-  constexpr int FNO = Cfg::PLANAR ? FN / 2 : FN;
-  constexpr int FMH = Cfg::PLANAR ? FM / 2 : FM;
+  constexpr int NVO = Cfg::COLS_LANE ? 2 : NV;                // values per lane and block that C / D see
+  constexpr int CB = Cfg::COLS_LANE ? MI / 2 : MI;            // columns of C / D per block
+  auto slot = [](int v) { return Cfg::COLS_LANE ? 2 * v : v; };
+  // COLS_FRAG: C / D see the left half of the column blocks (the right half holds the products with the imaginary
+  // parts of B until they are combined).  Planar complex: row block fi is complex rows of the real plane for
+  // fi < FM / 2, of the imaginary plane above
+  constexpr int FNO = Cfg::COLS_FRAG ? FN / 2 : FN;
+  constexpr int FMH = Cfg::ROWS_FRAG ? FM / 2 : FM;
   AccV acc[FM][FN];
-  const int mrow = Cfg::PLANAR ? (m0 + wm * Cfg::WTM) / 2 + (lane % MI) : m0 + wm * Cfg::WTM + (lane % MI);
-  const int ncol = Cfg::PAIR ? (n0 + wn * Cfg::WTN) / 2 + 2 * (lane / MI)
-                 : (Cfg::PLANAR ? (n0 + wn * Cfg::WTN) / 2 + 4 * (lane / MI) : n0 + wn * Cfg::WTN + 4 * (lane / MI));
+  const int mrow = Cfg::ROWS_FRAG ? (m0 + wm * Cfg::WTM) / 2 + (lane % MI) : m0 + wm * Cfg::WTM + (lane % MI);   // ROWS_FRAG: a complex row
+  const int ncol = Cfg::COLS_LANE ? (n0 + wn * Cfg::WTN) / 2 + 2 * (lane / MI)
+                 : (Cfg::COLS_FRAG ? (n0 + wn * Cfg::WTN) / 2 + 4 * (lane / MI) : n0 + wn * Cfg::WTN + 4 * (lane / MI));
   // complex C / D: row block fi of this lane holds imaginary parts (interleaved: the odd lanes, whatever fi; planar:
   // the lower half of the row blocks)
-  [[maybe_unused]] auto imag_rows = [&](int fi) { return Cfg::PLANAR ? fi >= FMH : (Cfg::COMPLEX && (lane & 1) != 0); };
+  [[maybe_unused]] auto imag_rows = [&](int fi) { return Cfg::ROWS_FRAG ? fi >= FMH : (Cfg::COMPLEX && (lane & 1) != 0); };
   // element offset of the lane's first element of accumulator block (fi, fj) in C / D, and the
   // stride between its consecutive columns.
   // contractions: offset of the lane's row of row block fi (gett_om) and of the first of its four columns of
@@ -708,6 +707,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   auto cd_offset = [&](int fi, int fj, long long ld, [[maybe_unused]] long long plane) -> long long {
     if constexpr (Cfg::PLANAR) {
       return (long long)(mrow + MI * (fi % FMH)) + (long long)(ncol + MI * fj) * ld + (fi >= FMH ? plane : 0ll);
+    } else if constexpr (Cfg::ROWS_FRAG) {
+      // interleaved C / D seen as a real matrix: complex row m is its rows 2m (real part) and 2m + 1
+      return 2ll * (mrow + MI * (fi % FMH)) + (fi >= FMH ? 1 : 0) + (long long)(ncol + CB * fj) * ld;
     } else if constexpr (!Cfg::GETT) {
       return (long long)(mrow + MI * fi) + (long long)(ncol + CB * fj) * ld;
     } else {
@@ -774,11 +776,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     gett_origins();
     // column blocks outermost: with 16-row blocks the two halves of a 128-byte line of C / D belong to
     // neighbouring row blocks, which are then read (and, below, written) right after each other
-    if constexpr (Cfg::PLANAR) {
+    if constexpr (Cfg::COLS_FRAG) {
 #pragma unroll
       for (int fj = FNO; fj < FN; ++fj)
 #pragma unroll
-        for (int fi = 0; fi < FM; ++fi) acc[fi][fj] = AccV{};     // the products with B_im start from zero
+        for (int fi = 0; fi < FM; ++fi) acc[fi][fj] = AccV{};     // the products with the imaginary parts of B start from zero
     }
 #pragma unroll
     for (int fj = 0; fj < FNO; ++fj)
@@ -786,7 +788,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fi = 0; fi < FM; ++fi) {
         const long long off = cd_offset(fi, fj, args.ldc, args.plane_c);
         const long long ns = cd_nstride(args.ldc);
-        if constexpr (Cfg::PAIR) acc[fi][fj] = AccV{};      // the values between the complex columns start from zero
+        if constexpr (Cfg::COLS_LANE) acc[fi][fj] = AccV{};      // the values between the complex columns start from zero
         if (args.c_dtype == DT_F32) {
           const float* cp = (const float*)args.c + off;
 #pragma unroll
@@ -838,8 +840,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const bool fast_b = std::is_same<T, _Float16>::value && args.fast_scale_b != 0;
   const float scale_a = args.scale_a, scale_b = args.scale_b;
 
-  typedef FragReader<BM, BK, Cfg::A_KIND, Cfg::EXPAND_A, FM, MI> RA;
-  typedef FragReader<BN, BK, Cfg::B_KIND, false, FN, MI> RB;
+  typedef FragReader<BM, BK, Cfg::A_KIND, FM, MI> RA;
+  typedef FragReader<BN, BK, Cfg::B_KIND, FN, MI> RB;
   RA ra;
   RB rb;
   ra.init(wm * Cfg::WTM, lane);
@@ -852,7 +854,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // the current set has arrived.
   typename RA::Raw fa[2][FM];
   typename RB::Raw fb[2][FN];
-  constexpr int FRAG_OPS = FM * RA::OPS + FN * RB::OPS;
+  constexpr int FRAG_OPS = RA::NREAD * RA::OPS + RB::NREAD * RB::OPS;
 
   // The whole K loop is a generic lambda whose MODE says at compile time what happens to the fragments
   // (bits 0 / 1: A / B multiplied by an FP16 factor): a flag tested inside the loop costs a branch around
@@ -860,6 +862,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // away, and the generic functor kernels).
   auto k_loop = [&](auto mode_c) __attribute__((always_inline)) {
   constexpr int MODE = decltype(mode_c)::value;
+  // the B fragments of a k-step, made once for both halves of A; the imaginary fragments of A
+  [[maybe_unused]] int4v vb_keep[(Cfg::B_KIND == OPK_KSPLIT || Cfg::A_KIND == OPK_KSPLIT) ? FN : 1];
+  [[maybe_unused]] int4v va_keep[Cfg::A_KIND == OPK_KSPLIT ? FM / 2 : 1];
   // runs after the wait that covers the reads of buffer ks & 1
   // With Cfg::SPLIT_A the A fragments live in two half buffers fa[h][0 .. FM/2) and `half_c` says which half
   // (rows fi = h * FM/2 + i) this call multiplies; otherwise fa[ks & 1] holds all FM fragments and half_c is -1.
@@ -868,17 +873,25 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     constexpr int half = decltype(half_c)::value;
     constexpr int NA = half < 0 ? FM : FM / 2;             // A fragments of this call
     constexpr int FI0 = half < 0 ? 0 : half * (FM / 2);     // the accumulator row block of the first one
+    constexpr bool B_BOTH = Cfg::B_KIND == OPK_KSPLIT;      // (an OPK_KSPLIT A has its own loop below)
     constexpr int ABUF = half < 0 ? (ks & 1) : half;
     int4v va[NA], vb[FN];
 #pragma unroll
     for (int fi = 0; fi < NA; ++fi) {
       RA::pin_raw(fa[ABUF][fi]);
-      va[fi] = expand_fixup<Cfg::FIX>(RA::finish(fa[ABUF][fi], lane), lane);
+      va[fi] = RA::finish(fa[ABUF][fi], lane);
     }
+    if constexpr (B_BOTH && half == 1) {
+      // the fragments of B were made by the call for the first half of A
 #pragma unroll
-    for (int fj = 0; fj < FN; ++fj) {
-      RB::pin_raw(fb[ks & 1][fj]);
-      vb[fj] = RB::finish(fb[ks & 1][fj], lane);
+      for (int fj = 0; fj < FN; ++fj) vb[fj] = vb_keep[fj];
+    } else {
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) {
+        if (fj < RB::NREAD) RB::pin_raw(fb[ks & 1][fj]);
+        vb[fj] = RB::finish(fb[ks & 1][fj % RB::NREAD], lane, fj >= RB::NREAD);
+        if constexpr (B_BOTH && half == 0) vb_keep[fj] = vb[fj];
+      }
     }
     if constexpr (MODE >= 0) {
       // A is scaled one fragment ahead of the MFMAs that use it: in this order the compiler lets part of
@@ -928,6 +941,17 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj) {
         acc[FI0 + fi][fj] = Mfma<T, MI>::run(vb[fj], va[fi], acc[FI0 + fi][fj]);
       }
+    if constexpr (B_BOTH && half == 0) {
+      // the four byte permutes that make fragment fj + 1 of B issue in the shadow of the MFMA on fragment fj
+      // (left to itself the compiler puts all sixteen in front of the first MFMA)
+      __builtin_amdgcn_sched_group_barrier(0x2, 4, 0);
+#pragma unroll
+      for (int fj = 1; fj < FN; ++fj) {
+        __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x2, 4, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x8, NA * FN - (FN - 1), 0);
+    }
   };
   typedef std::integral_constant<int, -1> Whole;
 
@@ -944,7 +968,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       const bool issue = (kt + STAGES - 1 < KT);
       if constexpr (Cfg::SPLIT_A) {
         constexpr int HF = FM / 2;
-        constexpr int OPS_AH = HF * RA::OPS, OPS_B = FN * RB::OPS;
+        constexpr int OPS_AH = HF * RA::OPS, OPS_B = RB::NREAD * RB::OPS;
         // reads of A half H of k-step KS into fa[H], of B of k-step KS into fb[KS & 1]
         auto load_a_half = [&](auto ks2_c, auto h_c) __attribute__((always_inline)) {
           constexpr int KS2 = decltype(ks2_c)::value, H = decltype(h_c)::value;
@@ -955,11 +979,89 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         };
         auto load_b = [&](auto ks2_c) __attribute__((always_inline)) {
           constexpr int KS2 = decltype(ks2_c)::value;
-          static_for<0, FN>([&](auto j_c) {
+          static_for<0, RB::NREAD>([&](auto j_c) {
             constexpr int J = decltype(j_c)::value;
             rb.template read<J, KS2, Cfg::SYNC_FRAGS>(fb[KS2 & 1][J]);
           });
         };
+        if constexpr (Cfg::A_KIND == OPK_KSPLIT) {
+          // One set of reads per k-step serves both halves: once it has arrived, the real and the imaginary fragments
+          // of A (and the fragments of B) are made from it and kept, which frees the registers of the reads for those
+          // of the next k-step; they are in flight under the MFMAs of both halves.  One buffer each for A and B.
+          auto load_both = [&](auto ks2_c) __attribute__((always_inline)) {
+            constexpr int KS2 = decltype(ks2_c)::value;
+            static_for<0, HF>([&](auto i_c) {
+              constexpr int I = decltype(i_c)::value;
+              ra.template read<I, KS2, Cfg::SYNC_FRAGS>(fa[0][I]);
+            });
+            static_for<0, RB::NREAD>([&](auto j_c) {
+              constexpr int J = decltype(j_c)::value;
+              rb.template read<J, KS2, Cfg::SYNC_FRAGS>(fb[0][J]);
+            });
+          };
+          load_both(std::integral_constant<int, 0>{});
+          static_for<0, 2 * Cfg::KSTEPS>([&](auto u_c) {
+            constexpr int u = decltype(u_c)::value;
+            constexpr int ks = u / 2, h = u % 2;
+            if (issue) issue_part(u_c, std::integral_constant<int, 2 * Cfg::KSTEPS>{}, (kt + STAGES - 1) % STAGES);
+            if constexpr (h == 0) {
+              wait_lgkmcnt<0>();                          // the reads of this k-step have arrived
+              // Program order = the order the instructions should issue in (the scheduling groups below pin it): the
+              // byte permutes that make a fragment stand right before the MFMAs that first need it, those of the
+              // imaginary fragments of A (needed by the second half) between the MFMA groups of the first half, so
+              // that all but the first eight run in the shadow of MFMAs; the reads of the next k-step follow the
+              // last permute (they reuse the registers the permutes read) and have the whole second half to land.
+              constexpr bool B_BOTH = Cfg::B_KIND == OPK_KSPLIT;
+              int4v va[HF];
+#pragma unroll
+              for (int i = 0; i < HF; ++i) RA::pin_raw(fa[0][i]);
+#pragma unroll
+              for (int fj = 0; fj < RB::NREAD; ++fj) RB::pin_raw(fb[0][fj]);
+              va[0] = RA::finish(fa[0][0], lane, false);
+#pragma unroll
+              for (int fj = 0; fj < FN; ++fj) {
+                vb_keep[fj] = RB::finish(fb[0][fj % RB::NREAD], lane, fj >= RB::NREAD);
+                acc[0][fj] = Mfma<T, MI>::run(vb_keep[fj], va[0], acc[0][fj]);
+              }
+#pragma unroll
+              for (int i = 1; i < HF; ++i) {
+                va[i] = RA::finish(fa[0][i], lane, false);
+                va_keep[i - 1] = RA::finish(fa[0][i - 1], lane, true);
+                pin(va_keep[i - 1]);          // made here, not where the second half uses it
+#pragma unroll
+                for (int fj = 0; fj < FN; ++fj) acc[i][fj] = Mfma<T, MI>::run(vb_keep[fj], va[i], acc[i][fj]);
+              }
+              va_keep[HF - 1] = RA::finish(fa[0][HF - 1], lane, true);
+              pin(va_keep[HF - 1]);
+              if constexpr (B_BOTH) {
+                __builtin_amdgcn_sched_group_barrier(0x2, 8, 0);
+                __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+#pragma unroll
+                for (int fj = 1; fj < FN; ++fj) {
+                  __builtin_amdgcn_sched_group_barrier(0x2, 4, 0);
+                  __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+                }
+              } else {
+                __builtin_amdgcn_sched_group_barrier(0x2, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x8, FN, 0);
+              }
+#pragma unroll
+              for (int i = 1; i < HF; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x2, 8, 0);
+                __builtin_amdgcn_sched_group_barrier(0x8, FN, 0);
+              }
+              __builtin_amdgcn_sched_group_barrier(0x2, 4, 0);
+              if constexpr (ks + 1 < Cfg::KSTEPS) load_both(std::integral_constant<int, ks + 1>{});
+            } else {
+#pragma unroll
+              for (int i = 0; i < HF; ++i)
+#pragma unroll
+                for (int fj = 0; fj < FN; ++fj) acc[HF + i][fj] = Mfma<T, MI>::run(vb_keep[fj], va_keep[i], acc[HF + i][fj]);
+            }
+          });
+          // (the last reads of the stage were waited for before its last MFMAs: complete before the next barrier)
+          continue;
+        }
         load_a_half(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
         load_b(std::integral_constant<int, 0>{});
         static_for<0, 2 * Cfg::KSTEPS>([&](auto u_c) {
@@ -1111,7 +1213,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
                 ra.template read<H * HF + I, ks, true>(fa[H][I]);
               });
               if constexpr (H == 0) {
-                static_for<0, FN>([&](auto j_c) {
+                static_for<0, RB::NREAD>([&](auto j_c) {
                   constexpr int J = decltype(j_c)::value;
                   rb.template read<J, ks, true>(fb[ks & 1][J]);
                 });
@@ -1150,7 +1252,22 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if (args.acc_post_scale != 1.0f) scale_acc(args.acc_post_scale);
   }
 
-  if constexpr (Cfg::PAIR) {
+  if constexpr (Cfg::ROWS_LANE && Cfg::COLS_FRAG) {
+    // As below, with the products of the imaginary parts of B in the column blocks fj + FN / 2: lane 2i holds
+    // re A * re B in block fj and re A * im B in block fj + FN / 2, lane 2i+1 im A * re B and im A * im B.
+#pragma unroll
+    for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FNO; ++fj)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+          const float own = acc[fi][fj][v];
+          const float mine = acc[fi][fj + FNO][v];
+          const float other = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, mine), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+          acc[fi][fj][v] = (lane & 1) ? own + other : (Cfg::FIX == FIX_PAIR_DUAL ? own : own - other);
+        }
+  }
+  if constexpr (Cfg::ROWS_LANE && Cfg::COLS_LANE) {
     // The four real products of a complex element of D = (re A + i im A)(re B + i im B): lane 2i holds, for
     // each of its two complex columns, re A * re B (value 0 / 2) and re A * im B (value 1 / 3), lane 2i+1
     // im A * re B and im A * im B.  The neighbours trade their odd values: lane 2i becomes the real part
@@ -1172,17 +1289,30 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
   }
 
-  if constexpr (Cfg::PLANAR) {
-    // The four real products of the elements of D lie in four blocks of the lane: (row blocks of A_re | A_im) x
-    // (column blocks of B_re | B_im).  Real part re*re - im*im into the upper left block, imaginary part
-    // im*re + re*im into the lower left one; C came in through the same two.
+  if constexpr (Cfg::ROWS_FRAG && Cfg::COLS_FRAG) {
+    // The four real products of the elements of D lie in four blocks of the lane: (row blocks of re A | im A) x
+    // (column blocks of re B | im B).  Real part re*re - im*im into the upper left block, imaginary part
+    // im*re + re*im into the lower left one (dual numbers: re*re, and du*re + re*du); C came in through the same two.
 #pragma unroll
     for (int fi = 0; fi < FMH; ++fi)
 #pragma unroll
       for (int fj = 0; fj < FNO; ++fj) {
-        acc[fi][fj] = acc[fi][fj] - acc[fi + FMH][fj + FNO];
+        if constexpr (Cfg::FIX != FIX_PAIR_DUAL) acc[fi][fj] = acc[fi][fj] - acc[fi + FMH][fj + FNO];
         acc[fi + FMH][fj] = acc[fi + FMH][fj] + acc[fi][fj + FNO];
       }
+  }
+  if constexpr (Cfg::ROWS_FRAG && Cfg::COLS_LANE) {
+    // re A | im A in the row blocks fi | fi + FM / 2, re B | im B in the values 2v | 2v + 1 of a block
+#pragma unroll
+    for (int fi = 0; fi < FMH; ++fi)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+          const float rr = acc[fi][fj][2 * v], ri = acc[fi][fj][2 * v + 1], ir = acc[fi + FMH][fj][2 * v], ii = acc[fi + FMH][fj][2 * v + 1];
+          acc[fi][fj][2 * v] = Cfg::FIX == FIX_PAIR_DUAL ? rr : rr - ii;
+          acc[fi + FMH][fj][2 * v] = ir + ri;
+        }
   }
 
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
@@ -1206,7 +1336,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       } else if (args.epi_kind == 2) {   // one bias value per row of D
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const int r = Cfg::PLANAR ? mrow + MI * (fi % FMH) : (Cfg::COMPLEX ? (mrow + MI * fi) >> 1 : mrow + MI * fi);
+          const int r = Cfg::ROWS_FRAG ? mrow + MI * (fi % FMH) : (Cfg::COMPLEX ? (mrow + MI * fi) >> 1 : mrow + MI * fi);
           const float bv = args.bias[(Cfg::RAGGED_OK && r >= args.M) ? 0 : r];
 #pragma unroll
           for (int v = 0; v < NVO; ++v) acc[fi][fj][slot(v)] = imag_rows(fi) ? acc[fi][fj][slot(v)] : acc[fi][fj][slot(v)] + bv;

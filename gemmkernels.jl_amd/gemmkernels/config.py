@@ -174,8 +174,9 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
     ``b_kmajor``: B is stored K x N ('N'); they admit the tiles with a side of 192."""
     M, N, K = gemm_shape["M"], gemm_shape["N"], gemm_shape["K"]
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
-        # a small Float32 product in whole 32 x 32 x 32 tiles: one wave per workgroup, four times the workgroups
-        # of the 64 x 64 tile (256^3: 64 workgroups instead of 16; every output is still one fma chain in k)
+        # a small Float32 product in whole 32 x 32 x 32 tiles: four times the workgroups of the 64 x 64 tile
+        # (256^3: 64 workgroups instead of 16) with 2 x 2 outputs per lane on four waves, so that a lane works
+        # through 4 fma chains instead of 16 (every output is still one fma chain in k: the same bits)
         if (operator.kind == Operator.FPU and operator.CT.name == "Float32" and operator.AT.name == "Float32" and tile_sized
                 and M % 32 == 0 and N % 32 == 0 and K % 32 == 0 and -(-M // 64) * -(-N // 64) < NUM_CUS // 2):
             return NT(M=32, N=32, K=32)
@@ -221,32 +222,22 @@ _MFMA_TILE_RATE = {(256, 256, 64): 1.0, (256, 256, 32): 0.95, (256, 128, 64): 0.
                    (256, 192, 64): 0.90, (192, 256, 64): 0.90}
 
 
-# complex / dual tiles (complex elements) -> waves, for interleaved A and B of which at least one is contiguous
-# along m or n: one real product of the real views of A and B, whose real tile has twice the rows and columns.
-# ('T','T' runs the first tile with the wave grid transposed, see _complex_tiles.)
+# complex / dual tiles (complex elements) -> waves: one real product of the real views of A and B, whose real tile
+# has twice the rows and columns; the same table for every transpose
 _COMPLEX_PAIR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
-# ... and for 'T','N' (both contiguous along k): the A fragments are expanded to [re -im; im re] in registers
-_COMPLEX_TN_TILES = [((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
-_DUAL_TN_TILES = [((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
 
 # complex tiles (complex elements) of the kernel for planar global matrices -> waves; the real tile has twice
 # the rows and columns (both planes of A, B and D)
 _PLANAR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
 
 # tiles of the vector-ALU kernel and of the bounds-checked MFMA kernel
-_FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (1, 1))]
+_FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (2, 2)), ((32, 32, 32), (1, 1))]
 _CHECKED_TILES = [((64, 64, 32), (2, 2))]
 
 
 def _complex_tiles(operator, planar, a_kmajor, b_kmajor):
     """(tile, waves) of the complex / dual instances for these layouts, in order of preference."""
-    if planar:
-        return _PLANAR_TILES
-    if a_kmajor and b_kmajor:
-        return _DUAL_TN_TILES if operator.kind == Operator.MFMA_DUAL else _COMPLEX_TN_TILES
-    if a_kmajor:      # 'T','T': A is the operand that is read twice from LDS, so the waves line up along m
-        return [(t, (w[1], w[0])) for t, w in _COMPLEX_PAIR_TILES]
-    return _COMPLEX_PAIR_TILES
+    return _PLANAR_TILES if planar else _COMPLEX_PAIR_TILES
 
 
 def _default_waves(operator, block_shape, checked=False, planar=False, gett=False, a_kmajor=False, b_kmajor=True):

@@ -341,17 +341,11 @@ const MFMA_TILES = [((256, 256, 64), (2, 4)), ((256, 256, 32), (2, 4)), ((256, 1
 # relative throughput of a CU running each tile (256 x 256 x 64 = 1), measured
 const MFMA_TILE_RATE = Dict((256, 256, 64) => 1.0, (256, 256, 32) => 0.95, (256, 128, 64) => 0.81, (128, 256, 64) => 0.82,
                             (128, 128, 32) => 0.63, (128, 128, 64) => 0.62, (64, 64, 64) => 0.47, (64, 64, 32) => 0.42)
-# complex / dual tiles (complex elements): interleaved A and B of which at least one is contiguous along m or n run as
-# one real product of their real views ('T','T' with the wave grid transposed); 'T','N' expands A in registers
+# complex / dual tiles (complex elements): one real product of the real views of A and B (interleaved or planar),
+# the same table for every transpose
 const COMPLEX_PAIR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
-const COMPLEX_TN_TILES = [((64, 128, 32), (2, 2)), ((128, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
-const DUAL_TN_TILES = [((64, 128, 32), (2, 2)), ((64, 64, 32), (4, 2)), ((32, 64, 32), (2, 2))]
-function complex_tiles(operator::Type, a_kmajor::Bool, b_kmajor::Bool; planar::Bool = false)
-    planar && return COMPLEX_PAIR_TILES            # planar global matrices: the planes are plain real matrices, one table for all transposes
-    a_kmajor && b_kmajor && return nameof(operator) in (:WMMADualOp, :MFMADualOp) ? DUAL_TN_TILES : COMPLEX_TN_TILES
-    a_kmajor ? [(t, (w[2], w[1])) for (t, w) in COMPLEX_PAIR_TILES] : COMPLEX_PAIR_TILES
-end
-const FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (1, 1))]
+complex_tiles(operator::Type, a_kmajor::Bool, b_kmajor::Bool; planar::Bool = false) = COMPLEX_PAIR_TILES
+const FPU_TILES = [((64, 64, 32), (2, 2)), ((128, 128, 16), (2, 2)), ((32, 32, 32), (2, 2)), ((32, 32, 32), (1, 1))]
 
 "reference src/config.jl:84-120, unchanged (the reference-compatible answer; the launch uses the tile table)"
 function heuristic_block_shape(shared_a::Type, shared_b::Type, shared_c::Type, shared_d::Type)

@@ -219,6 +219,4 @@ def test_tile_tables_match_the_python_tables():
 
     assert jl_table("MFMA_TILES") == [(t, w) for t, w in cfg._MFMA_TILES]
     assert jl_table("COMPLEX_PAIR_TILES") == cfg._COMPLEX_PAIR_TILES == cfg._PLANAR_TILES
-    assert jl_table("COMPLEX_TN_TILES") == cfg._COMPLEX_TN_TILES
-    assert jl_table("DUAL_TN_TILES") == cfg._DUAL_TN_TILES
     assert jl_table("FPU_TILES") == cfg._FPU_TILES
