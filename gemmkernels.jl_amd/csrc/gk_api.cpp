@@ -160,7 +160,7 @@ const gk_transforms* fold_pow2_scales(const gk_config* c, const gk_transforms* t
 
 // Builds the run-time key of the kernel instance for a configuration.
 // allow_ragged_fast = false: bounds-checked layouts run on the bounds-checked kernel whatever their alignment.
-int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
+int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast) {
   memset(key, 0, sizeof(*key));
   const int ak = c->global_a_layout.kind, bk = c->global_b_layout.kind;
   const int ck = c->global_c_layout.kind, dk = c->global_d_layout.kind;
@@ -239,6 +239,20 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   }
   if (key->fused && !t && c->global_a_layout.eltype != GK_F16 && (key->family == gk::FAMILY_MFMA || key->family == gk::FAMILY_GETT))
     key->fused = 2;
+  return GK_OK;
+}
+
+// The arrangement of four waves with 128 x 128 wave tiles (one wave per SIMD, see Cfg::SOLO) is compiled for plain
+// products without hooks whose extents are whole numbers of tiles.  Any other launch of such a configuration runs the
+// eight-wave arrangement of the same block shape, which gives the same bits (the order of the k-steps and of the
+// products inside them does not depend on how the tile is dealt out to waves).
+int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
+  const int rc = make_key_as_configured(c, t, e, key, allow_ragged_fast);
+  if (rc != GK_OK) return rc;
+  if (key->family == gk::FAMILY_MFMA && key->BM == 256 && key->BN == 256 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2) {
+    const bool whole = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0;
+    if (key->fused != 0 || !whole) key->waves_n = 4;
+  }
   return GK_OK;
 }
 
@@ -640,7 +654,7 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   // the instance that would run; its LDS request is what Kernel.shmem_size returns
   int rc = GK_OK;
   if (custom) {      // a kernel specialised at run time: its resources are known to the caller
-    rc = make_key(c, t, e, key, allow_ragged_fast);
+    rc = make_key_as_configured(c, t, e, key, allow_ragged_fast);     // (compiled for exactly this configuration)
     *info = *custom;
   } else {
     rc = find_instance(c, t, e, key, info, allow_ragged_fast);
@@ -659,9 +673,17 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
   if (threads > threads_max)
     return fail(GK_ERR_THREADS, "Requested too many threads for this kernel: This kernel can be launched using at most %d threads, while this configuration required %lld",
                 threads_max, threads);
-  if (threads != info->threads)
+  // (the instance that runs may be the eight-wave arrangement of a four-wave configuration, see make_key)
+  const long long configured_waves = (long long)(c->block_shape.M / c->compute_warp.M) * (c->block_shape.N / c->compute_warp.N);
+  const bool other_arrangement = key->waves_m * key->waves_n != configured_waves;
+  if (other_arrangement && info->threads > threads_max)
+    return fail(GK_ERR_THREADS, "Requested too many threads for this kernel: This kernel can be launched using at most %d threads, while this configuration required %d",
+                threads_max, info->threads);
+  if (!other_arrangement && threads != info->threads)
     return fail(GK_ERR_UNSUPPORTED, "warps_per_block = %d does not match the %d waves of block_shape / compute_warp", c->warps_per_block,
                 info->threads / gk::kWaveSize);
+  if (other_arrangement && c->warps_per_block != configured_waves)
+    return fail(GK_ERR_UNSUPPORTED, "warps_per_block = %d does not match the %lld waves of block_shape / compute_warp", c->warps_per_block, configured_waves);
   return GK_OK;
 }
 

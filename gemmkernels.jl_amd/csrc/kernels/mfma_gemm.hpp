@@ -268,6 +268,18 @@ struct FragReader {
       asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.hi) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K + 4) * G::ROW_BYTES) : "memory");
     }
   }
+  // one LDS instruction of read<FI, KS>: H < OPS
+  template <int FI, int KS, int H>
+  __device__ __forceinline__ void read_op(Raw& r) const {
+    static_assert(!opk_complex_k(KIND), "plain operands");
+    if constexpr (KIND == OPK_KMAJOR) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
+    } else if constexpr (H == 0) {
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.lo) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K) * G::ROW_BYTES) : "memory");
+    } else {
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.hi) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K + 4) * G::ROW_BYTES) : "memory");
+    }
+  }
   template <int FI>
   __device__ __forceinline__ unsigned mmajor_addr() const {
     if constexpr (PAIRED) return (FI & 1) ? (cur[FI / 2] ^ 32u) : cur[FI / 2];
@@ -400,14 +412,19 @@ struct MfmaGemmConfig {
   // the generic A / B hooks, and wave tiles of more than eight 32x32 blocks (256 accumulator registers),
   // need so many registers that the kernel spills: their fragment reads wait for their data inside the
   // assembly statement that issues them (see FragReader::read)
+  // One wave per SIMD: four waves with wave tiles of 64 16x16 blocks (all 256 accumulation registers), two LDS stages.
+  // The K loop of these instances is written out instruction slot by instruction slot (see the SOLO loop).
+  static constexpr bool SOLO = MI_ == 16 && WAVES_M_ * WAVES_N_ == 4 && (BM_ / WAVES_M_ / 16) * (BN_ / WAVES_N_ / 16) == 64 && STAGES_ == 2 &&
+                               (BK_ / 32) % 2 == 0 && FUSE_ == 0 && !GETT_ && FIX_ == FIX_NONE && !SPLITK_ &&
+                               A_KIND_ != OPK_KSPLIT && B_KIND_ != OPK_KSPLIT && (GK_FORCE_SYNC_FRAGS == 0);
   // plain real products may have a last tile row / column that sticks out over M / N and a last, partial K
   // tile (the host asks for it only with 16-byte aligned columns, M or N a multiple of 8 where that index is
   // the contiguous one of A or B, and K a multiple of 8): loads are clamped, the C load and the D store
   // masked, the part of the last K tile beyond K zeroed in LDS
   // (the K-split instances take tiles over M and N, not a partial K tile)
-  static constexpr bool RAGGED_OK = !GETT_ && FIX_ == FIX_NONE;
+  static constexpr bool RAGGED_OK = !GETT_ && FIX_ == FIX_NONE && !SOLO;
   static constexpr bool RAGGED_K_OK = RAGGED_OK && !SPLITK_;
-  static constexpr bool SYNC_FRAGS = FUSE_ == 2 || ((BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
+  static constexpr bool SYNC_FRAGS = FUSE_ == 2 || (!SOLO && (BM_ / WAVES_M_ / 32) * (BN_ / WAVES_N_ / 32) > 8) || (GK_FORCE_SYNC_FRAGS != 0);
   static constexpr bool PLANAR = (FIX_ == FIX_PLANAR);
   static constexpr bool PAIR = (FIX_ == FIX_PAIR || FIX_ == FIX_PAIR_DUAL);     // complex / dual product as one real product (see FIX_PAIR)
   static constexpr bool COMPLEX = FIX_ != FIX_NONE;                             // C / D hold complex numbers
@@ -644,8 +661,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 
   // --- prologue: start the first STAGES-1 tiles on their way ---
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s)
-    if (s < KT) issue_tile(s);
+  for (int s = 0; s < (Cfg::SOLO ? STAGES : STAGES - 1); ++s)
+    if (s < KT) issue_tile(s);      // (SOLO: both stages are free and the loop issues tile kt + 2 from tile kt)
 
   // --- accumulators: C tile (two transforms) or zeros -------------------------------------------
   // 32x32 blocks: lane l owns row m = 32*fi + l%32 and columns n = 32*fj + 8*(v/4) + 4*(l/32) + v%4, v < 16;
@@ -754,6 +771,40 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   [[maybe_unused]] const bool ragged = Cfg::RAGGED_OK && (m0 + BM > args.M || n0 + BN > args.N);   // wave-uniform
   // K-split launches: the first slice of K starts from C, the others from zero
   const bool load_c = args.c_mode != 0 && (!Cfg::SPLITK || blockIdx.z == 0);
+  // SOLO: the A fragment is the first MFMA operand, so a lane owns the rows 4 * (lane / 16) .. + 3 of column lane % 16 of
+  // a block: 16 contiguous bytes of a column-major FP32 C / D.  The loads go straight into the accumulation registers.
+  [[maybe_unused]] const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane / MI), solo_col = n0 + wn * Cfg::WTN + (lane % MI);
+  if constexpr (Cfg::SOLO) {
+    // (16-byte accesses where the pointer and the leading dimension allow them, else element by element)
+    if (load_c && args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0) {
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          const float* cp = (const float*)args.c + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc;
+          asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(acc[fi][fj]) : "v"(cp) : "memory");
+        }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) asm volatile("" : "+a"(acc[fi][fj]));
+    } else if (load_c) {
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[fi][fj][v] = load_cd(args.c, args.c_dtype, off + v);
+        }
+    } else {
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+        for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = AccV{};
+    }
+  } else
   if (Cfg::RAGGED_OK && ragged && load_c) {
     // tile over the edge: element by element, out-of-range elements start from zero
 #pragma unroll
@@ -955,7 +1006,99 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   };
   typedef std::integral_constant<int, -1> Whole;
 
-  if constexpr (!Cfg::PREFETCH) {
+  if constexpr (Cfg::SOLO) {
+    constexpr int KS = Cfg::KSTEPS;
+    constexpr int NM = FM * FN;                       // MFMAs per k-step
+    constexpr int NOPA = RA::NREAD * RA::OPS, NOPS = NOPA + RB::NREAD * RB::OPS;    // LDS instructions of the fragment reads of a k-step
+    // One side instruction behind an MFMA: a wave issues at most one instruction every four clocks, an MFMA keeps the
+    // matrix core busy for sixteen, and with a single wave on the SIMD every further instruction between two MFMAs
+    // is time in which the matrix core idles.  A DMA instruction (with its LDS address in M0) goes behind every GD-th
+    // MFMA of the k-step that follows the barrier, an LDS read behind every other MFMA.
+    constexpr int GD = 4, RSP = 1;
+    static_assert(GD * (DPT - 1) < NM, "the DMA of a tile is issued in the k-step behind the barrier that frees its stage");
+    static_assert(NOPS * RSP <= NM, "the fragment reads fit the MFMAs of a k-step");
+    // DMA instruction I of the tile that ga / gb stand at
+    auto dma_one = [&](auto i_c, int stage) __attribute__((always_inline)) {
+      constexpr int I = decltype(i_c)::value;
+      char* sa = smem + stage * Cfg::STAGE_BYTES;
+      char* sb = sa + GA::BYTES;
+      // (the offset passes through an empty assembly statement so that its widening to 64 bits stays next to the DMA
+      // instruction, which then takes the tile pointer from scalar registers and the 32-bit offset from the lane)
+      unsigned& o = I < DMA_A ? offa[I < DMA_A ? I : 0] : offb[I < DMA_A ? 0 : I - DMA_A];
+      asm volatile("" : "+v"(o));
+      if constexpr (I < DMA_A) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + o), GK_LDS_PTR(void, sa + (wave + I * NWAVES) * 1024), 16, 0, 0);
+      else __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + o), GK_LDS_PTR(void, sb + (wave + (I - DMA_A) * NWAVES) * 1024), 16, 0, 0);
+    };
+    // LDS instruction R of the fragment reads of k-step KS2 (of the stage the readers stand at), into buffer KS2 & 1
+    auto read_op = [&](auto r_c, auto ks2_c) __attribute__((always_inline)) {
+      constexpr int R = decltype(r_c)::value, KS2 = decltype(ks2_c)::value;
+      if constexpr (R < NOPA) ra.template read_op<R / RA::OPS, KS2, R % RA::OPS>(fa[KS2 & 1][R / RA::OPS]);
+      else rb.template read_op<(R - NOPA) / RB::OPS, KS2, (R - NOPA) % RB::OPS>(fb[KS2 & 1][(R - NOPA) / RB::OPS]);
+    };
+    // The MFMAs of k-step ks.  The fragments of k-step (ks + 1) % KS -- of this tile, or of the next one when ks is the
+    // last k-step -- are read in the slots behind the first MFMAs.  DMA: the k-step also issues the DMA of a tile.
+    auto phase = [&](auto ks_c, auto dma_c, int dma_stage) __attribute__((always_inline)) {
+      constexpr int ks = decltype(ks_c)::value;
+      constexpr bool DMA = decltype(dma_c)::value;
+      constexpr int NKS = (ks + 1) % KS;
+      int4v va[FM], vb[FN];
+      __builtin_amdgcn_sched_barrier(0);       // no MFMA of the k-step before moves behind the waits in front of this one
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi) { RA::pin_raw(fa[ks & 1][fi]); va[fi] = RA::finish(fa[ks & 1][fi], lane); }
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[ks & 1][fj]); vb[fj] = RB::finish(fb[ks & 1][fj], lane); }
+      static_for<0, NM>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        constexpr int fi = i / FN, fj = (fi & 1) ? FN - 1 - (i % FN) : i % FN;
+        acc[fi][fj] = Mfma<T, MI>::run(va[fi], vb[fj], acc[fi][fj]);
+        // (the scheduling barriers keep every instruction in the slot it is written in)
+        if constexpr (DMA && i % GD == 0 && i / GD < DPT) {
+          __builtin_amdgcn_sched_barrier(0);
+          dma_one(std::integral_constant<int, i / GD>{}, dma_stage);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr ((i % RSP) == 0 && i / RSP < NOPS) {
+          __builtin_amdgcn_sched_barrier(0);
+          read_op(std::integral_constant<int, i / RSP>{}, std::integral_constant<int, NKS>{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+    };
+    typedef std::integral_constant<bool, true> Yes;
+    typedef std::integral_constant<bool, false> No;
+    // tiles 0 and 1 were issued before the C load.  From here on ga / gb stand at the tile that the next DMA fetches:
+    // tile kt + 2 in step kt, and the last tile once more where there is no such tile (the DMA is unconditional: a
+    // branch around it costs more issue slots than the instruction; the data lands in a stage nobody reads any more)
+    if (KT < 3 && KT > 0) { ga -= a_step; gb -= b_step; }
+    if (KT > 1) wait_vmcnt<DPT>(); else wait_vmcnt<0>();
+    block_barrier();
+    ra.set_stage(lds_base);
+    rb.set_stage(lds_base + GA::BYTES);
+    static_for<0, NOPS>([&](auto r_c) { read_op(r_c, std::integral_constant<int, 0>{}); });
+    // (no copy of the loop body for the last tile: what it reads ahead and fetches there is never used)
+    for (int kt = 0; kt < KT; ++kt) {
+      static_for<0, KS>([&](auto ks_c) {
+        constexpr int ks = decltype(ks_c)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        wait_lgkmcnt<0>();                              // the fragments of this k-step have arrived
+        if constexpr (ks == KS - 1) {
+          // tile kt+1 has landed (its DMA was issued a k-step or more ago); behind the barrier it is visible to all
+          // waves, and all are done reading tile kt: its stage takes tile kt+2
+          wait_vmcnt<0>();
+          block_barrier();
+          const unsigned stage_addr = lds_base + (unsigned)((kt + 1) & 1) * Cfg::STAGE_BYTES;
+          ra.set_stage(stage_addr);
+          rb.set_stage(stage_addr + GA::BYTES);
+          phase(ks_c, Yes{}, kt & 1);
+          if (kt + 3 < KT) { ga += a_step; gb += b_step; }
+        } else {
+          phase(ks_c, No{}, 0);
+        }
+      });
+    }
+    wait_vmcnt<0>();     // (the last DMA of the loop may still be on its way; so are reads
+    wait_lgkmcnt<0>();   // of fragments)
+  } else if constexpr (!Cfg::PREFETCH) {
     // Two LDS stages: the DMA of tile kt+1 runs while tile kt is consumed; the first fragments of a
     // tile are read after the barrier that publishes it.
     for (int kt = 0; kt < KT; ++kt) {
@@ -1315,6 +1458,32 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
   }
 
+  if constexpr (Cfg::SOLO) {
+    // (the lane number is asked for again: nothing of the store addresses is then kept in registers across the K loop)
+    int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(lane_e));
+    const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane_e / MI), solo_col = n0 + wn * Cfg::WTN + (lane_e % MI);
+    if (args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0) {
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          float* dp = (float*)args.d + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd;
+          asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
+        }
+    } else {
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          asm volatile("" : "+a"(acc[fi][fj]));      // (stays where it is until this branch is taken)
+          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) store_cd(args.d, args.d_dtype, off + v, acc[fi][fj][v]);
+        }
+    }
+    return;
+  }
   // --- epilogue: regs -> (transform, bias, transform) -> global ------------------------------------
   gett_origins();
 #pragma unroll

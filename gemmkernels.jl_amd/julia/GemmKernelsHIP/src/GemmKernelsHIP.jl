@@ -385,8 +385,15 @@ function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true
     (M = best[1], N = best[2], K = best[3])
 end
 
-function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_kmajor::Bool = true, planar::Bool = false)
+# One wave per SIMD: 256 x 256 x 64 on four waves with 128 x 128 wave tiles, compiled for plain products without hooks
+# whose extents are whole numbers of tiles.  The library runs the 2 x 4 arrangement of the same block shape, with the
+# same bits, for any other launch of such a configuration.
+const SOLO_TILE = (256, 256, 64)
+const SOLO_WAVES = (2, 2)
+
+function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_kmajor::Bool = true, planar::Bool = false, whole_tiles::Bool = false)
     key = (block_shape.M, block_shape.N, block_shape.K)
+    Operator.is_mfma(operator) && key == SOLO_TILE && whole_tiles && return SOLO_WAVES
     table = Operator.is_fpu(operator) ? FPU_TILES : (Operator.is_mfma(operator) ? MFMA_TILES : complex_tiles(operator, a_kmajor, b_kmajor; planar = planar))
     for (t, w) in table
         t == key && return w
@@ -420,7 +427,8 @@ function get_config(; gemm_shape, operator, global_a_layout, global_c_layout, kw
     block_shape = get(params, :block_shape, default_block_shape(operator, gemm_shape; tile_sized = tile_sized, a_kmajor = a_kmajor, b_kmajor = b_kmajor, planar = planar))
     op_shape = Operator.shape(operator)
 
-    waves = default_waves(operator, block_shape; a_kmajor = a_kmajor, b_kmajor = b_kmajor, planar = planar)
+    whole_tiles = gemm_shape.M % block_shape.M == 0 && gemm_shape.N % block_shape.N == 0 && gemm_shape.K % block_shape.K == 0
+    waves = default_waves(operator, block_shape; a_kmajor = a_kmajor, b_kmajor = b_kmajor, planar = planar, whole_tiles = whole_tiles)
     if waves !== nothing
         warps_default = waves[1] * waves[2]
         compute_warp_default = (M = block_shape.M ÷ waves[1], N = block_shape.N ÷ waves[2], K = op_shape.K)

@@ -84,7 +84,13 @@ def base_kwargs(M=4096, N=4096, K=4096, **kw):
 def test_get_config_defaults_for_the_headline_problem():
     conf = gk.get_config(**base_kwargs())
     assert conf.block_shape == NT(M=256, N=256, K=64)
-    assert conf.warps_per_block == 8 and conf.compute_warp == NT(M=128, N=64, K=16)
+    # whole 256 x 256 x 64 tiles: four waves, one per SIMD, with 128 x 128 wave tiles
+    assert conf.warps_per_block == 4 and conf.compute_warp == NT(M=128, N=128, K=16)
+    # ... and eight waves with 128 x 64 wave tiles for extents that are not whole tiles
+    col = Layout.ColMajor
+    ragged = gk.get_config(**base_kwargs(M=4000, N=4000, K=4000, global_a_layout=col[F16], global_c_layout=col[F32],
+                                         block_shape=NT(M=256, N=256, K=64)))
+    assert ragged.warps_per_block == 8 and ragged.compute_warp == NT(M=128, N=64, K=16)
     assert conf.compute_op_shape == NT(M=32, N=32, K=16)
     # 64-lane waves, 16 bytes per lane (src/config.jl:240-260 with 64 lanes)
     assert conf.mem_a_warp == NT(M=256, K=2) and conf.mem_a_thread == NT(M=8, K=1)
@@ -154,7 +160,7 @@ def test_lds_stage_and_thread_limits():
         with pytest.raises(ConfigError) as ei:
             gk.check_config(conf, Kernel.matmul_pipelined)
         assert ei.value.status == _lib.GK_ERR_LDS and "shared memory" in ei.value.message
-        _lib.lib().gk_set_device_limits(0, 256)                # src/matmul.jl:41
+        _lib.lib().gk_set_device_limits(0, 128)                # src/matmul.jl:41 (the configuration runs 256 threads)
         with pytest.raises(ConfigError) as ei:
             gk.check_config(conf, Kernel.matmul_pipelined)
         assert ei.value.status == _lib.GK_ERR_THREADS

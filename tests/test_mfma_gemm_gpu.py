@@ -14,6 +14,7 @@ TOL = 1e-3
 
 TILES = [  # block shape, (waves_m, waves_n)
     ((256, 256, 64), (2, 4)),
+    ((256, 256, 64), (2, 2)),     # one wave per SIMD
     ((256, 256, 32), (2, 4)),
     ((256, 256, 32), (4, 2)),
     ((256, 128, 64), (2, 2)),

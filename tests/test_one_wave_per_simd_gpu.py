@@ -1,0 +1,148 @@
+"""The 256 x 256 x 64 tile on four waves (one per SIMD, 128 x 128 wave tiles) against the same tile on eight waves
+and against the CPU oracle.  The two arrangements run the k-steps and the products inside them in the same order,
+so FP32 results are compared bit for bit; the oracle with the tolerance of the other MFMA tests (relative
+Frobenius error <= 1e-3).  Launches the four-wave arrangement is not compiled for (hooks, a bias, extents that
+are not whole tiles) run the eight-wave arrangement of the same configuration."""
+import numpy as np
+import pytest
+
+import gemmkernels as gk
+from gemmkernels import Layout, Operator, Kernel, Transform, Epilogue, NT, Float16, Float32, BFloat16, rng
+import helpers
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+BLOCK = (256, 256, 64)
+
+
+def config(M, N, K, ta, tb, waves, ab=Float16, c=Float32, d=Float32, zero_c=False, checked=False):
+    col = Layout.ColMajor if checked else Layout.UnsafeAlignedColMajor
+    row = Layout.RowMajor if checked else Layout.UnsafeAlignedRowMajor
+    return gk.get_config(
+        gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=BLOCK[0], N=BLOCK[1], K=BLOCK[2]),
+        warps_per_block=waves[0] * waves[1], compute_warp=NT(M=BLOCK[0] // waves[0], N=BLOCK[1] // waves[1], K=16),
+        operator=Operator.MFMAOp[32, 32, 16, ab, Float32],
+        global_a_layout=(row if ta else col)[ab], global_b_layout=(row if tb else col)[ab],
+        global_c_layout=Layout.Zero[c] if zero_c else col[c], global_d_layout=col[d],
+        is_a_col_major=not ta, is_b_col_major=not tb)
+
+
+def operands(M, N, K, ta, tb, seed):
+    a = rng.matrix("upm1_f16", seed + 1, (K, M) if ta else (M, K))
+    b = rng.matrix("upm1_f16", seed + 2, (N, K) if tb else (K, N))
+    c = rng.matrix("upm1_f32", seed + 3, (M, N))
+    return a, b, c
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("K", [64, 128, 192, 448])
+def test_same_bits_as_eight_waves(gpu, ta, tb, K):
+    """One, two, three and seven K tiles: the pipeline start, the superfluous read-ahead of the last tile."""
+    M, N = 512, 768
+    a, b, c = operands(M, N, K, ta, tb, 7000 + K)
+    four, eight = config(M, N, K, ta, tb, (2, 2)), config(M, N, K, ta, tb, (2, 4))
+    name = gk.kernel_name(four, Kernel.matmul_pipelined)
+    print("case", ta, tb, K, name, flush=True)
+    assert "_w2x2_" in name and "_w2x4_" in gk.kernel_name(eight, Kernel.matmul_pipelined)
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    d8 = helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, d8)
+    assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N))) <= TOL
+    assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= TOL
+
+
+def test_zero_c_and_d_in_place(gpu):
+    M, N, K = 256, 512, 320
+    a, b, c = operands(M, N, K, False, False, 7100)
+    conf = config(M, N, K, False, False, (2, 2), zero_c=True)
+    d = helpers.run_gpu(conf, a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d, helpers.run_gpu(config(M, N, K, False, False, (2, 4), zero_c=True), a, b, None, (M, N), kernel=Kernel.matmul_pipelined))
+    assert oracle.rel_frobenius(d, oracle.gemm_f64(a, b, None, 1.0, 0.0, False, False)) <= TOL
+    # d aliases c (reference src/matmul.jl:198)
+    conf = config(M, N, K, False, False, (2, 2))
+    d_alias = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined, alias_cd=True)
+    assert np.array_equal(d_alias, helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined))
+
+
+@pytest.mark.parametrize("c16,d16", [(True, True), (False, True), (True, False)])
+def test_16_bit_c_and_d(gpu, c16, d16):
+    """C / D that are not FP32 go element by element (the 16-byte accesses are those of FP32 columns)."""
+    import torch
+    M, N, K = 512, 256, 256
+    a, b, c32 = operands(M, N, K, True, False, 7200)
+    c = rng.matrix("upm1_f16", 7204, (M, N)) if c16 else c32
+    kw = dict(c=Float16 if c16 else Float32, d=Float16 if d16 else Float32)
+    dt = torch.float16 if d16 else torch.float32
+    d4 = helpers.run_gpu(config(M, N, K, True, False, (2, 2), **kw), a, b, c, (M, N), d_dtype=dt, kernel=Kernel.matmul_pipelined)
+    d8 = helpers.run_gpu(config(M, N, K, True, False, (2, 4), **kw), a, b, c, (M, N), d_dtype=dt, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, d8)
+    assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, True, False)) <= TOL
+
+
+def test_bf16_operands(gpu):
+    import torch
+    M, N, K = 256, 256, 192
+    a = gk.bf16_bits(rng.matrix("upm1_f32", 7301, (M, K)))      # uint16 arrays are bfloat16 bit patterns
+    b = gk.bf16_bits(rng.matrix("upm1_f32", 7302, (K, N)))
+    c = rng.matrix("upm1_f32", 7303, (M, N))
+    four, eight = config(M, N, K, False, False, (2, 2), ab=BFloat16), config(M, N, K, False, False, (2, 4), ab=BFloat16)
+    assert "_w2x2_" in gk.kernel_name(four, Kernel.matmul_pipelined)
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined))
+    assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N))) <= TOL
+
+
+def test_c_and_d_off_a_16_byte_boundary(gpu):
+    """Bounds-checked layouts take any pointer: C and D that start 4 bytes into a 16-byte line go element by element."""
+    import torch
+    M, N, K = 256, 256, 128
+    a, b, c = operands(M, N, K, False, False, 7400)
+    conf = config(M, N, K, False, False, (2, 2), checked=True)
+    assert "_w2x2_" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    A, B = gk.colmajor(a), gk.colmajor(b)
+    cbuf = torch.zeros(M * N + 1, dtype=torch.float32, device="cuda")
+    dbuf = torch.full((M * N + 1,), float("nan"), dtype=torch.float32, device="cuda")
+    C = cbuf[1:].view(N, M).t()
+    D = dbuf[1:].view(N, M).t()
+    C.copy_(torch.from_numpy(c).cuda())
+    assert C.data_ptr() % 16 == 4 and D.data_ptr() % 16 == 4
+    gk.matmul(conf, A, B, C, D, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    d = D.cpu().numpy()
+    assert np.array_equal(d, helpers.run_gpu(config(M, N, K, False, False, (2, 4)), a, b, c, (M, N), kernel=Kernel.matmul_pipelined))
+
+
+def test_launches_with_hooks_or_ragged_extents_run_on_eight_waves(gpu):
+    M, N, K = 512, 256, 128
+    a, b, c = operands(M, N, K, False, False, 7500)
+    conf = config(M, N, K, False, False, (2, 2))
+    hooks = dict(transform_regs_to_shared_d=Transform.Elementwise(Transform.relu))
+    bias = rng.normal_f32(7504, N)
+    name = gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=hooks)
+    print("with a hook:", name, flush=True)
+    assert "_w2x4_" in name and "fused" in name
+    d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=hooks, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
+    ref = helpers.run_gpu(config(M, N, K, False, False, (2, 4)), a, b, c, (M, N), transforms=hooks, epilogue_cls=Epilogue.Bias, bias=bias,
+                          kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d, ref)
+    assert oracle.rel_frobenius(d, np.maximum(oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False), 0.0) + bias[None, :]) <= TOL
+    # extents that are not whole tiles (bounds-checked layouts)
+    M2, N2, K2 = 300, 520, 136
+    a2, b2, c2 = operands(M2, N2, K2, False, False, 7510)
+    ragged = config(M2, N2, K2, False, False, (2, 2), checked=True)
+    assert "_w2x4_" in gk.kernel_name(ragged, Kernel.matmul_pipelined)
+    d2 = helpers.run_gpu(ragged, a2, b2, c2, (M2, N2), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(d2, oracle.gemm_f64(a2, b2, c2, 1.0, 1.0, False, False)) <= TOL
+
+
+def test_default_configuration_of_a_large_product(gpu):
+    """get_config picks the four-wave arrangement for plain products made of whole 256 x 256 x 64 tiles."""
+    M = N = K = 1024
+    col = Layout.UnsafeAlignedColMajor
+    conf = gk.get_config(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+                         global_a_layout=col[Float16], global_c_layout=col[Float32], block_shape=NT(M=256, N=256, K=64))
+    assert conf.warps_per_block == 4 and (conf.compute_warp.M, conf.compute_warp.N) == (128, 128)
+    a, b, c = operands(M, N, K, False, False, 7600)
+    d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(d, helpers.run_oracle(conf, a, b, c, (M, N))) <= TOL
