@@ -243,7 +243,7 @@ int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_
 }
 
 // The arrangement of four waves with 128 x 128 wave tiles (one wave per SIMD, see Cfg::SOLO) is compiled for plain
-// products without hooks whose extents are whole numbers of tiles.  Any other launch of such a configuration runs the
+// products without hooks or bias whose extents are whole numbers of tiles.  Any other launch of such a configuration runs the
 // eight-wave arrangement of the same block shape, which gives the same bits (the order of the k-steps and of the
 // products inside them does not depend on how the tile is dealt out to waves).
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {

@@ -482,8 +482,13 @@ struct MfmaGemmConfig {
   static_assert(PAIR || (!opk_complex_k(A_KIND_) && !opk_complex_k(B_KIND_)), "OPK_KSPLIT belongs to the complex-pair products");
 };
 
-template <class Cfg>
+// CPATH (Cfg::SOLO only; 0 elsewhere): how C comes in and D goes out.  1: FP32 C and D with 16-byte accesses, straight into
+// and out of the accumulation registers; 2: no C, D as in 1; 0: anything else.  One kernel per path, chosen by the host
+// (solo_cd_path): where the paths met in one kernel, the register allocator gave the accumulators different registers
+// on each and shuffled 250 of them in front of the K loop.
+template <class Cfg, int CPATH = 0>
 __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs args) {
+  static_assert(CPATH == 0 || Cfg::SOLO, "the C / D paths belong to the one-wave-per-SIMD instances");
   typedef typename Cfg::T T;
   typedef typename Cfg::GA GA;
   typedef typename Cfg::GB GB;
@@ -775,8 +780,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // a block: 16 contiguous bytes of a column-major FP32 C / D.  The loads go straight into the accumulation registers.
   [[maybe_unused]] const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane / MI), solo_col = n0 + wn * Cfg::WTN + (lane % MI);
   if constexpr (Cfg::SOLO) {
-    // (16-byte accesses where the pointer and the leading dimension allow them, else element by element)
-    if (load_c && args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0) {
+    if constexpr (CPATH == 1) {
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
@@ -789,6 +793,33 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) asm volatile("" : "+a"(acc[fi][fj]));
+    } else if (load_c && args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0) {
+      // (FP32 C next to a D that is not: 16-byte loads through ordinary registers)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi)
+          acc[fi][fj] = *(const float4v*)((const float*)args.c + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc);
+    } else if (load_c && args.c_dtype != DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 1)) & 7u) == 0) {
+      // 16-bit C: the lane's four rows are 8 contiguous bytes
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc;
+          const int2v raw = *(const int2v*)((const char*)args.c + off * 2);
+          if (args.c_dtype == DT_F16) {
+            typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+            const half4 h = __builtin_bit_cast(half4, raw);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[fi][fj][v] = (float)h[v];
+          } else {
+            acc[fi][fj][0] = __builtin_bit_cast(float, raw[0] << 16);
+            acc[fi][fj][1] = __builtin_bit_cast(float, (int)((unsigned)raw[0] & 0xFFFF0000u));
+            acc[fi][fj][2] = __builtin_bit_cast(float, raw[1] << 16);
+            acc[fi][fj][3] = __builtin_bit_cast(float, (int)((unsigned)raw[1] & 0xFFFF0000u));
+          }
+        }
     } else if (load_c) {
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
@@ -1463,13 +1494,39 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
     const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane_e / MI), solo_col = n0 + wn * Cfg::WTN + (lane_e % MI);
-    if (args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0) {
+    if constexpr (CPATH != 0) {
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           float* dp = (float*)args.d + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd;
           asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
+        }
+    } else if (args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0) {
+      // (FP32 D next to a C that is not)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          asm volatile("" : "+a"(acc[fi][fj]));
+          *(float4v*)((float*)args.d + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd) = acc[fi][fj];
+        }
+    } else if (args.d_dtype != DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 1)) & 7u) == 0) {
+      // 16-bit D: one rounding per value, 8 contiguous bytes per lane and block
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          asm volatile("" : "+a"(acc[fi][fj]));
+          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd;
+          unsigned short b[4];
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            b[v] = args.d_dtype == DT_F16 ? __builtin_bit_cast(unsigned short, (_Float16)acc[fi][fj][v]) : __builtin_bit_cast(unsigned short, (__bf16)acc[fi][fj][v]);
+          int2v out;
+          out[0] = (int)((unsigned)b[0] | ((unsigned)b[1] << 16));
+          out[1] = (int)((unsigned)b[2] | ((unsigned)b[3] << 16));
+          *(int2v*)((char*)args.d + off * 2) = out;
         }
     } else {
 #pragma unroll
@@ -1546,6 +1603,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       }
     }
   }
+}
+
+// Which of the C / D paths of a Cfg::SOLO instance a launch takes (16-byte accesses where the pointers and the leading
+// dimensions allow them).
+inline int solo_cd_path(const GemmArgs& args) {
+  const bool d_wide = args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0;
+  const bool c_wide = args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0;
+  if (d_wide && args.c_mode != 0 && c_wide) return 1;
+  if (d_wide && args.c_mode == 0) return 2;
+  return 0;
 }
 
 }  // namespace gk

@@ -31,7 +31,8 @@ struct InstanceInfo {
 typedef int (*FamilyFn)(const InstanceKey& key, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode,
                         InstanceInfo* info, hipError_t* err);
 
-template <class Cfg, class Kernel>
+// (TAG tells the kernels of one configuration apart: the record of raised LDS limits below is per instantiation)
+template <class Cfg, int TAG = 0, class Kernel>
 inline int run_instance(Kernel kernel, const char* name, const GemmArgs& args, dim3 grid, hipStream_t stream, int mode,
                         InstanceInfo* info, hipError_t* err, int lds_bytes, int threads) {
   info->name = name;

@@ -113,21 +113,31 @@ def test_c_and_d_off_a_16_byte_boundary(gpu):
     assert np.array_equal(d, helpers.run_gpu(config(M, N, K, False, False, (2, 4)), a, b, c, (M, N), kernel=Kernel.matmul_pipelined))
 
 
-def test_launches_with_hooks_or_ragged_extents_run_on_eight_waves(gpu):
-    M, N, K = 512, 256, 128
-    a, b, c = operands(M, N, K, False, False, 7500)
-    conf = config(M, N, K, False, False, (2, 2))
-    hooks = dict(transform_regs_to_shared_d=Transform.Elementwise(Transform.relu))
-    bias = rng.normal_f32(7504, N)
-    name = gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=hooks)
-    print("with a hook:", name, flush=True)
-    assert "_w2x4_" in name and "fused" in name
-    d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=hooks, epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
-    ref = helpers.run_gpu(config(M, N, K, False, False, (2, 4)), a, b, c, (M, N), transforms=hooks, epilogue_cls=Epilogue.Bias, bias=bias,
-                          kernel=Kernel.matmul_pipelined)
-    assert np.array_equal(d, ref)
-    assert oracle.rel_frobenius(d, np.maximum(oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False), 0.0) + bias[None, :]) <= TOL
-    # extents that are not whole tiles (bounds-checked layouts)
+@pytest.mark.parametrize("epilogue_cls", [Epilogue.Bias, Epilogue.BiasRow])
+def test_launches_with_hooks_or_a_bias_run_on_eight_waves(gpu, epilogue_cls):
+    M, N, K = 512, 256, 192
+    a, b, c = operands(M, N, K, False, True, 7500)
+    E = Transform.Elementwise
+    hooks = dict(transform_global_to_shared_a=E(lambda x: x * 0.5), transform_global_to_shared_c=E(lambda x: x * 0.25),
+                 transform_shared_to_regs_c=E(lambda x: x + 1.0), transform_regs_to_shared_d=E(Transform.relu),
+                 transform_shared_to_global_d=E(lambda x: x * 3.0))
+    bias = rng.normal_f32(7504, N if epilogue_cls is Epilogue.Bias else M)
+    four, eight = config(M, N, K, False, True, (2, 2)), config(M, N, K, False, True, (2, 4))
+    name = gk.kernel_name(four, Kernel.matmul_pipelined, transforms=hooks, epilogue=epilogue_cls(None))
+    print("with hooks:", name, flush=True)
+    assert "_w2x4_" in name and name.endswith("_fused_cd")
+    assert "_w2x4_" in gk.kernel_name(four, Kernel.matmul_pipelined, epilogue=epilogue_cls(None))       # a bias alone
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), transforms=hooks, epilogue_cls=epilogue_cls, bias=bias, kernel=Kernel.matmul_pipelined)
+    d8 = helpers.run_gpu(eight, a, b, c, (M, N), transforms=hooks, epilogue_cls=epilogue_cls, bias=bias, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, d8)
+    ref = helpers.run_oracle(four, a, b, c, (M, N), transforms=hooks, epilogue=epilogue_cls(0), bias=bias)
+    assert oracle.rel_frobenius(d4, ref) <= TOL
+    bias2d = bias[None, :] if epilogue_cls is Epilogue.Bias else bias[:, None]
+    acc = 0.5 * (a.astype(np.float64) @ b.astype(np.float64).T) + (0.25 * c.astype(np.float64) + 1.0)
+    assert oracle.rel_frobenius(d4, 3.0 * (np.maximum(acc, 0.0) + bias2d)) <= TOL
+
+
+def test_ragged_extents_run_on_eight_waves(gpu):
     M2, N2, K2 = 300, 520, 136
     a2, b2, c2 = operands(M2, N2, K2, False, False, 7510)
     ragged = config(M2, N2, K2, False, False, (2, 2), checked=True)
