@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0
 HEADLINE_SETTLE_SECONDS = 0.4
 # HBM bytes per launch of the headline kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # summarised in profiles/ (None until measured)
-MEASURED_TRAFFIC_BYTES = 337_020_314   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131427.6 * 2.0 + 66266.2) KiB
+MEASURED_TRAFFIC_BYTES = 338_074_624   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131153.1 * 2.0 + 67844.8) KiB
 
 
 def parse_args():
