@@ -249,9 +249,19 @@ int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
   const int rc = make_key_as_configured(c, t, e, key, allow_ragged_fast);
   if (rc != GK_OK) return rc;
-  if (key->family == gk::FAMILY_MFMA && key->BM == 256 && key->BN == 256 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2) {
-    const bool whole = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0;
-    if (key->fused != 0 || !whole) key->waves_n = 4;
+  const bool plain = key->family == gk::FAMILY_MFMA, contraction = key->family == gk::FAMILY_GETT;
+  if ((plain || contraction) && key->BM == 256 && key->BN == 256 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2) {
+    bool ok = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0 && key->fused == 0;
+    if (contraction) {
+      // contractions: four consecutive m of a lane are 16 contiguous, aligned bytes of an FP32 C / D
+      const gk_gett_dim& gm = c->gett.m; const gk_gett_dim& gn = c->gett.n;
+      ok = ok && c->global_d_layout.eltype == GK_F32 && (c->global_c_layout.kind == GK_LAYOUT_ZERO || c->global_c_layout.eltype == GK_F32);
+      ok = ok && gm.nmodes >= 1 && gm.stride1[0] == 1 && gm.extent[0] % 4 == 0;
+      ok = ok && c->matmul_shape.K / 64 <= 1024;          // the K tiles the offset table of these instances holds (KTABLE_TILES)
+      for (int i = 1; i < gm.nmodes && i < GK_MAX_MODES; ++i) ok = ok && gm.stride1[i] % 4 == 0;
+      for (int i = 0; i < gn.nmodes && i < GK_MAX_MODES; ++i) ok = ok && gn.stride1[i] % 4 == 0;
+    }
+    if (!ok) key->waves_n = 4;
   }
   return GK_OK;
 }
@@ -854,6 +864,14 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
 
   gk::GemmArgs& args = out->args;
   make_args(conf, a, b, c, d, transforms, epilogue, &args);
+  if (!custom && key.family == gk::FAMILY_GETT && key.BM == 256 && key.waves_m == 2 && key.waves_n == 2 && gk::solo_cd_path(args) == 0) {
+    // a contraction on the four-wave arrangement moves C and D 16 bytes at a time: pointers that do not allow it
+    // run the eight-wave arrangement (see make_key)
+    key.waves_n = 4;
+    gk::FamilyFn fn8 = family_fn(key);
+    hipError_t e8 = hipSuccess;
+    if (!fn8 || !fn8(key, args, dim3(1), nullptr, 0, &info, &e8)) return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance for this contraction");
+  }
 
   // aligned layouts move 16-byte vectors (reference src/layout.jl:22-34 traps on the device; here it is a host check)
   auto check_aligned = [&](const gk_layout& l, const void* p, long long ld, const char* what) -> int {

@@ -392,4 +392,14 @@ __device__ __forceinline__ void wait_vmcnt() {
 __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
+// Which of the C / D paths of a one-wave-per-SIMD instance (MfmaGemmConfig::SOLO) a launch takes (16-byte accesses where the pointers and the leading
+// dimensions allow them).
+inline int solo_cd_path(const GemmArgs& args) {
+  const bool d_wide = args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0;
+  const bool c_wide = args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0;
+  if (d_wide && args.c_mode != 0 && c_wide) return 1;
+  if (d_wide && args.c_mode == 0) return 2;
+  return 0;
+}
+
 }  // namespace gk

@@ -415,7 +415,7 @@ struct MfmaGemmConfig {
   // One wave per SIMD: four waves with wave tiles of 64 16x16 blocks (all 256 accumulation registers), two LDS stages.
   // The K loop of these instances is written out instruction slot by instruction slot (see the SOLO loop).
   static constexpr bool SOLO = MI_ == 16 && WAVES_M_ * WAVES_N_ == 4 && (BM_ / WAVES_M_ / 16) * (BN_ / WAVES_N_ / 16) == 64 && STAGES_ == 2 &&
-                               (BK_ / 32) % 2 == 0 && FUSE_ == 0 && !GETT_ && FIX_ == FIX_NONE && !SPLITK_ &&
+                               (BK_ / 32) % 2 == 0 && FUSE_ == 0 && FIX_ == FIX_NONE && !SPLITK_ &&
                                A_KIND_ != OPK_KSPLIT && B_KIND_ != OPK_KSPLIT && (GK_FORCE_SYNC_FRAGS == 0);
   // plain real products may have a last tile row / column that sticks out over M / N and a last, partial K
   // tile (the host asks for it only with 16-byte aligned columns, M or N a multiple of 8 where that index is
@@ -462,7 +462,12 @@ struct MfmaGemmConfig {
   typedef OperandGeom<BM, BK, A_KIND> GA;
   typedef OperandGeom<BN, BK, B_KIND> GB;
   static constexpr int STAGE_BYTES = GA::BYTES + GB::BYTES;
-  static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
+  // Contractions on the one-wave-per-SIMD arrangement keep the element offsets of every K tile in A and in B in a table
+  // behind the LDS stages (two 64-bit offsets per tile, filled before the loop): walking the K modes tile by tile takes
+  // some sixty scalar instructions and a dozen branches, which a lone wave on a SIMD cannot hide.
+  static constexpr int KTABLE_BYTES = (SOLO && GETT_) ? 16 * 1024 : 0;     // 1024 K tiles
+  static constexpr int KTABLE_TILES = KTABLE_BYTES / 16;
+  static constexpr int LDS_BYTES = STAGE_BYTES * STAGES + KTABLE_BYTES;
   static constexpr int DMA_A = (GA::NDMA + NWAVES - 1) / NWAVES;   // per wave, per tile
   static constexpr int DMA_B = (GB::NDMA + NWAVES - 1) / NWAVES;
   static constexpr int DMA_PER_TILE = DMA_A + DMA_B;
@@ -668,6 +673,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
   for (int s = 0; s < (Cfg::SOLO ? STAGES : STAGES - 1); ++s)
     if (s < KT) issue_tile(s);      // (SOLO: both stages are free and the loop issues tile kt + 2 from tile kt)
+  if constexpr (Cfg::SOLO && Cfg::GETT) {
+    // element offsets of K tile t in A and in B (published by the barrier in front of the K loop)
+    long long* table = (long long*)(smem + Cfg::STAGE_BYTES * STAGES);
+    for (int t = (int)threadIdx.x; t < KT; t += Cfg::THREADS) {
+      long long oa, ob;
+      gett_offsets32(args.gk, t * BK, oa, ob);
+      table[2 * t] = oa;
+      table[2 * t + 1] = ob;
+    }
+  }
 
   // --- accumulators: C tile (two transforms) or zeros -------------------------------------------
   // 32x32 blocks: lane l owns row m = 32*fi + l%32 and columns n = 32*fj + 8*(v/4) + 4*(l/32) + v%4, v < 16;
@@ -779,13 +794,32 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // SOLO: the A fragment is the first MFMA operand, so a lane owns the rows 4 * (lane / 16) .. + 3 of column lane % 16 of
   // a block: 16 contiguous bytes of a column-major FP32 C / D.  The loads go straight into the accumulation registers.
   [[maybe_unused]] const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane / MI), solo_col = n0 + wn * Cfg::WTN + (lane % MI);
+  // Element offset of the lane's first row of block (fi, fj) in C / D.  Contractions: the lane walks the M modes for its
+  // first row of every row block (the other three follow in the first M mode, whose stride in C / D is 1 and whose extent
+  // is a multiple of 4: the host runs these instances on nothing else) and the N modes for its column of every block column.
+  [[maybe_unused]] long long solo_om[Cfg::GETT ? FM : 1], solo_on[Cfg::GETT ? FN : 1];
+  [[maybe_unused]] auto solo_origins = [&](int row, int col) __attribute__((always_inline)) {
+    if constexpr (Cfg::GETT) {
+      long long t0;
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi) gett_offsets32(args.gm, row + MI * fi, t0, solo_om[fi]);
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj) gett_offsets32(args.gn, col + MI * fj, t0, solo_on[fj]);
+    }
+  };
+  [[maybe_unused]] auto solo_off = [&](int row, int col, int fi, int fj, long long ld) -> long long {
+    if constexpr (Cfg::GETT) return solo_om[fi] + solo_on[fj];
+    else return (long long)(row + MI * fi) + (long long)(col + MI * fj) * ld;
+  };
   if constexpr (Cfg::SOLO) {
+    static_assert(!Cfg::GETT || CPATH != 0, "contractions run the four waves with 16-byte C / D accesses only");
+    if (load_c) solo_origins(solo_row, solo_col);
     if constexpr (CPATH == 1) {
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const float* cp = (const float*)args.c + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc;
+          const float* cp = (const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc);
           asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(acc[fi][fj]) : "v"(cp) : "memory");
         }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -799,14 +833,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
-          acc[fi][fj] = *(const float4v*)((const float*)args.c + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc);
+          acc[fi][fj] = *(const float4v*)((const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc));
     } else if (load_c && args.c_dtype != DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 1)) & 7u) == 0) {
       // 16-bit C: the lane's four rows are 8 contiguous bytes
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc;
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc);
           const int2v raw = *(const int2v*)((const char*)args.c + off * 2);
           if (args.c_dtype == DT_F16) {
             typedef _Float16 half4 __attribute__((ext_vector_type(4)));
@@ -825,7 +859,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldc;
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc);
 #pragma unroll
           for (int v = 0; v < 4; ++v) acc[fi][fj][v] = load_cd(args.c, args.c_dtype, off + v);
         }
@@ -833,7 +867,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
       for (int fi = 0; fi < FM; ++fi)
 #pragma unroll
-        for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = AccV{};
+        for (int fj = 0; fj < FN; ++fj) {
+          acc[fi][fj] = AccV{};
+          asm volatile("" : "+a"(acc[fi][fj]));     // (zeroed in place, in the accumulation registers)
+        }
     }
   } else
   if (Cfg::RAGGED_OK && ragged && load_c) {
@@ -1057,8 +1094,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       // instruction, which then takes the tile pointer from scalar registers and the 32-bit offset from the lane)
       unsigned& o = I < DMA_A ? offa[I < DMA_A ? I : 0] : offb[I < DMA_A ? 0 : I - DMA_A];
       asm volatile("" : "+v"(o));
-      if constexpr (I < DMA_A) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(ga + o), GK_LDS_PTR(void, sa + (wave + I * NWAVES) * 1024), 16, 0, 0);
-      else __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(gb + o), GK_LDS_PTR(void, sb + (wave + (I - DMA_A) * NWAVES) * 1024), 16, 0, 0);
+      if constexpr (I < DMA_A) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR((Cfg::GETT ? part_a : ga) + o), GK_LDS_PTR(void, sa + (wave + I * NWAVES) * 1024), 16, 0, 0);
+      else __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR((Cfg::GETT ? part_b : gb) + o), GK_LDS_PTR(void, sb + (wave + (I - DMA_A) * NWAVES) * 1024), 16, 0, 0);
     };
     // LDS instruction R of the fragment reads of k-step KS2 (of the stage the readers stand at), into buffer KS2 & 1
     auto read_op = [&](auto r_c, auto ks2_c) __attribute__((always_inline)) {
@@ -1101,6 +1138,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // tile kt + 2 in step kt, and the last tile once more where there is no such tile (the DMA is unconditional: a
     // branch around it costs more issue slots than the instruction; the data lands in a stage nobody reads any more)
     if (KT < 3 && KT > 0) { ga -= a_step; gb -= b_step; }
+    [[maybe_unused]] int4v ktab;                              // contractions: a table entry on its way from LDS
     if (KT > 1) wait_vmcnt<DPT>(); else wait_vmcnt<0>();
     block_barrier();
     ra.set_stage(lds_base);
@@ -1120,9 +1158,24 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           const unsigned stage_addr = lds_base + (unsigned)((kt + 1) & 1) * Cfg::STAGE_BYTES;
           ra.set_stage(stage_addr);
           rb.set_stage(stage_addr + GA::BYTES);
+          if constexpr (Cfg::GETT) {
+            // (read a k-step ago; the same value in every lane)
+            asm volatile("" : "+v"(ktab));
+            const unsigned long long oa = ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane(ktab[1]) << 32) | (unsigned)__builtin_amdgcn_readfirstlane(ktab[0]);
+            const unsigned long long ob = ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane(ktab[3]) << 32) | (unsigned)__builtin_amdgcn_readfirstlane(ktab[2]);
+            part_a = ga + (long long)oa * 2;
+            part_b = gb + (long long)ob * 2;
+          }
           phase(ks_c, Yes{}, kt & 1);
           if (kt + 3 < KT) { ga += a_step; gb += b_step; }
         } else {
+          if constexpr (Cfg::GETT && ks == 0) {
+            // the table entry of the tile that the next k-step fetches (tile kt + 2, or the last tile once more); it
+            // arrives with the fragments of that k-step
+            const int t = kt + 2 < KT ? kt + 2 : KT - 1;
+            const unsigned addr = lds_base + (unsigned)(Cfg::STAGE_BYTES * STAGES) + 16u * (unsigned)t;
+            asm volatile("ds_read_b128 %0, %1" : "=v"(ktab) : "v"(addr) : "memory");
+          }
           phase(ks_c, No{}, 0);
         }
       });
@@ -1494,12 +1547,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
     const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane_e / MI), solo_col = n0 + wn * Cfg::WTN + (lane_e % MI);
+    solo_origins(solo_row, solo_col);
     if constexpr (CPATH != 0) {
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          float* dp = (float*)args.d + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd;
+          float* dp = (float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd);
           asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
         }
     } else if (args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0) {
@@ -1509,7 +1563,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));
-          *(float4v*)((float*)args.d + (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd) = acc[fi][fj];
+          *(float4v*)((float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd)) = acc[fi][fj];
         }
     } else if (args.d_dtype != DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 1)) & 7u) == 0) {
       // 16-bit D: one rounding per value, 8 contiguous bytes per lane and block
@@ -1518,7 +1572,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));
-          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd;
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd);
           unsigned short b[4];
 #pragma unroll
           for (int v = 0; v < 4; ++v)
@@ -1534,7 +1588,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));      // (stays where it is until this branch is taken)
-          const long long off = (long long)(solo_row + MI * fi) + (long long)(solo_col + MI * fj) * args.ldd;
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd);
 #pragma unroll
           for (int v = 0; v < 4; ++v) store_cd(args.d, args.d_dtype, off + v, acc[fi][fj][v]);
         }
@@ -1603,16 +1657,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       }
     }
   }
-}
-
-// Which of the C / D paths of a Cfg::SOLO instance a launch takes (16-byte accesses where the pointers and the leading
-// dimensions allow them).
-inline int solo_cd_path(const GemmArgs& args) {
-  const bool d_wide = args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0;
-  const bool c_wide = args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0;
-  if (d_wide && args.c_mode != 0 && c_wide) return 1;
-  if (d_wide && args.c_mode == 0) return 2;
-  return 0;
 }
 
 }  // namespace gk

@@ -251,7 +251,7 @@ def _default_waves(operator, block_shape, checked=False, planar=False, gett=Fals
     key = (block_shape["M"], block_shape["N"], block_shape["K"])
     if gett and key == (64, 64, 32):
         return (1, 1)
-    if operator.kind == Operator.MFMA and not gett and key == _SOLO_TILE and whole_tiles:
+    if operator.kind == Operator.MFMA and key == _SOLO_TILE and whole_tiles:
         return _SOLO_WAVES
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         table = _FPU_TILES

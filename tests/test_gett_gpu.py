@@ -175,3 +175,52 @@ def test_general_mode_extents_are_exact_against_einsum(gpu, ext, block, what):
               transform_shared_to_global_d=Transform.Elementwise(lambda x: x * 2.0))
     torch.cuda.synchronize()
     assert np.array_equal(gk.to_numpy(d).astype(np.float64), 2.0 * (want + C))
+
+
+def _four_wave_case(d_modes, with_c):
+    """D = sum_{e,f} A[a,e,b,f] * B[d,f,c,e] (+ C) on 256 x 256 x 64 tiles: M = a*b = 512, N = c*d = 256, K = e*f = 128."""
+    ext = dict(a=64, b=8, c=4, d=64, e=64, f=2)
+    kw = dict(block_shape=(256, 256, 64), zero_c=not with_c)
+    conf, gmap = configs.gett_config("aebf", "dfce", d_modes, ext, **kw)
+    eight, _ = configs.gett_config("aebf", "dfce", d_modes, ext, warps_per_block=8,
+                                   compute_warp=gk.NT(M=128, N=64, K=16), **kw)
+    A = rng.matrix("upm1_f16", 5101, tuple(ext[ch] for ch in "aebf"))
+    B = rng.matrix("upm1_f16", 5102, tuple(ext[ch] for ch in "dfce"))
+    d_shape = tuple(ext[ch] for ch in d_modes)
+    C = rng.matrix("upm1_f32", 5103, d_shape) if with_c else None
+
+    def run(cf):
+        a, b = gk.colmajor(A), gk.colmajor(B)
+        c = gk.colmajor(C) if with_c else None
+        d = gk.colmajor_empty(d_shape, torch.float32)
+        d.fill_(float("nan"))
+        gk.matmul(cf, a, b, c, d, kernel=Kernel.matmul_pipelined)
+        torch.cuda.synchronize()
+        return gk.to_numpy(d)
+
+    want = np.einsum(f"aebf,dfce->{d_modes}", A.astype(np.float64), B.astype(np.float64)) + (C.astype(np.float64) if with_c else 0.0)
+    return conf, eight, run, want
+
+
+@pytest.mark.parametrize("with_c", [False, True])
+def test_four_waves_give_the_bits_of_eight_waves(gpu, with_c):
+    """The first M mode is the contiguous one of C and D: four consecutive m of a lane are 16 bytes, and the
+    contraction runs on the one-wave-per-SIMD arrangement of the 256 x 256 x 64 tile."""
+    conf, eight, run, want = _four_wave_case("abcd", with_c)
+    assert conf.warps_per_block == 4
+    name = gk.kernel_name(conf, Kernel.matmul_pipelined)
+    print("case", with_c, name, flush=True)
+    assert "_w2x2_" in name and name.endswith("_gett")
+    assert "_w2x4_" in gk.kernel_name(eight, Kernel.matmul_pipelined)
+    d4, d8 = run(conf), run(eight)
+    assert np.array_equal(d4, d8)
+    assert oracle.rel_frobenius(d4, want) <= 1e-3
+
+
+def test_four_wave_contraction_falls_back_where_c_and_d_are_not_contiguous_along_m(gpu):
+    """D[c,a,b,d]: an N mode is the contiguous one, a lane's four rows are 4 * 4 bytes apart: eight waves."""
+    conf, eight, run, want = _four_wave_case("cabd", True)
+    assert "_w2x4_" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    d = run(conf)
+    assert np.array_equal(d, run(eight))
+    assert oracle.rel_frobenius(d, want) <= 1e-3
