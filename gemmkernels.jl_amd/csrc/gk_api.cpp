@@ -251,7 +251,26 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   if (rc != GK_OK) return rc;
   const bool plain = key->family == gk::FAMILY_MFMA, contraction = key->family == gk::FAMILY_GETT;
   if ((plain || contraction) && key->BM == 256 && key->BN == 256 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2) {
-    bool ok = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0 && key->fused == 0;
+    bool ok = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0;
+    if (key->fused == 3 && plain) {
+      // hooks of C and D and a bias: the four waves take what has a closed form (fuse level 4 of the kernel): no hook on
+      // C, at most one op in each hook of D, and a power-of-two scale of A or B folded into the accumulators only where
+      // there is no C to scale the other way
+      gk_transforms folded_storage;
+      float post = 1.0f;
+      const gk_transforms* tf = fold_pow2_scales(c, t, &folded_storage, &post);
+      auto real_ops = [&](int h) {
+        int n = 0;
+        if (tf) for (int i = 0; i < tf->hook[h].n_ops && i < GK_MAX_OPS; ++i) if (tf->hook[h].ops[i].kind != GK_T_IDENTITY) ++n;
+        return n;
+      };
+      const bool closed = real_ops(GK_HOOK_GLOBAL_TO_SHARED_C) == 0 && real_ops(GK_HOOK_SHARED_TO_REGS_C) == 0 &&
+                          real_ops(GK_HOOK_REGS_TO_SHARED_D) <= 1 && real_ops(GK_HOOK_SHARED_TO_GLOBAL_D) <= 1 &&
+                          (post == 1.0f || c->global_c_layout.kind == GK_LAYOUT_ZERO);
+      if (closed) key->fused = 4; else ok = false;
+    } else if (key->fused != 0) {
+      ok = false;
+    }
     if (contraction) {
       // contractions: four consecutive m of a lane are 16 contiguous, aligned bytes of an FP32 C / D
       const gk_gett_dim& gm = c->gett.m; const gk_gett_dim& gn = c->gett.n;
@@ -261,6 +280,16 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
       for (int i = 1; i < gm.nmodes && i < GK_MAX_MODES; ++i) ok = ok && gm.stride1[i] % 4 == 0;
       for (int i = 0; i < gn.nmodes && i < GK_MAX_MODES; ++i) ok = ok && gn.stride1[i] % 4 == 0;
     }
+    if (!ok) {
+      key->waves_n = 4;
+      if (key->fused == 4) key->fused = 3;
+    }
+  }
+  // ... and for the complex / dual product on interleaved matrices of an 'N','N' launch (real tile 256 x 256 x 64)
+  if (key->family == gk::FAMILY_COMPLEX && key->variant <= 1 && key->BM == 128 && key->BN == 128 && key->BK == 64 && key->waves_m == 2 &&
+      key->waves_n == 2) {
+    const bool ok = c->matmul_shape.M % 128 == 0 && c->matmul_shape.N % 128 == 0 && c->matmul_shape.K % 64 == 0 && key->fused == 0 &&
+                    key->a_kmajor == 0 && key->b_kmajor == 1;
     if (!ok) key->waves_n = 4;
   }
   return GK_OK;

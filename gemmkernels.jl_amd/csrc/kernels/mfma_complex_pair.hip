@@ -31,6 +31,20 @@ int family_complex_pair(const InstanceKey& key, const GemmArgs& args, dim3 grid,
   GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, 0, 0, dual_, "mfma_" TAG "_nt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, 1, 1, dual_, "mfma_" TAG "_tn_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_PAIR(bm_, bn_, bk_, wm_, wn_, st_, 1, 0, dual_, "mfma_" TAG "_tt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)
+  // 'N','N' on four waves, one per SIMD (MfmaGemmConfig::SOLO; launches without hooks): one kernel per way of moving C and D
+#define GK_PAIR_SOLO(dual_, NAME)                                                                                         \
+  if (key.BM == 128 && key.BN == 128 && key.BK == 64 && key.waves_m == 2 && key.waves_n == 2 && key.a_kmajor == 0 &&     \
+      key.b_kmajor == 1 && key.variant == dual_ && key.fused == 0) {                                                      \
+    typedef MfmaGemmConfig<256, 256, 64, 2, 2, 2, OPK_MMAJOR, OPK_KSPLIT, _Float16, 0, false, (dual_ ? FIX_PAIR_DUAL : FIX_PAIR), false, 16> Cfg; \
+    static_assert(Cfg::SOLO, "the four-wave arrangement");                                                               \
+    const int path = mode == 1 ? solo_cd_path(args) : 0;                                                                 \
+    if (path == 1) return run_instance<Cfg, 1>(mfma_gemm_kernel<Cfg, 1>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
+    if (path == 2) return run_instance<Cfg, 2>(mfma_gemm_kernel<Cfg, 2>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
+    return run_instance<Cfg, 0>(mfma_gemm_kernel<Cfg, 0>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
+  }
+  GK_PAIR_SOLO(0, "mfma_complex_pair_nn_128x128x64_w2x2")
+  GK_PAIR_SOLO(1, "mfma_dual_pair_nn_128x128x64_w2x2")
+#undef GK_PAIR_SOLO
   GK_PAIR_T(128, 128, 64, 2, 4, 2, 0, "complex_pair")
   GK_PAIR_T(64, 64, 64, 2, 2, 2, 0, "complex_pair")
   GK_PAIR_T(64, 64, 32, 2, 2, 4, 0, "complex_pair")

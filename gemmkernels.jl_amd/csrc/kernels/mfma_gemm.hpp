@@ -271,8 +271,10 @@ struct FragReader {
   // one LDS instruction of read<FI, KS>: H < OPS
   template <int FI, int KS, int H>
   __device__ __forceinline__ void read_op(Raw& r) const {
-    static_assert(!opk_complex_k(KIND), "plain operands");
-    if constexpr (KIND == OPK_KMAJOR) {
+    if constexpr (opk_complex_k(KIND)) {
+      if constexpr (H == 0) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[2 * KS]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
+      else asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q1) : "v"(cur[2 * KS + 1]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
+    } else if constexpr (KIND == OPK_KMAJOR) {
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r.q) : "v"(cur[KS < NBASE ? KS : 0]), "n"(FI * FRAG_ROWS * G::ROW_BYTES) : "memory");
     } else if constexpr (H == 0) {
       asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r.lo) : "v"(mmajor_addr<FI>()), "n"((KS * KSTEP_K) * G::ROW_BYTES) : "memory");
@@ -405,7 +407,9 @@ struct MfmaGemmConfig {
   // 0: no transform and no bias; 1: C / D hooks, bias and at most one exact 16-bit scale on A and on B
   // (a packed multiply per fragment); 2: arbitrary op lists on A and B as well (evaluated in fp32 per
   // element inside the K loop: complete, and markedly slower); 3: C / D hooks and bias only, the K loop of
-  // level 0 (also what a power-of-two scale of A or B runs on: the host folds it into the accumulators)
+  // level 0 (also what a power-of-two scale of A or B runs on: the host folds it into the accumulators);
+  // 4 (one-wave-per-SIMD instances only): level 3 narrowed to what the host can name in closed form -- no hook on C, at
+  // most one op in each hook of D, a bias, a folded scale when there is no C -- which needs no op list walked on the device
   static constexpr int FUSE = FUSE_;
   static constexpr bool FUSED = FUSE_ != 0;
   static constexpr bool FUSED_AB_GENERIC = FUSE_ == 2;
@@ -415,8 +419,10 @@ struct MfmaGemmConfig {
   // One wave per SIMD: four waves with wave tiles of 64 16x16 blocks (all 256 accumulation registers), two LDS stages.
   // The K loop of these instances is written out instruction slot by instruction slot (see the SOLO loop).
   static constexpr bool SOLO = MI_ == 16 && WAVES_M_ * WAVES_N_ == 4 && (BM_ / WAVES_M_ / 16) * (BN_ / WAVES_N_ / 16) == 64 && STAGES_ == 2 &&
-                               (BK_ / 32) % 2 == 0 && FUSE_ == 0 && FIX_ == FIX_NONE && !SPLITK_ &&
-                               A_KIND_ != OPK_KSPLIT && B_KIND_ != OPK_KSPLIT && (GK_FORCE_SYNC_FRAGS == 0);
+                               (BK_ / 32) % 2 == 0 && !SPLITK_ && (GK_FORCE_SYNC_FRAGS == 0) &&
+                               ((FIX_ == FIX_NONE && (FUSE_ == 0 || FUSE_ == 4) && A_KIND_ != OPK_KSPLIT && B_KIND_ != OPK_KSPLIT) ||
+                                // ... and the complex / dual real-view product of an 'N','N' launch (A contiguous along m, B along k)
+                                ((FIX_ == FIX_PAIR || FIX_ == FIX_PAIR_DUAL) && FUSE_ == 0 && !GETT_ && A_KIND_ == OPK_MMAJOR && B_KIND_ == OPK_KSPLIT));
   // plain real products may have a last tile row / column that sticks out over M / N and a last, partial K
   // tile (the host asks for it only with 16-byte aligned columns, M or N a multiple of 8 where that index is
   // the contiguous one of A or B, and K a multiple of 8): loads are clamped, the C load and the D store
@@ -637,12 +643,21 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     }
     const char* pa = Cfg::GETT ? part_a : ga;
     const char* pb = Cfg::GETT ? part_b : gb;
+    // (the offsets pass through an empty assembly statement: their widening to 64 bits then stays next to the DMA
+    // instruction, which takes the tile pointer from scalar registers and the 32-bit offset from the lane, instead of
+    // being hoisted out of the loop as sixteen register pairs and a 64-bit addition per instruction)
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i)
-      if ((i % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      if ((i % NP) == P) {
+        asm volatile("" : "+v"(offa[i]));
+        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      }
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i)
-      if (((DMA_A + i) % NP) == P) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      if (((DMA_A + i) % NP) == P) {
+        asm volatile("" : "+v"(offb[i]));
+        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+      }
     if constexpr (P == NP - 1 && !Cfg::GETT) {
       ga += a_step;
       gb += b_step;
@@ -793,7 +808,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const bool load_c = args.c_mode != 0 && (!Cfg::SPLITK || blockIdx.z == 0);
   // SOLO: the A fragment is the first MFMA operand, so a lane owns the rows 4 * (lane / 16) .. + 3 of column lane % 16 of
   // a block: 16 contiguous bytes of a column-major FP32 C / D.  The loads go straight into the accumulation registers.
-  [[maybe_unused]] const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane / MI), solo_col = n0 + wn * Cfg::WTN + (lane % MI);
+  // (complex products: rows of the real view -- a lane's four rows are two complex numbers -- and complex columns, of which
+  // the block columns fj and fj + FN / 2 hold the products with the real and with the imaginary parts of B)
+  constexpr int SFN = Cfg::COLS_FRAG ? FN / 2 : FN;          // block columns that C / D see
+  [[maybe_unused]] const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane / MI);
+  [[maybe_unused]] const int solo_col = (Cfg::COLS_FRAG ? (n0 + wn * Cfg::WTN) / 2 : n0 + wn * Cfg::WTN) + (lane % MI);
   // Element offset of the lane's first row of block (fi, fj) in C / D.  Contractions: the lane walks the M modes for its
   // first row of every row block (the other three follow in the first M mode, whose stride in C / D is 1 and whose extent
   // is a multiple of 4: the host runs these instances on nothing else) and the N modes for its column of every block column.
@@ -816,7 +835,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if (load_c) solo_origins(solo_row, solo_col);
     if constexpr (CPATH == 1) {
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           const float* cp = (const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc);
@@ -824,20 +843,20 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) asm volatile("" : "+a"(acc[fi][fj]));
     } else if (load_c && args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0) {
       // (FP32 C next to a D that is not: 16-byte loads through ordinary registers)
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
           acc[fi][fj] = *(const float4v*)((const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc));
     } else if (load_c && args.c_dtype != DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 1)) & 7u) == 0) {
       // 16-bit C: the lane's four rows are 8 contiguous bytes
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc);
@@ -856,7 +875,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
     } else if (load_c) {
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc);
@@ -871,6 +890,18 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           acc[fi][fj] = AccV{};
           asm volatile("" : "+a"(acc[fi][fj]));     // (zeroed in place, in the accumulation registers)
         }
+    }
+    if constexpr (Cfg::COLS_FRAG) {
+      // the products with the imaginary parts of B start from zero (C came in through the block columns of the real parts)
+      if (load_c) {
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+          for (int fj = SFN; fj < FN; ++fj) {
+            acc[fi][fj] = AccV{};
+            asm volatile("" : "+a"(acc[fi][fj]));
+          }
+      }
     }
   } else
   if (Cfg::RAGGED_OK && ragged && load_c) {
@@ -947,7 +978,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int v = 0; v < NV; ++v) acc[fi][fj][v] = acc[fi][fj][v] * f;
   };
-  if constexpr (Cfg::FUSED) {
+  if constexpr (Cfg::FUSED && !Cfg::SOLO) {
     if (load_c && args.acc_pre_scale != 1.0f) scale_acc(args.acc_pre_scale);
   }
 
@@ -1113,11 +1144,22 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       __builtin_amdgcn_sched_barrier(0);       // no MFMA of the k-step before moves behind the waits in front of this one
 #pragma unroll
       for (int fi = 0; fi < FM; ++fi) { RA::pin_raw(fa[ks & 1][fi]); va[fi] = RA::finish(fa[ks & 1][fi], lane); }
+      // B read as OPK_KSPLIT: a fragment of real parts (block column fj) and one of imaginary parts (fj + FN / 2) are made
+      // of each set of registers read, four byte permutes each, right before the MFMAs that use them first: the block
+      // columns are the outer loop there
+      constexpr bool B_BOTH = Cfg::B_KIND == OPK_KSPLIT;
+      if constexpr (!B_BOTH) {
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[ks & 1][fj]); vb[fj] = RB::finish(fb[ks & 1][fj], lane); }
+        for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[ks & 1][fj]); vb[fj] = RB::finish(fb[ks & 1][fj], lane); }
+      } else {
+#pragma unroll
+        for (int fj = 0; fj < RB::NREAD; ++fj) RB::pin_raw(fb[ks & 1][fj]);
+      }
       static_for<0, NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
-        constexpr int fi = i / FN, fj = (fi & 1) ? FN - 1 - (i % FN) : i % FN;
+        constexpr int o_ = B_BOTH ? i / FM : i / FN, q_ = B_BOTH ? ((o_ & 1) ? FM - 1 - (i % FM) : i % FM) : ((o_ & 1) ? FN - 1 - (i % FN) : i % FN);
+        constexpr int fi = B_BOTH ? q_ : o_, fj = B_BOTH ? o_ : q_;
+        if constexpr (B_BOTH && (i % FM) == 0) vb[fj] = RB::finish(fb[ks & 1][fj % RB::NREAD], lane, fj >= RB::NREAD);
         acc[fi][fj] = Mfma<T, MI>::run(va[fi], vb[fj], acc[fi][fj]);
         // (the scheduling barriers keep every instruction in the slot it is written in)
         if constexpr (DMA && i % GD == 0 && i / GD < DPT) {
@@ -1475,11 +1517,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     }
   }
 
-  if constexpr (Cfg::FUSED) {
+  if constexpr (Cfg::FUSED && !Cfg::SOLO) {      // (SOLO: in its own epilogue)
     if (args.acc_post_scale != 1.0f) scale_acc(args.acc_post_scale);
   }
 
-  if constexpr (Cfg::ROWS_LANE && Cfg::COLS_FRAG) {
+  if constexpr (Cfg::ROWS_LANE && Cfg::COLS_FRAG && !Cfg::SOLO) {
     // As below, with the products of the imaginary parts of B in the column blocks fj + FN / 2: lane 2i holds
     // re A * re B in block fj and re A * im B in block fj + FN / 2, lane 2i+1 im A * re B and im A * im B.
 #pragma unroll
@@ -1494,7 +1536,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           acc[fi][fj][v] = (lane & 1) ? own + other : (Cfg::FIX == FIX_PAIR_DUAL ? own : own - other);
         }
   }
-  if constexpr (Cfg::ROWS_LANE && Cfg::COLS_LANE) {
+  if constexpr (Cfg::ROWS_LANE && Cfg::COLS_LANE && !Cfg::SOLO) {
     // The four real products of a complex element of D = (re A + i im A)(re B + i im B): lane 2i holds, for
     // each of its two complex columns, re A * re B (value 0 / 2) and re A * im B (value 1 / 3), lane 2i+1
     // im A * re B and im A * im B.  The neighbours trade their odd values: lane 2i becomes the real part
@@ -1516,7 +1558,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
   }
 
-  if constexpr (Cfg::ROWS_FRAG && Cfg::COLS_FRAG) {
+  if constexpr (Cfg::ROWS_FRAG && Cfg::COLS_FRAG && !Cfg::SOLO) {
     // The four real products of the elements of D lie in four blocks of the lane: (row blocks of re A | im A) x
     // (column blocks of re B | im B).  Real part re*re - im*im into the upper left block, imaginary part
     // im*re + re*im into the lower left one (dual numbers: re*re, and du*re + re*du); C came in through the same two.
@@ -1528,7 +1570,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         acc[fi + FMH][fj] = acc[fi + FMH][fj] + acc[fi][fj + FNO];
       }
   }
-  if constexpr (Cfg::ROWS_FRAG && Cfg::COLS_LANE) {
+  if constexpr (Cfg::ROWS_FRAG && Cfg::COLS_LANE && !Cfg::SOLO) {
     // re A | im A in the row blocks fi | fi + FM / 2, re B | im B in the values 2v | 2v + 1 of a block
 #pragma unroll
     for (int fi = 0; fi < FMH; ++fi)
@@ -1546,11 +1588,91 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // (the lane number is asked for again: nothing of the store addresses is then kept in registers across the K loop)
     int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
-    const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane_e / MI), solo_col = n0 + wn * Cfg::WTN + (lane_e % MI);
+    const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane_e / MI);
+    const int solo_col = (Cfg::COLS_FRAG ? (n0 + wn * Cfg::WTN) / 2 : n0 + wn * Cfg::WTN) + (lane_e % MI);      // (as before the K loop)
     solo_origins(solo_row, solo_col);
+    if constexpr (Cfg::PAIR) {
+      // The four real products of two complex elements of D in one lane: its rows 0 .. 3 of block (fi, fj) are
+      // re A re B, im A re B of complex row m and of m + 1, those of block (fi, fj + FN / 2) re A im B, im A im B.
+      // Real part re*re - im*im, imaginary part im*re + re*im (dual numbers: re*re, and du*re + re*du), left where
+      // the real view of D has them: values 0 .. 3 of block (fi, fj).  C came in through the same values.
+#pragma unroll
+      for (int fj = 0; fj < SFN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          asm volatile("" : "+a"(acc[fi][fj]));
+          asm volatile("" : "+a"(acc[fi][fj + SFN]));
+          const AccV a = acc[fi][fj], b = acc[fi][fj + SFN];
+          AccV o;
+          o[0] = Cfg::FIX == FIX_PAIR_DUAL ? a[0] : a[0] - b[1];
+          o[1] = a[1] + b[0];
+          o[2] = Cfg::FIX == FIX_PAIR_DUAL ? a[2] : a[2] - b[3];
+          o[3] = a[3] + b[2];
+          acc[fi][fj] = o;
+          asm volatile("" : "+a"(acc[fi][fj]));
+        }
+    }
+    if constexpr (Cfg::FUSE == 4) {
+      // D = op1(op0(s * acc) + bias): one block column at a time leaves the accumulation registers (32 values per lane),
+      // is transformed and stored; the switch on an op is paid once per block column
+      const int k0 = args.t[H_RF2SH_D].n > 0 ? args.t[H_RF2SH_D].kind[0] : (int)T_IDENTITY;
+      const int k1 = args.t[H_SH2GL_D].n > 0 ? args.t[H_SH2GL_D].kind[0] : (int)T_IDENTITY;
+      const float p00 = args.t[H_RF2SH_D].p0[0], p01 = args.t[H_RF2SH_D].p1[0], p10 = args.t[H_SH2GL_D].p0[0], p11 = args.t[H_SH2GL_D].p1[0];
+      const float post = args.acc_post_scale;
+      const int epi = args.epi_kind;
+      const float* bias = args.bias;
+      const bool d_wide = args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0;
+      // the lane's bias values, fetched once and together: its column of every block column, or its rows of every row block
+      float bcol[FN], brow[FM * 4];
+#pragma unroll
+      for (int j = 0; j < FN; ++j) bcol[j] = epi == 1 ? bias[solo_col + MI * j] : 0.0f;
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) brow[4 * fi + v] = epi == 2 ? bias[solo_row + MI * fi + v] : 0.0f;
+      static_for<0, SFN>([&](auto fj_c) __attribute__((always_inline)) {
+        constexpr int fj = decltype(fj_c)::value;
+        float x[FM * 4];
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          asm volatile("" : "+a"(acc[fi][fj]));
+#pragma unroll
+          for (int v = 0; v < 4; ++v) x[4 * fi + v] = acc[fi][fj][v] * post;
+        }
+        dispatch_op(k0, p00, p01, [&](auto f) __attribute__((always_inline)) {
+#pragma unroll
+          for (int e = 0; e < FM * 4; ++e) x[e] = f(x[e]);
+        });
+        if (epi == 1) {            // one bias value per column of D
+#pragma unroll
+          for (int e = 0; e < FM * 4; ++e) x[e] = x[e] + bcol[fj];
+        } else if (epi == 2) {     // one bias value per row of D
+#pragma unroll
+          for (int e = 0; e < FM * 4; ++e) x[e] = x[e] + brow[e];
+        }
+        dispatch_op(k1, p10, p11, [&](auto f) __attribute__((always_inline)) {
+#pragma unroll
+          for (int e = 0; e < FM * 4; ++e) x[e] = f(x[e]);
+        });
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd);
+          if (d_wide) {
+            float4v o;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[v] = x[4 * fi + v];
+            *(float4v*)((float*)args.d + off) = o;
+          } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) store_cd(args.d, args.d_dtype, off + v, x[4 * fi + v]);
+          }
+        }
+      });
+      return;
+    }
     if constexpr (CPATH != 0) {
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           float* dp = (float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd);
@@ -1559,7 +1681,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     } else if (args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0) {
       // (FP32 D next to a C that is not)
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));
@@ -1568,7 +1690,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     } else if (args.d_dtype != DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 1)) & 7u) == 0) {
       // 16-bit D: one rounding per value, 8 contiguous bytes per lane and block
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));
@@ -1584,7 +1706,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
     } else {
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj)
+      for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));      // (stays where it is until this branch is taken)

@@ -245,6 +245,7 @@ def _complex_tiles(operator, planar, a_kmajor, b_kmajor):
 # without hooks whose extents are whole numbers of tiles; the library runs the 2 x 4 arrangement of the same block
 # shape, with the same bits, for any other launch of such a configuration.
 _SOLO_TILE, _SOLO_WAVES = (256, 256, 64), (2, 2)
+_SOLO_COMPLEX_TILE = (128, 128, 64)        # in complex elements
 
 
 def _default_waves(operator, block_shape, checked=False, planar=False, gett=False, a_kmajor=False, b_kmajor=True, whole_tiles=False):
@@ -252,6 +253,10 @@ def _default_waves(operator, block_shape, checked=False, planar=False, gett=Fals
     if gett and key == (64, 64, 32):
         return (1, 1)
     if operator.kind == Operator.MFMA and key == _SOLO_TILE and whole_tiles:
+        return _SOLO_WAVES
+    # ... and the complex / dual product on interleaved matrices of an 'N','N' launch, whose real tile is that tile
+    if (operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL) and not planar and key == _SOLO_COMPLEX_TILE and whole_tiles
+            and not a_kmajor and b_kmajor):
         return _SOLO_WAVES
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         table = _FPU_TILES

@@ -390,10 +390,13 @@ end
 # same bits, for any other launch of such a configuration.
 const SOLO_TILE = (256, 256, 64)
 const SOLO_WAVES = (2, 2)
+const SOLO_COMPLEX_TILE = (128, 128, 64)       # in complex elements
 
 function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_kmajor::Bool = true, planar::Bool = false, whole_tiles::Bool = false)
     key = (block_shape.M, block_shape.N, block_shape.K)
     Operator.is_mfma(operator) && key == SOLO_TILE && whole_tiles && return SOLO_WAVES
+    # ... and the complex / dual product on interleaved matrices of an 'N','N' launch, whose real tile is that tile
+    !Operator.is_fpu(operator) && !Operator.is_mfma(operator) && !planar && key == SOLO_COMPLEX_TILE && whole_tiles && !a_kmajor && b_kmajor && return SOLO_WAVES
     table = Operator.is_fpu(operator) ? FPU_TILES : (Operator.is_mfma(operator) ? MFMA_TILES : complex_tiles(operator, a_kmajor, b_kmajor; planar = planar))
     for (t, w) in table
         t == key && return w

@@ -341,3 +341,46 @@ def test_config4a_planar_full_size(gpu):
     ref = planar_to_c128(h["a"]).astype(np.complex64) @ planar_to_c128(h["b"]).astype(np.complex64)
     assert oracle.rel_frobenius(d.real, ref.real) <= TOL
     assert oracle.rel_frobenius(d.imag, ref.imag) <= TOL
+
+
+@pytest.mark.parametrize("dual", [False, True])
+@pytest.mark.parametrize("zero_c", [True, False])
+def test_four_waves_give_the_bits_of_eight_waves(gpu, dual, zero_c):
+    """'N','N' on interleaved matrices: the 256 x 256 x 64 real tile on four waves, one per SIMD (a lane's four rows
+    of a block are two complex numbers; the four real products of an element of D lie in two blocks of the lane)."""
+    M, N, K = 256, 384, 320
+    blk = dict(block_shape=gk.NT(M=128, N=128, K=64))
+    four = configs.complex_config(M, N, K, zero_c=zero_c, dual=dual, **blk)
+    eight = configs.complex_config(M, N, K, zero_c=zero_c, dual=dual, warps_per_block=8, compute_warp=gk.NT(M=64, N=32, K=16), **blk)
+    n4, n8 = gk.kernel_name(four, Kernel.matmul_pipelined), gk.kernel_name(eight, Kernel.matmul_pipelined)
+    print("case", dual, zero_c, n4, n8, flush=True)
+    assert four.warps_per_block == 4 and n4.endswith("_w2x2") and n8.endswith("_w2x4")
+    a, b = configs.complex_matrix(71, M, K), configs.complex_matrix(72, K, N)
+    c = None if zero_c else rng.matrix("upm1_f32", 73, (2, M, N))
+    d4, d8 = run(four, a, b, c, M, N), run(eight, a, b, c, M, N)
+    assert np.array_equal(d4, d8)
+    if not dual:
+        want = to_c128(a) @ to_c128(b) + (0 if zero_c else to_c128(c))
+        assert oracle.rel_frobenius(d4[0], want.real) <= TOL and oracle.rel_frobenius(d4[1], want.imag) <= TOL
+
+
+def test_four_wave_complex_configuration_falls_back(gpu):
+    """Other transposes, hooks and a bias run the eight-wave arrangement of the same tile."""
+    from gemmkernels import Transform, Epilogue
+    M, N, K = 256, 256, 128
+    blk = dict(block_shape=gk.NT(M=128, N=128, K=64), warps_per_block=4, compute_warp=gk.NT(M=64, N=64, K=16))
+    for ta, tb in [(False, True), (True, False), (True, True)]:
+        conf = configs.complex_config(M, N, K, ta, tb, **blk)
+        assert gk.kernel_name(conf, Kernel.matmul_pipelined).endswith("_w2x4")
+    conf = configs.complex_config(M, N, K, **blk)
+    assert gk.kernel_name(conf, Kernel.matmul_pipelined).endswith("_w2x2")
+    hooks = dict(transform_shared_to_global_d=Transform.Elementwise(lambda x: x * 2.0))
+    assert gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=hooks).endswith("_w2x4")
+    a, b = configs.complex_matrix(74, M, K), configs.complex_matrix(75, K, N)
+    ta_, tb_ = gk.colmajor(a), gk.colmajor(b)
+    td = gk.colmajor_empty((2, M, N), torch.float32)
+    gk.matmul(conf, ta_, tb_, None, td, kernel=Kernel.matmul_pipelined, **hooks)
+    torch.cuda.synchronize()
+    want = 2.0 * (to_c128(a) @ to_c128(b))
+    d = gk.to_numpy(td)
+    assert oracle.rel_frobenius(d[0], want.real) <= TOL and oracle.rel_frobenius(d[1], want.imag) <= TOL

@@ -226,6 +226,8 @@ def test_every_tile_of_the_python_tables_has_a_compiled_instance():
                 for (bm, bn, bk), (wm, wn) in cfg._complex_tiles(op[16, 16, 16, F16, F32], False, ta, not tb):
                     conf = configs.complex_config(2 * bm, 2 * bn, 4 * bk, ta, tb, dual=dual, block_shape=NT(M=bm, N=bn, K=bk))
                     name = gk.kernel_name(conf, Kernel.matmul_pipelined)
+                    if (bm, bn, bk) == cfg._SOLO_COMPLEX_TILE and not ta and not tb:
+                        wm, wn = cfg._SOLO_WAVES          # whole tiles of an 'N','N' launch: one wave per SIMD
                     assert f"_{'nt'[ta]}{'nt'[tb]}_{bm}x{bn}x{bk}_w{wm}x{wn}" in name, name
                     assert "pair" in name, name
     for (bm, bn, bk), (wm, wn) in cfg._PLANAR_TILES:

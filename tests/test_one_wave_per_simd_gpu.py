@@ -1,8 +1,8 @@
 """The 256 x 256 x 64 tile on four waves (one per SIMD, 128 x 128 wave tiles) against the same tile on eight waves
 and against the CPU oracle.  The two arrangements run the k-steps and the products inside them in the same order,
 so FP32 results are compared bit for bit; the oracle with the tolerance of the other MFMA tests (relative
-Frobenius error <= 1e-3).  Launches the four-wave arrangement is not compiled for (hooks, a bias, extents that
-are not whole tiles) run the eight-wave arrangement of the same configuration."""
+Frobenius error <= 1e-3).  Launches the four-wave arrangement is not compiled for (hooks on A, B or C, more than
+one op in a hook of D, extents that are not whole tiles) run the eight-wave arrangement of the same configuration."""
 import numpy as np
 import pytest
 
@@ -114,27 +114,57 @@ def test_c_and_d_off_a_16_byte_boundary(gpu):
 
 
 @pytest.mark.parametrize("epilogue_cls", [Epilogue.Bias, Epilogue.BiasRow])
-def test_launches_with_hooks_or_a_bias_run_on_eight_waves(gpu, epilogue_cls):
+@pytest.mark.parametrize("with_c", [False, True])
+def test_hooks_of_d_in_closed_form_and_a_bias_run_on_four_waves(gpu, epilogue_cls, with_c):
+    """At most one op in each hook of D, a bias, and (where there is no C) a power-of-two scale of A folded into the
+    accumulators: the shape of benchmark config 3.  The four waves apply them without walking op lists."""
     M, N, K = 512, 256, 192
     a, b, c = operands(M, N, K, False, True, 7500)
     E = Transform.Elementwise
-    hooks = dict(transform_global_to_shared_a=E(lambda x: x * 0.5), transform_global_to_shared_c=E(lambda x: x * 0.25),
-                 transform_shared_to_regs_c=E(lambda x: x + 1.0), transform_regs_to_shared_d=E(Transform.relu),
-                 transform_shared_to_global_d=E(lambda x: x * 3.0))
+    hooks = dict(transform_regs_to_shared_d=E(Transform.relu), transform_shared_to_global_d=E(lambda x: x * 3.0))
+    if not with_c:
+        hooks["transform_global_to_shared_a"] = E(lambda x: x * 0.5)
     bias = rng.normal_f32(7504, N if epilogue_cls is Epilogue.Bias else M)
-    four, eight = config(M, N, K, False, True, (2, 2)), config(M, N, K, False, True, (2, 4))
+    four, eight = config(M, N, K, False, True, (2, 2), zero_c=not with_c), config(M, N, K, False, True, (2, 4), zero_c=not with_c)
     name = gk.kernel_name(four, Kernel.matmul_pipelined, transforms=hooks, epilogue=epilogue_cls(None))
     print("with hooks:", name, flush=True)
-    assert "_w2x4_" in name and name.endswith("_fused_cd")
-    assert "_w2x4_" in gk.kernel_name(four, Kernel.matmul_pipelined, epilogue=epilogue_cls(None))       # a bias alone
-    d4 = helpers.run_gpu(four, a, b, c, (M, N), transforms=hooks, epilogue_cls=epilogue_cls, bias=bias, kernel=Kernel.matmul_pipelined)
-    d8 = helpers.run_gpu(eight, a, b, c, (M, N), transforms=hooks, epilogue_cls=epilogue_cls, bias=bias, kernel=Kernel.matmul_pipelined)
+    assert "_w2x2_" in name and name.endswith("_fused_d")
+    assert "_w2x4_" in gk.kernel_name(eight, Kernel.matmul_pipelined, transforms=hooks, epilogue=epilogue_cls(None))
+    cc = c if with_c else None
+    d4 = helpers.run_gpu(four, a, b, cc, (M, N), transforms=hooks, epilogue_cls=epilogue_cls, bias=bias, kernel=Kernel.matmul_pipelined)
+    d8 = helpers.run_gpu(eight, a, b, cc, (M, N), transforms=hooks, epilogue_cls=epilogue_cls, bias=bias, kernel=Kernel.matmul_pipelined)
     assert np.array_equal(d4, d8)
-    ref = helpers.run_oracle(four, a, b, c, (M, N), transforms=hooks, epilogue=epilogue_cls(0), bias=bias)
+    ref = helpers.run_oracle(four, a, b, cc, (M, N), transforms=hooks, epilogue=epilogue_cls(0), bias=bias)
     assert oracle.rel_frobenius(d4, ref) <= TOL
     bias2d = bias[None, :] if epilogue_cls is Epilogue.Bias else bias[:, None]
-    acc = 0.5 * (a.astype(np.float64) @ b.astype(np.float64).T) + (0.25 * c.astype(np.float64) + 1.0)
+    acc = (1.0 if with_c else 0.5) * (a.astype(np.float64) @ b.astype(np.float64).T) + (c.astype(np.float64) if with_c else 0.0)
     assert oracle.rel_frobenius(d4, 3.0 * (np.maximum(acc, 0.0) + bias2d)) <= TOL
+    # a bias alone, and one op alone
+    assert gk.kernel_name(four, Kernel.matmul_pipelined, epilogue=epilogue_cls(None)).endswith("_fused_d")
+    only = dict(transform_shared_to_global_d=E(lambda x: Transform.clamp(x, -1.0, 2.0)))
+    d4 = helpers.run_gpu(four, a, b, cc, (M, N), transforms=only, kernel=Kernel.matmul_pipelined)
+    d8 = helpers.run_gpu(eight, a, b, cc, (M, N), transforms=only, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, d8)
+
+
+def test_other_hooks_run_on_eight_waves(gpu):
+    """Hooks on C, two ops in one hook of D, a scale folded next to a C, hooks on A that stay in the K loop."""
+    M, N, K = 512, 256, 128
+    a, b, c = operands(M, N, K, False, False, 7550)
+    conf = config(M, N, K, False, False, (2, 2))
+    E = Transform.Elementwise
+    cases = [dict(transform_global_to_shared_c=E(lambda x: x * 0.25)),
+             dict(transform_shared_to_global_d=E(lambda x: Transform.relu(x) * 2.0)),
+             dict(transform_global_to_shared_a=E(lambda x: x * 0.5)),                # folded, but C would have to be scaled the other way
+             dict(transform_global_to_shared_a=E(lambda x: x * 0.75))]               # not a power of two: runs in the K loop
+    for hooks in cases:
+        name = gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=hooks)
+        print("hooks", list(hooks), name, flush=True)
+        assert "_w2x4_" in name and "fused" in name
+        d = helpers.run_gpu(conf, a, b, c, (M, N), transforms=hooks, kernel=Kernel.matmul_pipelined)
+        ref = helpers.run_gpu(config(M, N, K, False, False, (2, 4)), a, b, c, (M, N), transforms=hooks, kernel=Kernel.matmul_pipelined)
+        assert np.array_equal(d, ref)
+        assert oracle.rel_frobenius(d, helpers.run_oracle(conf, a, b, c, (M, N), transforms=hooks)) <= TOL
 
 
 def test_ragged_extents_run_on_eight_waves(gpu):
