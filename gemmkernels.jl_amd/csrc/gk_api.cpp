@@ -286,10 +286,10 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
     }
   }
   // ... and for the complex / dual product on interleaved matrices of an 'N','N' launch (real tile 256 x 256 x 64)
-  if (key->family == gk::FAMILY_COMPLEX && key->variant <= 1 && key->BM == 128 && key->BN == 128 && key->BK == 64 && key->waves_m == 2 &&
-      key->waves_n == 2) {
+  // (planar matrices, variant 2: every transpose, the planes being plain real operands)
+  if (key->family == gk::FAMILY_COMPLEX && key->BM == 128 && key->BN == 128 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2) {
     const bool ok = c->matmul_shape.M % 128 == 0 && c->matmul_shape.N % 128 == 0 && c->matmul_shape.K % 64 == 0 && key->fused == 0 &&
-                    key->a_kmajor == 0 && key->b_kmajor == 1;
+                    (key->variant == 2 || (key->a_kmajor == 0 && key->b_kmajor == 1));
     if (!ok) key->waves_n = 4;
   }
   return GK_OK;

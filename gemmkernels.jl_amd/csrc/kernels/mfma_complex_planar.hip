@@ -30,6 +30,22 @@ int family_complex_planar(const InstanceKey& key, const GemmArgs& args, dim3 gri
   GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, 0, 0, "mfma_complex_planar_nt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, 1, 1, "mfma_complex_planar_tn_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)  \
   GK_PLANAR(bm_, bn_, bk_, wm_, wn_, st_, 1, 0, "mfma_complex_planar_tt_" #bm_ "x" #bn_ "x" #bk_ "_w" #wm_ "x" #wn_)
+  // four waves, one per SIMD (MfmaGemmConfig::SOLO; launches without hooks): one kernel per way of moving C and D
+#define GK_PLANAR_SOLO(akm_, bkm_, NAME)                                                                                  \
+  if (key.BM == 128 && key.BN == 128 && key.BK == 64 && key.waves_m == 2 && key.waves_n == 2 && key.a_kmajor == akm_ &&  \
+      key.b_kmajor == bkm_ && key.fused == 0) {                                                                           \
+    typedef MfmaGemmConfig<256, 256, 64, 2, 2, 2, (akm_ ? OPK_KMAJOR : OPK_MMAJOR), (bkm_ ? OPK_KMAJOR : OPK_MMAJOR), _Float16, 0, false, FIX_PLANAR, false, 16> Cfg; \
+    static_assert(Cfg::SOLO, "the four-wave arrangement");                                                               \
+    const int path = mode == 1 ? solo_cd_path(args) : 0;                                                                 \
+    if (path == 1) return run_instance<Cfg, 1>(mfma_gemm_kernel<Cfg, 1>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
+    if (path == 2) return run_instance<Cfg, 2>(mfma_gemm_kernel<Cfg, 2>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
+    return run_instance<Cfg, 0>(mfma_gemm_kernel<Cfg, 0>, NAME, args, grid, stream, mode, info, err, Cfg::LDS_BYTES, Cfg::THREADS); \
+  }
+  GK_PLANAR_SOLO(0, 1, "mfma_complex_planar_nn_128x128x64_w2x2")
+  GK_PLANAR_SOLO(0, 0, "mfma_complex_planar_nt_128x128x64_w2x2")
+  GK_PLANAR_SOLO(1, 1, "mfma_complex_planar_tn_128x128x64_w2x2")
+  GK_PLANAR_SOLO(1, 0, "mfma_complex_planar_tt_128x128x64_w2x2")
+#undef GK_PLANAR_SOLO
   GK_PLANAR_T(128, 128, 64, 2, 4, 2)
   GK_PLANAR_T(64, 64, 64, 2, 2, 2)
   GK_PLANAR_T(64, 64, 32, 2, 2, 4)

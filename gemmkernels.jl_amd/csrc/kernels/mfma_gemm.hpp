@@ -422,7 +422,9 @@ struct MfmaGemmConfig {
                                (BK_ / 32) % 2 == 0 && !SPLITK_ && (GK_FORCE_SYNC_FRAGS == 0) &&
                                ((FIX_ == FIX_NONE && (FUSE_ == 0 || FUSE_ == 4) && A_KIND_ != OPK_KSPLIT && B_KIND_ != OPK_KSPLIT) ||
                                 // ... and the complex / dual real-view product of an 'N','N' launch (A contiguous along m, B along k)
-                                ((FIX_ == FIX_PAIR || FIX_ == FIX_PAIR_DUAL) && FUSE_ == 0 && !GETT_ && A_KIND_ == OPK_MMAJOR && B_KIND_ == OPK_KSPLIT));
+                                ((FIX_ == FIX_PAIR || FIX_ == FIX_PAIR_DUAL) && FUSE_ == 0 && !GETT_ && A_KIND_ == OPK_MMAJOR && B_KIND_ == OPK_KSPLIT) ||
+                                // ... and the complex product on planar matrices, whose planes are plain real operands
+                                (FIX_ == FIX_PLANAR && FUSE_ == 0 && !GETT_ && A_KIND_ != OPK_KSPLIT && B_KIND_ != OPK_KSPLIT));
   // plain real products may have a last tile row / column that sticks out over M / N and a last, partial K
   // tile (the host asks for it only with 16-byte aligned columns, M or N a multiple of 8 where that index is
   // the contiguous one of A or B, and K a multiple of 8): loads are clamped, the C load and the D store
@@ -811,7 +813,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // (complex products: rows of the real view -- a lane's four rows are two complex numbers -- and complex columns, of which
   // the block columns fj and fj + FN / 2 hold the products with the real and with the imaginary parts of B)
   constexpr int SFN = Cfg::COLS_FRAG ? FN / 2 : FN;          // block columns that C / D see
-  [[maybe_unused]] const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane / MI);
+  // (planar complex: complex rows, of which the row blocks fi and fi + FM / 2 hold the products of the real and of the
+  // imaginary plane of A; C / D keep real parts in one plane and imaginary parts in the other)
+  constexpr int SFM = Cfg::PLANAR ? FM / 2 : FM;
+  [[maybe_unused]] const int solo_row = (Cfg::PLANAR ? (m0 + wm * Cfg::WTM) / 2 : m0 + wm * Cfg::WTM) + 4 * (lane / MI);
   [[maybe_unused]] const int solo_col = (Cfg::COLS_FRAG ? (n0 + wn * Cfg::WTN) / 2 : n0 + wn * Cfg::WTN) + (lane % MI);
   // Element offset of the lane's first row of block (fi, fj) in C / D.  Contractions: the lane walks the M modes for its
   // first row of every row block (the other three follow in the first M mode, whose stride in C / D is 1 and whose extent
@@ -826,8 +831,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj) gett_offsets32(args.gn, col + MI * fj, t0, solo_on[fj]);
     }
   };
-  [[maybe_unused]] auto solo_off = [&](int row, int col, int fi, int fj, long long ld) -> long long {
+  [[maybe_unused]] auto solo_off = [&](int row, int col, int fi, int fj, long long ld, [[maybe_unused]] long long plane) -> long long {
     if constexpr (Cfg::GETT) return solo_om[fi] + solo_on[fj];
+    else if constexpr (Cfg::PLANAR) return (long long)(row + MI * (fi % SFM)) + (long long)(col + MI * fj) * ld + (fi >= SFM ? plane : 0ll);
     else return (long long)(row + MI * fi) + (long long)(col + MI * fj) * ld;
   };
   if constexpr (Cfg::SOLO) {
@@ -838,7 +844,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const float* cp = (const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc);
+          const float* cp = (const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc, args.plane_c);
           asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(acc[fi][fj]) : "v"(cp) : "memory");
         }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -852,14 +858,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
-          acc[fi][fj] = *(const float4v*)((const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc));
+          acc[fi][fj] = *(const float4v*)((const float*)args.c + solo_off(solo_row, solo_col, fi, fj, args.ldc, args.plane_c));
     } else if (load_c && args.c_dtype != DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 1)) & 7u) == 0) {
       // 16-bit C: the lane's four rows are 8 contiguous bytes
 #pragma unroll
       for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc);
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc, args.plane_c);
           const int2v raw = *(const int2v*)((const char*)args.c + off * 2);
           if (args.c_dtype == DT_F16) {
             typedef _Float16 half4 __attribute__((ext_vector_type(4)));
@@ -878,7 +884,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc);
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldc, args.plane_c);
 #pragma unroll
           for (int v = 0; v < 4; ++v) acc[fi][fj][v] = load_cd(args.c, args.c_dtype, off + v);
         }
@@ -1588,9 +1594,26 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // (the lane number is asked for again: nothing of the store addresses is then kept in registers across the K loop)
     int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
-    const int solo_row = m0 + wm * Cfg::WTM + 4 * (lane_e / MI);
+    const int solo_row = (Cfg::PLANAR ? (m0 + wm * Cfg::WTM) / 2 : m0 + wm * Cfg::WTM) + 4 * (lane_e / MI);
     const int solo_col = (Cfg::COLS_FRAG ? (n0 + wn * Cfg::WTN) / 2 : n0 + wn * Cfg::WTN) + (lane_e % MI);      // (as before the K loop)
     solo_origins(solo_row, solo_col);
+    if constexpr (Cfg::PLANAR) {
+      // (row blocks of re A | im A) x (block columns of re B | im B): real part re*re - im*im into the upper left block,
+      // imaginary part im*re + re*im into the lower left one; C came in through the same two
+#pragma unroll
+      for (int fj = 0; fj < SFN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < SFM; ++fi) {
+          asm volatile("" : "+a"(acc[fi][fj]));
+          asm volatile("" : "+a"(acc[fi + SFM][fj + SFN]));
+          acc[fi][fj] = acc[fi][fj] - acc[fi + SFM][fj + SFN];
+          asm volatile("" : "+a"(acc[fi][fj]));
+          asm volatile("" : "+a"(acc[fi + SFM][fj]));
+          asm volatile("" : "+a"(acc[fi][fj + SFN]));
+          acc[fi + SFM][fj] = acc[fi + SFM][fj] + acc[fi][fj + SFN];
+          asm volatile("" : "+a"(acc[fi + SFM][fj]));
+        }
+    }
     if constexpr (Cfg::PAIR) {
       // The four real products of two complex elements of D in one lane: its rows 0 .. 3 of block (fi, fj) are
       // re A re B, im A re B of complex row m and of m + 1, those of block (fi, fj + FN / 2) re A im B, im A im B.
@@ -1656,7 +1679,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         });
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd);
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd, args.plane_d);
           if (d_wide) {
             float4v o;
 #pragma unroll
@@ -1675,7 +1698,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
-          float* dp = (float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd);
+          float* dp = (float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd, args.plane_d);
           asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
         }
     } else if (args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0) {
@@ -1685,7 +1708,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));
-          *(float4v*)((float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd)) = acc[fi][fj];
+          *(float4v*)((float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd, args.plane_d)) = acc[fi][fj];
         }
     } else if (args.d_dtype != DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 1)) & 7u) == 0) {
       // 16-bit D: one rounding per value, 8 contiguous bytes per lane and block
@@ -1694,7 +1717,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));
-          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd);
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd, args.plane_d);
           unsigned short b[4];
 #pragma unroll
           for (int v = 0; v < 4; ++v)
@@ -1710,7 +1733,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           asm volatile("" : "+a"(acc[fi][fj]));      // (stays where it is until this branch is taken)
-          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd);
+          const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd, args.plane_d);
 #pragma unroll
           for (int v = 0; v < 4; ++v) store_cd(args.d, args.d_dtype, off + v, acc[fi][fj][v]);
         }

@@ -255,8 +255,9 @@ def _default_waves(operator, block_shape, checked=False, planar=False, gett=Fals
     if operator.kind == Operator.MFMA and key == _SOLO_TILE and whole_tiles:
         return _SOLO_WAVES
     # ... and the complex / dual product on interleaved matrices of an 'N','N' launch, whose real tile is that tile
-    if (operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL) and not planar and key == _SOLO_COMPLEX_TILE and whole_tiles
-            and not a_kmajor and b_kmajor):
+    # (planar matrices: every transpose)
+    if (operator.kind in (Operator.MFMA_COMPLEX, Operator.MFMA_DUAL) and key == _SOLO_COMPLEX_TILE and whole_tiles
+            and (planar or (not a_kmajor and b_kmajor))):
         return _SOLO_WAVES
     if operator.kind in (Operator.FPU, Operator.FPU_TROPICAL):
         table = _FPU_TILES

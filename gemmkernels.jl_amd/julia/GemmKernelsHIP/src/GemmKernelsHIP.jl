@@ -396,7 +396,8 @@ function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_km
     key = (block_shape.M, block_shape.N, block_shape.K)
     Operator.is_mfma(operator) && key == SOLO_TILE && whole_tiles && return SOLO_WAVES
     # ... and the complex / dual product on interleaved matrices of an 'N','N' launch, whose real tile is that tile
-    !Operator.is_fpu(operator) && !Operator.is_mfma(operator) && !planar && key == SOLO_COMPLEX_TILE && whole_tiles && !a_kmajor && b_kmajor && return SOLO_WAVES
+    # (planar matrices: every transpose)
+    !Operator.is_fpu(operator) && !Operator.is_mfma(operator) && key == SOLO_COMPLEX_TILE && whole_tiles && (planar || (!a_kmajor && b_kmajor)) && return SOLO_WAVES
     table = Operator.is_fpu(operator) ? FPU_TILES : (Operator.is_mfma(operator) ? MFMA_TILES : complex_tiles(operator, a_kmajor, b_kmajor; planar = planar))
     for (t, w) in table
         t == key && return w

@@ -384,3 +384,34 @@ def test_four_wave_complex_configuration_falls_back(gpu):
     want = 2.0 * (to_c128(a) @ to_c128(b))
     d = gk.to_numpy(td)
     assert oracle.rel_frobenius(d[0], want.real) <= TOL and oracle.rel_frobenius(d[1], want.imag) <= TOL
+
+
+@pytest.mark.parametrize("ta,tb", TRANSPOSES)
+@pytest.mark.parametrize("zero_c", [True, False])
+def test_planar_four_waves_give_the_bits_of_eight_waves(gpu, ta, tb, zero_c):
+    """Planar matrices on the one-wave-per-SIMD arrangement (every transpose: the planes are plain real operands)."""
+    M, N, K = 256, 384, 192
+    blk = dict(block_shape=NT(M=128, N=128, K=64))
+    four = configs.complex_planar_config(M, N, K, ta, tb, zero_c=zero_c, **blk)
+    eight = configs.complex_planar_config(M, N, K, ta, tb, zero_c=zero_c, warps_per_block=8, compute_warp=NT(M=64, N=32, K=16), **blk)
+    n4, n8 = gk.kernel_name(four, Kernel.matmul_pipelined), gk.kernel_name(eight, Kernel.matmul_pipelined)
+    print("case", ta, tb, zero_c, n4, n8, flush=True)
+    assert four.warps_per_block == 4 and n4.endswith("_w2x2") and n8.endswith("_w2x4") and "planar" in n4
+    a = planar(101, K if ta else M, M if ta else K)
+    b = planar(102, N if tb else K, K if tb else N)
+    c = None if zero_c else planar(103, M, N, np.float32)
+    out = []
+    for conf in (four, eight):
+        td = gk.colmajor_empty((M, N, 2), torch.float32)
+        td.fill_(float("nan"))
+        gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), None if zero_c else gk.colmajor(c), td, kernel=Kernel.matmul_pipelined)
+        torch.cuda.synchronize()
+        out.append(gk.to_numpy(td))
+    assert np.array_equal(out[0], out[1])
+    A = planar_to_c128(a).T if ta else planar_to_c128(a)
+    B = planar_to_c128(b).T if tb else planar_to_c128(b)
+    assert oracle.rel_frobenius(planar_to_c128(out[0]), A @ B + (0 if zero_c else planar_to_c128(c))) <= TOL
+    # with a hook the launch runs on eight waves
+    from gemmkernels import Transform
+    hooks = dict(transform_shared_to_global_d=Transform.Elementwise(lambda x: x * 2.0))
+    assert gk.kernel_name(four, Kernel.matmul_pipelined, transforms=hooks).endswith("_w2x4")

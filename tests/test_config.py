@@ -232,6 +232,8 @@ def test_every_tile_of_the_python_tables_has_a_compiled_instance():
                     assert "pair" in name, name
     for (bm, bn, bk), (wm, wn) in cfg._PLANAR_TILES:
         conf = configs.complex_planar_config(2 * bm, 2 * bn, 4 * bk, block_shape=NT(M=bm, N=bn, K=bk))
+        if (bm, bn, bk) == cfg._SOLO_COMPLEX_TILE:
+            wm, wn = cfg._SOLO_WAVES          # whole tiles: one wave per SIMD
         assert f"{bm}x{bn}x{bk}_w{wm}x{wn}" in gk.kernel_name(conf, Kernel.matmul_pipelined)
 
 
