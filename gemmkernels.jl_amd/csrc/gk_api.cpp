@@ -243,7 +243,9 @@ int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_
 }
 
 // The arrangement of four waves with 128 x 128 wave tiles (one wave per SIMD, see Cfg::SOLO) is compiled for plain
-// products without hooks or bias whose extents are whole numbers of tiles.  Any other launch of such a configuration runs the
+// products without hooks or bias whose extents are whole numbers of tiles, and for plain products without hooks whose M and N
+// are multiples of 8 (tiles over the edges, a partial last K tile: path 3 of the kernel, which moves an FP32 C / D 16 bytes at a
+// time).  Any other launch of such a configuration runs the
 // eight-wave arrangement of the same block shape, which gives the same bits (the order of the k-steps and of the
 // products inside them does not depend on how the tile is dealt out to waves).
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
@@ -251,7 +253,15 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   if (rc != GK_OK) return rc;
   const bool plain = key->family == gk::FAMILY_MFMA, contraction = key->family == gk::FAMILY_GETT;
   if ((plain || contraction) && key->BM == 256 && key->BN == 256 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2) {
-    bool ok = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0;
+    const bool whole = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0;
+    bool ok = whole;
+    if (!whole && plain && key->fused == 0) {
+      const long long ldc = c->global_c_layout.ld > 0 ? c->global_c_layout.ld : c->matmul_shape.M;
+      const long long ldd = c->global_d_layout.ld > 0 ? c->global_d_layout.ld : c->matmul_shape.M;
+      const bool no_c = c->global_c_layout.kind == GK_LAYOUT_ZERO;
+      ok = c->matmul_shape.M % 8 == 0 && c->matmul_shape.N % 8 == 0 && c->matmul_shape.K >= 64 &&
+           c->global_d_layout.eltype == GK_F32 && ldd % 4 == 0 && (no_c || (c->global_c_layout.eltype == GK_F32 && ldc % 4 == 0));
+    }
     if (key->fused == 3 && plain) {
       // hooks of C and D and a bias: the four waves take what has a closed form (fuse level 4 of the kernel): no hook on
       // C, at most one op in each hook of D, and a power-of-two scale of A or B folded into the accumulators only where
@@ -287,6 +297,9 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
   }
   // ... and for the complex / dual product on interleaved matrices of an 'N','N' launch (real tile 256 x 256 x 64)
   // (planar matrices, variant 2: every transpose, the planes being plain real operands)
+  // (the bounds-checked kernel has no such arrangement)
+  if (key->family == gk::FAMILY_MFMA_CHECKED && key->BM == 256 && key->BN == 256 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2)
+    key->waves_n = 4;
   if (key->family == gk::FAMILY_COMPLEX && key->BM == 128 && key->BN == 128 && key->BK == 64 && key->waves_m == 2 && key->waves_n == 2) {
     const bool ok = c->matmul_shape.M % 128 == 0 && c->matmul_shape.N % 128 == 0 && c->matmul_shape.K % 64 == 0 && key->fused == 0 &&
                     (key->variant == 2 || (key->a_kmajor == 0 && key->b_kmajor == 1));
@@ -893,13 +906,15 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
 
   gk::GemmArgs& args = out->args;
   make_args(conf, a, b, c, d, transforms, epilogue, &args);
-  if (!custom && key.family == gk::FAMILY_GETT && key.BM == 256 && key.waves_m == 2 && key.waves_n == 2 && gk::solo_cd_path(args) == 0) {
-    // a contraction on the four-wave arrangement moves C and D 16 bytes at a time: pointers that do not allow it
-    // run the eight-wave arrangement (see make_key)
+  const bool solo_edges = key.family == gk::FAMILY_MFMA && key.fused == 0 && (args.M % 256 != 0 || args.N % 256 != 0 || args.K % 64 != 0);
+  if (!custom && (key.family == gk::FAMILY_GETT || solo_edges) && key.BM == 256 && key.BN == 256 && key.BK == 64 && key.waves_m == 2 && key.waves_n == 2 &&
+      gk::solo_cd_path(args) == 0) {
+    // a contraction on the four-wave arrangement, and a product with tiles over its edges, move C and D 16 bytes at a
+    // time: pointers that do not allow it run the eight-wave arrangement (see make_key)
     key.waves_n = 4;
     gk::FamilyFn fn8 = family_fn(key);
     hipError_t e8 = hipSuccess;
-    if (!fn8 || !fn8(key, args, dim3(1), nullptr, 0, &info, &e8)) return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance for this contraction");
+    if (!fn8 || !fn8(key, args, dim3(1), nullptr, 0, &info, &e8)) return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance for this %s", solo_edges ? "product" : "contraction");
   }
 
   // aligned layouts move 16-byte vectors (reference src/layout.jl:22-34 traps on the device; here it is a host check)

@@ -496,7 +496,8 @@ struct MfmaGemmConfig {
 };
 
 // CPATH (Cfg::SOLO only; 0 elsewhere): how C comes in and D goes out.  1: FP32 C and D with 16-byte accesses, straight into
-// and out of the accumulation registers; 2: no C, D as in 1; 0: anything else.  One kernel per path, chosen by the host
+// and out of the accumulation registers; 2: no C, D as in 1; 3: as 1 and 2 for products whose extents are not whole numbers of
+// tiles (M a multiple of 4: edge tiles leave out what lies outside D, a partial last K tile runs behind the loop); 0: anything else.  One kernel per path, chosen by the host
 // (solo_cd_path): where the paths met in one kernel, the register allocator gave the accumulators different registers
 // on each and shuffled 250 of them in front of the K loop.
 template <class Cfg, int CPATH = 0>
@@ -508,6 +509,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, STAGES = Cfg::STAGES;
   constexpr int FM = Cfg::FM, FN = Cfg::FN, NWAVES = Cfg::NWAVES;
   constexpr int DMA_A = Cfg::DMA_A, DMA_B = Cfg::DMA_B, DPT = Cfg::DMA_PER_TILE;
+  // tiles that stick out over the edges of the operands and a partial last K tile: the instances compiled for them
+  // (Cfg::RAGGED_OK) and path 3 of the one-wave-per-SIMD instances
+  constexpr bool RAGGED = Cfg::RAGGED_OK || (Cfg::SOLO && CPATH == 3);
+  constexpr bool RAGGED_K = Cfg::RAGGED_K_OK || (Cfg::SOLO && CPATH == 3);
+  static_assert(CPATH != 3 || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "path 3 is compiled for plain real products");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -557,7 +563,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         m = planar_index(m, Cfg::WTM, imag);
         offa[i] = (unsigned)(((long long)row * args.lda + col + (imag ? args.plane_a : 0ll)) * 2);
       } else {
-        if constexpr (Cfg::RAGGED_OK) {
+        if constexpr (RAGGED) {
           // a tile that sticks out over the last row of A: chunks beyond it re-read the last valid chunk
           // (their products land in rows of the tile that are never stored)
           int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
@@ -571,7 +577,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     for (int i = 0; i < DMA_B; ++i) {
       int row, col;
       dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
-      if constexpr (Cfg::RAGGED_OK) {
+      if constexpr (RAGGED) {
         int& n = Cfg::B_KIND == OPK_KMAJOR ? row : col;
         const int last = Cfg::B_KIND == OPK_KMAJOR ? args.N - n0 - 1 : ((args.N - n0 - 1) >> 3) << 3;
         n = n > last ? last : n;
@@ -672,7 +678,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // but a 16-byte chunk of this workgroup's tiles straddles the last row of an operand whose rows are contiguous in
   // memory (M, or N, not a multiple of 8): in the last k such a chunk would read past the end of the operand.
   [[maybe_unused]] int tail_k = 0;
-  if constexpr (Cfg::RAGGED_K_OK) {
+  if constexpr (RAGGED_K) {
     tail_k = args.K - KT * BK;
     const bool straddle = (Cfg::A_KIND == OPK_MMAJOR && (args.M & 7) != 0 && m0 + BM > args.M) ||
                           (Cfg::B_KIND == OPK_MMAJOR && (args.N & 7) != 0 && n0 + BN > args.N);
@@ -684,6 +690,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if (KT <= 0) return;       // the whole workgroup leaves together, before any barrier
     ga += (long long)kt0 * a_step;
     gb += (long long)kt0 * b_step;
+  }
+
+  // (SOLO: the loop leaves ga / gb at the last tile it fetched, so the tile behind the loop is kept here)
+  [[maybe_unused]] const char* ga_tail = ga;
+  [[maybe_unused]] const char* gb_tail = gb;
+  if constexpr (Cfg::SOLO && RAGGED_K) {
+    ga_tail += (long long)KT * a_step;
+    gb_tail += (long long)KT * b_step;
   }
 
   // --- prologue: start the first STAGES-1 tiles on their way ---
@@ -839,7 +853,33 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   if constexpr (Cfg::SOLO) {
     static_assert(!Cfg::GETT || CPATH != 0, "contractions run the four waves with 16-byte C / D accesses only");
     if (load_c) solo_origins(solo_row, solo_col);
-    if constexpr (CPATH == 1) {
+    if constexpr (CPATH == 3) {
+      // FP32 C with 16-byte accesses, tiles over the edge included: M is a multiple of 4 (the host runs this path on nothing
+      // else), so a lane's four rows are inside or outside together; rows and columns outside are read from the last ones
+      // inside, and what is accumulated on them is never stored
+      if (load_c) {
+#pragma unroll
+        for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+          for (int fi = 0; fi < FM; ++fi) {
+            int r = solo_row + MI * fi, cc = solo_col + MI * fj;
+            r = r < args.M - 4 ? r : args.M - 4;
+            cc = cc < args.N - 1 ? cc : args.N - 1;
+            const float* cp = (const float*)args.c + ((long long)r + (long long)cc * args.ldc);
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(acc[fi][fj]) : "v"(cp) : "memory");
+          }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      } else {
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+          for (int fj = 0; fj < FN; ++fj) acc[fi][fj] = AccV{};
+      }
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) asm volatile("" : "+a"(acc[fi][fj]));
+    } else if constexpr (CPATH == 1) {
 #pragma unroll
       for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll
@@ -1109,6 +1149,63 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       __builtin_amdgcn_sched_group_barrier(0x8, NA * FN - (FN - 1), 0);
     }
   };
+  // The last K tile of a product whose K is not a whole number of tiles (or that has a chunk over the end of an operand,
+  // see tail_k): fetched into the first stage from gta / gtb with clamped coordinates and repaired there, outside the pipeline.
+  [[maybe_unused]] auto fetch_tail_tile = [&](auto gta, auto gtb) __attribute__((always_inline)) {
+    block_barrier();                                     // every wave is done with the stages of the loop
+    char* sa = smem;
+    char* sb = sa + GA::BYTES;
+    // per chunk: elements it was fetched too far back (0 .. 7), leading elements that keep their value (0 .. 8)
+    int shift_a[DMA_A], keep_a[DMA_A], shift_b[DMA_B], keep_b[DMA_B];
+    auto fetch = [&](auto kind_c, auto geom, int q, const char* g, long long ld, int rows_valid, char* dst, int& shift, int& keep)
+        __attribute__((always_inline)) {
+      constexpr int KIND = decltype(kind_c)::value;
+      typedef decltype(geom) G;
+      int row, col;
+      dma_lane_coords<G, KIND>(q, lane, row, col);
+      int& r = KIND == OPK_KMAJOR ? row : col;           // index along M (A) or N (B), from the tile origin
+      int& k = KIND == OPK_KMAJOR ? col : row;
+      const int last_r = KIND == OPK_KMAJOR ? rows_valid - 1 : ((rows_valid - 1) >> 3) << 3;
+      r = r > last_r ? last_r : r;
+      keep = 8;
+      if (KIND == OPK_KMAJOR) {                          // the chunk runs along k
+        if (k >= tail_k) { keep = 0; k = ((tail_k - 1) >> 3) << 3; }
+        else if (k + 8 > tail_k) keep = tail_k - k;
+      } else if (k >= tail_k) { keep = 0; k = tail_k - 1; }
+      long long e = (long long)row * ld + col;
+      // one past the last element of the operand, counted from the tile origin
+      const long long end = KIND == OPK_KMAJOR ? (long long)(rows_valid - 1) * ld + tail_k : (long long)(tail_k - 1) * ld + rows_valid;
+      shift = 0;
+      if (e + 8 > end) { shift = (int)(e + 8 - end); e -= shift; }
+      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(g + e * 2), GK_LDS_PTR(void, dst + q * 1024), 16, 0, 0);
+    };
+#pragma unroll
+    for (int i = 0; i < DMA_A; ++i)
+      fetch(std::integral_constant<int, Cfg::A_KIND>{}, GA{}, wave + i * NWAVES, gta, args.lda, args.M - m0, sa, shift_a[i], keep_a[i]);
+#pragma unroll
+    for (int i = 0; i < DMA_B; ++i)
+      fetch(std::integral_constant<int, Cfg::B_KIND>{}, GB{}, wave + i * NWAVES, gtb, args.ldb, args.N - n0, sb, shift_b[i], keep_b[i]);
+    wait_vmcnt<0>();                                     // this lane's own slots have landed
+    auto repair = [&](char* slot, int shift, int keep) __attribute__((always_inline)) {
+      if (shift == 0 && keep == 8) return;
+      short8v v = *(const short8v*)slot, out;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        short x = 0;
+#pragma unroll
+        for (int f = 0; f < 8; ++f) x = (f == e + shift) ? v[f] : x;      // element e was fetched into place e + shift
+        out[e] = e < keep ? x : (short)0;
+      }
+      *(short8v*)slot = out;
+    };
+#pragma unroll
+    for (int i = 0; i < DMA_A; ++i) repair(sa + (wave + i * NWAVES) * 1024 + lane * 16, shift_a[i], keep_a[i]);
+#pragma unroll
+    for (int i = 0; i < DMA_B; ++i) repair(sb + (wave + i * NWAVES) * 1024 + lane * 16, shift_b[i], keep_b[i]);
+    __syncthreads();                                     // waits for the LDS writes as well
+    ra.set_stage(lds_base);
+    rb.set_stage(lds_base + GA::BYTES);
+  };
   typedef std::integral_constant<int, -1> Whole;
 
   if constexpr (Cfg::SOLO) {
@@ -1230,6 +1327,21 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     }
     wait_vmcnt<0>();     // (the last DMA of the loop may still be on its way; so are reads
     wait_lgkmcnt<0>();   // of fragments)
+    if constexpr (RAGGED_K) {
+      // the last, partial K tile, outside the schedule of the loop: the k-steps that hold valid values
+      if (tail_k > 0) {
+        fetch_tail_tile(ga_tail, gb_tail);
+        static_for<0, KS>([&](auto ks_c) {
+          constexpr int ks = decltype(ks_c)::value;
+          if (ks * Cfg::KSTEP_K < tail_k) {
+            static_for<0, NOPS>([&](auto r_c) { read_op(r_c, ks_c); });
+            wait_lgkmcnt<0>();
+            phase(ks_c, No{}, 0);        // (what it reads ahead for the next k-step is read again there, or never used)
+            wait_lgkmcnt<0>();
+          }
+        });
+      }
+    }
   } else if constexpr (!Cfg::PREFETCH) {
     // Two LDS stages: the DMA of tile kt+1 runs while tile kt is consumed; the first fragments of a
     // tile are read after the barrier that publishes it.
@@ -1423,59 +1535,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // then repairs its own chunks in LDS: shifted into place, values whose k is beyond K set to zero.  Then the
     // k-steps that hold valid values are multiplied.  ga / gb stand at this tile: every earlier tile has been issued.
     if (tail_k > 0) {
-      block_barrier();                                     // every wave is done with the stages of the loop
-      char* sa = smem;
-      char* sb = sa + GA::BYTES;
-      // per chunk: elements it was fetched too far back (0 .. 7), leading elements that keep their value (0 .. 8)
-      int shift_a[DMA_A], keep_a[DMA_A], shift_b[DMA_B], keep_b[DMA_B];
-      auto fetch = [&](auto kind_c, auto geom, int q, const char* g, long long ld, int rows_valid, char* dst, int& shift, int& keep)
-          __attribute__((always_inline)) {
-        constexpr int KIND = decltype(kind_c)::value;
-        typedef decltype(geom) G;
-        int row, col;
-        dma_lane_coords<G, KIND>(q, lane, row, col);
-        int& r = KIND == OPK_KMAJOR ? row : col;           // index along M (A) or N (B), from the tile origin
-        int& k = KIND == OPK_KMAJOR ? col : row;
-        const int last_r = KIND == OPK_KMAJOR ? rows_valid - 1 : ((rows_valid - 1) >> 3) << 3;
-        r = r > last_r ? last_r : r;
-        keep = 8;
-        if (KIND == OPK_KMAJOR) {                          // the chunk runs along k
-          if (k >= tail_k) { keep = 0; k = ((tail_k - 1) >> 3) << 3; }
-          else if (k + 8 > tail_k) keep = tail_k - k;
-        } else if (k >= tail_k) { keep = 0; k = tail_k - 1; }
-        long long e = (long long)row * ld + col;
-        // one past the last element of the operand, counted from the tile origin
-        const long long end = KIND == OPK_KMAJOR ? (long long)(rows_valid - 1) * ld + tail_k : (long long)(tail_k - 1) * ld + rows_valid;
-        shift = 0;
-        if (e + 8 > end) { shift = (int)(e + 8 - end); e -= shift; }
-        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(g + e * 2), GK_LDS_PTR(void, dst + q * 1024), 16, 0, 0);
-      };
-#pragma unroll
-      for (int i = 0; i < DMA_A; ++i)
-        fetch(std::integral_constant<int, Cfg::A_KIND>{}, GA{}, wave + i * NWAVES, ga, args.lda, args.M - m0, sa, shift_a[i], keep_a[i]);
-#pragma unroll
-      for (int i = 0; i < DMA_B; ++i)
-        fetch(std::integral_constant<int, Cfg::B_KIND>{}, GB{}, wave + i * NWAVES, gb, args.ldb, args.N - n0, sb, shift_b[i], keep_b[i]);
-      wait_vmcnt<0>();                                     // this lane's own slots have landed
-      auto repair = [&](char* slot, int shift, int keep) __attribute__((always_inline)) {
-        if (shift == 0 && keep == 8) return;
-        short8v v = *(const short8v*)slot, out;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          short x = 0;
-#pragma unroll
-          for (int f = 0; f < 8; ++f) x = (f == e + shift) ? v[f] : x;      // element e was fetched into place e + shift
-          out[e] = e < keep ? x : (short)0;
-        }
-        *(short8v*)slot = out;
-      };
-#pragma unroll
-      for (int i = 0; i < DMA_A; ++i) repair(sa + (wave + i * NWAVES) * 1024 + lane * 16, shift_a[i], keep_a[i]);
-#pragma unroll
-      for (int i = 0; i < DMA_B; ++i) repair(sb + (wave + i * NWAVES) * 1024 + lane * 16, shift_b[i], keep_b[i]);
-      __syncthreads();                                     // waits for the LDS writes as well
-      ra.set_stage(lds_base);
-      rb.set_stage(lds_base + GA::BYTES);
+      fetch_tail_tile(ga, gb);
       static_for<0, Cfg::KSTEPS>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
         if (ks * Cfg::KSTEP_K < tail_k) {
@@ -1693,7 +1753,19 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       });
       return;
     }
-    if constexpr (CPATH != 0) {
+    if constexpr (CPATH == 3) {
+      // (blocks of four rows and a column that lie outside D are left out)
+#pragma unroll
+      for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+        for (int fi = 0; fi < FM; ++fi) {
+          const int r = solo_row + MI * fi, cc = solo_col + MI * fj;
+          if (r < args.M && cc < args.N) {
+            float* dp = (float*)args.d + ((long long)r + (long long)cc * args.ldd);
+            asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
+          }
+        }
+    } else if constexpr (CPATH != 0) {
 #pragma unroll
       for (int fj = 0; fj < SFN; ++fj)
 #pragma unroll

@@ -378,7 +378,7 @@ def _skinny() -> Workload:
 def _mul4000() -> Workload:
     """Not one of the five benchmark configurations: mul!(C, A, B) at a size that is not a whole number of
     tiles, through the BLAS-level front end (bounds-checked layouts with 16-byte aligned columns, which the
-    library runs on the aligned kernel with masked edge tiles)."""
+    library runs on the aligned kernel with masked edge tiles: four waves, one per SIMD, as M and N are multiples of 8)."""
     M = N = K = 4000
 
     def host():
@@ -399,7 +399,7 @@ def _mul4000() -> Workload:
         name="mul4000",
         description="mul!(C, A, B), M=N=K=4000 (not whole tiles), FP16 A/B, FP32 C, 'N','N', C not read",
         flops=2 * M * N * K, bytes=M * K * 2 + K * N * 2 + M * N * 4, bound="mfma", make_host=host, make_launch=launch,
-        kernel_name="mfma_gemm_nn_256x256x64_w2x4_s2__Float16")
+        kernel_name="mfma_gemm_nn_256x256x64_w2x2_s2__Float16_edges")
 
 
 def benchmark_config(n, variant: Optional[str] = None) -> Workload:

@@ -2,7 +2,7 @@
 and against the CPU oracle.  The two arrangements run the k-steps and the products inside them in the same order,
 so FP32 results are compared bit for bit; the oracle with the tolerance of the other MFMA tests (relative
 Frobenius error <= 1e-3).  Launches the four-wave arrangement is not compiled for (hooks on A, B or C, more than
-one op in a hook of D, extents that are not whole tiles) run the eight-wave arrangement of the same configuration."""
+one op in a hook of D, an M or N that is not a multiple of 8) run the eight-wave arrangement of the same configuration."""
 import numpy as np
 import pytest
 
@@ -167,7 +167,74 @@ def test_other_hooks_run_on_eight_waves(gpu):
         assert oracle.rel_frobenius(d, helpers.run_oracle(conf, a, b, c, (M, N), transforms=hooks)) <= TOL
 
 
-def test_ragged_extents_run_on_eight_waves(gpu):
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(264, 520, 136), (512, 776, 104), (1000, 8, 197), (256, 256, 100), (8, 1032, 64)])
+def test_tiles_over_the_edges_same_bits_as_eight_waves(gpu, ta, tb, M, N, K):
+    """M and N multiples of 8: edge tiles leave out what lies outside D, the partial last K tile runs behind the loop
+    (one whole tile in front of it, several, none after it; a K that is odd)."""
+    a, b, c = operands(M, N, K, ta, tb, 7700 + M + K)
+    four, eight = config(M, N, K, ta, tb, (2, 2), checked=True), config(M, N, K, ta, tb, (2, 4), checked=True)
+    name = gk.kernel_name(four, Kernel.matmul_pipelined)
+    print("case", ta, tb, M, N, K, name, flush=True)
+    assert "_w2x2_" in name and "_w2x4_" in gk.kernel_name(eight, Kernel.matmul_pipelined)
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    d8 = helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, d8)
+    assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N))) <= TOL
+    assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= TOL
+
+
+def test_tiles_over_the_edges_without_c_in_place_and_off_a_16_byte_boundary(gpu):
+    import torch
+    M, N, K = 520, 264, 232
+    a, b, c = operands(M, N, K, False, False, 7800)
+    four, eight = config(M, N, K, False, False, (2, 2), checked=True), config(M, N, K, False, False, (2, 4), checked=True)
+    zero4, zero8 = (config(M, N, K, False, False, w, zero_c=True, checked=True) for w in ((2, 2), (2, 4)))
+    assert "_w2x2_" in gk.kernel_name(zero4, Kernel.matmul_pipelined)
+    d = helpers.run_gpu(zero4, a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d, helpers.run_gpu(zero8, a, b, None, (M, N), kernel=Kernel.matmul_pipelined))
+    assert oracle.rel_frobenius(d, oracle.gemm_f64(a, b, None, 1.0, 0.0, False, False)) <= TOL
+    # d aliases c (reference src/matmul.jl:198)
+    ref = helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined, alias_cd=True), ref)
+    # C and D that start 4 bytes into a 16-byte line: the library runs the eight waves; nothing outside D is written
+    A, B = gk.colmajor(a), gk.colmajor(b)
+    cbuf = torch.zeros(M * N + 1, dtype=torch.float32, device="cuda")
+    dbuf = torch.full((M * N + 9,), float("nan"), dtype=torch.float32, device="cuda")
+    C = cbuf[1:].view(N, M).t()
+    D = dbuf[1:1 + M * N].view(N, M).t()
+    C.copy_(torch.from_numpy(c).cuda())
+    gk.matmul(four, A, B, C, D, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    assert np.array_equal(D.cpu().numpy(), ref)
+    assert bool(torch.isnan(dbuf[0])) and bool(torch.isnan(dbuf[1 + M * N:]).all())
+
+
+def test_nothing_is_written_outside_d(gpu):
+    """D as a window of a larger matrix (leading dimension beyond M) whose other elements keep their values."""
+    import torch
+    M, N, K, LD = 264, 136, 128, 272
+    a, b, c = operands(M, N, K, False, True, 7850)
+    col = Layout.ColMajor
+    conf = gk.get_config(
+        gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=256, N=256, K=64), warps_per_block=4, compute_warp=NT(M=128, N=128, K=16),
+        operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+        global_a_layout=col[Float16], global_b_layout=Layout.RowMajor[Float16], global_c_layout=col[Float32], global_d_layout=col[Float32],
+        is_a_col_major=True, is_b_col_major=False)
+    assert "_w2x2_" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    big = torch.full((N + 3, LD), float("nan"), dtype=torch.float32, device="cuda")
+    Dw = big[1:1 + N, :M].t()                     # M x N, column-major with leading dimension LD
+    Cw = torch.zeros((N, LD), dtype=torch.float32, device="cuda")[:, :M].t()
+    Cw.copy_(torch.from_numpy(c).cuda())
+    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), Cw, Dw, kernel=Kernel.matmul_pipelined)      # ('T' B: stored N x K)
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(Dw.cpu().numpy(), oracle.gemm_f64(a, b, c, 1.0, 1.0, False, True)) <= TOL
+    outside = big.clone()
+    outside[1:1 + N, :M] = float("nan")
+    assert bool(torch.isnan(outside).all()) and not bool(torch.isnan(big[1:1 + N, :M]).any())
+
+
+def test_extents_that_are_not_multiples_of_8_run_on_eight_waves(gpu):
     M2, N2, K2 = 300, 520, 136
     a2, b2, c2 = operands(M2, N2, K2, False, False, 7510)
     ragged = config(M2, N2, K2, False, False, (2, 2), checked=True)
