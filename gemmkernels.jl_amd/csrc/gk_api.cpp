@@ -434,6 +434,7 @@ int find_instance(const gk_config* c, const gk_transforms* t, const gk_epilogue*
   gk::FamilyFn fn = family_fn(*key);
   gk::GemmArgs dummy;
   memset(&dummy, 0, sizeof(dummy));
+  dummy.M = c->matmul_shape.M; dummy.N = c->matmul_shape.N; dummy.K = c->matmul_shape.K;     // (instances that depend on the extents: tiles over the edges)
   hipError_t err = hipSuccess;
   if (key->family == gk::FAMILY_MFMA && allow_ragged_fast && ragged_fast_path(c) && (!fn || !fn(*key, dummy, dim3(1), nullptr, 0, info, &err))) {
     // no aligned instance of this tile: the bounds-checked kernel after all

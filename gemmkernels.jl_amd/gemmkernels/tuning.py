@@ -27,7 +27,7 @@ from .tiling import NT
 
 # every MFMA instance of the library: (block shape, waves M x N)
 MFMA_CANDIDATES = [
-    ((256, 256, 64), (2, 4)), ((256, 256, 64), (2, 2)),     # (2, 2): one wave per SIMD, plain whole-tile products only
+    ((256, 256, 64), (2, 4)), ((256, 256, 64), (2, 2)),     # (2, 2): one wave per SIMD, plain products only
     ((256, 256, 32), (2, 4)), ((256, 256, 32), (4, 2)),
     ((256, 128, 64), (2, 2)), ((128, 256, 64), (2, 2)),
     ((128, 128, 64), (2, 2)), ((128, 128, 64), (4, 2)), ((128, 128, 32), (2, 2)),

@@ -176,7 +176,7 @@ def test_tiles_over_the_edges_same_bits_as_eight_waves(gpu, ta, tb, M, N, K):
     four, eight = config(M, N, K, ta, tb, (2, 2), checked=True), config(M, N, K, ta, tb, (2, 4), checked=True)
     name = gk.kernel_name(four, Kernel.matmul_pipelined)
     print("case", ta, tb, M, N, K, name, flush=True)
-    assert "_w2x2_" in name and "_w2x4_" in gk.kernel_name(eight, Kernel.matmul_pipelined)
+    assert "_w2x2_" in name and name.endswith("_edges") and "_w2x4_" in gk.kernel_name(eight, Kernel.matmul_pipelined)
     d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
     d8 = helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
     assert np.array_equal(d4, d8)
