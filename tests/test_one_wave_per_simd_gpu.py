@@ -2,7 +2,7 @@
 and against the CPU oracle.  The two arrangements run the k-steps and the products inside them in the same order,
 so FP32 results are compared bit for bit; the oracle with the tolerance of the other MFMA tests (relative
 Frobenius error <= 1e-3).  Launches the four-wave arrangement is not compiled for (hooks on A, B or C, more than
-one op in a hook of D, an M or N that is not a multiple of 8) run the eight-wave arrangement of the same configuration."""
+one op in a hook of D, extents the edge instances do not take) run the eight-wave arrangement of the same configuration."""
 import numpy as np
 import pytest
 
@@ -232,6 +232,26 @@ def test_nothing_is_written_outside_d(gpu):
     outside = big.clone()
     outside[1:1 + N, :M] = float("nan")
     assert bool(torch.isnan(outside).all()) and not bool(torch.isnan(big[1:1 + N, :M]).any())
+
+
+@pytest.mark.parametrize("ta,tb,M,N,K,four_waves", [
+    (False, False, 264, 515, 100, True),     # 'N' B is contiguous along k: any N
+    (True, False, 260, 515, 136, True),      # 'T' A as well: M in fours (the 16-byte accesses to C / D)
+    (True, True, 260, 520, 197, True),
+    (False, False, 260, 515, 100, False),    # 'N' A is contiguous along M: M in eights
+    (True, True, 260, 516, 100, False),      # 'T' B is contiguous along N: N in eights
+    (True, False, 258, 512, 128, False)])    # M not in fours
+def test_extents_in_fours_and_eights(gpu, ta, tb, M, N, K, four_waves):
+    """Which extents the four waves take with tiles over the edges: M in fours, and in eights along an operand whose
+    16-byte chunks run along M or N; the rest runs on eight waves.  Same bits either way."""
+    a, b, c = operands(M, N, K, ta, tb, 7900 + M + N)
+    four, eight = config(M, N, K, ta, tb, (2, 2), checked=True), config(M, N, K, ta, tb, (2, 4), checked=True)
+    name = gk.kernel_name(four, Kernel.matmul_pipelined)
+    print("case", ta, tb, M, N, K, name, flush=True)
+    assert ("_w2x2_" in name and name.endswith("_edges")) if four_waves else "_w2x4_" in name
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined))
+    assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= TOL
 
 
 def test_extents_that_are_not_multiples_of_8_run_on_eight_waves(gpu):
