@@ -244,8 +244,7 @@ int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_
 
 // The arrangement of four waves with 128 x 128 wave tiles (one wave per SIMD, see Cfg::SOLO) is compiled for plain
 // products without hooks or bias whose extents are whole numbers of tiles, and for plain products without hooks whose M is a
-// multiple of 4 -- of 8, like N, where the operand is contiguous along it -- (tiles over the edges, a partial last K tile: path 3
-// of the kernel, which moves an FP32 C / D 16 bytes at a time).  Any other launch of such a configuration runs the
+// multiple of 4 (tiles over the edges, a partial last K tile: path 3 of the kernel, which moves an FP32 C / D 16 bytes at a time).  Any other launch of such a configuration runs the
 // eight-wave arrangement of the same block shape, which gives the same bits (the order of the k-steps and of the
 // products inside them does not depend on how the tile is dealt out to waves).
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
@@ -259,9 +258,8 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
       const long long ldc = c->global_c_layout.ld > 0 ? c->global_c_layout.ld : c->matmul_shape.M;
       const long long ldd = c->global_d_layout.ld > 0 ? c->global_d_layout.ld : c->matmul_shape.M;
       const bool no_c = c->global_c_layout.kind == GK_LAYOUT_ZERO;
-      // (M in fours for the 16-byte accesses to C / D; in eights along an operand whose 16-byte chunks run along M or N)
-      ok = c->matmul_shape.M % 4 == 0 && (key->a_kmajor || c->matmul_shape.M % 8 == 0) && (key->b_kmajor || c->matmul_shape.N % 8 == 0) &&
-           c->matmul_shape.K >= 64 &&
+      // (M in fours: a lane's four rows of C / D are inside or outside together)
+      ok = c->matmul_shape.M % 4 == 0 && c->matmul_shape.K >= 64 &&
            c->global_d_layout.eltype == GK_F32 && ldd % 4 == 0 && (no_c || (c->global_c_layout.eltype == GK_F32 && ldc % 4 == 0));
     }
     if (key->fused == 3 && plain) {

@@ -86,7 +86,7 @@ def test_get_config_defaults_for_the_headline_problem():
     assert conf.block_shape == NT(M=256, N=256, K=64)
     # whole 256 x 256 x 64 tiles: four waves, one per SIMD, with 128 x 128 wave tiles
     assert conf.warps_per_block == 4 and conf.compute_warp == NT(M=128, N=128, K=16)
-    # ... also with tiles over the edges where M is a multiple of 8 ('N' A; 'N' B takes any N); eight waves with 128 x 64 wave tiles otherwise
+    # ... also with tiles over the edges where M is a multiple of 4; eight waves with 128 x 64 wave tiles otherwise
     col = Layout.ColMajor
     ragged = gk.get_config(**base_kwargs(M=4000, N=4000, K=4000, global_a_layout=col[F16], global_c_layout=col[F32],
                                          block_shape=NT(M=256, N=256, K=64)))

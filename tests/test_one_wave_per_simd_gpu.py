@@ -235,15 +235,17 @@ def test_nothing_is_written_outside_d(gpu):
 
 
 @pytest.mark.parametrize("ta,tb,M,N,K,four_waves", [
-    (False, False, 264, 515, 100, True),     # 'N' B is contiguous along k: any N
-    (True, False, 260, 515, 136, True),      # 'T' A as well: M in fours (the 16-byte accesses to C / D)
-    (True, True, 260, 520, 197, True),
-    (False, False, 260, 515, 100, False),    # 'N' A is contiguous along M: M in eights
-    (True, True, 260, 516, 100, False),      # 'T' B is contiguous along N: N in eights
-    (True, False, 258, 512, 128, False)])    # M not in fours
-def test_extents_in_fours_and_eights(gpu, ta, tb, M, N, K, four_waves):
-    """Which extents the four waves take with tiles over the edges: M in fours, and in eights along an operand whose
-    16-byte chunks run along M or N; the rest runs on eight waves.  Same bits either way."""
+    (False, False, 264, 515, 100, True),     # an odd N
+    (True, False, 260, 515, 136, True),      # M in fours (the 16-byte accesses to C / D)
+    (True, True, 260, 517, 197, True),
+    # operands whose 16-byte chunks run along M or N and reach over the edge: the last K tile runs behind the loop
+    (False, False, 260, 515, 128, True), (False, False, 260, 515, 100, True), (False, False, 260, 515, 64, True),
+    (True, True, 260, 517, 192, True), (False, True, 516, 262, 320, True),
+    (True, False, 258, 512, 128, False),     # M not in fours
+    (False, False, 261, 512, 128, False)])
+def test_extents_in_fours(gpu, ta, tb, M, N, K, four_waves):
+    """Which extents the four waves take with tiles over the edges: M in fours, any N and K; the rest runs on eight
+    waves.  Same bits either way."""
     a, b, c = operands(M, N, K, ta, tb, 7900 + M + N)
     four, eight = config(M, N, K, ta, tb, (2, 2), checked=True), config(M, N, K, ta, tb, (2, 4), checked=True)
     name = gk.kernel_name(four, Kernel.matmul_pipelined)
@@ -254,8 +256,8 @@ def test_extents_in_fours_and_eights(gpu, ta, tb, M, N, K, four_waves):
     assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= TOL
 
 
-def test_extents_that_are_not_multiples_of_8_run_on_eight_waves(gpu):
-    M2, N2, K2 = 300, 520, 136
+def test_extents_that_are_not_multiples_of_4_run_on_eight_waves(gpu):
+    M2, N2, K2 = 302, 520, 136
     a2, b2, c2 = operands(M2, N2, K2, False, False, 7510)
     ragged = config(M2, N2, K2, False, False, (2, 2), checked=True)
     assert "_w2x4_" in gk.kernel_name(ragged, Kernel.matmul_pipelined)
