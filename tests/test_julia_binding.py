@@ -191,7 +191,7 @@ def test_every_name_the_integration_notes_use_is_defined():
     exported = set(re.findall(r"\w+!?", re.search(r"^export (.*?)\n\n", SRC, re.S | re.M).group(1)))
     for name in ("Layout", "Operator", "Transform", "Epilogue", "Kernel", "to_device", "DeviceArray", "get_config", "matmul", "mul!", "matmatmul!"):
         assert name in exported and name in defined, name
-    # what the reference's API needs from the host layer (SURVEY of src/matmul.jl, src/config.jl)
+    # what the reference's API needs from the host layer (reference src/matmul.jl:58-215, src/config.jl:180-316)
     for name in ("Config", "get_config", "create_config", "matmatmul!", "mul!", "matmul", "lower", "lower_layout", "lower_operator",
                  "lower_swizzle", "lower_transform", "lower_epilogue", "empty_gett", "devptr", "heuristic_block_shape", "adjacent_elements",
                  "validate", "shmem_size", "specialize", "last_error"):
