@@ -243,8 +243,8 @@ int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_
 }
 
 // The arrangement of four waves with 128 x 128 wave tiles (one wave per SIMD, see Cfg::SOLO) is compiled for plain
-// products without hooks or bias whose extents are whole numbers of tiles, and for plain products without hooks whose M is a
-// multiple of 4 (tiles over the edges, a partial last K tile: path 3 of the kernel, which moves an FP32 C / D 16 bytes at a time).  Any other launch of such a configuration runs the
+// products without hooks or bias whose extents are whole numbers of tiles, and for plain products without hooks of any extents
+// (tiles over the edges, a partial last K tile: path 3 of the kernel, which moves an FP32 C / D 16 bytes at a time).  Any other launch of such a configuration runs the
 // eight-wave arrangement of the same block shape, which gives the same bits (the order of the k-steps and of the
 // products inside them does not depend on how the tile is dealt out to waves).
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
@@ -255,12 +255,8 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
     const bool whole = c->matmul_shape.M % 256 == 0 && c->matmul_shape.N % 256 == 0 && c->matmul_shape.K % 64 == 0;
     bool ok = whole;
     if (!whole && plain && key->fused == 0) {
-      const long long ldc = c->global_c_layout.ld > 0 ? c->global_c_layout.ld : c->matmul_shape.M;
-      const long long ldd = c->global_d_layout.ld > 0 ? c->global_d_layout.ld : c->matmul_shape.M;
       const bool no_c = c->global_c_layout.kind == GK_LAYOUT_ZERO;
-      // (M in fours: a lane's four rows of C / D are inside or outside together)
-      ok = c->matmul_shape.M % 4 == 0 && c->matmul_shape.K >= 64 &&
-           c->global_d_layout.eltype == GK_F32 && ldd % 4 == 0 && (no_c || (c->global_c_layout.eltype == GK_F32 && ldc % 4 == 0));
+      ok = c->matmul_shape.M >= 8 && c->matmul_shape.K >= 64 && c->global_d_layout.eltype == GK_F32 && (no_c || c->global_c_layout.eltype == GK_F32);
     }
     if (key->fused == 3 && plain) {
       // hooks of C and D and a bias: the four waves take what has a closed form (fuse level 4 of the kernel): no hook on
@@ -908,8 +904,10 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
   gk::GemmArgs& args = out->args;
   make_args(conf, a, b, c, d, transforms, epilogue, &args);
   const bool solo_edges = key.family == gk::FAMILY_MFMA && key.fused == 0 && (args.M % 256 != 0 || args.N % 256 != 0 || args.K % 64 != 0);
+  // (16-byte accesses to an FP32 C / D: at 16-byte boundaries for a contraction, at those of an element for a product with tiles over its edges)
+  const bool cd_fit = solo_edges ? ((((uintptr_t)args.d) | (args.c_mode != 0 ? (uintptr_t)args.c : 0)) & 3u) == 0 : gk::solo_cd_path(args) != 0;
   if (!custom && (key.family == gk::FAMILY_GETT || solo_edges) && key.BM == 256 && key.BN == 256 && key.BK == 64 && key.waves_m == 2 && key.waves_n == 2 &&
-      gk::solo_cd_path(args) == 0) {
+      !cd_fit) {
     // a contraction on the four-wave arrangement, and a product with tiles over its edges, move C and D 16 bytes at a
     // time: pointers that do not allow it run the eight-wave arrangement (see make_key)
     key.waves_n = 4;

@@ -497,7 +497,8 @@ struct MfmaGemmConfig {
 
 // CPATH (Cfg::SOLO only; 0 elsewhere): how C comes in and D goes out.  1: FP32 C and D with 16-byte accesses, straight into
 // and out of the accumulation registers; 2: no C, D as in 1; 3: as 1 and 2 for products whose extents are not whole numbers of
-// tiles (M a multiple of 4: edge tiles leave out what lies outside D, a partial last K tile runs behind the loop); 0: anything else.  One kernel per path, chosen by the host
+// tiles (FP32 C / D at any 4-byte alignment: edge tiles leave out what lies outside D, a partial last K tile runs behind the loop);
+// 0: anything else.  One kernel per path, chosen by the host
 // (solo_cd_path): where the paths met in one kernel, the register allocator gave the accumulators different registers
 // on each and shuffled 250 of them in front of the K loop.
 template <class Cfg, int CPATH = 0>
@@ -854,9 +855,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     static_assert(!Cfg::GETT || CPATH != 0, "contractions run the four waves with 16-byte C / D accesses only");
     if (load_c) solo_origins(solo_row, solo_col);
     if constexpr (CPATH == 3) {
-      // FP32 C with 16-byte accesses, tiles over the edge included: M is a multiple of 4 (the host runs this path on nothing
-      // else), so a lane's four rows are inside or outside together; rows and columns outside are read from the last ones
-      // inside, and what is accumulated on them is never stored
+      // FP32 C with 16-byte accesses (at any 4-byte alignment), tiles over the edge included: rows and columns outside are
+      // read from the last ones inside, and what is accumulated on them is never stored
       if (load_c) {
 #pragma unroll
         for (int fj = 0; fj < FN; ++fj)
@@ -869,6 +869,27 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(acc[fi][fj]) : "v"(cp) : "memory");
           }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const int m4 = args.M & 3;
+        if (m4 != 0) {
+          // M not in fours: the lane whose four rows reach over the last row was loaded 4 - m4 rows early (the clamp
+          // above); its rows inside C are the last m4 values of what arrived
+#pragma unroll
+          for (int fj = 0; fj < FN; ++fj)
+#pragma unroll
+            for (int fi = 0; fi < FM; ++fi) {
+              const int r = solo_row + MI * fi;
+              asm volatile("" : "+a"(acc[fi][fj]));         // (one block at a time)
+              if (r < args.M && r + 4 > args.M) {
+                const AccV t = acc[fi][fj];
+                AccV o = t;
+                o[0] = m4 == 3 ? t[1] : (m4 == 2 ? t[2] : t[3]);
+                o[1] = m4 == 3 ? t[2] : t[3];
+                o[2] = t[3];
+                acc[fi][fj] = o;
+              }
+              asm volatile("" : "+a"(acc[fi][fj]));
+            }
+        }
       } else {
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi)
@@ -1754,7 +1775,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       return;
     }
     if constexpr (CPATH == 3) {
-      // (blocks of four rows and a column that lie outside D are left out)
+      // (what lies outside D is left out: columns, groups of four rows, and the last rows of the group that reaches over
+      // the last row of a D whose M is not in fours)
 #pragma unroll
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
@@ -1762,7 +1784,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           const int r = solo_row + MI * fi, cc = solo_col + MI * fj;
           if (r < args.M && cc < args.N) {
             float* dp = (float*)args.d + ((long long)r + (long long)cc * args.ldd);
-            asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
+            if (r + 4 <= args.M) {
+              asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
+            } else {
+              const int left = args.M - r;     // 1 .. 3
+              asm volatile("global_store_dword %0, %1, off" :: "v"(dp), "a"(acc[fi][fj][0]) : "memory");
+              if (left > 1) asm volatile("global_store_dword %0, %1, off offset:4" :: "v"(dp), "a"(acc[fi][fj][1]) : "memory");
+              if (left > 2) asm volatile("global_store_dword %0, %1, off offset:8" :: "v"(dp), "a"(acc[fi][fj][2]) : "memory");
+            }
           }
         }
     } else if constexpr (CPATH != 0) {

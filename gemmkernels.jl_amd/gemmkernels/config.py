@@ -330,9 +330,9 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
     checked = any(l.kind in (Layout.COL_MAJOR, Layout.ROW_MAJOR) for l in (global_a_layout, global_b_layout, global_c_layout, global_d_layout))
     whole_tiles = gemm_shape.M % block_shape.M == 0 and gemm_shape.N % block_shape.N == 0 and gemm_shape.K % block_shape.K == 0
     if operator.kind == Operator.MFMA and not is_gett:
-        # (the plain product also where tiles stick out over the edges, for an M that is a multiple of 4; the library
-        # runs the eight-wave arrangement where C / D do not take 16-byte accesses)
-        whole_tiles = whole_tiles or (gemm_shape.M % 4 == 0 and gemm_shape.K >= 64)
+        # (the plain product also where tiles stick out over the edges; the library runs the eight-wave arrangement
+        # where C / D are not FP32)
+        whole_tiles = whole_tiles or (gemm_shape.M >= 8 and gemm_shape.K >= 64)
     waves = _default_waves(operator, block_shape, checked, planar, is_gett, a_kmajor, b_kmajor, whole_tiles)
     if waves is not None:
         warps_default = waves[0] * waves[1]

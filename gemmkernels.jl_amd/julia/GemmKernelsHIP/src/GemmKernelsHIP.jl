@@ -433,9 +433,9 @@ function get_config(; gemm_shape, operator, global_a_layout, global_c_layout, kw
 
     whole_tiles = gemm_shape.M % block_shape.M == 0 && gemm_shape.N % block_shape.N == 0 && gemm_shape.K % block_shape.K == 0
     if Operator.is_mfma(operator) && !haskey(params, :gett)
-        # (the plain product also where tiles stick out over the edges, for an M that is a multiple of 4; the library
-        # runs the eight-wave arrangement where C / D do not take 16-byte accesses)
-        whole_tiles = whole_tiles || (gemm_shape.M % 4 == 0 && gemm_shape.K >= 64)
+        # (the plain product also where tiles stick out over the edges; the library runs the eight-wave arrangement
+        # where C / D are not FP32)
+        whole_tiles = whole_tiles || (gemm_shape.M >= 8 && gemm_shape.K >= 64)
     end
     waves = default_waves(operator, block_shape; a_kmajor = a_kmajor, b_kmajor = b_kmajor, planar = planar, whole_tiles = whole_tiles)
     if waves !== nothing

@@ -86,14 +86,15 @@ def test_get_config_defaults_for_the_headline_problem():
     assert conf.block_shape == NT(M=256, N=256, K=64)
     # whole 256 x 256 x 64 tiles: four waves, one per SIMD, with 128 x 128 wave tiles
     assert conf.warps_per_block == 4 and conf.compute_warp == NT(M=128, N=128, K=16)
-    # ... also with tiles over the edges where M is a multiple of 4; eight waves with 128 x 64 wave tiles otherwise
+    # ... also with tiles over the edges; eight waves with 128 x 64 wave tiles for a K of less than one tile
     col = Layout.ColMajor
-    ragged = gk.get_config(**base_kwargs(M=4000, N=4000, K=4000, global_a_layout=col[F16], global_c_layout=col[F32],
-                                         block_shape=NT(M=256, N=256, K=64)))
-    assert ragged.warps_per_block == 4 and ragged.compute_warp == NT(M=128, N=128, K=16)
-    ragged = gk.get_config(**base_kwargs(M=4001, N=4003, K=4005, global_a_layout=col[F16], global_c_layout=col[F32],
-                                         block_shape=NT(M=256, N=256, K=64)))
-    assert ragged.warps_per_block == 8 and ragged.compute_warp == NT(M=128, N=64, K=16)
+    for size in (4000, 4001):
+        ragged = gk.get_config(**base_kwargs(M=size, N=size + 2, K=size + 4, global_a_layout=col[F16], global_c_layout=col[F32],
+                                             block_shape=NT(M=256, N=256, K=64)))
+        assert ragged.warps_per_block == 4 and ragged.compute_warp == NT(M=128, N=128, K=16)
+    short = gk.get_config(**base_kwargs(M=4000, N=4000, K=40, global_a_layout=col[F16], global_c_layout=col[F32],
+                                        block_shape=NT(M=256, N=256, K=64)))
+    assert short.warps_per_block == 8 and short.compute_warp == NT(M=128, N=64, K=16)
     assert conf.compute_op_shape == NT(M=32, N=32, K=16)
     # 64-lane waves, 16 bytes per lane (src/config.jl:240-260 with 64 lanes)
     assert conf.mem_a_warp == NT(M=256, K=2) and conf.mem_a_thread == NT(M=8, K=1)

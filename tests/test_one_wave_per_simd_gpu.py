@@ -197,7 +197,7 @@ def test_tiles_over_the_edges_without_c_in_place_and_off_a_16_byte_boundary(gpu)
     # d aliases c (reference src/matmul.jl:198)
     ref = helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
     assert np.array_equal(helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined, alias_cd=True), ref)
-    # C and D that start 4 bytes into a 16-byte line: the library runs the eight waves; nothing outside D is written
+    # C and D that start 4 bytes into a 16-byte line; nothing outside D is written
     A, B = gk.colmajor(a), gk.colmajor(b)
     cbuf = torch.zeros(M * N + 1, dtype=torch.float32, device="cuda")
     dbuf = torch.full((M * N + 9,), float("nan"), dtype=torch.float32, device="cuda")
@@ -210,10 +210,11 @@ def test_tiles_over_the_edges_without_c_in_place_and_off_a_16_byte_boundary(gpu)
     assert bool(torch.isnan(dbuf[0])) and bool(torch.isnan(dbuf[1 + M * N:]).all())
 
 
-def test_nothing_is_written_outside_d(gpu):
+@pytest.mark.parametrize("M", [264, 261, 263])
+def test_nothing_is_written_outside_d(gpu, M):
     """D as a window of a larger matrix (leading dimension beyond M) whose other elements keep their values."""
     import torch
-    M, N, K, LD = 264, 136, 128, 272
+    N, K, LD = 136, 128, 272
     a, b, c = operands(M, N, K, False, True, 7850)
     col = Layout.ColMajor
     conf = gk.get_config(
@@ -234,35 +235,44 @@ def test_nothing_is_written_outside_d(gpu):
     assert bool(torch.isnan(outside).all()) and not bool(torch.isnan(big[1:1 + N, :M]).any())
 
 
-@pytest.mark.parametrize("ta,tb,M,N,K,four_waves", [
-    (False, False, 264, 515, 100, True),     # an odd N
-    (True, False, 260, 515, 136, True),      # M in fours (the 16-byte accesses to C / D)
-    (True, True, 260, 517, 197, True),
+@pytest.mark.parametrize("ta,tb,M,N,K", [
+    (False, False, 264, 515, 100),     # an odd N
+    (True, False, 260, 515, 136),
+    (True, True, 260, 517, 197),
     # operands whose 16-byte chunks run along M or N and reach over the edge: the last K tile runs behind the loop
-    (False, False, 260, 515, 128, True), (False, False, 260, 515, 100, True), (False, False, 260, 515, 64, True),
-    (True, True, 260, 517, 192, True), (False, True, 516, 262, 320, True),
-    (True, False, 258, 512, 128, False),     # M not in fours
-    (False, False, 261, 512, 128, False)])
-def test_extents_in_fours(gpu, ta, tb, M, N, K, four_waves):
-    """Which extents the four waves take with tiles over the edges: M in fours, any N and K; the rest runs on eight
-    waves.  Same bits either way."""
+    (False, False, 260, 515, 128), (False, False, 260, 515, 100), (False, False, 260, 515, 64),
+    (True, True, 260, 517, 192), (False, True, 516, 262, 320),
+    # M not in fours: the group of four rows that reaches over the last row of C / D goes element by element, and the
+    # columns of C / D are not 16-byte aligned
+    (False, False, 257, 512, 128), (False, False, 258, 300, 64), (False, False, 259, 513, 197), (False, False, 261, 512, 128),
+    (True, False, 258, 512, 128), (False, True, 511, 258, 100), (True, True, 1001, 33, 203), (False, False, 1001, 1003, 1005)])
+def test_any_extents(gpu, ta, tb, M, N, K):
+    """Tiles over the edges at any M, N and K (M of at least 8, K of at least 64): same bits as eight waves."""
     a, b, c = operands(M, N, K, ta, tb, 7900 + M + N)
     four, eight = config(M, N, K, ta, tb, (2, 2), checked=True), config(M, N, K, ta, tb, (2, 4), checked=True)
     name = gk.kernel_name(four, Kernel.matmul_pipelined)
     print("case", ta, tb, M, N, K, name, flush=True)
-    assert ("_w2x2_" in name and name.endswith("_edges")) if four_waves else "_w2x4_" in name
+    assert "_w2x2_" in name and name.endswith("_edges")
     d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
     assert np.array_equal(d4, helpers.run_gpu(eight, a, b, c, (M, N), kernel=Kernel.matmul_pipelined))
     assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= TOL
+    # ... without C, and with D in the place of C
+    zero4, zero8 = (config(M, N, K, ta, tb, w, zero_c=True, checked=True) for w in ((2, 2), (2, 4)))
+    assert np.array_equal(helpers.run_gpu(zero4, a, b, None, (M, N), kernel=Kernel.matmul_pipelined),
+                          helpers.run_gpu(zero8, a, b, None, (M, N), kernel=Kernel.matmul_pipelined))
+    assert np.array_equal(helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined, alias_cd=True), d4)
 
 
-def test_extents_that_are_not_multiples_of_4_run_on_eight_waves(gpu):
+def test_16_bit_d_and_short_products_with_tiles_over_the_edges_run_on_eight_waves(gpu):
+    import torch
     M2, N2, K2 = 302, 520, 136
     a2, b2, c2 = operands(M2, N2, K2, False, False, 7510)
-    ragged = config(M2, N2, K2, False, False, (2, 2), checked=True)
+    ragged = config(M2, N2, K2, False, False, (2, 2), d=Float16, checked=True)
     assert "_w2x4_" in gk.kernel_name(ragged, Kernel.matmul_pipelined)
-    d2 = helpers.run_gpu(ragged, a2, b2, c2, (M2, N2), kernel=Kernel.matmul_pipelined)
+    d2 = helpers.run_gpu(ragged, a2, b2, c2, (M2, N2), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
     assert oracle.rel_frobenius(d2, oracle.gemm_f64(a2, b2, c2, 1.0, 1.0, False, False)) <= TOL
+    short = config(M2, N2, 40, False, False, (2, 2), checked=True)
+    assert "_w2x4_" in gk.kernel_name(short, Kernel.matmul_pipelined)
 
 
 def test_default_configuration_of_a_large_product(gpu):
