@@ -210,6 +210,34 @@ def test_create_config_choices():
         create_config(F16, (128, 64), (1, 128), False, F16, (128, 128), (1, 128), False, F32, (128, 128), (1, 128), float, False, float, False, None)
 
 
+def test_which_launches_of_the_headline_tile_run_on_four_waves():
+    """What the library runs for a configuration of the 256 x 256 x 64 tile with four waves (one per SIMD): that
+    arrangement where it is compiled for the launch, the eight-wave arrangement of the same tile elsewhere (same bits)."""
+    from gemmkernels import Transform, Epilogue
+    col = Layout.ColMajor
+
+    def name(M, N, K, c=F32, d=F32, checked=False, **kw):
+        lay = col if checked else ACM
+        conf = gk.get_config(gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=256, N=256, K=64), warps_per_block=4,
+                             compute_warp=NT(M=128, N=128, K=16), operator=Operator.MFMAOp[32, 32, 16, F16, F32],
+                             global_a_layout=lay[F16], global_b_layout=lay[F16], global_c_layout=lay[c], global_d_layout=lay[d])
+        return gk.kernel_name(conf, Kernel.matmul_pipelined, **kw)
+
+    assert name(4096, 4096, 4096) == "mfma_gemm_nn_256x256x64_w2x2_s2__Float16"
+    assert name(4096, 4096, 4096, c=F16, d=F16) == "mfma_gemm_nn_256x256x64_w2x2_s2__Float16"
+    # tiles over the edges, a partial last K tile, odd extents: an instance of its own
+    for size in ((4000, 4000, 4000), (4001, 4003, 4005), (8, 1032, 64)):
+        assert name(*size, checked=True) == "mfma_gemm_nn_256x256x64_w2x2_s2__Float16_edges"
+    # ... for FP32 C / D and at least one whole K tile
+    assert "_w2x4_" in name(4000, 4000, 4000, d=F16, checked=True)
+    assert "_w2x4_" in name(4000, 4000, 40, checked=True)
+    # hooks of D in closed form and a bias; any other hook runs on eight waves
+    E = Transform.Elementwise
+    assert name(512, 512, 512, transforms=dict(transform_shared_to_global_d=E(Transform.relu)), epilogue=Epilogue.Bias(None)).endswith("_w2x2_s2__Float16_fused_d")
+    assert "_w2x4_" in name(512, 512, 512, transforms=dict(transform_global_to_shared_c=E(lambda x: x * 0.25)))
+    assert "_w2x4_" in name(4000, 4000, 4000, checked=True, transforms=dict(transform_shared_to_global_d=E(Transform.relu)))
+
+
 def test_every_tile_of_the_python_tables_has_a_compiled_instance():
     """The tile tables the defaults are drawn from and the instances compiled into the library
     must not drift apart: every entry resolves to a kernel name."""
