@@ -242,8 +242,8 @@ def _complex_tiles(operator, planar, a_kmajor, b_kmajor):
 
 # One wave per SIMD: 256 x 256 x 64 on four waves with 128 x 128 wave tiles (a third fewer LDS reads per MFMA than
 # 2 x 4 waves, and a K loop written out slot by slot: 105 against 116 us at 4096^3).  Compiled for plain products
-# without hooks whose extents are whole numbers of tiles; the library runs the 2 x 4 arrangement of the same block
-# shape, with the same bits, for any other launch of such a configuration.
+# without hooks (whole tiles, or any extents with an FP32 C / D) and with hooks of D in closed form; the library runs
+# the 2 x 4 arrangement of the same block shape, with the same bits, for any other launch of such a configuration.
 _SOLO_TILE, _SOLO_WAVES = (256, 256, 64), (2, 2)
 _SOLO_COMPLEX_TILE = (128, 128, 64)        # in complex elements
 

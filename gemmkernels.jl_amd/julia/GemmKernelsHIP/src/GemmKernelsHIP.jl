@@ -386,8 +386,8 @@ function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true
 end
 
 # One wave per SIMD: 256 x 256 x 64 on four waves with 128 x 128 wave tiles, compiled for plain products without hooks
-# whose extents are whole numbers of tiles.  The library runs the 2 x 4 arrangement of the same block shape, with the
-# same bits, for any other launch of such a configuration.
+# (whole tiles, or any extents with an FP32 C / D) and with hooks of D in closed form.  The library runs the 2 x 4
+# arrangement of the same block shape, with the same bits, for any other launch of such a configuration.
 const SOLO_TILE = (256, 256, 64)
 const SOLO_WAVES = (2, 2)
 const SOLO_COMPLEX_TILE = (128, 128, 64)       # in complex elements
