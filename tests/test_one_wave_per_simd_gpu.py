@@ -210,11 +210,12 @@ def test_tiles_over_the_edges_without_c_in_place_and_off_a_16_byte_boundary(gpu)
     assert bool(torch.isnan(dbuf[0])) and bool(torch.isnan(dbuf[1 + M * N:]).all())
 
 
-@pytest.mark.parametrize("M", [264, 261, 263])
-def test_nothing_is_written_outside_d(gpu, M):
-    """D as a window of a larger matrix (leading dimension beyond M) whose other elements keep their values."""
+@pytest.mark.parametrize("M,LD", [(264, 272), (261, 272), (263, 272), (264, 273), (262, 275)])
+def test_nothing_is_written_outside_d(gpu, M, LD):
+    """D as a window of a larger matrix (leading dimension beyond M, columns on and off 16-byte boundaries) whose other
+    elements keep their values."""
     import torch
-    N, K, LD = 136, 128, 272
+    N, K = 136, 128
     a, b, c = operands(M, N, K, False, True, 7850)
     col = Layout.ColMajor
     conf = gk.get_config(
