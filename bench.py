@@ -28,6 +28,7 @@ HEADLINE_SETTLE_SECONDS = 0.4
 # HBM bytes per launch of the headline kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # summarised in profiles/ (None until measured)
 MEASURED_TRAFFIC_BYTES = 338_074_624   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131153.1 * 2.0 + 67844.8) KiB
+TRAFFIC_SOURCE = "profiles/mfma_gemm_config2_hbm_traffic.txt (a constant from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE passes, not a reading of this run)"
 
 
 def parse_args():
@@ -130,6 +131,35 @@ def time_launches(fn, steps, warmup, settle_seconds=0.0):
     return start.elapsed_time(stop) * 1e3 / steps, wall
 
 
+def settle_then_time(fn, steps, warmup, settle_seconds):
+    """time_launches, and the number of untimed launches of the settle phase."""
+    count = {"n": 0}
+
+    def counted():
+        count["n"] += 1
+        fn()
+    us, wall = time_launches(counted, steps, warmup, settle_seconds)
+    return us, wall, count["n"] - steps - warmup
+
+
+def verify_slab(wl, run, cols=256):
+    """Outside every timed region: the output the timed launches of the headline workload ('N','N') left in `run.d`, its
+    first and its last `cols` columns, against the float64 product D = A*B + C of the same seeded inputs.
+    Returns (ok, relative Frobenius error)."""
+    import numpy as np
+    import gemmkernels as gk
+    h = wl.host()
+    a, b, c = h["a"].astype(np.float64), h["b"], h["c"]
+    d = gk.to_numpy(run.d)
+    num = den = 0.0
+    for sl in (slice(0, cols), slice(c.shape[1] - cols, c.shape[1])):
+        ref = a @ b[:, sl].astype(np.float64) + c[:, sl]
+        num += float(((d[:, sl] - ref) ** 2).sum())
+        den += float((ref ** 2).sum())
+    err = (num / den) ** 0.5
+    return bool(err <= 1e-3), err
+
+
 def launch_distribution(fn, launches=40):
     """Min and median duration in microseconds of single launches, each bracketed by its own pair of events."""
     import torch
@@ -195,8 +225,9 @@ def main():
     # the W warm-up launches are followed by a time-based settle phase (untimed, like the warm-up): a short run
     # such as --steps 20 --warmup 5 would otherwise time the first milliseconds after idle, while the shader
     # clock is still coming up (the secondary figures below have always been taken after such a phase)
-    us, wall = time_launches(run, args.steps, args.warmup, HEADLINE_SETTLE_SECONDS)
+    us, wall, settle_launches = settle_then_time(run, args.steps, args.warmup, HEADLINE_SETTLE_SECONDS)
     tflops = wl.flops / us / 1e6
+    ok, err = verify_slab(wl, run)
     result = {
         "metric": METRIC,
         "value": round(tflops, 2),
@@ -204,6 +235,8 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_s": HEADLINE_SETTLE_SECONDS,
+        "settle_launches": settle_launches,
         "ms_per_step": round(us / 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",
@@ -211,10 +244,13 @@ def main():
         "dtype": "f16 multiplicands, f32 accumulate",
         "data": "synthetic (counter-based splitmix64 streams, seeds 2001-2003)",
         "config": {"workload": wl.description, "kernel": wl.kernel_name},
+        "verified": ok,
+        "verified_rel_frobenius_error": float(f"{err:.3e}"),
+        "verified_against": "float64 product of the same inputs on the first and the last 256 columns of the D the timed launches wrote",
         "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_FP16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": wl.kernel_name, "avg_launch_us": round(us, 2), "flop_per_launch": wl.flops},
+                     "traffic_source": TRAFFIC_SOURCE, "kernel": wl.kernel_name, "avg_launch_us": round(us, 2), "flop_per_launch": wl.flops},
     }
 
     if not args.no_extras:

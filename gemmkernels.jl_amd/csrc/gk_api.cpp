@@ -992,7 +992,13 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
 
 namespace {
 
-constexpr size_t kCounterAlign = 256;
+// The arrival counters of a K-split launch take a region of fixed size at the head of the workspace, whatever the
+// product: a launch is split only when its tiles leave CUs idle (split_k_slices gives one slice from 2 * kNumCUs tiles
+// on), so kSplitCounterBytes / 4 counters are enough for every launch that uses them.  With a region whose size followed
+// the tile count, a workspace reused by a product with more tiles would have found the float bits of old partial sums
+// where its counters are.
+constexpr size_t kSplitCounterBytes = 2048;
+static_assert(kSplitCounterBytes / sizeof(unsigned) >= 2 * (size_t)gk::kNumCUs - 1, "one counter for every tile of a launch that is split");
 
 // K slices of a K-split launch, from a sweep of slice counts on 4096 x 64 x 4096, 256 x 256 x 16384 and
 // 8192 x 128 x 8192: about two workgroups per CU, and slices at least 1024 deep in K -- a slice pays for its
@@ -1005,8 +1011,6 @@ int split_k_slices(int tiles, int k_tiles, int block_k) {
   if (slices > k_tiles / min_tiles) slices = k_tiles / min_tiles;
   return slices < 1 ? 1 : slices;
 }
-
-size_t split_k_counter_bytes(int tiles) { return ((size_t)tiles * sizeof(unsigned) + kCounterAlign - 1) / kCounterAlign * kCounterAlign; }
 
 }  // namespace
 
@@ -1034,7 +1038,9 @@ int launch_split_k(const gk_config* conf, const void* a, const void* b, const vo
   if (slices > 1 && !L.ragged && sk_fn && sk_fn(L.key, L.args, dim3(1), nullptr, 0, &sk_info, &err)) {
     const int per = (kt + slices - 1) / slices;
     slices = (kt + per - 1) / per;           // no empty slice: every slice arrives at its tile's counter
-    const size_t counters = split_k_counter_bytes(tiles);
+    const size_t counters = kSplitCounterBytes;
+    if ((size_t)tiles * sizeof(unsigned) > counters)
+      return fail(GK_ERR_INVALID_ARGUMENT, "a K-split launch of %d tiles has no room for its arrival counters (%zu bytes)", tiles, counters);
     const size_t need = counters + (size_t)tiles * slices * conf->block_shape.M * conf->block_shape.N * sizeof(float);
     if (!workspace || workspace_bytes < need)
       return fail(GK_ERR_INVALID_ARGUMENT, "the K-split launch needs a workspace of %zu bytes (%d tiles x %d slices of %d x %d floats); %s holds %zu",
@@ -1067,7 +1073,7 @@ int gk_split_k_workspace_size(const gk_config* conf, size_t* bytes) {
   const int kt = (g.K + b.K - 1) / b.K;
   const long long slices = split_k_slices((int)(tiles > (1 << 30) ? (1 << 30) : tiles), kt, b.K);
   if (slices < 2) { *bytes = 0; return GK_OK; }      // runs unsplit
-  *bytes = split_k_counter_bytes((int)tiles) + (size_t)tiles * (size_t)slices * b.M * b.N * sizeof(float);
+  *bytes = kSplitCounterBytes + (size_t)tiles * (size_t)slices * b.M * b.N * sizeof(float);
   return GK_OK;
 }
 

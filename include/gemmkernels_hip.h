@@ -275,10 +275,12 @@ int gk_matmul(const gk_config* conf, const void* a, const void* b, const void* c
 /* The K-split kind of launch (GK_KERNEL_SPLIT_K above; no counterpart in the reference, whose launcher
  * src/matmul.jl:7-44 has one kernel per product).  gk_split_k_workspace_size gives an upper bound of
  * the workspace a launch of `conf` needs (0: it runs unsplit); gk_matmul_split_k is gk_matmul plus the
- * workspace: device memory owned by the caller, 16-byte aligned, ZEROED BEFORE ITS FIRST USE.  Its head
- * holds one arrival counter per output tile, which every launch leaves at zero again, so one workspace
- * serves any number of launches one after the other; launches that overlap in time (two streams) need
- * a workspace each. */
+ * workspace: device memory owned by the caller, 16-byte aligned, ZEROED BEFORE ITS FIRST USE.  Its first
+ * 2048 bytes hold the arrival counters of the output tiles -- a region of the same size for every product,
+ * so that launches of different shapes find their counters in the same place -- which every launch leaves
+ * at zero again: one workspace serves any number of launches of any products one after the other; launches
+ * that overlap in time (two streams) need a workspace each.  A launch that faulted or was aborted may leave
+ * counters behind: zero the first 2048 bytes again before the workspace is used after such a failure. */
 int gk_split_k_workspace_size(const gk_config* conf, size_t* bytes);
 int gk_matmul_split_k(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
                       const gk_transforms* transforms, const gk_epilogue* epilogue, void* workspace,
@@ -291,7 +293,10 @@ int gk_matmul_split_k(const gk_config* conf, const void* a, const void* b, const
  * GPU the library is used on, for the life of the process).  A launch that needs more is refused with
  * GK_ERR_INVALID_ARGUMENT and a message that names both sizes; nothing is allocated or freed by the call,
  * on the device or through any library.  All calls on one GPU share the array: calls that overlap in time
- * (two streams, two host threads) race on it and must be serialised by the caller. */
+ * (two streams, two host threads) race on it and must be serialised by the caller.  The first call on a
+ * device asks the runtime for the array's address, which may load the library's device code at that moment:
+ * make that first call (any product will do) outside of a stream capture; every later call on that device
+ * only launches the kernel. */
 size_t gk_split_k_noalloc_capacity(void);
 int gk_matmul_split_k_noalloc(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
                               const gk_transforms* transforms, const gk_epilogue* epilogue, void* stream);

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import gemmkernels as gk
-from gemmkernels import Layout, Operator, Kernel, CTASwizzle, NT, Float16, Float32, rng
+from gemmkernels import Layout, Operator, Kernel, CTASwizzle, NT, Float16, Float32, configs, rng
 import helpers
 from oracle import oracle
 
@@ -136,19 +136,38 @@ def test_wmma_compat_operator(gpu):
     assert oracle.rel_frobenius(d, oracle.gemm_f64(a, b, c, 1.0, 1.0)) <= TOL
 
 
+@pytest.mark.parametrize("waves", [(2, 4), "default"])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-def test_full_size_4096(gpu, ta, tb):
+def test_full_size_4096(gpu, ta, tb, waves):
     """Benchmark config 2 at full size, checked against the CPU BLAS path (OpenBLAS sgemm on the
-    exactly converted inputs) and through linearity: D(C) - D(0) == C."""
+    exactly converted inputs) and through linearity: D(C) - D(0) == C.  `default` is the configuration of the
+    benchmark itself (configs.benchmark_config(2, variant): the tile, wave arrangement and tile walk that bench.py times),
+    (2, 4) the eight-wave arrangement of the same tile.  Comparison as in reference test/matmul.jl:12-20."""
     M = N = K = 4096
     a, b, c = inputs(M, N, K, ta, tb, 2000)
-    conf = make_config(M, N, K, ta, tb, (256, 256, 64), (2, 4))
+    if waves == "default":
+        variant = ("T" if ta else "N") + ("T" if tb else "N")
+        wl = configs.benchmark_config(2, variant=variant)
+        conf = configs.mfma_config(M, N, K, ta, tb)
+        assert gk.kernel_name(conf, Kernel.matmul_pipelined) == wl.kernel_name        # the kernel that the benchmark times
+        assert "w2x2" in wl.kernel_name
+        conf0 = configs.mfma_config(M, N, K, ta, tb, zero_c=True)
+    else:
+        conf = make_config(M, N, K, ta, tb, (256, 256, 64), waves)
+        conf0 = make_config(M, N, K, ta, tb, (256, 256, 64), waves, zero_c=True)
     d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
     ref = oracle.gemm_blas_f32(a, b, c, 1.0, 1.0, ta, tb)
     assert oracle.rel_frobenius(d, ref) <= TOL
-    conf0 = make_config(M, N, K, ta, tb, (256, 256, 64), (2, 4), zero_c=True)
     d0 = helpers.run_gpu(conf0, a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
     assert oracle.rel_frobenius(d - d0, c) <= 1e-4
+    if waves == "default":
+        # the benchmark's own inputs and prepared launch: what bench.py times is what is checked here
+        run = wl.prepare()
+        run()
+        import torch
+        torch.cuda.synchronize()
+        ha, hb, hc = wl.host_inputs()
+        assert oracle.rel_frobenius(gk.to_numpy(run.d), oracle.gemm_blas_f32(ha, hb, hc, 1.0, 1.0, ta, tb)) <= TOL
 
 
 @pytest.mark.parametrize("block,waves", [((256, 256, 64), (2, 4)), ((128, 128, 64), (2, 2)), ((64, 64, 32), (1, 1))])

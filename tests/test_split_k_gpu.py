@@ -178,3 +178,72 @@ def test_skinny_products_with_tiles_over_the_edge_are_split_too(gpu, beta):
     out = full.cpu().numpy()
     assert (out[M:, :] == 555.0).all() and (out[:, N:] == 555.0).all()
     assert oracle.rel_frobenius(out[:M, :N], oracle.gemm_f64(a, b, c, 1.0, beta, False, False)) <= 1e-3
+
+
+def _split_on(ws, M, N, K, block, seed, swizzle=None):
+    """One K-split launch of small-integer data on the workspace `ws`, through the C ABI; returns (D, exact reference)."""
+    import ctypes
+    kw = {} if swizzle is None else {"cta_swizzle": swizzle}
+    conf = configs.mfma_config(M, N, K, block_shape=block, **kw)
+    rs = np.random.RandomState(seed)
+    ai = np.asfortranarray(rs.randint(-4, 5, size=(M, K)).astype(np.float16))
+    bi = np.asfortranarray(rs.randint(-4, 5, size=(K, N)).astype(np.float16))
+    ci = np.asfortranarray(rs.randint(-64, 65, size=(M, N)).astype(np.float32))
+    A, B, C = gk.colmajor(ai), gk.colmajor(bi), gk.colmajor(ci)
+    D = gk.colmajor_empty((M, N), torch.float32)
+    D.fill_(float("nan"))
+    cconf = conf.to_c(M, K, M, M)
+    need = ctypes.c_size_t()
+    assert _lib.lib().gk_split_k_workspace_size(ctypes.byref(cconf), ctypes.byref(need)) == 0 and 0 < need.value <= ws.numel()
+    rc = _lib.lib().gk_matmul_split_k(ctypes.byref(cconf), A.data_ptr(), B.data_ptr(), C.data_ptr(), D.data_ptr(), None, None,
+                                      ws.data_ptr(), ws.numel(), None)
+    assert rc == _lib.GK_OK, _lib.last_error()
+    torch.cuda.synchronize()
+    return gk.to_numpy(D).astype(np.float64), ai.astype(np.float64) @ bi.astype(np.float64) + ci
+
+
+def test_one_workspace_serves_products_with_different_tile_counts(gpu):
+    """The arrival counters sit in a region of fixed size at the head of the workspace.  (With a region as large as the
+    tile count asked for, a product of 128 tiles found the partial sums of an earlier product of 64 tiles where its
+    counters 64 .. 127 are: no workgroup of those tiles ever saw itself arrive last and D stayed unwritten.)  Small-integer
+    data: every sum is exact, so D must equal the float64 product whatever is left in the workspace."""
+    ws = torch.zeros(16 << 20, dtype=torch.uint8, device="cuda")
+    seq = [((4096, 64, 8192), (64, 64, 64)),      # 64 tiles x 8 slices
+           ((1024, 512, 2048), (64, 64, 64)),     # 128 tiles x 2 slices
+           ((4096, 64, 4096), (64, 64, 64)),      # 64 tiles again
+           ((1024, 1024, 2048), (64, 64, 64)),    # 256 tiles x 2 slices
+           ((256, 256, 8192), (128, 128, 64)),    # 4 tiles
+           ((1024, 512, 2048), (64, 64, 64))]
+    for i, (dims, block) in enumerate(seq):
+        print("K-split on a shared workspace:", dims, block, flush=True)
+        got, ref = _split_on(ws, *dims, block, 9000 + i)
+        assert np.array_equal(got, ref), (dims, block)
+    # ... and every counter is back at zero
+    assert int(ws[:2048].to(torch.int32).abs().sum()) == 0
+
+
+def test_many_launches_on_one_workspace_with_other_data_and_other_tile_walks(gpu):
+    """The partial tiles cross from one XCD's L2 to another's through memory (device-scope stores and loads).  A line of
+    the workspace that a launch reads was written by the launch before as well: forty launches on one workspace, each
+    with data of its own and every other one with another tile-to-XCD mapping, must each give the exact product -- a
+    stale line from an earlier launch would show."""
+    from gemmkernels import CTASwizzle
+    ws = torch.zeros(8 << 20, dtype=torch.uint8, device="cuda")
+    walks = [None, CTASwizzle.Identity, CTASwizzle.XCDAware[2], CTASwizzle.HorizontallyTiled[2]]
+    for i in range(40):
+        got, ref = _split_on(ws, 512, 256, 4096, (64, 64, 64), 9100 + i, walks[i % 4])
+        assert np.array_equal(got, ref), i
+
+
+def test_blas_entry_after_a_product_with_fewer_tiles(gpu):
+    """mul! on 4096 x 64 x 8192 (64 tiles) and then on 1024 x 512 x 2048 (128 tiles): both take the K-split kernel and
+    share the workspace the host layer keeps per stream."""
+    for (M, N, K), seed in (((4096, 64, 8192), 9300), ((1024, 512, 2048), 9301), ((4096, 64, 8192), 9302)):
+        rs = np.random.RandomState(seed)
+        ai = np.asfortranarray(rs.randint(-4, 5, size=(M, K)).astype(np.float16))
+        bi = np.asfortranarray(rs.randint(-4, 5, size=(K, N)).astype(np.float16))
+        ci = np.asfortranarray(rs.randint(-64, 65, size=(M, N)).astype(np.float32))
+        C = gk.colmajor(ci)
+        gk.matmatmul_(C, "N", "N", gk.colmajor(ai), gk.colmajor(bi), 1.0, 1.0)
+        torch.cuda.synchronize()
+        assert np.array_equal(gk.to_numpy(C).astype(np.float64), ai.astype(np.float64) @ bi.astype(np.float64) + ci), (M, N, K)

@@ -55,6 +55,12 @@ def test_two_calls_in_a_row_the_second_smaller(gpu):
     _both_ways(256, 256, 8192, (128, 128, 64), 7300)
     print("no-alloc K-split: 64 x 64 x 4096", flush=True)
     _both_ways(64, 64, 4096, (64, 64, 64), 7400)
+    # more tiles than any call before: the counters of the tiles 64 .. 127 lie where, with a counter region sized by
+    # the tile count, the partial sums of the calls above would have been
+    print("no-alloc K-split: 1024 x 512 x 2048 (128 tiles)", flush=True)
+    _both_ways(1024, 512, 2048, (64, 64, 64), 7500)
+    print("no-alloc K-split: 4096 x 64 x 4096 again", flush=True)
+    _both_ways(4096, 64, 4096, (64, 64, 64), 7600)
 
 
 def test_a_product_beyond_the_static_workspace_is_refused(gpu):
