@@ -354,11 +354,23 @@ template <> struct Mfma<_Float16, 16> {
   __device__ static __forceinline__ float4v run(int4v a, int4v b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
   }
+  // ... on the accumulator block in the accumulation registers a[R : R + 3], named in the instruction text: kernels that
+  // manage the accumulation registers themselves (see CPATH 4 of mfma_gemm_kernel).  FIRST: the block starts from zero.
+  template <int R, bool FIRST>
+  __device__ static __forceinline__ void run_fixed(int4v a, int4v b) {
+    if constexpr (FIRST) asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, 0" :: "v"(a), "v"(b), "n"(R), "n"(R + 3));
+    else asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]" :: "v"(a), "v"(b), "n"(R), "n"(R + 3));
+  }
 };
 template <> struct Mfma<__bf16, 16> {
   typedef float4v Acc;
   __device__ static __forceinline__ float4v run(int4v a, int4v b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  template <int R, bool FIRST>
+  __device__ static __forceinline__ void run_fixed(int4v a, int4v b) {
+    if constexpr (FIRST) asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" :: "v"(a), "v"(b), "n"(R), "n"(R + 3));
+    else asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" :: "v"(a), "v"(b), "n"(R), "n"(R + 3));
   }
 };
 
@@ -498,6 +510,9 @@ struct MfmaGemmConfig {
 // CPATH (Cfg::SOLO only; 0 elsewhere): how C comes in and D goes out.  1: FP32 C and D with 16-byte accesses, straight into
 // and out of the accumulation registers; 2: no C, D as in 1; 3: as 1 and 2 for products whose extents are not whole numbers of
 // tiles (FP32 C / D at any 4-byte alignment: edge tiles leave out what lies outside D, a partial last K tile runs behind the loop);
+// 4: as 1 for products of at least kSoloStreamTiles K tiles, with C on its way while the matrix cores run: the accumulators start
+// at zero, the C tile arrives one block column per K tile in registers of its own during the first K tiles and is added to the
+// accumulators there (so the sum is (products of the first K tiles) + C + (the rest), where path 1 starts from C);
 // 0: anything else.  One kernel per path, chosen by the host
 // (solo_cd_path): where the paths met in one kernel, the register allocator gave the accumulators different registers
 // on each and shuffled 250 of them in front of the K loop.
@@ -515,6 +530,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr bool RAGGED = Cfg::RAGGED_OK || (Cfg::SOLO && CPATH == 3);
   constexpr bool RAGGED_K = Cfg::RAGGED_K_OK || (Cfg::SOLO && CPATH == 3);
   static_assert(CPATH != 3 || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "path 3 is compiled for plain real products");
+  static_assert(CPATH != 4 || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "path 4 is compiled for plain real products");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -853,7 +869,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   };
   if constexpr (Cfg::SOLO) {
     static_assert(!Cfg::GETT || CPATH != 0, "contractions run the four waves with 16-byte C / D accesses only");
-    if (load_c) solo_origins(solo_row, solo_col);
+    if (load_c && CPATH != 4) solo_origins(solo_row, solo_col);
     if constexpr (CPATH == 3) {
       // FP32 C with 16-byte accesses (at any 4-byte alignment), tiles over the edge included: rows and columns outside are
       // read from the last ones inside, and what is accumulated on them is never stored
@@ -900,6 +916,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) asm volatile("" : "+a"(acc[fi][fj]));
+    } else if constexpr (CPATH == 4) {
+      // (the accumulators start from zero in the first k-step and C comes in during the first K tiles, see the K loop)
     } else if constexpr (CPATH == 1) {
 #pragma unroll
       for (int fj = 0; fj < SFN; ++fj)
@@ -1253,53 +1271,138 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       else __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR((Cfg::GETT ? part_b : gb) + o), GK_LDS_PTR(void, sb + (wave + (I - DMA_A) * NWAVES) * 1024), 16, 0, 0);
     };
     // LDS instruction R of the fragment reads of k-step KS2 (of the stage the readers stand at), into buffer KS2 & 1
-    auto read_op = [&](auto r_c, auto ks2_c) __attribute__((always_inline)) {
-      constexpr int R = decltype(r_c)::value, KS2 = decltype(ks2_c)::value;
-      if constexpr (R < NOPA) ra.template read_op<R / RA::OPS, KS2, R % RA::OPS>(fa[KS2 & 1][R / RA::OPS]);
-      else rb.template read_op<(R - NOPA) / RB::OPS, KS2, (R - NOPA) % RB::OPS>(fb[KS2 & 1][(R - NOPA) / RB::OPS]);
+    // (into buffer BUF)
+    auto read_op = [&](auto r_c, auto ks2_c, auto buf_c) __attribute__((always_inline)) {
+      constexpr int R = decltype(r_c)::value, KS2 = decltype(ks2_c)::value, BUF = decltype(buf_c)::value;
+      if constexpr (R < NOPA) ra.template read_op<R / RA::OPS, KS2, R % RA::OPS>(fa[BUF][R / RA::OPS]);
+      else rb.template read_op<(R - NOPA) / RB::OPS, KS2, (R - NOPA) % RB::OPS>(fb[BUF][(R - NOPA) / RB::OPS]);
     };
     // The MFMAs of k-step ks.  The fragments of k-step (ks + 1) % KS -- of this tile, or of the next one when ks is the
     // last k-step -- are read in the slots behind the first MFMAs.  DMA: the k-step also issues the DMA of a tile.
-    auto phase = [&](auto ks_c, auto dma_c, int dma_stage) __attribute__((always_inline)) {
+    // Path 4: the kernel manages the accumulation registers itself.  Block (fi, fj) of the wave tile lives in a[R : R + 3],
+    // R = 4 * (fj * FM + fi), and every instruction that touches it -- MFMA, the moves below, the store of D -- names these
+    // registers in its text; the compiler never sees them (they are listed as clobbered once, so that the kernel is given
+    // the whole register file).  The accumulators start from zero (the MFMAs of the very first k-step take the constant 0 as
+    // their third operand) and C comes in while the matrix cores run, block column by block column (group G = block
+    // column G: FM blocks, 16 contiguous bytes per lane and block).  K tile G fetches group G in its first k-step, behind the
+    // fragment reads, into one of two sets of FM * 4 registers; these loads are younger than the DMA of the next tile, so
+    // the wait in front of the barrier lets them stay in flight (memory reads return in order) and the wait of K tile G + 1
+    // covers them; the last k-step of K tile G + 1 adds the group to the accumulators: an accumulation register is read,
+    // added to and written back by the vector ALU, two values per MFMA slot, starting four slots behind the MFMA of the block
+    // (a block whose turn would reach the end of the k-step takes the first slots instead, before its MFMA and a dozen slots
+    // after the one of the k-step before): the matrix core has long delivered the block and does not need it again for fifty
+    // slots.  So the sum is (products of the first K tiles) + C + (the rest), where the other paths start from C.
+    constexpr int CGROUPS = CPATH == 4 ? FN : 0;
+    static_assert(CGROUPS + 3 <= kSoloStreamTiles, "the K tiles that bring C in are written out in front of the loop, the last two behind it");
+    static_assert(CPATH != 4 || KS >= 2, "the loads of C go into the first k-step of a tile, the additions into the last");
+    [[maybe_unused]] float4v cland[CPATH == 4 ? 2 : 1][CPATH == 4 ? FM : 1];
+    [[maybe_unused]] float ctmp[2][4];
+    [[maybe_unused]] unsigned c_voff = 0;              // byte offset of the lane's four rows of block (0, 0) from the wave tile's origin in C
+    [[maybe_unused]] const char* c_tile = nullptr;     // the wave tile's origin in C (the same in every lane)
+    [[maybe_unused]] long long c_col16 = 0;            // bytes from a block column to the next
+    if constexpr (CPATH == 4) {
+      c_voff = (unsigned)((4 * (lane / MI) + (long long)(lane % MI) * args.ldc) * 4);
+      c_tile = (const char*)args.c + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldc) * 4;
+      c_col16 = (long long)args.ldc * (MI * 4);
+      asm volatile("" ::: "a255");           // (the highest one: the kernel is given all 256)
+    }
+    // the load of block (J, G)
+    [[maybe_unused]] auto c_load = [&](auto g_c, auto j_c) __attribute__((always_inline)) {
+      constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value;
+      const char* base = c_tile + c_col16 * G;
+      float4v& dst = cland[G & 1][J];         // (named here: an operand of an assembly statement does not capture by itself)
+      const unsigned vo = c_voff;
+      asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(vo), "s"(base), "n"(J * MI * 4) : "memory");
+    };
+    // Step Q (0 .. 5) of the addition of block (J, G): two accumulation registers read, two values added, two registers
+    // written back
+    [[maybe_unused]] auto c_add_step = [&](auto g_c, auto j_c, auto q_c) __attribute__((always_inline)) {
+      constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value, Q = decltype(q_c)::value;
+      constexpr int R = 4 * (G * FM + J), E = 2 * (Q & 1);
+      float4v& src = cland[G & 1][J];
+      float& t0 = ctmp[J & 1][E];
+      float& t1 = ctmp[J & 1][E + 1];
+      if constexpr (Q == 0) asm volatile("" : "+v"(src));
+      if constexpr (Q < 2) {
+        asm volatile("v_accvgpr_read_b32 %0, a[%2]\n\tv_accvgpr_read_b32 %1, a[%3]" : "=v"(t0), "=v"(t1) : "n"(R + E), "n"(R + E + 1));
+      } else if constexpr (Q < 4) {
+        t0 = t0 + src[E];
+        t1 = t1 + src[E + 1];
+      } else {
+        asm volatile("v_accvgpr_write_b32 a[%2], %0\n\tv_accvgpr_write_b32 a[%3], %1" :: "v"(t0), "v"(t1), "n"(R + E), "n"(R + E + 1));
+      }
+    };
+    // PAR: the fragment buffer that the MFMAs of this k-step read (the reads go into the other one)
+    // RD: the k-step reads the fragments of the next one
+    auto phase = [&](auto ks_c, auto dma_c, int dma_stage, auto lg_c, auto ag_c, auto first_c, auto par_c, auto rd_c) __attribute__((always_inline)) {
       constexpr int ks = decltype(ks_c)::value;
+      constexpr int PAR = decltype(par_c)::value;
+      constexpr bool RD = decltype(rd_c)::value;
       constexpr bool DMA = decltype(dma_c)::value;
+      constexpr int LG = decltype(lg_c)::value, AG = decltype(ag_c)::value;     // groups of C to fetch / to add in this k-step (-1: none)
+      [[maybe_unused]] constexpr bool FIRST = decltype(first_c)::value;         // path 4: the accumulators start from zero here
       constexpr int NKS = (ks + 1) % KS;
       int4v va[FM], vb[FN];
       __builtin_amdgcn_sched_barrier(0);       // no MFMA of the k-step before moves behind the waits in front of this one
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi) { RA::pin_raw(fa[ks & 1][fi]); va[fi] = RA::finish(fa[ks & 1][fi], lane); }
+      for (int fi = 0; fi < FM; ++fi) { RA::pin_raw(fa[PAR][fi]); va[fi] = RA::finish(fa[PAR][fi], lane); }
       // B read as OPK_KSPLIT: a fragment of real parts (block column fj) and one of imaginary parts (fj + FN / 2) are made
       // of each set of registers read, four byte permutes each, right before the MFMAs that use them first: the block
       // columns are the outer loop there
       constexpr bool B_BOTH = Cfg::B_KIND == OPK_KSPLIT;
       if constexpr (!B_BOTH) {
 #pragma unroll
-        for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[ks & 1][fj]); vb[fj] = RB::finish(fb[ks & 1][fj], lane); }
+        for (int fj = 0; fj < FN; ++fj) { RB::pin_raw(fb[PAR][fj]); vb[fj] = RB::finish(fb[PAR][fj], lane); }
       } else {
 #pragma unroll
-        for (int fj = 0; fj < RB::NREAD; ++fj) RB::pin_raw(fb[ks & 1][fj]);
+        for (int fj = 0; fj < RB::NREAD; ++fj) RB::pin_raw(fb[PAR][fj]);
       }
       static_for<0, NM>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
         constexpr int o_ = B_BOTH ? i / FM : i / FN, q_ = B_BOTH ? ((o_ & 1) ? FM - 1 - (i % FM) : i % FM) : ((o_ & 1) ? FN - 1 - (i % FN) : i % FN);
         constexpr int fi = B_BOTH ? q_ : o_, fj = B_BOTH ? o_ : q_;
-        if constexpr (B_BOTH && (i % FM) == 0) vb[fj] = RB::finish(fb[ks & 1][fj % RB::NREAD], lane, fj >= RB::NREAD);
-        acc[fi][fj] = Mfma<T, MI>::run(va[fi], vb[fj], acc[fi][fj]);
+        if constexpr (B_BOTH && (i % FM) == 0) vb[fj] = RB::finish(fb[PAR][fj % RB::NREAD], lane, fj >= RB::NREAD);
+        if constexpr (CPATH == 4) Mfma<T, MI>::template run_fixed<4 * (fj * FM + fi), FIRST>(va[fi], vb[fj]);
+        else acc[fi][fj] = Mfma<T, MI>::run(va[fi], vb[fj], acc[fi][fj]);
         // (the scheduling barriers keep every instruction in the slot it is written in)
         if constexpr (DMA && i % GD == 0 && i / GD < DPT) {
           __builtin_amdgcn_sched_barrier(0);
           dma_one(std::integral_constant<int, i / GD>{}, dma_stage);
           __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr ((i % RSP) == 0 && i / RSP < NOPS) {
+        if constexpr (RD && (i % RSP) == 0 && i / RSP < NOPS) {
           __builtin_amdgcn_sched_barrier(0);
-          read_op(std::integral_constant<int, i / RSP>{}, std::integral_constant<int, NKS>{});
+          read_op(std::integral_constant<int, i / RSP>{}, std::integral_constant<int, NKS>{}, std::integral_constant<int, (PAR ^ 1)>{});
           __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (CPATH == 4 && !B_BOTH) {
+          constexpr int LSLOT0 = NOPS * RSP + 2, LSTEP = 4;        // (behind the fragment reads)
+          static_assert(LG < 0 || LSLOT0 + LSTEP * (FM - 1) < NM, "the loads of a group of C fit the k-step");
+          if constexpr (LG >= 0 && i >= LSLOT0 && (i - LSLOT0) % LSTEP == 0 && (i - LSLOT0) / LSTEP < FM) {
+            __builtin_amdgcn_sched_barrier(0);
+            c_load(lg_c, std::integral_constant<int, (i - LSLOT0) / LSTEP>{});
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          if constexpr (AG >= 0) {
+            static_for<0, FM * 6>([&](auto u_c) {
+              constexpr int u = decltype(u_c)::value, j = u / 6, q = u % 6;
+              constexpr int p = j * FN + ((j & 1) ? FN - 1 - AG : AG);       // the MFMA of block (j, AG) in this k-step
+              constexpr int s0 = (p + 9 < NM) ? p + 4 : p + 4 - NM + 8;
+              // (the two halves of a step trade places so that a value is read, added and written two slots apart)
+              constexpr int at = s0 + (q / 2) * 2 + (q & 1);
+              if constexpr (at == i) {
+                __builtin_amdgcn_sched_barrier(0);
+                c_add_step(ag_c, std::integral_constant<int, j>{}, std::integral_constant<int, q>{});
+                __builtin_amdgcn_sched_barrier(0);
+              }
+            });
+          }
         }
       });
     };
     typedef std::integral_constant<bool, true> Yes;
     typedef std::integral_constant<bool, false> No;
+    typedef std::integral_constant<int, -1> NoGroup;
     // tiles 0 and 1 were issued before the C load.  From here on ga / gb stand at the tile that the next DMA fetches:
     // tile kt + 2 in step kt, and the last tile once more where there is no such tile (the DMA is unconditional: a
     // branch around it costs more issue slots than the instruction; the data lands in a stage nobody reads any more)
@@ -1309,21 +1412,26 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     block_barrier();
     ra.set_stage(lds_base);
     rb.set_stage(lds_base + GA::BYTES);
-    static_for<0, NOPS>([&](auto r_c) { read_op(r_c, std::integral_constant<int, 0>{}); });
+    static_for<0, NOPS>([&](auto r_c) { read_op(r_c, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
     // (no copy of the loop body for the last tile: what it reads ahead and fetches there is never used)
-    for (int kt = 0; kt < KT; ++kt) {
+    // DMA: the tile fetches tile kt + 2; LAST: there is no tile kt + 1 (nothing to wait for, nothing to read ahead)
+    auto tile_body = [&](int kt, auto lg_c, auto ag_c, auto first_c, auto dma_c, auto last_c) __attribute__((always_inline)) {
+      constexpr bool LAST = decltype(last_c)::value;
       static_for<0, KS>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
         __builtin_amdgcn_sched_barrier(0);
         wait_lgkmcnt<0>();                              // the fragments of this k-step have arrived
         if constexpr (ks == KS - 1) {
-          // tile kt+1 has landed (its DMA was issued a k-step or more ago); behind the barrier it is visible to all
-          // waves, and all are done reading tile kt: its stage takes tile kt+2
-          wait_vmcnt<0>();
-          block_barrier();
-          const unsigned stage_addr = lds_base + (unsigned)((kt + 1) & 1) * Cfg::STAGE_BYTES;
-          ra.set_stage(stage_addr);
-          rb.set_stage(stage_addr + GA::BYTES);
+          if constexpr (!LAST) {
+            // tile kt+1 has landed (its DMA was issued a k-step or more ago); behind the barrier it is visible to all
+            // waves, and all are done reading tile kt: its stage takes tile kt+2
+            // (the loads of C that this tile has issued stay in flight: memory reads return in order, and they are younger than the DMA)
+            wait_vmcnt<(decltype(lg_c)::value >= 0 ? FM : 0)>();
+            block_barrier();
+            const unsigned stage_addr = lds_base + (unsigned)((kt + 1) & 1) * Cfg::STAGE_BYTES;
+            ra.set_stage(stage_addr);
+            rb.set_stage(stage_addr + GA::BYTES);
+          }
           if constexpr (Cfg::GETT) {
             // (read a k-step ago; the same value in every lane)
             asm volatile("" : "+v"(ktab));
@@ -1332,7 +1440,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             part_a = ga + (long long)oa * 2;
             part_b = gb + (long long)ob * 2;
           }
-          phase(ks_c, Yes{}, kt & 1);
+          phase(ks_c, dma_c, kt & 1, NoGroup{}, ag_c, No{}, std::integral_constant<int, (ks & 1)>{}, std::integral_constant<bool, !LAST>{});
           if (kt + 3 < KT) { ga += a_step; gb += b_step; }
         } else {
           if constexpr (Cfg::GETT && ks == 0) {
@@ -1342,12 +1450,30 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             const unsigned addr = lds_base + (unsigned)(Cfg::STAGE_BYTES * STAGES) + 16u * (unsigned)t;
             asm volatile("ds_read_b128 %0, %1" : "=v"(ktab) : "v"(addr) : "memory");
           }
-          phase(ks_c, No{}, 0);
+          if constexpr (ks == 0) phase(ks_c, No{}, 0, lg_c, NoGroup{}, first_c, std::integral_constant<int, 0>{}, Yes{});
+          else phase(ks_c, No{}, 0, NoGroup{}, NoGroup{}, No{}, std::integral_constant<int, (ks & 1)>{}, Yes{});
         }
       });
+    };
+    if constexpr (CPATH == 4) {
+      // the first K tiles, written out: tile t fetches group t of C and adds group t - 1 (the host sends products of at
+      // least kSoloStreamTiles K tiles here) ...
+      static_for<0, CGROUPS + 1>([&](auto t_c) {
+        constexpr int t = decltype(t_c)::value;
+        tile_body(t, std::integral_constant<int, (t < CGROUPS ? t : -1)>{}, std::integral_constant<int, t - 1>{}, std::integral_constant<bool, t == 0>{}, Yes{}, No{});
+      });
+      for (int kt = CGROUPS + 1; kt < KT - 2; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{});
+      // ... and the last two, which have nothing left to fetch
+      tile_body(KT - 2, NoGroup{}, NoGroup{}, No{}, No{}, No{});
+      tile_body(KT - 1, NoGroup{}, NoGroup{}, No{}, No{}, Yes{});
+    } else {
+      for (int kt = 0; kt < KT; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{});
     }
     wait_vmcnt<0>();     // (the last DMA of the loop may still be on its way; so are reads
     wait_lgkmcnt<0>();   // of fragments)
+    // (path 4 issues its MFMAs from assembly statements, which the compiler does not see: the results of the last ones must
+    // have left the matrix core before anything else reads their registers)
+    if constexpr (CPATH == 4) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     if constexpr (RAGGED_K) {
       // the last, partial K tile, outside the schedule of the loop: the k-steps that hold valid values
       if (tail_k > 0) {
@@ -1355,9 +1481,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         static_for<0, KS>([&](auto ks_c) {
           constexpr int ks = decltype(ks_c)::value;
           if (ks * Cfg::KSTEP_K < tail_k) {
-            static_for<0, NOPS>([&](auto r_c) { read_op(r_c, ks_c); });
+            static_for<0, NOPS>([&](auto r_c) { read_op(r_c, ks_c, std::integral_constant<int, (ks & 1)>{}); });
             wait_lgkmcnt<0>();
-            phase(ks_c, No{}, 0);        // (what it reads ahead for the next k-step is read again there, or never used)
+            phase(ks_c, No{}, 0, NoGroup{}, NoGroup{}, No{}, std::integral_constant<int, (ks & 1)>{}, Yes{});        // (what it reads ahead for the next k-step is read again there, or never used)
             wait_lgkmcnt<0>();
           }
         });
@@ -1794,6 +1920,23 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             }
           }
         }
+    } else if constexpr (CPATH == 4) {
+      // from the accumulation registers the kernel manages itself: the wave tile's origin in D from scalar registers, the
+      // lane's offset in it from a vector register, the row block as an immediate
+      const unsigned d_voff = (unsigned)((4 * (lane_e / MI) + (long long)(lane_e % MI) * args.ldd) * 4);
+      const char* d_tile = (const char*)args.d + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldd) * 4;
+      const long long d_col16 = (long long)args.ldd * (MI * 4);
+      static_for<0, FN>([&](auto fj_c) {
+        constexpr int fj = decltype(fj_c)::value;
+        const char* base = d_tile + d_col16 * fj;
+        static_for<0, FM>([&](auto fi_c) {
+          constexpr int fi = decltype(fi_c)::value;
+          constexpr int R = 4 * (fj * FM + fi);
+          const unsigned vo = d_voff;             // (named here: an operand of an assembly statement does not capture by itself)
+          const char* sb = base;
+          asm volatile("global_store_dwordx4 %0, a[%2:%3], %1 offset:%4" :: "v"(vo), "s"(sb), "n"(R), "n"(R + 3), "n"(fi * MI * 4) : "memory");
+        });
+      });
     } else if constexpr (CPATH != 0) {
 #pragma unroll
       for (int fj = 0; fj < SFN; ++fj)

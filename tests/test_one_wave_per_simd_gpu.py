@@ -286,3 +286,67 @@ def test_default_configuration_of_a_large_product(gpu):
     a, b, c = operands(M, N, K, False, False, 7600)
     d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
     assert oracle.rel_frobenius(d, helpers.run_oracle(conf, a, b, c, (M, N))) <= TOL
+
+
+# --- C on its way during the first K tiles (products of at least eleven K tiles, FP32 C and D with 16-byte accesses) -------------
+# The sum runs (products of the first K tiles) + C + (the rest) there, where the eight-wave arrangement starts from C: results
+# are compared with the oracle and with float64 by norm, and exactly on data whose partial sums are all exact in FP32.
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("K", [704, 768, 1344])
+def test_c_streamed_during_the_first_k_tiles(gpu, ta, tb, K):
+    """Eleven K tiles (the fewest that take this route: nine that bring C in, none in between, the two last), twelve, twenty-one."""
+    M, N = 512, 768
+    a, b, c = operands(M, N, K, ta, tb, 7600 + K)
+    conf = config(M, N, K, ta, tb, (2, 2))
+    print("case", ta, tb, K, gk.kernel_name(conf, Kernel.matmul_pipelined), flush=True)
+    d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(d, helpers.run_oracle(conf, a, b, c, (M, N))) <= TOL
+    assert oracle.rel_frobenius(d, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= 1e-6
+    # linearity in C, which pins that every element of C went into its own accumulator exactly once: D(C) - D(0) = C
+    d0 = helpers.run_gpu(config(M, N, K, ta, tb, (2, 2), zero_c=True), a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.abs((d.astype(np.float64) - d0) - c).max() <= 1e-4
+    # small integers: every partial sum is exact, whatever the place of C in the sum
+    rs = np.random.RandomState(K)
+    ai = np.asfortranarray(rs.randint(-4, 5, size=a.shape).astype(np.float16))
+    bi = np.asfortranarray(rs.randint(-4, 5, size=b.shape).astype(np.float16))
+    ci = np.asfortranarray(rs.randint(-999, 1000, size=(M, N)).astype(np.float32))
+    di = helpers.run_gpu(conf, ai, bi, ci, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(di.astype(np.float64), oracle.gemm_f64(ai, bi, ci, 1.0, 1.0, ta, tb))
+    # the eight-wave arrangement adds the same products in the same order but for the place of C: same values to rounding
+    d8 = helpers.run_gpu(config(M, N, K, ta, tb, (2, 4)), a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(d, d8.astype(np.float64)) <= 1e-6
+
+
+def test_c_streamed_d_in_place_and_as_a_window(gpu):
+    """d aliases c (reference src/matmul.jl:198): every workgroup has read its C tile before it writes the same tile of D.
+    C and D as windows of larger matrices (leading dimension beyond M)."""
+    import torch
+    M, N, K = 256, 512, 960
+    a, b, c = operands(M, N, K, False, False, 7700)
+    conf = config(M, N, K, False, False, (2, 2))
+    ref = oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False)
+    d_alias = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined, alias_cd=True)
+    assert np.array_equal(d_alias, helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined))
+    assert oracle.rel_frobenius(d_alias, ref) <= 1e-6
+    ld = M + 64
+    cbig = torch.full((N, ld), 7.0, dtype=torch.float32, device="cuda")
+    dbig = torch.full((N, ld), float("nan"), dtype=torch.float32, device="cuda")
+    C, D = cbig.t()[:M, :], dbig.t()[:M, :]
+    C.copy_(torch.from_numpy(c).cuda())
+    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), C, D, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    assert np.array_equal(D.cpu().numpy(), d_alias)
+    assert bool(torch.isnan(dbig.t()[M:, :]).all())            # nothing written outside the window
+
+
+def test_c_streamed_bf16_operands(gpu):
+    M, N, K = 256, 256, 832
+    a = gk.bf16_bits(rng.matrix("upm1_f32", 7801, (M, K)))
+    b = gk.bf16_bits(rng.matrix("upm1_f32", 7802, (K, N)))
+    c = rng.matrix("upm1_f32", 7803, (M, N))
+    four = config(M, N, K, False, False, (2, 2), ab=BFloat16)
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N))) <= TOL
+    d8 = helpers.run_gpu(config(M, N, K, False, False, (2, 4), ab=BFloat16), a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(d4, d8.astype(np.float64)) <= 1e-6
