@@ -372,6 +372,40 @@ def main():
             torch.cuda.empty_cache()
         except Exception as e:
             extras["mul! 4000^3 (not whole tiles)"] = {"error": f"{type(e).__name__}: {e}"}
+        # the BLAS-level front end over the sizes of the reference's performance curve (media/performance-wmma-gemm.png sweeps
+        # N = 128 ... 16384): mul!(C, A, B, 1, 1) on FP16 A, B and an FP32 C that is read and written, default tile choice.
+        # Each size is checked once, before it is timed: 128 columns of the result of one launch against the float64 product
+        # of the same operands (generated on the device: the largest C alone is 1 GiB).  "vendor" is torch.mm on the same
+        # A and B with FP16 output and no C, for orientation.
+        try:
+            from gemmkernels.matmul import matmatmul_plan
+            sizes = {}
+            for (m, n, k) in [(1024, 1024, 1024), (2048, 2048, 2048), (3072, 3072, 3072), (4096, 4096, 4096), (6144, 6144, 6144),
+                              (8192, 8192, 8192), (4096, 4096, 16384), (8192, 8192, 4096), (16384, 16384, 4096)]:
+                gen = torch.Generator(device="cuda")
+                gen.manual_seed(m * 31 + n * 17 + k)
+                a_ = (torch.rand(k, m, device="cuda", generator=gen) * 2 - 1).to(torch.float16).t()      # column-major m x k
+                b_ = (torch.rand(n, k, device="cuda", generator=gen) * 2 - 1).to(torch.float16).t()
+                c_ = (torch.rand(n, m, device="cuda", generator=gen) * 2 - 1).t()
+                c0 = c_[:, :128].to(torch.float64).cpu().numpy()
+                p_ = matmatmul_plan(c_, "N", "N", a_, b_, 1.0, 1.0)
+                p_()
+                torch.cuda.synchronize()
+                got = c_[:, :128].to(torch.float64).cpu().numpy()
+                ref = a_.to(torch.float64).cpu().numpy() @ b_[:, :128].to(torch.float64).cpu().numpy() + c0
+                err_ = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+                u, _ = time_launches(p_, 30 if m * n * k > 2 ** 37 else 50, 5, 0.15)
+                out_ = torch.empty(m, n, device="cuda", dtype=torch.float16)
+                am, bm_ = a_.contiguous(), b_.contiguous()
+                uv, _ = time_launches(lambda: torch.mm(am, bm_, out=out_), 30 if m * n * k > 2 ** 37 else 50, 5, 0.15)
+                sizes[f"{m}x{n}x{k}"] = {"us": round(u, 2), "TFLOP/s": round(2.0 * m * n * k / u / 1e6, 1), "rel_error_128_columns": float(f"{err_:.2e}"),
+                                         "verified": bool(err_ <= 1e-3), "kernels": sorted(set(p_.kernel_names)),
+                                         "vendor_fp16_out_no_c_us": round(uv, 2)}
+                del a_, b_, c_, p_, out_, am, bm_
+                torch.cuda.empty_cache()
+            extras["sizes: mul!(C, A, B, 1, 1), FP16 x FP16 + FP32 C"] = sizes
+        except Exception as e:
+            extras["sizes: mul!(C, A, B, 1, 1), FP16 x FP16 + FP32 C"] = {"error": f"{type(e).__name__}: {e}"}
         # the vendor library on the headline shape, for orientation only: FP16 in, FP16 out, no C read
         # (torch.mm -> hipBLASLt), so it moves 96 MiB less per launch than config 2 does
         try:

@@ -122,14 +122,19 @@ bool needs_tail_tile(const gk_config* c) {
   return (c->matmul_shape.K % c->block_shape.K) != 0 || (!a_row && (c->matmul_shape.M % 8) != 0) || (b_row && (c->matmul_shape.N % 8) != 0);
 }
 
-// A multiplication of A (or B) by +-2^e commutes with every rounding of the sum (barring overflow and the
-// subnormal range of the operand's type, where the product on the operand would lose bits that the folded form
-// keeps): sum_k (s a) b + c = s (sum_k a b + c / s), bit for bit.  For the real matrix-core operator such a hook
-// therefore leaves the K loop: the accumulators start from T_c(C) / s and are multiplied by s before the hooks
-// of D.  Returns the transforms that remain (`storage` when something was folded) and the factor s.
+// A multiplication of A (or B) by +-2^e commutes with every rounding of the sum as long as the scaled operand stays
+// inside the normal range of its 16-bit type: sum_k (s a) b + c = s (sum_k a b + c / s), bit for bit.  For the
+// matrix-core operators (real, complex and dual: s is real, so it acts on both parts of a number) such a hook -- a scale
+// by +-2^e, or a negation -- therefore leaves the K loop: the accumulators start from T_c(C) / s and are multiplied by s
+// before the hooks of D.  Outside that range the two forms differ: the reference (and the in-loop form) rounds s * a to
+// the operand's type, so s = 2^20 turns finite FP16 values into Inf and s = 2^-20 flushes them into the subnormal range,
+// where the folded form returns the exact product.  The fold is therefore limited to |e| <= 4 (operands up to 4095 in
+// magnitude and down to 2^-10 keep every bit under the largest folded factor, 16); other powers of two run in the K loop
+// like any other scale.  Returns the transforms that remain (`storage` when something was folded) and the factor s.
 const gk_transforms* fold_pow2_scales(const gk_config* c, const gk_transforms* t, gk_transforms* storage, float* post) {
   *post = 1.0f;
-  if (!t || c->op.kind != GK_OP_MFMA || c->global_a_layout.kind == GK_LAYOUT_DIAGONAL) return t;
+  const bool matrix_core = c->op.kind == GK_OP_MFMA || c->op.kind == GK_OP_MFMA_COMPLEX || c->op.kind == GK_OP_MFMA_DUAL;
+  if (!t || !matrix_core || c->global_a_layout.kind == GK_LAYOUT_DIAGONAL) return t;
   float factor = 1.0f;
   bool folded = false;
   gk_transforms out = *t;
@@ -143,11 +148,12 @@ const gk_transforms* fold_pow2_scales(const gk_config* c, const gk_transforms* t
       for (int i = 0; i < tr.n_ops; ++i)
         if (tr.ops[i].kind != GK_T_IDENTITY) { ++n; one = &tr.ops[i]; }
     }
-    if (n != 1 || one->kind != GK_T_SCALE) continue;
+    if (n != 1 || (one->kind != GK_T_SCALE && one->kind != GK_T_NEG)) continue;
+    const float s = one->kind == GK_T_NEG ? -1.0f : one->p0;
     int e = 0;
-    const float m = frexpf(one->p0, &e);
-    if (!(m == 0.5f || m == -0.5f) || e < -23 || e > 24) continue;   // +-2^(e-1), a moderate exponent
-    factor *= one->p0;
+    const float m = frexpf(s, &e);
+    if (!(m == 0.5f || m == -0.5f) || e - 1 < -4 || e - 1 > 4) continue;   // +-2^(e-1), |e - 1| <= 4
+    factor *= s;
     out.hook[pr[0]].n_ops = 0;
     out.hook[pr[1]].n_ops = 0;
     folded = true;
@@ -177,6 +183,11 @@ int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_
     case GK_OP_FPU_TROPICAL:
       key->family = gk::FAMILY_FPU;
       key->variant = ((c->op.kind == GK_OP_FPU_TROPICAL) ? 1 : 0) + (any_checked ? 2 : 0);
+      if (c->op.mb != 8 && c->op.mb > 0) {          // another lane grid than 8 x 8: log2(OPERATOR_M_BASE) + 1 from bit 4 on
+        int lg = 0;
+        while ((1 << lg) < c->op.mb) ++lg;
+        key->variant += (lg + 1) << 4;
+      }
       break;
     case GK_OP_MFMA_COMPLEX:
     case GK_OP_MFMA_DUAL:
@@ -579,11 +590,23 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
       return fail(GK_ERR_OP_SHAPE, "The operator shape should adhere to the following constraint: OPERATOR_M, OPERATOR_N, OPERATOR_K are multiples of OPERATOR_M_BASE, OPERATOR_N_BASE, OPERATOR_K_BASE, respectively.");
     // The base shape says how the lanes of a wave are laid over a block of outputs; the operator shape, how many
     // outputs a lane owns.  Neither changes a result (every output is one fma chain in ascending k).  The
-    // vector-ALU kernels are compiled for the square 8 x 8 lane grid and own their outputs in 4-wide chunks
-    // whatever the operator shape says; another lane grid is refused rather than silently replaced.
-    if (op.mb != 8 || op.nb != 8)
-      return fail(GK_ERR_OP_SHAPE, "The vector-ALU kernels of this library are compiled for the base shape OPERATOR_M_BASE = OPERATOR_N_BASE = 8 "
-                                   "(a wave as an 8 x 8 grid of lanes), got %d x %d.", op.mb, op.nb);
+    // vector-ALU kernels own their outputs in chunks of up to 4 whatever the operator shape says.  The square 8 x 8
+    // lane grid is compiled for every tile, element type and layout; the other grids of the reference's sweep
+    // (configs/configs.jl:545-550, doubled for 64 lanes: 1 x 64, 2 x 32, 4 x 16, 16 x 4, 32 x 2, 64 x 1) for Float32 on
+    // aligned layouts and the 128 x 128 x 16 tile, whose 64 x 64 wave tiles every grid divides.  Anything else is
+    // refused rather than silently run on another grid.
+    if (op.mb != 8 || op.nb != 8) {
+      if ((op.mb & (op.mb - 1)) != 0)
+        return fail(GK_ERR_OP_SHAPE, "OPERATOR_M_BASE must be a power of two, got %d.", op.mb);
+      const bool f32 = c->global_a_layout.eltype == GK_F32 && c->global_b_layout.eltype == GK_F32 && c->global_d_layout.eltype == GK_F32;
+      auto aligned = [](int k) { return k == GK_LAYOUT_ALIGNED_COL_MAJOR || k == GK_LAYOUT_ALIGNED_ROW_MAJOR; };
+      const bool lay = aligned(c->global_a_layout.kind) && aligned(c->global_b_layout.kind) && c->global_d_layout.kind == GK_LAYOUT_ALIGNED_COL_MAJOR &&
+                       (c->global_c_layout.kind == GK_LAYOUT_ALIGNED_COL_MAJOR || c->global_c_layout.kind == GK_LAYOUT_ZERO);
+      if (op.kind != GK_OP_FPU || !f32 || !lay || b.M != 128 || b.N != 128 || b.K != 16 || c->compute_warp.M != 64 || c->compute_warp.N != 64)
+        return fail(GK_ERR_OP_SHAPE, "The base shape OPERATOR_M_BASE x OPERATOR_N_BASE = %d x %d (a wave as a %d x %d grid of lanes) is compiled for FPUOp on Float32 "
+                                     "with aligned layouts, block shape 128 x 128 x 16 and 64 x 64 wave tiles; every other configuration runs 8 x 8.",
+                    op.mb, op.nb, op.mb, op.nb);
+    }
   } else if (is_mfma_kind(op.kind)) {
     const bool native = (op.M == 32 && op.N == 32 && op.K == 16);
     const bool wmma_compat = (op.K == 16) && ((op.M == 16 && op.N == 16) || (op.M == 8 && op.N == 32) || (op.M == 32 && op.N == 8));
@@ -638,11 +661,17 @@ int validate_config(const gk_config* c, int kernel, const gk_transforms* t, cons
     // x * p0 and -x, and x + p0, which acts on the real part; max / abs / clamp have no complex counterpart of the
     // same type.  A bias value is real and goes to the real part.
     if (t) {
+      // (on A and B: what folds into the accumulators -- one scale by +-2^e, |e| <= 4, or one negation per operand: a real
+      // factor acts on both parts of a number and commutes with the product; see fold_pow2_scales)
+      gk_transforms folded_storage;
+      float post = 1.0f;
+      const gk_transforms* rest = fold_pow2_scales(c, t, &folded_storage, &post);
       const int ab_hooks[4] = {GK_HOOK_GLOBAL_TO_SHARED_A, GK_HOOK_SHARED_TO_REGS_A, GK_HOOK_GLOBAL_TO_SHARED_B, GK_HOOK_SHARED_TO_REGS_B};
       for (int h : ab_hooks)
-        for (int i = 0; i < t->hook[h].n_ops && i < GK_MAX_OPS; ++i)
-          if (t->hook[h].ops[i].kind != GK_T_IDENTITY)
-            return fail(GK_ERR_UNSUPPORTED, "the complex and dual operators take transforms on C and D only");
+        for (int i = 0; i < rest->hook[h].n_ops && i < GK_MAX_OPS; ++i)
+          if (rest->hook[h].ops[i].kind != GK_T_IDENTITY)
+            return fail(GK_ERR_UNSUPPORTED, "the complex and dual operators take transforms on C and D, and on A and B one scale by a power of two "
+                                            "between 1/16 and 16 or one negation each (anything else would have to run inside their K loop)");
       for (int h = 0; h < 8; ++h)
         for (int i = 0; i < t->hook[h].n_ops && i < GK_MAX_OPS; ++i) {
           const int k = t->hook[h].ops[i].kind;

@@ -78,10 +78,13 @@ std::string build_source(const gk_config* c, const char* const hooks[8], int sta
   src += "    return x;\n  }\n};\n}\n#include \"mfma_gemm.hpp\"\n";
   char buf[512];
   snprintf(buf, sizeof(buf),
-           "typedef gk::MfmaGemmConfig<%d, %d, %d, %d, %d, %d, %d, %d, %s, %d, false, gk::FIX_NONE, false, 16> GkUserCfg;\n"
+           "typedef gk::MfmaGemmConfig<%d, %d, %d, %d, %d, %d, %d, %d, %s, %d, false, gk::FIX_NONE, false, %d> GkUserCfg;\n"
            "template __global__ void gk::mfma_gemm_kernel<GkUserCfg>(const gk::GemmArgs);\n",
            c->block_shape.M, c->block_shape.N, c->block_shape.K, c->block_shape.M / c->compute_warp.M,
-           c->block_shape.N / c->compute_warp.N, stages, a_kind, b_kind, type, fuse);
+           c->block_shape.N / c->compute_warp.N, stages, a_kind, b_kind, type, fuse,
+           // v_mfma_f32_16x16x32 takes 32 values of k at a time; a BLOCK_K of 16 (the reference sweeps it,
+           // configs/configs.jl:601) runs on v_mfma_f32_32x32x16
+           c->block_shape.K % 32 == 0 ? 16 : 32);
   src += buf;
   return src;
 }
@@ -108,7 +111,7 @@ int gk_rtc_compile(const gk_config* conf, const char* const hooks[8], int32_t ke
   if (b.M <= 0 || b.N <= 0 || b.K <= 0 || w.M <= 0 || w.N <= 0 || b.M % w.M || b.N % w.N)
     return fail(GK_ERR_BLOCK_SHAPE, "block_shape must be a positive multiple of compute_warp");
   const int wm = b.M / w.M, wn = b.N / w.N, nwaves = wm * wn;
-  if (w.M % 32 || w.N % 32 || b.K % 32 || b.K > 128) return fail(GK_ERR_BLOCK_SHAPE, "compute_warp must be made of 32x32 blocks and BLOCK_K be 32, 64 or 128");
+  if (w.M % 32 || w.N % 32 || (b.K != 16 && b.K % 32) || b.K > 128) return fail(GK_ERR_BLOCK_SHAPE, "compute_warp must be made of 32x32 blocks and BLOCK_K be 16, 32, 64 or 128");
   if ((w.M / 32) * (w.N / 32) > 16) return fail(GK_ERR_BLOCK_SHAPE, "a wave tile holds at most sixteen 32x32 accumulator blocks");
   if (nwaves > 16 || nwaves != c->warps_per_block) return fail(GK_ERR_UNSUPPORTED, "warps_per_block must equal block_shape / compute_warp (at most 16)");
   if (((long long)b.M * b.K * 2 / 1024) % nwaves || ((long long)b.N * b.K * 2 / 1024) % nwaves || ((long long)b.M * b.K * 2) % 1024 || ((long long)b.N * b.K * 2) % 1024)
@@ -244,7 +247,10 @@ int gk_rtc_matmul(gk_rtc_kernel* k, const gk_config* conf, const void* a, const 
   // a bias epilogue makes the host layer choose a fused path; the hooks themselves are compiled in,
   // so no op lists travel with the launch
   gk_internal::Launch L;
-  int rc = gk_internal::prepare_launch(conf, a, b, c, d, nullptr, epilogue, GK_KERNEL_PIPELINED, &k->info, &L);
+  // (a block that is a single operator k-step deep -- BLOCK_K = 16 -- is what the reference can only run on its
+  // single-stage kernel, src/matmul.jl:34-36; the compiled code is the same pipeline either way)
+  const int kind = conf->block_shape.K < 2 * conf->compute_op_shape.K ? GK_KERNEL_SINGLESTAGE : GK_KERNEL_PIPELINED;
+  int rc = gk_internal::prepare_launch(conf, a, b, c, d, nullptr, epilogue, kind, &k->info, &L);
   if (rc != GK_OK) return rc;
   L.args.fast_scale_a = L.args.fast_scale_b = 0;
   if (k->info.lds_bytes > 64 * 1024 && !k->lds_raised) {

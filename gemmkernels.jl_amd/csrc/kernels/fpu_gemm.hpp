@@ -8,9 +8,10 @@
 // the multiplicands are converted to it before the fma, which is what Julia's promotion makes of
 // fma(a::CT, b::CT, c::AT) for the type triples the reference runs (configs/configs.jl:489-497):
 // Float16 -> Float32, Float32 -> Float32, Float32 -> Float64, Float64 -> Float64 and Int16 / Int32 /
-// Int64 with wrap-around.  A wave is an 8 x 8 grid of lanes (the reference's base shape mb x nb =
-// 32 lanes becomes 64 here); a lane owns TM x TN outputs in 4-wide chunks so that LDS reads and D
-// stores are vector accesses.  Tiles go global -> registers -> LDS with the next tile's global
+// Int64 with wrap-around.  A wave is a LANES_M x LANES_N grid of lanes (the reference's base shape
+// OPERATOR_M_BASE x OPERATOR_N_BASE, src/operator.jl:58-61: 32 lanes there, 64 here; 8 x 8 unless a
+// configuration asks for another grid); a lane owns TM x TN outputs in chunks of up to 4 so that LDS
+// reads and D stores are vector accesses.  Tiles go global -> registers -> LDS with the next tile's global
 // loads in flight during the fmas of the current one.  With CHECKED the loads and stores are per
 // element and bounds-checked (reference Layout.ColMajor / RowMajor, src/layout.jl:117-184:
 // out-of-range loads give 0, out-of-range stores are dropped), so any problem size and any leading
@@ -107,8 +108,11 @@ __device__ __forceinline__ TACC fpu_fma(TACC a, TACC b, TACC c) {
 }
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, typename TIN_, bool A_KMAJOR_, bool B_KMAJOR_, bool CHECKED_,
-          bool TROPICAL_, typename TACC_ = float, bool FUSED_ = true>
+          bool TROPICAL_, typename TACC_ = float, bool FUSED_ = true, int LANES_M_ = 8>
 struct FpuGemmConfig {
+  // the lane grid of a wave: lane l stands at row l % LANES_M, column l / LANES_M of it (reference src/operator.jl:61)
+  static constexpr int LANES_M = LANES_M_, LANES_N = kWaveSize / LANES_M_;
+  static_assert(LANES_M_ > 0 && kWaveSize % LANES_M_ == 0, "the lane grid is LANES_M x (64 / LANES_M)");
   // FUSED: the kernel carries the eight transform hooks and the bias; without, none of that code exists
   static constexpr bool FUSED = FUSED_;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
@@ -117,8 +121,8 @@ struct FpuGemmConfig {
   typedef TACC_ TACC;
   static constexpr int THREADS = WAVES_M * WAVES_N * kWaveSize;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
-  static constexpr int TM = WTM / 8, TN = WTN / 8;          // outputs per lane
-  // a lane's outputs come in chunks of consecutive rows (columns), 4 wide, or 2 wide for the smallest wave tile
+  static constexpr int TM = WTM / LANES_M, TN = WTN / LANES_N;          // outputs per lane
+  // a lane's outputs come in chunks of consecutive rows (columns), 4 wide, or fewer where a lane owns fewer
   static constexpr int CWM = TM < 4 ? TM : 4, CWN = TN < 4 ? TN : 4;
   static constexpr int CM = TM / CWM, CN = TN / CWN;        // chunks per lane
   static constexpr int PAD = 4;
@@ -132,7 +136,9 @@ struct FpuGemmConfig {
   // -- four tiles without hooks, two with; the bounds-checked and the 64-bit kernels stay with one (their
   // per-element loads and wide registers make deeper buffers expensive to compile and to hold)
   static constexpr int DEPTH = (CHECKED_ || sizeof(TIN_) > 4) ? 1 : (FUSED_ ? 2 : 4);
-  static_assert(TM >= 2 && TN >= 2 && TM % CWM == 0 && TN % CWN == 0, "a lane owns whole chunks of 2 or 4 outputs");
+  static_assert(WTM % LANES_M == 0 && WTN % LANES_N == 0 && TM >= 1 && TN >= 1 && TM % CWM == 0 && TN % CWN == 0,
+                "the lane grid divides the wave tile and a lane owns whole chunks");
+  static_assert(LANES_M_ != 8 || (TM >= 2 && TN >= 2), "8 x 8 lanes: a lane owns whole chunks of 2 or 4 outputs");
   static_assert(A_CHUNKS % THREADS == 0 && B_CHUNKS % THREADS == 0, "tile loads divide evenly over the threads");
   static_assert(!TROPICAL || std::is_same<TACC, float>::value, "the max-plus product is compiled for fp32");
 };
@@ -202,7 +208,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
   if (ti >= args.nbm || tj >= args.nbn) return;
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
-  const int ly = lane & 7, lx = lane >> 3;
+  const int ly = lane % Cfg::LANES_M, lx = lane / Cfg::LANES_M;
   const int m0 = ti * BM, n0 = tj * BN;
   const TIN* A = (const TIN*)args.a;
   const TIN* B = (const TIN*)args.b;
@@ -211,13 +217,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
   const bool xf_a = Cfg::FUSED && (args.t[H_GL2SH_A].n > 0 || args.t[H_SH2RF_A].n > 0);
   const bool xf_b = Cfg::FUSED && (args.t[H_GL2SH_B].n > 0 || args.t[H_SH2RF_B].n > 0);
 
-  // accumulators: acc[i][j] is row wm*WTM + (i/CW)*8*CW + CW*ly + i%CW (CW = 4, or 2), columns likewise with lx
+  // accumulators: acc[i][j] is row wm*WTM + (i/CW)*LANES_M*CW + CW*ly + i%CW (CW = 4, or fewer), columns likewise with lx
   constexpr int CWM = Cfg::CWM, CWN = Cfg::CWN;
   typedef TACC accm __attribute__((ext_vector_type(CWM)));
   typedef TACC accn __attribute__((ext_vector_type(CWN)));
   TACC acc[TM][TN];
-  auto row_of = [&](int i) { return m0 + wm * Cfg::WTM + (i / CWM) * 8 * CWM + CWM * ly + (i % CWM); };
-  auto col_of = [&](int j) { return n0 + wn * Cfg::WTN + (j / CWN) * 8 * CWN + CWN * lx + (j % CWN); };
+  auto row_of = [&](int i) { return m0 + wm * Cfg::WTM + (i / CWM) * Cfg::LANES_M * CWM + CWM * ly + (i % CWM); };
+  auto col_of = [&](int j) { return n0 + wn * Cfg::WTN + (j / CWN) * Cfg::LANES_N * CWN + CWN * lx + (j % CWN); };
 #pragma unroll
   for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -338,13 +344,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) fpu_gemm_kernel(const GemmArgs a
       TACC a[TM], b[TN];
 #pragma unroll
       for (int c = 0; c < Cfg::CM; ++c) {
-        const accm v = *(const accm*)&ap[k * Cfg::LDA_S + c * 8 * CWM];
+        const accm v = *(const accm*)&ap[k * Cfg::LDA_S + c * Cfg::LANES_M * CWM];
 #pragma unroll
         for (int e = 0; e < CWM; ++e) a[CWM * c + e] = v[e];
       }
 #pragma unroll
       for (int c = 0; c < Cfg::CN; ++c) {
-        const accn v = *(const accn*)&bp[k * Cfg::LDB_S + c * 8 * CWN];
+        const accn v = *(const accn*)&bp[k * Cfg::LDB_S + c * Cfg::LANES_N * CWN];
 #pragma unroll
         for (int e = 0; e < CWN; ++e) b[CWN * c + e] = v[e];
       }

@@ -918,6 +918,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         for (int fi = 0; fi < FM; ++fi) asm volatile("" : "+a"(acc[fi][fj]));
     } else if constexpr (CPATH == 4) {
       // (the accumulators start from zero in the first k-step and C comes in during the first K tiles, see the K loop)
+    } else if constexpr (CPATH == 2) {
+      // (no C: zeroed in place, in the accumulation registers)
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+        for (int fj = 0; fj < FN; ++fj) {
+          acc[fi][fj] = AccV{};
+          asm volatile("" : "+a"(acc[fi][fj]));
+        }
     } else if constexpr (CPATH == 1) {
 #pragma unroll
       for (int fj = 0; fj < SFN; ++fj)
@@ -1404,16 +1413,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     typedef std::integral_constant<bool, false> No;
     typedef std::integral_constant<int, -1> NoGroup;
     // tiles 0 and 1 were issued before the C load.  From here on ga / gb stand at the tile that the next DMA fetches:
-    // tile kt + 2 in step kt, and the last tile once more where there is no such tile (the DMA is unconditional: a
-    // branch around it costs more issue slots than the instruction; the data lands in a stage nobody reads any more)
-    if (KT < 3 && KT > 0) { ga -= a_step; gb -= b_step; }
+    // tile kt + 2 in step kt.  The last two tiles have nothing left to fetch and are written out behind the loop without
+    // the DMA (a branch around every DMA instruction would cost more issue slots than the instruction; fetching the last
+    // tile again into a stage nobody reads, as an earlier version did, costs the memory pipeline two tiles' worth of time).
     [[maybe_unused]] int4v ktab;                              // contractions: a table entry on its way from LDS
     if (KT > 1) wait_vmcnt<DPT>(); else wait_vmcnt<0>();
     block_barrier();
     ra.set_stage(lds_base);
     rb.set_stage(lds_base + GA::BYTES);
     static_for<0, NOPS>([&](auto r_c) { read_op(r_c, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
-    // (no copy of the loop body for the last tile: what it reads ahead and fetches there is never used)
     // DMA: the tile fetches tile kt + 2; LAST: there is no tile kt + 1 (nothing to wait for, nothing to read ahead)
     auto tile_body = [&](int kt, auto lg_c, auto ag_c, auto first_c, auto dma_c, auto last_c) __attribute__((always_inline)) {
       constexpr bool LAST = decltype(last_c)::value;
@@ -1441,7 +1449,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             part_b = gb + (long long)ob * 2;
           }
           phase(ks_c, dma_c, kt & 1, NoGroup{}, ag_c, No{}, std::integral_constant<int, (ks & 1)>{}, std::integral_constant<bool, !LAST>{});
-          if (kt + 3 < KT) { ga += a_step; gb += b_step; }
+          if constexpr (decltype(dma_c)::value) { ga += a_step; gb += b_step; }
         } else {
           if constexpr (Cfg::GETT && ks == 0) {
             // the table entry of the tile that the next k-step fetches (tile kt + 2, or the last tile once more); it
@@ -1467,7 +1475,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       tile_body(KT - 2, NoGroup{}, NoGroup{}, No{}, No{}, No{});
       tile_body(KT - 1, NoGroup{}, NoGroup{}, No{}, No{}, Yes{});
     } else {
-      for (int kt = 0; kt < KT; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{});
+      for (int kt = 0; kt < KT - 2; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{});
+      if (KT >= 2) tile_body(KT - 2, NoGroup{}, NoGroup{}, No{}, No{}, No{});
+      if (KT >= 1) tile_body(KT - 1, NoGroup{}, NoGroup{}, No{}, No{}, Yes{});
     }
     wait_vmcnt<0>();     // (the last DMA of the loop may still be on its way; so are reads
     wait_lgkmcnt<0>();   // of fragments)

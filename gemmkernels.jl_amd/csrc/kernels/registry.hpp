@@ -67,6 +67,7 @@ int family_mfma_nt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, 
 int family_mfma_tt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_fpu(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_fpu_types(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+int family_fpu_lanes(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_fpu_more(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_splitk(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_complex(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);

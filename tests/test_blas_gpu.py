@@ -221,7 +221,7 @@ def test_odd_sizes_with_16_bit_c(gpu, beta, dtype):
 def test_fpu_operator_shapes(gpu, ta, tb):
     """The operator-shape sweep of the reference (configs/configs.jl:521-551) on 64-lane waves: operator shapes that
     are multiples of the 8 x 8 lane grid run and give, bit for bit, the sequential fma chain (the shape only says
-    which lane owns which output); other lane grids are refused with the operator-shape error, not replaced."""
+    which lane owns which output); the other lane grids run on the tile they are compiled for, see below."""
     from gemmkernels import Kernel, Layout, NT, Operator
     M = N = K = 128
     a, b, c = operands(M, N, K, ta, tb, np.float32, 900)
@@ -240,7 +240,28 @@ def test_fpu_operator_shapes(gpu, ta, tb):
             if ref is None:
                 ref = helpers.run_oracle(conf, a, b, c, (M, N))
             assert np.array_equal(d, ref), (shape, block)
-    for shape in [(4, 64, 1, 1, 64, 1), (4, 32, 1, 2, 32, 1), (16, 16, 1, 4, 16, 1), (16, 16, 1, 16, 4, 1), (32, 4, 1, 32, 2, 1), (64, 4, 1, 64, 1, 1)]:
+    # The other lane grids of the reference's sweep (base shapes 1 x 32 ... 32 x 1 there, 1 x 64 ... 64 x 1 on 64 lanes) run on the
+    # 128 x 128 x 16 tile, whose 64 x 64 wave tiles every grid divides: which lane owns which output changes, the fma chain of
+    # an output does not -- same bits as the oracle.  On other tiles they are refused with the operator-shape error, not replaced.
+    grids = [(4, 64, 1, 1, 64, 1), (4, 32, 1, 2, 32, 1), (16, 16, 1, 4, 16, 1), (16, 16, 1, 16, 4, 1), (32, 4, 1, 32, 2, 1), (64, 4, 1, 64, 1, 1)]
+    for shape in grids:
+        conf = gk.get_config(gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=128, N=128, K=16), warps_per_block=4,
+                             compute_warp=NT(M=64, N=64, K=shape[2]),
+                             operator=Operator.FPUOp[(*shape, Float32, Float32)], global_a_layout=la, global_b_layout=lb,
+                             global_c_layout=Layout.UnsafeAlignedColMajor[Float32], global_d_layout=Layout.UnsafeAlignedColMajor[Float32],
+                             is_a_col_major=not ta, is_b_col_major=not tb)
+        name = gk.kernel_name(conf, Kernel.matmul_pipelined)
+        print("lane grid", shape[3], "x", shape[4], name, flush=True)
+        assert f"lanes{shape[3]}x{shape[4]}" in name
+        d = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+        assert np.array_equal(d, ref), shape
+        # ... with hooks: scale on A, bias per column, ReLU on D
+        from gemmkernels import Epilogue, Transform
+        hooks = dict(transform_shared_to_regs_a=Transform.Elementwise(lambda x: x * 0.75), transform_shared_to_global_d=Transform.Elementwise(Transform.relu))
+        bias = rng.matrix("upm1_f32", 905, (N, 1))[:, 0] * 30
+        dh = helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined, transforms=hooks, epilogue_cls=Epilogue.Bias, bias=bias)
+        assert np.array_equal(dh, helpers.run_oracle(conf, a, b, c, (M, N), transforms=hooks, epilogue=Epilogue.Bias(0), bias=bias)), shape
+    for shape in grids:
         with pytest.raises(gk.ConfigError) as ei:
             conf = conf_for(shape, (128, 128, 32))
             helpers.run_gpu(conf, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)

@@ -17,12 +17,33 @@ LLVM = "/opt/rocm/llvm/bin"
 MAGIC = b"__CLANG_OFFLOAD_BUNDLE__"
 
 
+COMPRESSED_MAGIC = b"CCOB"
+
+
 def code_objects(tmp_path):
-    """The gfx950 code objects bundled into the library (one per translation unit)."""
+    """The gfx950 code objects bundled into the library (one per translation unit).  The library is built with
+    --offload-compress: every bundle is a compressed one (magic CCOB, total size in its header), which the bundler of
+    the toolchain unpacks; plain bundles (magic __CLANG_OFFLOAD_BUNDLE__) are read directly."""
     fat = tmp_path / "fatbin"
     subprocess.run([f"{LLVM}/llvm-objcopy", f"--dump-section=.hip_fatbin={fat}", LIB, os.devnull], check=True)
     data = fat.read_bytes()
     out = []
+    for m in re.finditer(re.escape(COMPRESSED_MAGIC), data):
+        p = m.start()
+        version, method = struct.unpack_from("<HH", data, p + 4)
+        if version >= 3:
+            (total,) = struct.unpack_from("<Q", data, p + 8)
+        else:
+            (total,) = struct.unpack_from("<I", data, p + 8)
+        if method not in (0, 1) or total < 24 or p + total > len(data):       # (a chance match inside other data)
+            continue
+        piece = tmp_path / f"bundle{len(out)}.ccob"
+        piece.write_bytes(data[p:p + total])
+        path = tmp_path / f"co{len(out)}.elf"
+        r = subprocess.run([f"{LLVM}/clang-offload-bundler", "--type=o", f"--input={piece}", "--targets=hipv4-amdgcn-amd-amdhsa--gfx950",
+                            f"--output={path}", "--unbundle"], capture_output=True, text=True)
+        if r.returncode == 0 and path.exists() and path.stat().st_size > 0:
+            out.append(path)
     for m in re.finditer(re.escape(MAGIC), data):
         p = m.start()
         (count,) = struct.unpack_from("<Q", data, p + len(MAGIC))

@@ -122,6 +122,40 @@ def test_hooks_and_bias_on_complex(gpu, ta, tb, dual):
         assert oracle.rel_frobenius(d[0], want.real) <= TOL and oracle.rel_frobenius(d[1], want.imag) <= TOL
 
 
+@pytest.mark.parametrize("ta,tb", TRANSPOSES)
+@pytest.mark.parametrize("dual", [False, True])
+def test_scale_and_negation_of_a_and_b_on_complex(gpu, ta, tb, dual):
+    """Hooks on A and B of the complex and dual operators (the reference's hooks are operator-agnostic,
+    src/kernel.jl:224-236, 311-319): a scale by a power of two and a negation are real factors, act on both parts and
+    commute with the product, so they are folded into the accumulators.  Against the oracle, which applies them to the
+    operands, against numpy, and exactly on dyadic data (the fold must not cost a single bit)."""
+    from gemmkernels import Transform
+    M, N, K = 128, 192, 128
+    conf = configs.complex_config(M, N, K, ta, tb, zero_c=False, dual=dual)
+    a = configs.complex_matrix(166, K if ta else M, M if ta else K)
+    b = configs.complex_matrix(167, N if tb else K, K if tb else N)
+    c = rng.matrix("upm1_f32", 168, (2, M, N))
+    transforms = dict(transform_global_to_shared_a=Transform.Elementwise(lambda x: x * 0.25),
+                      transform_shared_to_regs_b=Transform.Elementwise(lambda x: -x),
+                      transform_shared_to_global_d=Transform.Elementwise(lambda x: x * 2.0))
+    print("case", ta, tb, dual, gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=transforms), flush=True)
+    d, ref = _hooked(conf, a, b, c, M, N, transforms, None)
+    assert np.isfinite(d).all()
+    assert oracle.rel_frobenius(d[0], ref[0]) <= 1e-5 and oracle.rel_frobenius(d[1], ref[1]) <= 1e-5
+    if not dual:
+        A = to_c128(a).T if ta else to_c128(a)
+        B = to_c128(b).T if tb else to_c128(b)
+        want = 2.0 * ((0.25 * A) @ (-B) + to_c128(c))
+        assert oracle.rel_frobenius(d[0], want.real) <= TOL and oracle.rel_frobenius(d[1], want.imag) <= TOL
+    # dyadic data: every product and every partial sum is exact in FP32, folded or not
+    rs = np.random.RandomState(170)
+    ai = np.asfortranarray(rs.randint(-4, 5, size=a.shape).astype(np.float16))
+    bi = np.asfortranarray(rs.randint(-4, 5, size=b.shape).astype(np.float16))
+    ci = np.asfortranarray(rs.randint(-64, 65, size=c.shape).astype(np.float32))
+    di, refi = _hooked(conf, ai, bi, ci, M, N, transforms, None)
+    assert np.array_equal(di, refi)
+
+
 def test_complex_fp16_c_and_d(gpu):
     """Complex{Float16} C and D: fp32 accumulation, one rounding at the store."""
     from gemmkernels import Float16
@@ -148,7 +182,9 @@ def test_complex_hooks_that_are_not_defined_are_refused(gpu):
     d = gk.colmajor_empty((2, M, N), torch.float32)
     for kw in (dict(transform_shared_to_global_d=Transform.Elementwise(Transform.relu)),          # max(z, 0) has no complex method
                dict(transform_regs_to_shared_d=Transform.Elementwise(lambda x: abs(x))),         # abs(z) is real
-               dict(transform_global_to_shared_a=Transform.Elementwise(lambda x: x * 2.0))):     # A / B hooks: C and D only
+               dict(transform_global_to_shared_a=Transform.Elementwise(lambda x: x * 3.0)),      # A / B hooks: what folds into the accumulators only
+               dict(transform_shared_to_regs_b=Transform.Elementwise(lambda x: x * 64.0)),       # a power of two beyond the folded range
+               dict(transform_shared_to_regs_a=Transform.Elementwise(lambda x: x + 1.0))):
         with pytest.raises(ConfigError) as ei:
             gk.matmul(conf, a, b, None, d, kernel=Kernel.matmul_pipelined, **kw)
         assert ei.value.status == _lib.GK_ERR_UNSUPPORTED, ei.value.message

@@ -184,3 +184,27 @@ def test_config3_full_size(gpu):
     ref = np.maximum(0.5 * oracle.gemm_blas_f32(h["a"], h["b"], None) + h["bias"][None, :], 0.0)
     assert oracle.rel_frobenius(d, ref) <= TOL
     assert (d >= 0).all()
+
+
+def test_power_of_two_scales_beyond_the_folded_range_run_in_the_k_loop(gpu):
+    """A scale of A by 2^e leaves the K loop only for |e| <= 4.  2^-20 takes U[-1,1) FP16 values into the subnormal range
+    of FP16, where the reference's hook (and the oracle, and the in-loop scale) rounds s * a to FP16 and loses bits that
+    a fold into the accumulators would keep: the result must be the oracle's, not the exact product."""
+    import torch
+    from gemmkernels import Kernel, Transform, configs, rng
+    M, N, K = 256, 256, 256
+    conf = configs.mfma_config(M, N, K, block_shape=(128, 128, 64), zero_c=True)
+    a, b = rng.matrix("upm1_f16", 9401, (M, K)), rng.matrix("upm1_f16", 9402, (K, N))
+    small = dict(transform_global_to_shared_a=Transform.Elementwise(lambda x: x * 2.0 ** -20))
+    assert "fused_cd" not in gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=small)          # (the level that runs folded scales)
+    d = helpers.run_gpu(conf, a, b, None, (M, N), kernel=Kernel.matmul_pipelined, transforms=small)
+    ref = helpers.run_oracle(conf, a, b, None, (M, N), transforms=small)
+    exact = 2.0 ** -20 * oracle.gemm_f64(a, b, None, 1.0, 0.0)
+    assert oracle.rel_frobenius(d, ref) <= 1e-5
+    assert oracle.rel_frobenius(ref, exact) > 1e-3           # the rounding of s * a to FP16 shows: a fold would not have it
+    # at the edge of the range, 2^-4, the scale is folded: the plain product times 2^-4, bit for bit
+    edge = dict(transform_global_to_shared_a=Transform.Elementwise(lambda x: x * 2.0 ** -4))
+    assert "fused_cd" in gk.kernel_name(conf, Kernel.matmul_pipelined, transforms=edge)
+    d4 = helpers.run_gpu(conf, a, b, None, (M, N), kernel=Kernel.matmul_pipelined, transforms=edge)
+    plain = helpers.run_gpu(conf, a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, plain * np.float32(2.0 ** -4))

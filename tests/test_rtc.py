@@ -158,3 +158,60 @@ def test_a_specialised_kernel_refuses_bounds_checked_layouts_at_launch(gpu):
         Plan(loose, A[:M - 8, :], B, None, D[:M - 8, :], {}, _DEFAULT_EPILOGUE, Kernel.matmul_pipelined, specialized=k)()
     k(A, B, None, D)                                  # the configuration it was compiled for still runs
     torch.cuda.synchronize()
+
+
+# The reference's parameter sweep of the tensor-core GEMM (configs/configs.jl:597-612): M = N = K = 256, block shapes of at
+# most 128 x 128 outputs out of {64, 128, 256}^2, BLOCK_K in {16, 32, 64}, 1 / 2 / 4 warps along M and N with at least four in
+# all.  Every tile that the kernel template can be built for is compiled on demand and checked against the oracle; the
+# others are refused with a configuration error before anything is compiled, which the reference's test counts as
+# skipped (test/matmul.jl:21-27).  'N','N' for every tile, 'T','T' as well for BLOCK_K = 16 (which runs on the 32 x 32 x 16
+# instruction: the k-step of v_mfma_f32_16x16x32 is 32).
+SWEEP_BLOCKS = [(bm, bn, bk) for bm in (64, 128, 256) for bn in (64, 128, 256) if bm * bn <= 128 * 128 for bk in (16, 32, 64)]
+SWEEP_WAVES = [(wm, wn) for wm in (1, 2, 4) for wn in (1, 2, 4) if wm * wn >= 4]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("block", SWEEP_BLOCKS)
+def test_the_reference_sweep_of_block_shapes_and_warp_arrangements(gpu, block):
+    import torch
+    from gemmkernels import ConfigError
+    from oracle import oracle
+    BM, BN, BK = block
+    M = N = K = 256
+    ran = refused = 0
+    for ta, tb in ([(False, False), (True, True)] if BK == 16 else [(False, False)]):
+        a = rng.matrix("upm1_f16", 41, (K, M) if ta else (M, K))
+        b = rng.matrix("upm1_f16", 42, (N, K) if tb else (K, N))
+        c = rng.matrix("upm1_f32", 43, (M, N))
+        A, B, C = gk.colmajor(a), gk.colmajor(b), gk.colmajor(c)
+        ref = oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)
+        for wm, wn in SWEEP_WAVES:
+            try:
+                conf = gk.get_config(gemm_shape=NT(M=M, N=N, K=K), operator=Operator.MFMAOp[32, 32, 16, Float16, Float32],
+                                     global_a_layout=(Layout.UnsafeAlignedRowMajor if ta else Layout.UnsafeAlignedColMajor)[Float16],
+                                     global_b_layout=(Layout.UnsafeAlignedRowMajor if tb else Layout.UnsafeAlignedColMajor)[Float16],
+                                     global_c_layout=Layout.UnsafeAlignedColMajor[Float32], global_d_layout=Layout.UnsafeAlignedColMajor[Float32],
+                                     is_a_col_major=not ta, is_b_col_major=not tb, block_shape=NT(M=BM, N=BN, K=BK), warps_per_block=wm * wn,
+                                     compute_warp=NT(M=BM // wm, N=BN // wn, K=16), specialize=True)
+                k = gk.specialize(conf)
+            except ConfigError as e:
+                refused += 1
+                print("refused", block, (wm, wn), "TT" if ta else "NN", e.message[:90], flush=True)
+                continue
+            print("runs   ", block, (wm, wn), "TT" if ta else "NN", k.name, flush=True)
+            D = gk.colmajor_empty((M, N), torch.float32)
+            D.fill_(float("nan"))
+            k(A, B, C, D)
+            torch.cuda.synchronize()
+            assert oracle.rel_frobenius(gk.to_numpy(D), ref) <= 1e-3, (block, wm, wn, ta, tb)
+            ran += 1
+    print(f"block {block}: {ran} ran, {refused} refused", flush=True)
+    # what runs is exactly what the kernel template can be built for: wave tiles made of 32 x 32 blocks (at most sixteen),
+    # and an A tile and a B tile whose 1 KiB pieces divide evenly over the waves (64 x 64 x 16 has two pieces per operand
+    # and no arrangement of four or more waves: the whole block shape counts as skipped, like a ConfigError of the reference)
+    def buildable(wm, wn):
+        wtm, wtn = BM // wm, BN // wn
+        pieces_a, pieces_b = BM * BK * 2 // 1024, BN * BK * 2 // 1024
+        return (wtm % 32 == 0 and wtn % 32 == 0 and (wtm // 32) * (wtn // 32) <= 16 and pieces_a % (wm * wn) == 0 and pieces_b % (wm * wn) == 0)
+    expected = sum(buildable(wm, wn) for wm, wn in SWEEP_WAVES) * (2 if BK == 16 else 1)
+    assert ran == expected, (block, ran, expected)
