@@ -258,6 +258,14 @@ int make_key_as_configured(const gk_config* c, const gk_transforms* t, const gk_
 // (tiles over the edges, a partial last K tile: path 3 of the kernel, which moves an FP32 C / D 16 bytes at a time).  Any other launch of such a configuration runs the
 // eight-wave arrangement of the same block shape, which gives the same bits (the order of the k-steps and of the
 // products inside them does not depend on how the tile is dealt out to waves).
+bool wide_tile(const gk::InstanceKey& key) {
+  return key.BK == 64 && ((key.BM == 256 && key.BN == 192) || (key.BM == 192 && key.BN == 256));
+}
+void wide_tile_on_eight_waves(gk::InstanceKey* key) {
+  key->waves_m = key->BM == 256 ? 4 : 2;
+  key->waves_n = key->BM == 256 ? 2 : 4;
+}
+
 int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, gk::InstanceKey* key, bool allow_ragged_fast = true) {
   const int rc = make_key_as_configured(c, t, e, key, allow_ragged_fast);
   if (rc != GK_OK) return rc;
@@ -301,6 +309,12 @@ int make_key(const gk_config* c, const gk_transforms* t, const gk_epilogue* e, g
       key->waves_n = 4;
       if (key->fused == 4) key->fused = 3;
     }
+  }
+  // ... for the tiles with a side of 192 (wave tiles of 128 x 96 or 96 x 128): plain products without hooks or bias
+  // in whole tiles; any other launch runs the eight waves that have the 192 side to themselves in pairs
+  if ((plain || key->family == gk::FAMILY_MFMA_CHECKED) && wide_tile(*key) && key->waves_m == 2 && key->waves_n == 2) {
+    const bool whole = c->matmul_shape.M % key->BM == 0 && c->matmul_shape.N % key->BN == 0 && c->matmul_shape.K % 64 == 0;
+    if (!(plain && whole && key->fused == 0 && key->variant == 0)) wide_tile_on_eight_waves(key);
   }
   // ... and for the complex / dual product on interleaved matrices of an 'N','N' launch (real tile 256 x 256 x 64)
   // (planar matrices, variant 2: every transpose, the planes being plain real operands)
@@ -418,6 +432,12 @@ void make_args(const gk_config* c, const void* a, const void* b, const void* cc,
 gk::FamilyFn family_fn(const gk::InstanceKey& key) {
   switch (key.family) {
     case gk::FAMILY_MFMA:
+      if (wide_tile(key) && key.waves_m == 2 && key.waves_n == 2) {
+        // the tiles with a side of 192 on four waves are compiled in translation units of their own
+        if (key.a_kmajor) return key.b_kmajor ? gk::family_mfma_wide_tn : gk::family_mfma_wide_tt;
+        return key.b_kmajor ? gk::family_mfma_wide_nn : gk::family_mfma_wide_nt;
+      }
+      [[fallthrough]];
     case gk::FAMILY_GETT:
       if (key.a_kmajor) return key.b_kmajor ? gk::family_mfma_tn : gk::family_mfma_tt;
       return key.b_kmajor ? gk::family_mfma_nn : gk::family_mfma_nt;
@@ -943,6 +963,14 @@ int prepare_launch(const gk_config* conf, const void* a, const void* b, const vo
     gk::FamilyFn fn8 = family_fn(key);
     hipError_t e8 = hipSuccess;
     if (!fn8 || !fn8(key, args, dim3(1), nullptr, 0, &info, &e8)) return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance for this %s", solo_edges ? "product" : "contraction");
+  }
+
+  if (!custom && key.family == gk::FAMILY_MFMA && wide_tile(key) && key.waves_m == 2 && key.waves_n == 2 && gk::solo_cd_path(args) == 0) {
+    // the four waves of a tile with a side of 192 move an FP32 C / D 16 bytes at a time as well
+    wide_tile_on_eight_waves(&key);
+    gk::FamilyFn fn8 = family_fn(key);
+    hipError_t e8 = hipSuccess;
+    if (!fn8 || !fn8(key, args, dim3(1), nullptr, 0, &info, &e8)) return fail(GK_ERR_UNSUPPORTED, "no compiled kernel instance for this product");
   }
 
   // aligned layouts move 16-byte vectors (reference src/layout.jl:22-34 traps on the device; here it is a host check)

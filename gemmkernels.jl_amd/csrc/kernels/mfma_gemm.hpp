@@ -430,7 +430,9 @@ struct MfmaGemmConfig {
   // assembly statement that issues them (see FragReader::read)
   // One wave per SIMD: four waves with wave tiles of 64 16x16 blocks (all 256 accumulation registers), two LDS stages.
   // The K loop of these instances is written out instruction slot by instruction slot (see the SOLO loop).
-  static constexpr bool SOLO = MI_ == 16 && WAVES_M_ * WAVES_N_ == 4 && (BM_ / WAVES_M_ / 16) * (BN_ / WAVES_N_ / 16) == 64 && STAGES_ == 2 &&
+  // (64 accumulator blocks: all 256 accumulation registers; 48 for the tiles with a side of 192)
+  static constexpr int SOLO_BLOCKS = (BM_ / WAVES_M_ / 16) * (BN_ / WAVES_N_ / 16);
+  static constexpr bool SOLO = MI_ == 16 && WAVES_M_ * WAVES_N_ == 4 && (SOLO_BLOCKS == 64 || (SOLO_BLOCKS == 48 && FIX_ == FIX_NONE && !GETT_)) && STAGES_ == 2 &&
                                (BK_ / 32) % 2 == 0 && !SPLITK_ && (GK_FORCE_SYNC_FRAGS == 0) &&
                                ((FIX_ == FIX_NONE && (FUSE_ == 0 || FUSE_ == 4) && A_KIND_ != OPK_KSPLIT && B_KIND_ != OPK_KSPLIT) ||
                                 // ... and the complex / dual real-view product of an 'N','N' launch (A contiguous along m, B along k)
@@ -1264,7 +1266,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // matrix core busy for sixteen, and with a single wave on the SIMD every further instruction between two MFMAs
     // is time in which the matrix core idles.  A DMA instruction (with its LDS address in M0) goes behind every GD-th
     // MFMA of the k-step that follows the barrier, an LDS read behind every other MFMA.
-    constexpr int GD = 4, RSP = 1;
+    constexpr int GD = (4 * (DPT - 1) < NM) ? 4 : 3, RSP = 1;
     static_assert(GD * (DPT - 1) < NM, "the DMA of a tile is issued in the k-step behind the barrier that frees its stage");
     static_assert(NOPS * RSP <= NM, "the fragment reads fit the MFMAs of a k-step");
     // DMA instruction I of the tile that ga / gb stand at
@@ -1305,7 +1307,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     static_assert(CGROUPS + 3 <= kSoloStreamTiles, "the K tiles that bring C in are written out in front of the loop, the last two behind it");
     static_assert(CPATH != 4 || KS >= 2, "the loads of C go into the first k-step of a tile, the additions into the last");
     [[maybe_unused]] float4v cland[CPATH == 4 ? 2 : 1][CPATH == 4 ? FM : 1];
-    [[maybe_unused]] float ctmp[2][4];
+    [[maybe_unused]] float ctmp[4][4];                 // values on their way from an accumulation register and back (see c_add_step)
     [[maybe_unused]] unsigned c_voff = 0;              // byte offset of the lane's four rows of block (0, 0) from the wave tile's origin in C
     [[maybe_unused]] const char* c_tile = nullptr;     // the wave tile's origin in C (the same in every lane)
     [[maybe_unused]] long long c_col16 = 0;            // bytes from a block column to the next
@@ -1325,12 +1327,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     };
     // Step Q (0 .. 5) of the addition of block (J, G): two accumulation registers read, two values added, two registers
     // written back
-    [[maybe_unused]] auto c_add_step = [&](auto g_c, auto j_c, auto q_c) __attribute__((always_inline)) {
-      constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value, Q = decltype(q_c)::value;
+    // (T: the set of temporaries.  The additions of two blocks overlap in time when their slots do: blocks two rows apart
+    // never do, a block that takes the first slots of the k-step may meet any of the first rows and has sets of its own)
+    [[maybe_unused]] auto c_add_step = [&](auto g_c, auto j_c, auto q_c, auto t_c) __attribute__((always_inline)) {
+      constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value, Q = decltype(q_c)::value, T = decltype(t_c)::value;
       constexpr int R = 4 * (G * FM + J), E = 2 * (Q & 1);
       float4v& src = cland[G & 1][J];
-      float& t0 = ctmp[J & 1][E];
-      float& t1 = ctmp[J & 1][E + 1];
+      float& t0 = ctmp[T][E];
+      float& t1 = ctmp[T][E + 1];
       if constexpr (Q == 0) asm volatile("" : "+v"(src));
       if constexpr (Q < 2) {
         asm volatile("v_accvgpr_read_b32 %0, a[%2]\n\tv_accvgpr_read_b32 %1, a[%3]" : "=v"(t0), "=v"(t1) : "n"(R + E), "n"(R + E + 1));
@@ -1385,7 +1389,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (CPATH == 4 && !B_BOTH) {
-          constexpr int LSLOT0 = NOPS * RSP + 2, LSTEP = 4;        // (behind the fragment reads)
+          constexpr int LSLOT0 = NOPS * RSP + 2;                   // (behind the fragment reads)
+          constexpr int LSTEP = (LSLOT0 + 4 * (FM - 1) < NM) ? 4 : (LSLOT0 + 3 * (FM - 1) < NM) ? 3 : 2;
           static_assert(LG < 0 || LSLOT0 + LSTEP * (FM - 1) < NM, "the loads of a group of C fit the k-step");
           if constexpr (LG >= 0 && i >= LSLOT0 && (i - LSLOT0) % LSTEP == 0 && (i - LSLOT0) / LSTEP < FM) {
             __builtin_amdgcn_sched_barrier(0);
@@ -1396,12 +1401,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             static_for<0, FM * 6>([&](auto u_c) {
               constexpr int u = decltype(u_c)::value, j = u / 6, q = u % 6;
               constexpr int p = j * FN + ((j & 1) ? FN - 1 - AG : AG);       // the MFMA of block (j, AG) in this k-step
-              constexpr int s0 = (p + 9 < NM) ? p + 4 : p + 4 - NM + 8;
+              constexpr bool early = !(p + 9 < NM);
+              constexpr int s0 = early ? p + 4 - NM + 8 : p + 4;
               // (the two halves of a step trade places so that a value is read, added and written two slots apart)
               constexpr int at = s0 + (q / 2) * 2 + (q & 1);
               if constexpr (at == i) {
                 __builtin_amdgcn_sched_barrier(0);
-                c_add_step(ag_c, std::integral_constant<int, j>{}, std::integral_constant<int, q>{});
+                c_add_step(ag_c, std::integral_constant<int, j>{}, std::integral_constant<int, q>{}, std::integral_constant<int, (j & 1) + (early ? 2 : 0)>{});
                 __builtin_amdgcn_sched_barrier(0);
               }
             });
@@ -1423,7 +1429,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     rb.set_stage(lds_base + GA::BYTES);
     static_for<0, NOPS>([&](auto r_c) { read_op(r_c, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
     // DMA: the tile fetches tile kt + 2; LAST: there is no tile kt + 1 (nothing to wait for, nothing to read ahead)
-    auto tile_body = [&](int kt, auto lg_c, auto ag_c, auto first_c, auto dma_c, auto last_c) __attribute__((always_inline)) {
+    // PEND: loads of C, younger than the DMA of tile kt + 1, that stay in flight over the wait for that tile
+    auto tile_body = [&](int kt, auto lg_c, auto ag_c, auto first_c, auto dma_c, auto last_c, auto pend_c) __attribute__((always_inline)) {
       constexpr bool LAST = decltype(last_c)::value;
       static_for<0, KS>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
@@ -1434,7 +1441,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             // tile kt+1 has landed (its DMA was issued a k-step or more ago); behind the barrier it is visible to all
             // waves, and all are done reading tile kt: its stage takes tile kt+2
             // (the loads of C that this tile has issued stay in flight: memory reads return in order, and they are younger than the DMA)
-            wait_vmcnt<(decltype(lg_c)::value >= 0 ? FM : 0)>();
+            wait_vmcnt<decltype(pend_c)::value>();
             block_barrier();
             const unsigned stage_addr = lds_base + (unsigned)((kt + 1) & 1) * Cfg::STAGE_BYTES;
             ra.set_stage(stage_addr);
@@ -1466,18 +1473,22 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if constexpr (CPATH == 4) {
       // the first K tiles, written out: tile t fetches group t of C and adds group t - 1 (the host sends products of at
       // least kSoloStreamTiles K tiles here) ...
+      typedef std::integral_constant<int, 0> Pend0;
       static_for<0, CGROUPS + 1>([&](auto t_c) {
         constexpr int t = decltype(t_c)::value;
-        tile_body(t, std::integral_constant<int, (t < CGROUPS ? t : -1)>{}, std::integral_constant<int, t - 1>{}, std::integral_constant<bool, t == 0>{}, Yes{}, No{});
+        constexpr int LGT = t < CGROUPS ? t : -1;
+        tile_body(t, std::integral_constant<int, LGT>{}, std::integral_constant<int, t - 1>{}, std::integral_constant<bool, t == 0>{}, Yes{}, No{},
+                  std::integral_constant<int, (LGT >= 0 ? FM : 0)>{});
       });
-      for (int kt = CGROUPS + 1; kt < KT - 2; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{});
+      for (int kt = CGROUPS + 1; kt < KT - 2; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{}, Pend0{});
       // ... and the last two, which have nothing left to fetch
-      tile_body(KT - 2, NoGroup{}, NoGroup{}, No{}, No{}, No{});
-      tile_body(KT - 1, NoGroup{}, NoGroup{}, No{}, No{}, Yes{});
+      tile_body(KT - 2, NoGroup{}, NoGroup{}, No{}, No{}, No{}, Pend0{});
+      tile_body(KT - 1, NoGroup{}, NoGroup{}, No{}, No{}, Yes{}, Pend0{});
     } else {
-      for (int kt = 0; kt < KT - 2; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{});
-      if (KT >= 2) tile_body(KT - 2, NoGroup{}, NoGroup{}, No{}, No{}, No{});
-      if (KT >= 1) tile_body(KT - 1, NoGroup{}, NoGroup{}, No{}, No{}, Yes{});
+      typedef std::integral_constant<int, 0> Pend0;
+      for (int kt = 0; kt < KT - 2; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{}, Pend0{});
+      if (KT >= 2) tile_body(KT - 2, NoGroup{}, NoGroup{}, No{}, No{}, No{}, Pend0{});
+      if (KT >= 1) tile_body(KT - 1, NoGroup{}, NoGroup{}, No{}, No{}, Yes{}, Pend0{});
     }
     wait_vmcnt<0>();     // (the last DMA of the loop may still be on its way; so are reads
     wait_lgkmcnt<0>();   // of fragments)
@@ -1901,7 +1912,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             float4v o;
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[v] = x[4 * fi + v];
-            *(float4v*)((float*)args.d + off) = o;
+            float* dp = (float*)args.d + off;
+            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(dp), "v"(o) : "memory");       // (write-through, see path 4)
           } else {
 #pragma unroll
             for (int v = 0; v < 4; ++v) store_cd(args.d, args.d_dtype, off + v, x[4 * fi + v]);
@@ -1921,7 +1933,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           if (r < args.M && cc < args.N) {
             float* dp = (float*)args.d + ((long long)r + (long long)cc * args.ldd);
             if (r + 4 <= args.M) {
-              asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
+              asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
             } else {
               const int left = args.M - r;     // 1 .. 3
               asm volatile("global_store_dword %0, %1, off" :: "v"(dp), "a"(acc[fi][fj][0]) : "memory");
@@ -1932,7 +1944,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
     } else if constexpr (CPATH == 4) {
       // from the accumulation registers the kernel manages itself: the wave tile's origin in D from scalar registers, the
-      // lane's offset in it from a vector register, the row block as an immediate
+      // lane's offset in it from a vector register, the row block as an immediate.  The stores write through to memory
+      // (sc0 sc1): D is not read again by this launch, and what stays dirty in the L2s has to be written back after the
+      // last wave has ended, before the launch counts as complete (a kernel that only stores such tiles: 11.3 us from
+      // launch to launch with plain stores, 10.1 us with these; the GEMM gains about one microsecond)
       const unsigned d_voff = (unsigned)((4 * (lane_e / MI) + (long long)(lane_e % MI) * args.ldd) * 4);
       const char* d_tile = (const char*)args.d + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldd) * 4;
       const long long d_col16 = (long long)args.ldd * (MI * 4);
@@ -1944,7 +1959,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           constexpr int R = 4 * (fj * FM + fi);
           const unsigned vo = d_voff;             // (named here: an operand of an assembly statement does not capture by itself)
           const char* sb = base;
-          asm volatile("global_store_dwordx4 %0, a[%2:%3], %1 offset:%4" :: "v"(vo), "s"(sb), "n"(R), "n"(R + 3), "n"(fi * MI * 4) : "memory");
+          asm volatile("global_store_dwordx4 %0, a[%2:%3], %1 offset:%4 sc0 sc1" :: "v"(vo), "s"(sb), "n"(R), "n"(R + 3), "n"(fi * MI * 4) : "memory");
         });
       });
     } else if constexpr (CPATH != 0) {
@@ -1953,7 +1968,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) {
           float* dp = (float*)args.d + solo_off(solo_row, solo_col, fi, fj, args.ldd, args.plane_d);
-          asm volatile("global_store_dwordx4 %0, %1, off" :: "v"(dp), "a"(acc[fi][fj]) : "memory");
+          asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(dp), "a"(acc[fi][fj]) : "memory");       // (write-through, see path 4)
         }
     } else if (args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0) {
       // (FP32 D next to a C that is not)

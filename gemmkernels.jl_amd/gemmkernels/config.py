@@ -152,7 +152,7 @@ _MFMA_TILES = [
     ((64, 64, 32), (2, 2)),       # four stages; the one-wave instance (the tensor-contraction kernels have only that) is 1.5 - 2.7 times slower
 ]
 # Tiles with a side of 192: they fill the chip where 256 x 256 leaves CUs idle (3072^2: 192 tiles instead of 144,
-# 59 us instead of 72).  Compiled per transpose: 256 x 192 for 'N','N', 'T','N' and 'N','T'; 192 x 256 for
+# 56 us instead of 68).  Compiled per transpose: 256 x 192 for 'N','N', 'T','N' and 'N','T'; 192 x 256 for
 # 'T','N' and 'T','T' (the third entry says whether a transpose (a_kmajor, b_kmajor) has the tile).
 _MFMA_TILES_192 = [((256, 192, 64), (4, 2), lambda a_kmajor, b_kmajor: b_kmajor or not a_kmajor),
                    ((192, 256, 64), (2, 4), lambda a_kmajor, b_kmajor: a_kmajor)]
@@ -205,8 +205,8 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
         tiles = -(-M // t[0]) * -(-N // t[1])
         rounds = -(-tiles // NUM_CUS)
         rate = _MFMA_TILE_RATE.get(t, 0.5)
-        if t == (256, 192, 64) and not a_kmajor and not b_kmajor:
-            rate = 0.78      # 'N','T': the 192 side is read with transposing LDS reads (3072^3: 69.7 us, 256 x 256: 72.6 us)
+        if t == (256, 192, 64) and not a_kmajor and not b_kmajor and (M % t[0] or N % t[1] or K % t[2]):
+            rate = 0.78      # 'N','T' on eight waves (tiles over the edges): the 192 side is read with transposing LDS reads
         if isinstance(rate, tuple):
             rate = rate[0] if rounds == 1 else rate[1]
         return rounds * t[0] * t[1] / rate
@@ -253,6 +253,11 @@ def _default_waves(operator, block_shape, checked=False, planar=False, gett=Fals
     if gett and key == (64, 64, 32):
         return (1, 1)
     if operator.kind == Operator.MFMA and key == _SOLO_TILE and whole_tiles:
+        return _SOLO_WAVES
+    # ... and the tiles with a side of 192 (wave tiles of 128 x 96 / 96 x 128; 3072^3: 56 us against 62 on eight waves,
+    # 'N','T' 57 against 65); the library runs the eight waves for what these instances do not cover (hooks, a bias,
+    # tiles over the edges, a C / D that does not take 16-byte accesses)
+    if operator.kind == Operator.MFMA and not gett and whole_tiles and any(key == t for t, _, _ in _MFMA_TILES_192):
         return _SOLO_WAVES
     # ... and the complex / dual product on interleaved matrices of an 'N','N' launch, whose real tile is that tile
     # (planar matrices: every transpose)
@@ -369,9 +374,10 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
     mem_cd_thread = NT(params.get("mem_cd_thread", adjacent_elements(n_c, mn, is_cd_col_major)))
 
     # src/config.jl:277-279 defaults to Identity; on the MI355X the XCD-aware walk is the default
-    # (panels 4 tiles high; 8 once the tile grid has a thousand tiles: 8192^3 runs 4 % faster with it)
+    # (panels 4 tiles high; 8 once the tile grid has a thousand tiles: 8192^3 runs 10 % faster with it; 16 from four
+    # thousand tiles on: 16384 x 16384 x 4096 1771 us against 1789 and 1871 us with 8 and 4)
     n_tiles = -(-gemm_shape.M // block_shape.M) * -(-gemm_shape.N // block_shape.N)
-    cta_swizzle = params.get("cta_swizzle", CTASwizzle.XCDAware[8 if n_tiles >= 1024 else 4])
+    cta_swizzle = params.get("cta_swizzle", CTASwizzle.XCDAware[16 if n_tiles >= 4096 else (8 if n_tiles >= 1024 else 4)])
 
     conf = Config(gemm_shape, block_shape, warps_per_block, mem_a_warp, mem_a_thread, mem_b_warp, mem_b_thread,
                   mem_cd_warp, mem_cd_thread, compute_warp, op_shape,

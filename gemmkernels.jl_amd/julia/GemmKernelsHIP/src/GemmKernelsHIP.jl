@@ -395,6 +395,9 @@ const SOLO_COMPLEX_TILE = (128, 128, 64)       # in complex elements
 function default_waves(operator::Type, block_shape; a_kmajor::Bool = false, b_kmajor::Bool = true, planar::Bool = false, whole_tiles::Bool = false)
     key = (block_shape.M, block_shape.N, block_shape.K)
     Operator.is_mfma(operator) && key == SOLO_TILE && whole_tiles && return SOLO_WAVES
+    # the tiles with a side of 192 (a caller's choice of block_shape): four waves in whole tiles, else the eight waves that
+    # share the 192 side in pairs
+    Operator.is_mfma(operator) && key in ((256, 192, 64), (192, 256, 64)) && return whole_tiles ? SOLO_WAVES : (key[1] == 256 ? (4, 2) : (2, 4))
     # ... and the complex / dual product on interleaved matrices of an 'N','N' launch, whose real tile is that tile
     # (planar matrices: every transpose)
     !Operator.is_fpu(operator) && !Operator.is_mfma(operator) && key == SOLO_COMPLEX_TILE && whole_tiles && (planar || (!a_kmajor && b_kmajor)) && return SOLO_WAVES
@@ -472,7 +475,7 @@ function get_config(; gemm_shape, operator, global_a_layout, global_c_layout, kw
 
     # reference src/config.jl:277-279 defaults to Identity; here the XCD-aware walk is the default
     n_tiles = cld(gemm_shape.M, block_shape.M) * cld(gemm_shape.N, block_shape.N)
-    cta_swizzle = get(params, :cta_swizzle, CTASwizzle.XCDAware{n_tiles >= 1024 ? 8 : 4})
+    cta_swizzle = get(params, :cta_swizzle, CTASwizzle.XCDAware{n_tiles >= 4096 ? 16 : (n_tiles >= 1024 ? 8 : 4)})
 
     conf = Config(gemm_shape, block_shape, warps_per_block, mem_a_warp, mem_a_thread, mem_b_warp, mem_b_thread,
                   mem_cd_warp, mem_cd_thread, compute_warp, op_shape,

@@ -16,12 +16,12 @@ TOL = 1e-3
 BLOCK = (256, 256, 64)
 
 
-def config(M, N, K, ta, tb, waves, ab=Float16, c=Float32, d=Float32, zero_c=False, checked=False):
+def config(M, N, K, ta, tb, waves, ab=Float16, c=Float32, d=Float32, zero_c=False, checked=False, block=BLOCK):
     col = Layout.ColMajor if checked else Layout.UnsafeAlignedColMajor
     row = Layout.RowMajor if checked else Layout.UnsafeAlignedRowMajor
     return gk.get_config(
-        gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=BLOCK[0], N=BLOCK[1], K=BLOCK[2]),
-        warps_per_block=waves[0] * waves[1], compute_warp=NT(M=BLOCK[0] // waves[0], N=BLOCK[1] // waves[1], K=16),
+        gemm_shape=NT(M=M, N=N, K=K), block_shape=NT(M=block[0], N=block[1], K=block[2]),
+        warps_per_block=waves[0] * waves[1], compute_warp=NT(M=block[0] // waves[0], N=block[1] // waves[1], K=16),
         operator=Operator.MFMAOp[32, 32, 16, ab, Float32],
         global_a_layout=(row if ta else col)[ab], global_b_layout=(row if tb else col)[ab],
         global_c_layout=Layout.Zero[c] if zero_c else col[c], global_d_layout=col[d],
@@ -350,3 +350,87 @@ def test_c_streamed_bf16_operands(gpu):
     assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N))) <= TOL
     d8 = helpers.run_gpu(config(M, N, K, False, False, (2, 4), ab=BFloat16), a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
     assert oracle.rel_frobenius(d4, d8.astype(np.float64)) <= 1e-6
+
+
+# The tiles with a side of 192 on four waves (wave tiles of 128 x 96 and 96 x 128: 48 accumulator blocks per wave),
+# compiled per transpose like their eight-wave arrangements (4 x 2 and 2 x 4 waves).
+WIDE = [((256, 192, 64), (4, 2), [(False, False), (True, False), (False, True)]), ((192, 256, 64), (2, 4), [(True, False), (True, True)])]
+
+
+@pytest.mark.parametrize("block,eight,transposes", WIDE)
+def test_tiles_with_a_side_of_192_on_four_waves(gpu, block, eight, transposes):
+    """C added at the end (fewer than eleven K tiles) and no C: the same bits as the eight waves.  C on its way during
+    the first K tiles (from eleven K tiles on: 704 is the fewest, 1344 has generic tiles in between): the oracle,
+    linearity in C, exact sums of small integers."""
+    BM, BN, _ = block
+    M, N = 2 * BM, 3 * BN
+    for ta, tb in transposes:
+        for K in (64, 192, 448, 704, 768, 1344):
+            a, b, c = operands(M, N, K, ta, tb, 7900 + K)
+            four, eight8 = config(M, N, K, ta, tb, (2, 2), block=block), config(M, N, K, ta, tb, eight, block=block)
+            name = gk.kernel_name(four, Kernel.matmul_pipelined)
+            print("case", block, ta, tb, K, name, flush=True)
+            assert "_w2x2_" in name and "_w%dx%d_" % eight in gk.kernel_name(eight8, Kernel.matmul_pipelined)
+            d4 = helpers.run_gpu(four, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+            d8 = helpers.run_gpu(eight8, a, b, c, (M, N), kernel=Kernel.matmul_pipelined)
+            assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N))) <= TOL
+            assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= 1e-6
+            z4 = helpers.run_gpu(config(M, N, K, ta, tb, (2, 2), zero_c=True, block=block), a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
+            z8 = helpers.run_gpu(config(M, N, K, ta, tb, eight, zero_c=True, block=block), a, b, None, (M, N), kernel=Kernel.matmul_pipelined)
+            assert np.array_equal(z4, z8)
+            if K < 704:
+                assert np.array_equal(d4, d8)
+                continue
+            assert oracle.rel_frobenius(d4, d8.astype(np.float64)) <= 1e-6
+            # every element of C went into its own accumulator exactly once
+            assert np.abs((d4.astype(np.float64) - z4) - c).max() <= 1e-4
+            rs = np.random.RandomState(K)
+            ai = np.asfortranarray(rs.randint(-4, 5, size=a.shape).astype(np.float16))
+            bi = np.asfortranarray(rs.randint(-4, 5, size=b.shape).astype(np.float16))
+            ci = np.asfortranarray(rs.randint(-999, 1000, size=(M, N)).astype(np.float32))
+            di = helpers.run_gpu(four, ai, bi, ci, (M, N), kernel=Kernel.matmul_pipelined)
+            assert np.array_equal(di.astype(np.float64), oracle.gemm_f64(ai, bi, ci, 1.0, 1.0, ta, tb))
+
+
+@pytest.mark.parametrize("block,eight,transposes", WIDE)
+def test_what_the_four_waves_of_a_192_tile_leave_to_the_eight(gpu, block, eight, transposes):
+    """A hook, a bias, a 16-bit D, tiles over the edges and BF16 operands on a configuration of 2 x 2 waves: the first four
+    run the eight-wave arrangement of the same tile with the same bits, BF16 runs on the four waves."""
+    import torch
+    BM, BN, _ = block
+    ta, tb = transposes[0]
+    M, N, K = BM, 2 * BN, 832
+    a, b, c = operands(M, N, K, ta, tb, 8100)
+    four, eight8 = config(M, N, K, ta, tb, (2, 2), block=block), config(M, N, K, ta, tb, eight, block=block)
+    E = Transform.Elementwise
+    tr = dict(transform_shared_to_global_d=E(Transform.relu))
+    assert "_w%dx%d_" % eight in gk.kernel_name(four, Kernel.matmul_pipelined, transforms=tr)
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), transforms=tr, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, helpers.run_gpu(eight8, a, b, c, (M, N), transforms=tr, kernel=Kernel.matmul_pipelined))
+    assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N), transforms=tr)) <= TOL
+    bias = rng.normal_f32(8104, N)
+    d4 = helpers.run_gpu(four, a, b, c, (M, N), epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, helpers.run_gpu(eight8, a, b, c, (M, N), epilogue_cls=Epilogue.Bias, bias=bias, kernel=Kernel.matmul_pipelined))
+    assert oracle.rel_frobenius(d4, helpers.run_oracle(four, a, b, c, (M, N), epilogue=Epilogue.Bias(0), bias=bias)) <= TOL
+    # a 16-bit D is found out at the launch (the kernel's name still tells the configured arrangement)
+    kw = dict(d=Float16, block=block)
+    d4 = helpers.run_gpu(config(M, N, K, ta, tb, (2, 2), **kw), a, b, c, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
+    d8 = helpers.run_gpu(config(M, N, K, ta, tb, eight, **kw), a, b, c, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(d4, d8)
+    assert oracle.rel_frobenius(d4, oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)) <= TOL
+    # tiles over the edges (bounds-checked layouts)
+    Mr, Nr, Kr = BM + 40, BN + 72, 840
+    ar, br, cr = operands(Mr, Nr, Kr, ta, tb, 8200)
+    ragged = config(Mr, Nr, Kr, ta, tb, (2, 2), checked=True, block=block)
+    assert "_w%dx%d_" % eight in gk.kernel_name(ragged, Kernel.matmul_pipelined)
+    dr = helpers.run_gpu(ragged, ar, br, cr, (Mr, Nr), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(dr, oracle.gemm_f64(ar, br, cr, 1.0, 1.0, ta, tb)) <= 1e-6
+    # BF16 operands
+    ab = gk.bf16_bits(rng.matrix("upm1_f32", 8301, a.shape))
+    bb = gk.bf16_bits(rng.matrix("upm1_f32", 8302, b.shape))
+    fourb = config(M, N, K, ta, tb, (2, 2), ab=BFloat16, block=block)
+    assert "_w2x2_" in gk.kernel_name(fourb, Kernel.matmul_pipelined)
+    db = helpers.run_gpu(fourb, ab, bb, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(db, helpers.run_oracle(fourb, ab, bb, c, (M, N))) <= TOL
+    d8b = helpers.run_gpu(config(M, N, K, ta, tb, eight, ab=BFloat16, block=block), ab, bb, c, (M, N), kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(db, d8b.astype(np.float64)) <= 1e-6
