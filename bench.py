@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0
 HEADLINE_SETTLE_SECONDS = 0.4
 # HBM bytes per launch of the headline kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # summarised in profiles/ (None until measured)
-MEASURED_TRAFFIC_BYTES = 338_074_624   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131153.1 * 2.0 + 67844.8) KiB
+MEASURED_TRAFFIC_BYTES = 336_073_933   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131330.6 * 2.0 + 65536.0) KiB
 TRAFFIC_SOURCE = "profiles/mfma_gemm_config2_hbm_traffic.txt (a constant from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE passes, not a reading of this run)"
 
 
@@ -40,9 +40,10 @@ def parse_args():
     p.add_argument("--steps", type=int, default=1000)
     p.add_argument("--warmup", type=int, default=2000)
     p.add_argument("--no-extras", action="store_true", help="skip the secondary configs and the CPU baseline")
-    p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4a-planar", "4b", "5", "skinny", "mul4000"],
+    p.add_argument("--workload", default="2", choices=["1", "2", "3", "4a", "4a-planar", "4b", "4b-rotating", "5", "skinny", "mul4000", "size"],
                    help="benchmark config to time as the step (default: 2, the headline; the others are for profiling one "
                         "kernel at a time and imply --no-extras)")
+    p.add_argument("--dims", default="3072,3072,3072", help="M,N,K of --workload size: mul!(C, A, B, 1, 1) as in the sizes sweep")
     p.add_argument("--variant", default="NN", choices=["NN", "NT", "TN", "TT"], help="transposes of config 2")
     p.add_argument("--copy-calibration", action="store_true",
                    help="instead of the benchmark, run a plain 256 MiB device-to-device copy 10 times: the reference "
@@ -200,11 +201,41 @@ def main():
         print(json.dumps({"copy_calibration": {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 10}}))
         return
 
+    if args.workload == "size":
+        # one size of the sweep below as the step, for profiling its kernel: mul!(C, A, B, 1, 1), default tile choice
+        from gemmkernels.matmul import matmatmul_plan
+        m, n, k = (int(x) for x in args.dims.split(","))
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(m * 31 + n * 17 + k)
+        a_ = (torch.rand(k, m, device="cuda", generator=gen) * 2 - 1).to(torch.float16).t()
+        b_ = (torch.rand(n, k, device="cuda", generator=gen) * 2 - 1).to(torch.float16).t()
+        c_ = (torch.rand(n, m, device="cuda", generator=gen) * 2 - 1).t()
+        plan = matmatmul_plan(c_, "N", "N", a_, b_, 1.0, 1.0)
+        us, _ = time_launches(plan, args.steps, args.warmup, HEADLINE_SETTLE_SECONDS)
+        tf = 2.0 * m * n * k / us / 1e6
+        print(json.dumps({
+            "metric": "TFLOP/s", "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(us / 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f16 multiplicands, f32 accumulate", "data": "synthetic (torch.rand on the device, seeded)",
+            "config": {"workload": f"mul!(C, A, B, 1, 1), {m} x {n} x {k}, FP16 A/B, FP32 C read and written", "kernels": sorted(set(plan.kernel_names))},
+            "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_FP16_TFLOPS, 4),
+                         "traffic": None, "avg_launch_us": round(us, 2), "flop_per_launch": 2 * m * n * k}}))
+        return
+
     if args.workload != "2" or args.variant != "NN":
         # one of the other workloads as the step: same JSON shape, for profiling a single kernel
-        key = int(args.workload) if args.workload.isdigit() else args.workload
+        rotating = args.workload == "4b-rotating"
+        key = "4b" if rotating else (int(args.workload) if args.workload.isdigit() else args.workload)
         wl = configs.benchmark_config(key, variant=args.variant if key == 2 else None)
         run = wl.prepare()
+        if rotating:
+            # four buffer sets (384 MiB, more than the last-level cache) in rotation: no launch finds its operands cached
+            runs = [run] + [wl.prepare() for _ in range(3)]
+            turn = {"i": 0}
+
+            def run():
+                runs[turn["i"] & 3]()
+                turn["i"] += 1
         us, _ = time_launches(run, args.steps, args.warmup, HEADLINE_SETTLE_SECONDS)
         hbm = wl.bound == "hbm"
         achieved = wl.bytes / us / 1e3 if hbm else wl.flops / us / 1e6
@@ -213,7 +244,7 @@ def main():
             "metric": "GB/s" if hbm else "TFLOP/s", "value": round(achieved, 2), "unit": "GB/s" if hbm else "TFLOP/s", "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6), "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "f16 multiplicands, f32 accumulate" if key != 1 else "f32", "data": "synthetic (counter-based splitmix64 streams)",
-            "config": {"workload": wl.description, "kernel": wl.kernel_name},
+            "config": {"workload": wl.description + (", four buffer sets in rotation" if rotating else ""), "kernel": wl.kernel_name},
             "roofline": {"bound": "hbm" if hbm else "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s",
                          "frac": round(achieved / peak, 4), "traffic": None, "kernel": wl.kernel_name, "avg_launch_us": round(us, 2),
                          "bytes_per_launch": wl.bytes, "flop_per_launch": wl.flops}}))
