@@ -434,7 +434,7 @@ gk::FamilyFn family_fn(const gk::InstanceKey& key) {
     case gk::FAMILY_MFMA:
       if (wide_tile(key) && key.waves_m == 2 && key.waves_n == 2) {
         // the tiles with a side of 192 on four waves are compiled in translation units of their own
-        if (key.a_kmajor) return key.b_kmajor ? gk::family_mfma_wide_tn : gk::family_mfma_wide_tt;
+        if (key.a_kmajor) return key.b_kmajor ? (key.BM == 256 ? gk::family_mfma_wide_tn : gk::family_mfma_wide_tn_192x256) : gk::family_mfma_wide_tt;
         return key.b_kmajor ? gk::family_mfma_wide_nn : gk::family_mfma_wide_nt;
       }
       [[fallthrough]];

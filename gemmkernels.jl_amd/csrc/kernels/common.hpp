@@ -394,12 +394,19 @@ __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "
 
 // Which of the C / D paths of a one-wave-per-SIMD instance (MfmaGemmConfig::SOLO) a launch takes (16-byte accesses where the pointers and the leading
 // dimensions allow them).
-// (path 4: C on its way during the first K tiles, for products of at least kSoloStreamTiles K tiles; `stream_ok`: the instance has that path)
+// (path 4: C on its way during the first K tiles, for products of at least kSoloStreamTiles K tiles; `stream_ok`: the instance has that path;
+// path 5: C spread over more K tiles, kSoloSpreadBlocks of the wave tile's `blocks` accumulator blocks per K tile, for products of
+// at least `spread_tiles` = solo_spread_tiles(blocks) K tiles; 0: the instance has no such path)
 constexpr int kSoloStreamTiles = 11;
-inline int solo_cd_path(const GemmArgs& args, bool stream_ok = false, int block_k = 64) {
+constexpr int kSoloSpreadBlocks = 2;
+constexpr int solo_spread_tiles(int blocks) { return blocks / kSoloSpreadBlocks + 3; }
+inline int solo_cd_path(const GemmArgs& args, bool stream_ok = false, int block_k = 64, int spread_tiles = 0) {
   const bool d_wide = args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0;
   const bool c_wide = args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0;
-  if (d_wide && args.c_mode != 0 && c_wide) return (stream_ok && args.K / block_k >= kSoloStreamTiles) ? 4 : 1;
+  if (d_wide && args.c_mode != 0 && c_wide) {
+    if (stream_ok && spread_tiles > 0 && args.K / block_k >= spread_tiles) return 5;
+    return (stream_ok && args.K / block_k >= kSoloStreamTiles) ? 4 : 1;
+  }
   if (d_wide && args.c_mode == 0) return 2;
   return 0;
 }

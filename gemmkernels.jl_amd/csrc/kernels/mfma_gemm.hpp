@@ -515,6 +515,8 @@ struct MfmaGemmConfig {
 // 4: as 1 for products of at least kSoloStreamTiles K tiles, with C on its way while the matrix cores run: the accumulators start
 // at zero, the C tile arrives one block column per K tile in registers of its own during the first K tiles and is added to the
 // accumulators there (so the sum is (products of the first K tiles) + C + (the rest), where path 1 starts from C);
+// 5: as 4 with C spread thinner, kSoloSpreadBlocks blocks per K tile, for products with that many K tiles (solo_spread_tiles):
+// the loads of C share the path of the tile DMA, which has little to spare per K tile (4096^3: 105.5 us on path 4, 102.8 on 5);
 // 0: anything else.  One kernel per path, chosen by the host
 // (solo_cd_path): where the paths met in one kernel, the register allocator gave the accumulators different registers
 // on each and shuffled 250 of them in front of the K loop.
@@ -532,7 +534,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr bool RAGGED = Cfg::RAGGED_OK || (Cfg::SOLO && CPATH == 3);
   constexpr bool RAGGED_K = Cfg::RAGGED_K_OK || (Cfg::SOLO && CPATH == 3);
   static_assert(CPATH != 3 || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "path 3 is compiled for plain real products");
-  static_assert(CPATH != 4 || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "path 4 is compiled for plain real products");
+  constexpr bool STREAM_C = CPATH == 4 || CPATH == 5;
+  static_assert(!STREAM_C || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "paths 4 and 5 are compiled for plain real products");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -871,7 +874,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   };
   if constexpr (Cfg::SOLO) {
     static_assert(!Cfg::GETT || CPATH != 0, "contractions run the four waves with 16-byte C / D accesses only");
-    if (load_c && CPATH != 4) solo_origins(solo_row, solo_col);
+    if (load_c && !STREAM_C) solo_origins(solo_row, solo_col);
     if constexpr (CPATH == 3) {
       // FP32 C with 16-byte accesses (at any 4-byte alignment), tiles over the edge included: rows and columns outside are
       // read from the last ones inside, and what is accumulated on them is never stored
@@ -918,7 +921,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       for (int fj = 0; fj < FN; ++fj)
 #pragma unroll
         for (int fi = 0; fi < FM; ++fi) asm volatile("" : "+a"(acc[fi][fj]));
-    } else if constexpr (CPATH == 4) {
+    } else if constexpr (STREAM_C) {
       // (the accumulators start from zero in the first k-step and C comes in during the first K tiles, see the K loop)
     } else if constexpr (CPATH == 2) {
       // (no C: zeroed in place, in the accumulation registers)
@@ -1303,15 +1306,20 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // (a block whose turn would reach the end of the k-step takes the first slots instead, before its MFMA and a dozen slots
     // after the one of the k-step before): the matrix core has long delivered the block and does not need it again for fifty
     // slots.  So the sum is (products of the first K tiles) + C + (the rest), where the other paths start from C.
-    constexpr int CGROUPS = CPATH == 4 ? FN : 0;
-    static_assert(CGROUPS + 3 <= kSoloStreamTiles, "the K tiles that bring C in are written out in front of the loop, the last two behind it");
-    static_assert(CPATH != 4 || KS >= 2, "the loads of C go into the first k-step of a tile, the additions into the last");
-    [[maybe_unused]] float4v cland[CPATH == 4 ? 2 : 1][CPATH == 4 ? FM : 1];
+    // (a group: CBLK consecutive blocks of a block column, FM of them on path 4; group G holds blocks G * CBLK ... of the
+    // wave tile in the order of their registers, block b = fj * FM + fi)
+    constexpr int CBLK = CPATH == 4 ? FM : kSoloSpreadBlocks;
+    constexpr int CGROUPS = STREAM_C ? NM / CBLK : 0;
+    static_assert(FM % CBLK == 0, "a group of C lies in one block column");
+    static_assert(CPATH != 4 || CGROUPS + 3 <= kSoloStreamTiles, "the K tiles that bring C in are written out in front of the loop, the last two behind it");
+    static_assert(CPATH != 5 || CGROUPS + 3 == solo_spread_tiles(NM), "the host sends products with enough K tiles");
+    static_assert(!STREAM_C || KS >= 2, "the loads of C go into the first k-step of a tile, the additions into the last");
+    [[maybe_unused]] float4v cland[STREAM_C ? 2 : 1][STREAM_C ? CBLK : 1];
     [[maybe_unused]] float ctmp[4][4];                 // values on their way from an accumulation register and back (see c_add_step)
     [[maybe_unused]] unsigned c_voff = 0;              // byte offset of the lane's four rows of block (0, 0) from the wave tile's origin in C
     [[maybe_unused]] const char* c_tile = nullptr;     // the wave tile's origin in C (the same in every lane)
     [[maybe_unused]] long long c_col16 = 0;            // bytes from a block column to the next
-    if constexpr (CPATH == 4) {
+    if constexpr (STREAM_C) {
       c_voff = (unsigned)((4 * (lane / MI) + (long long)(lane % MI) * args.ldc) * 4);
       c_tile = (const char*)args.c + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldc) * 4;
       c_col16 = (long long)args.ldc * (MI * 4);
@@ -1320,10 +1328,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // the load of block (J, G)
     [[maybe_unused]] auto c_load = [&](auto g_c, auto j_c) __attribute__((always_inline)) {
       constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value;
-      const char* base = c_tile + c_col16 * G;
+      constexpr int B = G * CBLK + J, FI = B % FM, FJ = B / FM;
+      const char* base = c_tile + c_col16 * FJ;
       float4v& dst = cland[G & 1][J];         // (named here: an operand of an assembly statement does not capture by itself)
       const unsigned vo = c_voff;
-      asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(vo), "s"(base), "n"(J * MI * 4) : "memory");
+      asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(vo), "s"(base), "n"(FI * MI * 4) : "memory");
     };
     // Step Q (0 .. 5) of the addition of block (J, G): two accumulation registers read, two values added, two registers
     // written back
@@ -1331,7 +1340,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // never do, a block that takes the first slots of the k-step may meet any of the first rows and has sets of its own)
     [[maybe_unused]] auto c_add_step = [&](auto g_c, auto j_c, auto q_c, auto t_c) __attribute__((always_inline)) {
       constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value, Q = decltype(q_c)::value, T = decltype(t_c)::value;
-      constexpr int R = 4 * (G * FM + J), E = 2 * (Q & 1);
+      constexpr int R = 4 * (G * CBLK + J), E = 2 * (Q & 1);
       float4v& src = cland[G & 1][J];
       float& t0 = ctmp[T][E];
       float& t1 = ctmp[T][E + 1];
@@ -1375,7 +1384,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         constexpr int o_ = B_BOTH ? i / FM : i / FN, q_ = B_BOTH ? ((o_ & 1) ? FM - 1 - (i % FM) : i % FM) : ((o_ & 1) ? FN - 1 - (i % FN) : i % FN);
         constexpr int fi = B_BOTH ? q_ : o_, fj = B_BOTH ? o_ : q_;
         if constexpr (B_BOTH && (i % FM) == 0) vb[fj] = RB::finish(fb[PAR][fj % RB::NREAD], lane, fj >= RB::NREAD);
-        if constexpr (CPATH == 4) Mfma<T, MI>::template run_fixed<4 * (fj * FM + fi), FIRST>(va[fi], vb[fj]);
+        if constexpr (STREAM_C) Mfma<T, MI>::template run_fixed<4 * (fj * FM + fi), FIRST>(va[fi], vb[fj]);
         else acc[fi][fj] = Mfma<T, MI>::run(va[fi], vb[fj], acc[fi][fj]);
         // (the scheduling barriers keep every instruction in the slot it is written in)
         if constexpr (DMA && i % GD == 0 && i / GD < DPT) {
@@ -1388,26 +1397,27 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           read_op(std::integral_constant<int, i / RSP>{}, std::integral_constant<int, NKS>{}, std::integral_constant<int, (PAR ^ 1)>{});
           __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr (CPATH == 4 && !B_BOTH) {
+        if constexpr (STREAM_C && !B_BOTH) {
           constexpr int LSLOT0 = NOPS * RSP + 2;                   // (behind the fragment reads)
-          constexpr int LSTEP = (LSLOT0 + 4 * (FM - 1) < NM) ? 4 : (LSLOT0 + 3 * (FM - 1) < NM) ? 3 : 2;
-          static_assert(LG < 0 || LSLOT0 + LSTEP * (FM - 1) < NM, "the loads of a group of C fit the k-step");
-          if constexpr (LG >= 0 && i >= LSLOT0 && (i - LSLOT0) % LSTEP == 0 && (i - LSLOT0) / LSTEP < FM) {
+          constexpr int LSTEP = (LSLOT0 + 4 * (CBLK - 1) < NM) ? 4 : (LSLOT0 + 3 * (CBLK - 1) < NM) ? 3 : 2;
+          static_assert(LG < 0 || LSLOT0 + LSTEP * (CBLK - 1) < NM, "the loads of a group of C fit the k-step");
+          if constexpr (LG >= 0 && i >= LSLOT0 && (i - LSLOT0) % LSTEP == 0 && (i - LSLOT0) / LSTEP < CBLK) {
             __builtin_amdgcn_sched_barrier(0);
             c_load(lg_c, std::integral_constant<int, (i - LSLOT0) / LSTEP>{});
             __builtin_amdgcn_sched_barrier(0);
           }
           if constexpr (AG >= 0) {
-            static_for<0, FM * 6>([&](auto u_c) {
+            static_for<0, CBLK * 6>([&](auto u_c) {
               constexpr int u = decltype(u_c)::value, j = u / 6, q = u % 6;
-              constexpr int p = j * FN + ((j & 1) ? FN - 1 - AG : AG);       // the MFMA of block (j, AG) in this k-step
+              constexpr int b = AG * CBLK + j, bi = b % FM, bj = b / FM;
+              constexpr int p = bi * FN + ((bi & 1) ? FN - 1 - bj : bj);     // the MFMA of block (bi, bj) in this k-step
               constexpr bool early = !(p + 9 < NM);
               constexpr int s0 = early ? p + 4 - NM + 8 : p + 4;
               // (the two halves of a step trade places so that a value is read, added and written two slots apart)
               constexpr int at = s0 + (q / 2) * 2 + (q & 1);
               if constexpr (at == i) {
                 __builtin_amdgcn_sched_barrier(0);
-                c_add_step(ag_c, std::integral_constant<int, j>{}, std::integral_constant<int, q>{}, std::integral_constant<int, (j & 1) + (early ? 2 : 0)>{});
+                c_add_step(ag_c, std::integral_constant<int, j>{}, std::integral_constant<int, q>{}, std::integral_constant<int, (bi & 1) + (early ? 2 : 0)>{});
                 __builtin_amdgcn_sched_barrier(0);
               }
             });
@@ -1470,7 +1480,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         }
       });
     };
-    if constexpr (CPATH == 4) {
+    if constexpr (STREAM_C) {
       // the first K tiles, written out: tile t fetches group t of C and adds group t - 1 (the host sends products of at
       // least kSoloStreamTiles K tiles here) ...
       typedef std::integral_constant<int, 0> Pend0;
@@ -1478,7 +1488,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         constexpr int t = decltype(t_c)::value;
         constexpr int LGT = t < CGROUPS ? t : -1;
         tile_body(t, std::integral_constant<int, LGT>{}, std::integral_constant<int, t - 1>{}, std::integral_constant<bool, t == 0>{}, Yes{}, No{},
-                  std::integral_constant<int, (LGT >= 0 ? FM : 0)>{});
+                  std::integral_constant<int, (LGT >= 0 ? CBLK : 0)>{});
       });
       for (int kt = CGROUPS + 1; kt < KT - 2; ++kt) tile_body(kt, NoGroup{}, NoGroup{}, No{}, Yes{}, No{}, Pend0{});
       // ... and the last two, which have nothing left to fetch
@@ -1494,7 +1504,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     wait_lgkmcnt<0>();   // of fragments)
     // (path 4 issues its MFMAs from assembly statements, which the compiler does not see: the results of the last ones must
     // have left the matrix core before anything else reads their registers)
-    if constexpr (CPATH == 4) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    if constexpr (STREAM_C) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     if constexpr (RAGGED_K) {
       // the last, partial K tile, outside the schedule of the loop: the k-steps that hold valid values
       if (tail_k > 0) {
@@ -1942,7 +1952,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             }
           }
         }
-    } else if constexpr (CPATH == 4) {
+    } else if constexpr (STREAM_C) {
       // from the accumulation registers the kernel manages itself: the wave tile's origin in D from scalar registers, the
       // lane's offset in it from a vector register, the row block as an immediate.  The stores write through to memory
       // (sc0 sc1): D is not read again by this launch, and what stays dirty in the L2s has to be written back after the

@@ -2,5 +2,6 @@
 #define GK_A_KMAJOR false
 #define GK_B_KMAJOR true
 #define GK_FAMILY_FN family_mfma_nn
+#define GK_STREAM_FN family_mfma_stream_nn
 #define GK_TAG "nn"
 #include "mfma_instances.inc"

@@ -2,5 +2,6 @@
 #define GK_A_KMAJOR false
 #define GK_B_KMAJOR false
 #define GK_FAMILY_FN family_mfma_nt
+#define GK_STREAM_FN family_mfma_stream_nt
 #define GK_TAG "nt"
 #include "mfma_instances.inc"

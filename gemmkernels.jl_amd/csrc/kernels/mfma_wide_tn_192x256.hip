@@ -1,0 +1,7 @@
+// Four-wave instances of the 192 x 256 x 64 tile for the 'TN' transpose pair (A K-major, B K-major in memory).
+#define GK_A_KMAJOR true
+#define GK_B_KMAJOR true
+#define GK_WIDE_SECOND
+#define GK_FAMILY_FN family_mfma_wide_tn_192x256
+#define GK_TAG "tn"
+#include "mfma_wide_instances.inc"

@@ -66,9 +66,15 @@ int family_mfma_nn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, 
 int family_mfma_nt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_tt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_wide_tn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+int family_mfma_wide_tn_192x256(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_wide_nn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_wide_nt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_mfma_wide_tt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
+// (the instances that stream C in: called by the family functions above with the path they chose)
+int family_mfma_stream_tn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*, int path);
+int family_mfma_stream_nn(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*, int path);
+int family_mfma_stream_nt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*, int path);
+int family_mfma_stream_tt(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*, int path);
 int family_fpu(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_fpu_types(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);
 int family_fpu_lanes(const InstanceKey&, const GemmArgs&, dim3, hipStream_t, int, InstanceInfo*, hipError_t*);

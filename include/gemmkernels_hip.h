@@ -307,7 +307,7 @@ int gk_matmul_split_k_noalloc(const gk_config* conf, const void* a, const void* 
  * gk_rtc_compile closes that gap for the real MFMA operator with aligned layouts: hooks[h] is NULL
  * (identity) or a C expression in the fp32 variable x, e.g. "x > 0.0f ? x : 0.01f * x", for hook h
  * in the order of gk_hook; block_shape / compute_warp may be any tile the kernel template accepts
- * (32x32 accumulator blocks, BLOCK_K of 32, 64 or 128, at most 160 KiB of LDS).  Expressions are
+ * (32x32 accumulator blocks, BLOCK_K of 16, 32, 64 or 128, at most 160 KiB of LDS).  Expressions are
  * evaluated in fp32 without contraction and the result is rounded to the hook's destination type,
  * like the op lists of gk_matmul.  Compiled kernels are cached by configuration, expressions and
  * device and live until the process ends.  gk_rtc_matmul runs the same checks as gk_matmul. */

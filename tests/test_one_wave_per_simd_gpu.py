@@ -1,8 +1,17 @@
-"""The 256 x 256 x 64 tile on four waves (one per SIMD, 128 x 128 wave tiles) against the same tile on eight waves
-and against the CPU oracle.  The two arrangements run the k-steps and the products inside them in the same order,
-so FP32 results are compared bit for bit; the oracle with the tolerance of the other MFMA tests (relative
-Frobenius error <= 1e-3).  Launches the four-wave arrangement is not compiled for (hooks on A, B or C, more than
-one op in a hook of D, extents the edge instances do not take) run the eight-wave arrangement of the same configuration."""
+"""The tiles that run on four waves (one per SIMD: 256 x 256 x 64 with 128 x 128 wave tiles, the tiles with a side of 192
+with 128 x 96 / 96 x 128) against the CPU oracle and the float64 product, which are the gate (relative Frobenius error
+<= 1e-3 like the other MFMA tests; <= 1e-6 against float64 where the test says so).
+
+Comparisons with the eight-wave arrangement of the same tile come on top of that and say two different things.  Where the
+summation order is the same by construction -- C loaded before the K loop or absent, tiles over the edges, the fused,
+complex and contraction kernels: the k-steps and the products inside them run in the same order however a tile is dealt
+out to waves -- the two must agree bit for bit, which catches a wrong register, lane or address that a norm would let
+pass.  Where C is added during the first K tiles (plain products of at least eleven K tiles with FP32 C / D) the place of
+that one addition differs, so the two agree to rounding only; there the tests pin what the order cannot change: linearity
+in C, D(C) - D(0) = C, and sums of small integers, which are exact in any order.
+
+Launches the four waves are not compiled for (hooks on A, B or C, more than one op in a hook of D, extents the edge
+instances do not take) run the eight-wave arrangement of the same configuration."""
 import numpy as np
 import pytest
 
@@ -293,9 +302,11 @@ def test_default_configuration_of_a_large_product(gpu):
 # are compared with the oracle and with float64 by norm, and exactly on data whose partial sums are all exact in FP32.
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("K", [704, 768, 1344])
+@pytest.mark.parametrize("K", [704, 768, 1344, 2240, 2304, 2880])
 def test_c_streamed_during_the_first_k_tiles(gpu, ta, tb, K):
-    """Eleven K tiles (the fewest that take this route: nine that bring C in, none in between, the two last), twelve, twenty-one."""
+    """Eleven K tiles (the fewest that take this route: nine that bring C in, none in between, the two last), twelve, twenty-one;
+    from thirty-five K tiles on C comes in two blocks per K tile (thirty-three tiles that bring it in, the two last): the fewest,
+    one more, forty-five."""
     M, N = 512, 768
     a, b, c = operands(M, N, K, ta, tb, 7600 + K)
     conf = config(M, N, K, ta, tb, (2, 2))
@@ -360,12 +371,12 @@ WIDE = [((256, 192, 64), (4, 2), [(False, False), (True, False), (False, True)])
 @pytest.mark.parametrize("block,eight,transposes", WIDE)
 def test_tiles_with_a_side_of_192_on_four_waves(gpu, block, eight, transposes):
     """C added at the end (fewer than eleven K tiles) and no C: the same bits as the eight waves.  C on its way during
-    the first K tiles (from eleven K tiles on: 704 is the fewest, 1344 has generic tiles in between): the oracle,
-    linearity in C, exact sums of small integers."""
+    the first K tiles (from eleven K tiles on: 704 is the fewest, 1344 has generic tiles in between; from 27 on, 1728, in
+    thinner slices): the oracle, linearity in C, exact sums of small integers."""
     BM, BN, _ = block
     M, N = 2 * BM, 3 * BN
     for ta, tb in transposes:
-        for K in (64, 192, 448, 704, 768, 1344):
+        for K in (64, 192, 448, 704, 768, 1344, 1728, 1792, 2368):       # (from 27 K tiles on: C two blocks per K tile)
             a, b, c = operands(M, N, K, ta, tb, 7900 + K)
             four, eight8 = config(M, N, K, ta, tb, (2, 2), block=block), config(M, N, K, ta, tb, eight, block=block)
             name = gk.kernel_name(four, Kernel.matmul_pipelined)
