@@ -411,7 +411,7 @@ def main():
         try:
             from gemmkernels.matmul import matmatmul_plan
             sizes = {}
-            for (m, n, k) in [(1024, 1024, 1024), (2048, 2048, 2048), (3072, 3072, 3072), (4096, 4096, 4096), (6144, 6144, 6144),
+            for (m, n, k) in [(128, 128, 128), (256, 256, 256), (512, 512, 512), (1024, 1024, 1024), (2048, 2048, 2048), (3072, 3072, 3072), (4096, 4096, 4096), (6144, 6144, 6144),
                               (8192, 8192, 8192), (4096, 4096, 16384), (8192, 8192, 4096), (16384, 16384, 4096)]:
                 gen = torch.Generator(device="cuda")
                 gen.manual_seed(m * 31 + n * 17 + k)

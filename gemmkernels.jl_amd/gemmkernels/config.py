@@ -198,28 +198,49 @@ def default_block_shape(operator, gemm_shape, tile_sized: bool = True, gett: boo
         fitting = [t for t in fitting if t in _GETT_TILES]
     if not fitting:
         return NT(M=64, N=64, K=32)
-    # time of the launch in units of "one CU multiplying at the rate of the 256 x 256 x 64 tile": every CU
-    # works through ceil(tiles / 256) tiles one after the other, a tile costs its area over the measured
-    # relative rate of its kernel (ties go to the tile listed first)
+    # time of the launch in units of "one CU multiplying at the rate of the 256 x 256 x 64 tile": a tile costs its area
+    # over the rate of its kernel when it has a CU to itself (_MFMA_TILE_RATE), and a CU works through its share of the
+    # tiles in rounds (_rounds: whole rounds for the tiles of which a CU holds one at a time, overlapping ones for the
+    # smaller tiles).  Ties go to the tile listed first.
     def cost(t):
         tiles = -(-M // t[0]) * -(-N // t[1])
-        rounds = -(-tiles // NUM_CUS)
-        rate = _MFMA_TILE_RATE.get(t, 0.5)
-        if t == (256, 192, 64) and not a_kmajor and not b_kmajor and (M % t[0] or N % t[1] or K % t[2]):
-            rate = 0.78      # 'N','T' on eight waves (tiles over the edges): the 192 side is read with transposing LDS reads
+        per_cu = tiles / NUM_CUS
+        rate = _MFMA_TILE_RATE.get(t, 0.3)
         if isinstance(rate, tuple):
-            rate = rate[0] if rounds == 1 else rate[1]
-        return rounds * t[0] * t[1] / rate
+            rate = rate[0] if per_cu <= 1 else rate[1]
+        if t == (256, 192, 64) and not a_kmajor and not b_kmajor and (M % t[0] or N % t[1] or K % t[2]):
+            rate = 0.70      # 'N','T' on eight waves (tiles over the edges): the 192 side is read with transposing LDS reads
+        if t == (64, 64, 32) and per_cu <= 1 and K >= 2048:
+            rate = 0.24      # a lone workgroup on a long K: four stages in flight instead of two (1024 x 1024 x 4096: 23.4 us, 64 x 64 x 64: 34.1)
+        return _rounds(t, tiles) * t[0] * t[1] / rate
     best = min(fitting, key=lambda t: (cost(t), fitting.index(t)))
     return NT(M=best[0], N=best[1], K=best[2])
 
 
-# throughput of a CU running each tile, relative to 256 x 256 x 64; a pair: with at most one tile per CU, with
-# several in a row.  From timings of every tile at 1000^3 ... 6000^3 (4096 x 4096 x 2048 and 4032^3 for the
-# 64-wide ones): e.g. 6000^3 takes 436 us on 256 x 256 x 64, 562 us on 128 x 128 x 64, 617 us on 128 x 128 x 32.
-_MFMA_TILE_RATE = {(256, 256, 64): 1.0, (256, 256, 32): 0.95, (256, 128, 64): 0.81, (128, 256, 64): 0.82,
-                   (128, 128, 32): (0.66, 0.60), (128, 128, 64): (0.60, 0.65), (64, 64, 64): 0.47, (64, 64, 32): 0.42,
-                   (256, 192, 64): 0.90, (192, 256, 64): 0.90}
+# Throughput of a CU that has one tile at a time, relative to 256 x 256 x 64 on four waves; a pair: a launch with at most
+# one tile per CU, a launch with several (the small tiles are bound by latency when alone).  From timings of every tile
+# and panel height at 1024^3 ... 6144^3 and eight rectangular problems ('N','N', three interleaved passes each):
+# e.g. 4096^3 takes 99 us on 256 x 256 x 64, 131 on 128 x 128 x 64, 134 on 128 x 256 x 64, 194 on 64 x 64 x 64;
+# 2560^3 42.2 us on 128 x 128 x 64 (400 tiles), 45.5 on 128 x 256 x 64 (200), 53.1 on 256 x 256 x 64 (100).
+_MFMA_TILE_RATE = {(256, 256, 64): 1.0, (256, 256, 32): 0.68, (256, 128, 64): (0.61, 0.70), (128, 256, 64): (0.62, 0.72),
+                   (128, 128, 32): (0.415, 0.345), (128, 128, 64): 0.39, (64, 64, 64): 0.169, (64, 64, 32): (0.163, 0.13),
+                   (256, 192, 64): 0.86, (192, 256, 64): 0.86}
+
+
+def _rounds(t, tiles):
+    """How many tile times a launch of ``tiles`` tiles of shape ``t`` takes.  A CU holds one workgroup of the tiles with
+    144 or 128 KiB of LDS at a time: whole rounds.  Of the 128 x 128 tiles it holds two, which run side by side in 1.15
+    times the time of one (2560^3, 400 tiles: 1.17; 4096^3, 1024 tiles: 2.27 = two such rounds); of the 64 x 64 tiles
+    four and more, whose time grows by about a third of a tile time per further tile of a CU (1536^3, 2.25 per CU: 1.43;
+    3072^3, 9 per CU: 3.8)."""
+    per_cu = tiles / NUM_CUS
+    if t[0] * t[1] >= 128 * 256:
+        return -(-tiles // NUM_CUS)
+    if per_cu <= 1:
+        return 1.0
+    if t[0] * t[1] >= 128 * 128:
+        return 1.15 * -(-tiles // (2 * NUM_CUS))
+    return 1.0 + 0.36 * (per_cu - 1.0)
 
 
 # complex / dual tiles (complex elements) -> waves: one real product of the real views of A and B, whose real tile
@@ -374,10 +395,10 @@ def get_config(*, gemm_shape, operator, global_a_layout, global_c_layout, **para
     mem_cd_thread = NT(params.get("mem_cd_thread", adjacent_elements(n_c, mn, is_cd_col_major)))
 
     # src/config.jl:277-279 defaults to Identity; on the MI355X the XCD-aware walk is the default
-    # (panels 4 tiles high; 8 once the tile grid has a thousand tiles: 8192^3 runs 10 % faster with it; 16 from four
-    # thousand tiles on: 16384 x 16384 x 4096 1771 us against 1789 and 1871 us with 8 and 4)
+    # (panels 4 tiles high; 8 once every CU has a tile: 4096^3 is 0.2 - 1.0 us faster with it in every transpose, 8192^3
+    # 10 %; 16 from four thousand tiles on: 16384 x 16384 x 4096 1771 us against 1789 and 1871 us with 8 and 4)
     n_tiles = -(-gemm_shape.M // block_shape.M) * -(-gemm_shape.N // block_shape.N)
-    cta_swizzle = params.get("cta_swizzle", CTASwizzle.XCDAware[16 if n_tiles >= 4096 else (8 if n_tiles >= 1024 else 4)])
+    cta_swizzle = params.get("cta_swizzle", CTASwizzle.XCDAware[16 if n_tiles >= 4096 else (8 if n_tiles >= NUM_CUS else 4)])
 
     conf = Config(gemm_shape, block_shape, warps_per_block, mem_a_warp, mem_a_thread, mem_b_warp, mem_b_thread,
                   mem_cd_warp, mem_cd_thread, compute_warp, op_shape,

@@ -33,8 +33,9 @@ MFMA_CANDIDATES = [
     ((128, 128, 64), (2, 2)), ((128, 128, 64), (4, 2)), ((128, 128, 32), (2, 2)),
     ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((64, 64, 32), (1, 1)),
     ((256, 192, 64), (4, 2)), ((192, 256, 64), (2, 4)),     # compiled for the transposes whose 192 side is contiguous along k; skipped elsewhere
+    ((256, 192, 64), (2, 2)), ((192, 256, 64), (2, 2)),     # ... and on one wave per SIMD (plain products in whole tiles)
 ]
-SWIZZLE_PANELS = (1, 2, 4, 8)
+SWIZZLE_PANELS = (1, 2, 4, 8, 16)
 
 
 def mfma_config(M, N, K, ta, tb, block, waves, panel, zero_c=False, ab=Float16, cd=Float32):

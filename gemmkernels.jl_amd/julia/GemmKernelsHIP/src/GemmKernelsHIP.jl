@@ -338,9 +338,20 @@ end
 # block shape -> waves (M x N) of the instances compiled into the library
 const MFMA_TILES = [((256, 256, 64), (2, 4)), ((256, 256, 32), (2, 4)), ((256, 128, 64), (2, 2)), ((128, 256, 64), (2, 2)),
                     ((128, 128, 32), (2, 2)), ((128, 128, 64), (2, 2)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2))]
-# relative throughput of a CU running each tile (256 x 256 x 64 = 1), measured
-const MFMA_TILE_RATE = Dict((256, 256, 64) => 1.0, (256, 256, 32) => 0.95, (256, 128, 64) => 0.81, (128, 256, 64) => 0.82,
-                            (128, 128, 32) => 0.63, (128, 128, 64) => 0.62, (64, 64, 64) => 0.47, (64, 64, 32) => 0.42)
+# throughput of a CU that has one tile at a time, relative to 256 x 256 x 64 on four waves, measured; a pair: a launch with
+# at most one tile per CU, a launch with several (the small tiles are bound by latency when alone)
+const MFMA_TILE_RATE = Dict((256, 256, 64) => (1.0, 1.0), (256, 256, 32) => (0.68, 0.68), (256, 128, 64) => (0.61, 0.70),
+                            (128, 256, 64) => (0.62, 0.72), (128, 128, 32) => (0.415, 0.345), (128, 128, 64) => (0.39, 0.39),
+                            (64, 64, 64) => (0.169, 0.169), (64, 64, 32) => (0.163, 0.13))
+# tile times of a launch: whole rounds for the tiles of which a CU holds one at a time; two 128 x 128 tiles run side by side
+# in 1.15 times the time of one; the time of 64 x 64 tiles grows by about a third of a tile time per further tile of a CU
+function tile_rounds(t, tiles)
+    per_cu = tiles / NUM_CUS
+    t[1] * t[2] >= 128 * 256 && return Float64(cld(tiles, NUM_CUS))
+    per_cu <= 1 && return 1.0
+    t[1] * t[2] >= 128 * 128 && return 1.15 * cld(tiles, 2 * NUM_CUS)
+    1.0 + 0.36 * (per_cu - 1.0)
+end
 # complex / dual tiles (complex elements): one real product of the real views of A and B (interleaved or planar),
 # the same table for every transpose
 const COMPLEX_PAIR_TILES = [((128, 128, 64), (2, 4)), ((64, 64, 64), (2, 2)), ((64, 64, 32), (2, 2)), ((32, 32, 32), (2, 2))]
@@ -380,7 +391,12 @@ function default_block_shape(operator::Type, gemm_shape; tile_sized::Bool = true
     end
     fitting = [t for (t, _) in MFMA_TILES if !tile_sized || (M % t[1] == 0 && N % t[2] == 0 && K % t[3] == 0)]
     isempty(fitting) && return (M = 64, N = 64, K = 32)
-    cost(t) = cld(cld(M, t[1]) * cld(N, t[2]), NUM_CUS) * t[1] * t[2] / MFMA_TILE_RATE[t]
+    function cost(t)
+        tiles = cld(M, t[1]) * cld(N, t[2])
+        rate = MFMA_TILE_RATE[t][tiles <= NUM_CUS ? 1 : 2]
+        t == (64, 64, 32) && tiles <= NUM_CUS && K >= 2048 && (rate = 0.24)      # a lone workgroup on a long K: four stages in flight
+        tile_rounds(t, tiles) * t[1] * t[2] / rate
+    end
     best = fitting[argmin(map(cost, fitting))]
     (M = best[1], N = best[2], K = best[3])
 end
@@ -475,7 +491,7 @@ function get_config(; gemm_shape, operator, global_a_layout, global_c_layout, kw
 
     # reference src/config.jl:277-279 defaults to Identity; here the XCD-aware walk is the default
     n_tiles = cld(gemm_shape.M, block_shape.M) * cld(gemm_shape.N, block_shape.N)
-    cta_swizzle = get(params, :cta_swizzle, CTASwizzle.XCDAware{n_tiles >= 4096 ? 16 : (n_tiles >= 1024 ? 8 : 4)})
+    cta_swizzle = get(params, :cta_swizzle, CTASwizzle.XCDAware{n_tiles >= 4096 ? 16 : (n_tiles >= NUM_CUS ? 8 : 4)})
 
     conf = Config(gemm_shape, block_shape, warps_per_block, mem_a_warp, mem_a_thread, mem_b_warp, mem_b_thread,
                   mem_cd_warp, mem_cd_thread, compute_warp, op_shape,

@@ -102,7 +102,7 @@ def test_get_config_defaults_for_the_headline_problem():
     assert conf.mem_cd_warp == NT(M=256, N=1) and conf.mem_cd_thread == NT(M=4, N=1)
     assert conf.global_b_layout == conf.global_a_layout and conf.global_d_layout == conf.global_c_layout
     assert conf.shared_a_layout == Layout.Padded[ACM[F16], 8]           # src/config.jl:191-194
-    assert conf.cta_swizzle == CTASwizzle.XCDAware[4]
+    assert conf.cta_swizzle == CTASwizzle.XCDAware[8]            # (every CU has a tile: panels 8 tiles high)
     assert Kernel.shmem_size(conf, Kernel.matmul_pipelined) == 2 * (256 * 64 * 2 + 256 * 64 * 2)
     assert "block_shape:" in str(conf) and "(M = 256, N = 256, K = 64)" in str(conf)
 
