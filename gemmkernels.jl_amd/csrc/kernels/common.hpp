@@ -400,9 +400,14 @@ __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "
 constexpr int kSoloStreamTiles = 11;
 constexpr int kSoloSpreadBlocks = 2;
 constexpr int solo_spread_tiles(int blocks) { return blocks / kSoloSpreadBlocks + 3; }
-inline int solo_cd_path(const GemmArgs& args, bool stream_ok = false, int block_k = 64, int spread_tiles = 0) {
+// (path 6: 4 for an FP16 C and an FP16 D that take 8-byte accesses; `half_cd_ok`: the instance has it)
+inline int solo_cd_path(const GemmArgs& args, bool stream_ok = false, int block_k = 64, int spread_tiles = 0, bool half_cd_ok = false) {
   const bool d_wide = args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0;
   const bool c_wide = args.c_dtype == DT_F32 && ((((uintptr_t)args.c) | ((uintptr_t)args.ldc << 2)) & 15u) == 0;
+  if (half_cd_ok && stream_ok && args.c_mode != 0 && args.d_dtype == DT_F16 && args.c_dtype == DT_F16 &&
+      ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 1) | ((uintptr_t)args.c) | ((uintptr_t)args.ldc << 1)) & 7u) == 0 &&
+      args.K / block_k >= kSoloStreamTiles)
+    return 6;
   if (d_wide && args.c_mode != 0 && c_wide) {
     if (stream_ok && spread_tiles > 0 && args.K / block_k >= spread_tiles) return 5;
     return (stream_ok && args.K / block_k >= kSoloStreamTiles) ? 4 : 1;

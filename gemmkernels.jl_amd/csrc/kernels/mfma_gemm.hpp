@@ -517,6 +517,9 @@ struct MfmaGemmConfig {
 // accumulators there (so the sum is (products of the first K tiles) + C + (the rest), where path 1 starts from C);
 // 5: as 4 with C spread thinner, kSoloSpreadBlocks blocks per K tile, for products with that many K tiles (solo_spread_tiles):
 // the loads of C share the path of the tile DMA, which has little to spare per K tile (4096^3: 105.5 us on path 4, 102.8 on 5);
+// 6: as 4 for an FP16 C and an FP16 D (8 bytes per lane and block; C is widened where it is added, D rounded once where it is
+// stored; 4096^3: 107.2 us on path 0, 102.5 on 6; spread as on path 5 it took 103.7: the widening costs vector-ALU slots in
+// every K tile that adds);
 // 0: anything else.  One kernel per path, chosen by the host
 // (solo_cd_path): where the paths met in one kernel, the register allocator gave the accumulators different registers
 // on each and shuffled 250 of them in front of the K loop.
@@ -534,8 +537,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   constexpr bool RAGGED = Cfg::RAGGED_OK || (Cfg::SOLO && CPATH == 3);
   constexpr bool RAGGED_K = Cfg::RAGGED_K_OK || (Cfg::SOLO && CPATH == 3);
   static_assert(CPATH != 3 || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "path 3 is compiled for plain real products");
-  constexpr bool STREAM_C = CPATH == 4 || CPATH == 5;
-  static_assert(!STREAM_C || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "paths 4 and 5 are compiled for plain real products");
+  constexpr bool STREAM_C = CPATH >= 4 && CPATH <= 6;
+  constexpr bool HALF_CD = CPATH == 6;                      // FP16 C and D on a streamed path (8 bytes per lane and block)
+  constexpr int CDB = HALF_CD ? 2 : 4;                      // bytes per element of C and D there
+  static_assert(!STREAM_C || (!Cfg::GETT && Cfg::FIX == FIX_NONE && Cfg::FUSE == 0), "paths 4 to 6 are compiled for plain real products");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -1308,21 +1313,22 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // slots.  So the sum is (products of the first K tiles) + C + (the rest), where the other paths start from C.
     // (a group: CBLK consecutive blocks of a block column, FM of them on path 4; group G holds blocks G * CBLK ... of the
     // wave tile in the order of their registers, block b = fj * FM + fi)
-    constexpr int CBLK = CPATH == 4 ? FM : kSoloSpreadBlocks;
+    constexpr int CBLK = (CPATH == 4 || CPATH == 6) ? FM : kSoloSpreadBlocks;
     constexpr int CGROUPS = STREAM_C ? NM / CBLK : 0;
     static_assert(FM % CBLK == 0, "a group of C lies in one block column");
-    static_assert(CPATH != 4 || CGROUPS + 3 <= kSoloStreamTiles, "the K tiles that bring C in are written out in front of the loop, the last two behind it");
+    static_assert((CPATH != 4 && CPATH != 6) || CGROUPS + 3 <= kSoloStreamTiles, "the K tiles that bring C in are written out in front of the loop, the last two behind it");
     static_assert(CPATH != 5 || CGROUPS + 3 == solo_spread_tiles(NM), "the host sends products with enough K tiles");
     static_assert(!STREAM_C || KS >= 2, "the loads of C go into the first k-step of a tile, the additions into the last");
-    [[maybe_unused]] float4v cland[STREAM_C ? 2 : 1][STREAM_C ? CBLK : 1];
+    [[maybe_unused]] float4v cland[(STREAM_C && !HALF_CD) ? 2 : 1][(STREAM_C && !HALF_CD) ? CBLK : 1];
+    [[maybe_unused]] int2v cland16[HALF_CD ? 2 : 1][HALF_CD ? CBLK : 1];        // four FP16 values of C per lane and block
     [[maybe_unused]] float ctmp[4][4];                 // values on their way from an accumulation register and back (see c_add_step)
     [[maybe_unused]] unsigned c_voff = 0;              // byte offset of the lane's four rows of block (0, 0) from the wave tile's origin in C
     [[maybe_unused]] const char* c_tile = nullptr;     // the wave tile's origin in C (the same in every lane)
     [[maybe_unused]] long long c_col16 = 0;            // bytes from a block column to the next
     if constexpr (STREAM_C) {
-      c_voff = (unsigned)((4 * (lane / MI) + (long long)(lane % MI) * args.ldc) * 4);
-      c_tile = (const char*)args.c + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldc) * 4;
-      c_col16 = (long long)args.ldc * (MI * 4);
+      c_voff = (unsigned)((4 * (lane / MI) + (long long)(lane % MI) * args.ldc) * CDB);
+      c_tile = (const char*)args.c + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldc) * CDB;
+      c_col16 = (long long)args.ldc * (MI * CDB);
       asm volatile("" ::: "a255");           // (the highest one: the kernel is given all 256)
     }
     // the load of block (J, G)
@@ -1330,9 +1336,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value;
       constexpr int B = G * CBLK + J, FI = B % FM, FJ = B / FM;
       const char* base = c_tile + c_col16 * FJ;
-      float4v& dst = cland[G & 1][J];         // (named here: an operand of an assembly statement does not capture by itself)
-      const unsigned vo = c_voff;
-      asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(vo), "s"(base), "n"(FI * MI * 4) : "memory");
+      const unsigned vo = c_voff;             // (named here: an operand of an assembly statement does not capture by itself)
+      if constexpr (HALF_CD) {
+        int2v& dst = cland16[G & 1][J];
+        asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(vo), "s"(base), "n"(FI * MI * 2) : "memory");
+      } else {
+        float4v& dst = cland[G & 1][J];
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(vo), "s"(base), "n"(FI * MI * 4) : "memory");
+      }
     };
     // Step Q (0 .. 5) of the addition of block (J, G): two accumulation registers read, two values added, two registers
     // written back
@@ -1341,15 +1352,24 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     [[maybe_unused]] auto c_add_step = [&](auto g_c, auto j_c, auto q_c, auto t_c) __attribute__((always_inline)) {
       constexpr int G = decltype(g_c)::value, J = decltype(j_c)::value, Q = decltype(q_c)::value, T = decltype(t_c)::value;
       constexpr int R = 4 * (G * CBLK + J), E = 2 * (Q & 1);
-      float4v& src = cland[G & 1][J];
       float& t0 = ctmp[T][E];
       float& t1 = ctmp[T][E + 1];
-      if constexpr (Q == 0) asm volatile("" : "+v"(src));
+      if constexpr (Q == 0) {
+        if constexpr (HALF_CD) asm volatile("" : "+v"(cland16[G & 1][J]));
+        else asm volatile("" : "+v"(cland[G & 1][J]));
+      }
       if constexpr (Q < 2) {
         asm volatile("v_accvgpr_read_b32 %0, a[%2]\n\tv_accvgpr_read_b32 %1, a[%3]" : "=v"(t0), "=v"(t1) : "n"(R + E), "n"(R + E + 1));
       } else if constexpr (Q < 4) {
-        t0 = t0 + src[E];
-        t1 = t1 + src[E + 1];
+        if constexpr (HALF_CD) {
+          // (values E and E + 1 are the two halves of a register; FP16 widens exactly)
+          const unsigned w = (unsigned)cland16[G & 1][J][E / 2];
+          t0 = t0 + (float)__builtin_bit_cast(_Float16, (unsigned short)(w & 0xffffu));
+          t1 = t1 + (float)__builtin_bit_cast(_Float16, (unsigned short)(w >> 16));
+        } else {
+          t0 = t0 + cland[G & 1][J][E];
+          t1 = t1 + cland[G & 1][J][E + 1];
+        }
       } else {
         asm volatile("v_accvgpr_write_b32 a[%2], %0\n\tv_accvgpr_write_b32 a[%3], %1" :: "v"(t0), "v"(t1), "n"(R + E), "n"(R + E + 1));
       }
@@ -1958,9 +1978,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       // (sc0 sc1): D is not read again by this launch, and what stays dirty in the L2s has to be written back after the
       // last wave has ended, before the launch counts as complete (a kernel that only stores such tiles: 11.3 us from
       // launch to launch with plain stores, 10.1 us with these; the GEMM gains about one microsecond)
-      const unsigned d_voff = (unsigned)((4 * (lane_e / MI) + (long long)(lane_e % MI) * args.ldd) * 4);
-      const char* d_tile = (const char*)args.d + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldd) * 4;
-      const long long d_col16 = (long long)args.ldd * (MI * 4);
+      const unsigned d_voff = (unsigned)((4 * (lane_e / MI) + (long long)(lane_e % MI) * args.ldd) * CDB);
+      const char* d_tile = (const char*)args.d + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldd) * CDB;
+      const long long d_col16 = (long long)args.ldd * (MI * CDB);
       static_for<0, FN>([&](auto fj_c) {
         constexpr int fj = decltype(fj_c)::value;
         const char* base = d_tile + d_col16 * fj;
@@ -1969,7 +1989,18 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           constexpr int R = 4 * (fj * FM + fi);
           const unsigned vo = d_voff;             // (named here: an operand of an assembly statement does not capture by itself)
           const char* sb = base;
-          asm volatile("global_store_dwordx4 %0, a[%2:%3], %1 offset:%4 sc0 sc1" :: "v"(vo), "s"(sb), "n"(R), "n"(R + 3), "n"(fi * MI * 4) : "memory");
+          if constexpr (HALF_CD) {
+            // one rounding per value (to nearest even, as the conversion of the other paths), two values per register
+            float x0, x1, x2, x3;
+            asm volatile("v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\tv_accvgpr_read_b32 %2, a[%6]\n\tv_accvgpr_read_b32 %3, a[%7]"
+                         : "=v"(x0), "=v"(x1), "=v"(x2), "=v"(x3) : "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
+            int2v out;
+            out[0] = (int)((unsigned)__builtin_bit_cast(unsigned short, (_Float16)x0) | ((unsigned)__builtin_bit_cast(unsigned short, (_Float16)x1) << 16));
+            out[1] = (int)((unsigned)__builtin_bit_cast(unsigned short, (_Float16)x2) | ((unsigned)__builtin_bit_cast(unsigned short, (_Float16)x3) << 16));
+            asm volatile("global_store_dwordx2 %0, %1, %2 offset:%3 sc0 sc1" :: "v"(vo), "v"(out), "s"(sb), "n"(fi * MI * 2) : "memory");
+          } else {
+            asm volatile("global_store_dwordx4 %0, a[%2:%3], %1 offset:%4 sc0 sc1" :: "v"(vo), "s"(sb), "n"(R), "n"(R + 3), "n"(fi * MI * 4) : "memory");
+          }
         });
       });
     } else if constexpr (CPATH != 0) {

@@ -363,6 +363,58 @@ def test_c_streamed_bf16_operands(gpu):
     assert oracle.rel_frobenius(d4, d8.astype(np.float64)) <= 1e-6
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("K", [704, 1344])
+def test_c_streamed_fp16_c_and_d(gpu, ta, tb, K):
+    """An FP16 C and an FP16 D that take 8-byte accesses come in and go out the same way (C one block column per K tile,
+    widened where it is added; D rounded once, to nearest even, where it is stored)."""
+    import torch
+    M, N = 512, 768
+    a, b, _ = operands(M, N, K, ta, tb, 7900 + K)
+    c = rng.matrix("upm1_f16", 7904 + K, (M, N))
+    kw = dict(c=Float16, d=Float16)
+    conf = config(M, N, K, ta, tb, (2, 2), **kw)
+    d = helpers.run_gpu(conf, a, b, c, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
+    assert oracle.rel_frobenius(d, helpers.run_oracle(conf, a, b, c, (M, N), d_dtype=np.float16)) <= TOL
+    ref = oracle.gemm_f64(a, b, c, 1.0, 1.0, ta, tb)
+    # one rounding to FP16: half a unit in the last place of every element (2^-11 relative)
+    assert np.all(np.abs(d.astype(np.float64) - ref) <= np.abs(ref) * 2.0 ** -11 + 1e-4)
+    # sums of small integers that FP16 represents: exact wherever C enters the sum
+    rs = np.random.RandomState(K)
+    ai = np.asfortranarray(rs.randint(-1, 2, size=a.shape).astype(np.float16))
+    bi = np.asfortranarray(rs.randint(-1, 2, size=b.shape).astype(np.float16))
+    ci = np.asfortranarray(rs.randint(-500, 501, size=(M, N)).astype(np.float16))
+    di = helpers.run_gpu(conf, ai, bi, ci, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
+    assert np.array_equal(di.astype(np.float64), oracle.gemm_f64(ai, bi, ci, 1.0, 1.0, ta, tb))
+    # the eight waves start from C and round the same way: the same values but for the last place of a few
+    d8 = helpers.run_gpu(config(M, N, K, ta, tb, (2, 4), **kw), a, b, c, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
+    assert np.mean(d != d8) <= 1e-3
+    assert oracle.rel_frobenius(d, d8.astype(np.float64)) <= 1e-4
+
+
+def test_c_streamed_fp16_c_and_d_in_place_and_as_a_window(gpu):
+    """d aliases c; C and D as windows of larger FP16 matrices: nothing is written outside."""
+    import torch
+    M, N, K = 256, 512, 960
+    a, b, _ = operands(M, N, K, False, False, 7950)
+    c = rng.matrix("upm1_f16", 7953, (M, N))
+    conf = config(M, N, K, False, False, (2, 2), c=Float16, d=Float16)
+    ref = oracle.gemm_f64(a, b, c, 1.0, 1.0, False, False)
+    plain = helpers.run_gpu(conf, a, b, c, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined)
+    d_alias = helpers.run_gpu(conf, a, b, c, (M, N), d_dtype=torch.float16, kernel=Kernel.matmul_pipelined, alias_cd=True)
+    assert np.array_equal(d_alias, plain)
+    assert oracle.rel_frobenius(plain, ref) <= TOL
+    ld = M + 8
+    cbig = torch.full((N, ld), 7.0, dtype=torch.float16, device="cuda")
+    dbig = torch.full((N, ld), float("nan"), dtype=torch.float16, device="cuda")
+    C, D = cbig.t()[:M, :], dbig.t()[:M, :]
+    C.copy_(torch.from_numpy(c).cuda())
+    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), C, D, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    assert np.array_equal(D.cpu().numpy(), plain)
+    assert bool(torch.isnan(dbig.t()[M:, :]).all())            # nothing written outside the window
+
+
 # The tiles with a side of 192 on four waves (wave tiles of 128 x 96 and 96 x 128: 48 accumulator blocks per wave),
 # compiled per transpose like their eight-wave arrangements (4 x 2 and 2 x 4 waves).
 WIDE = [((256, 192, 64), (4, 2), [(False, False), (True, False), (False, True)]), ((192, 256, 64), (2, 4), [(True, False), (True, True)])]
