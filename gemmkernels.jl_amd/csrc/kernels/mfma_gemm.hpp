@@ -100,6 +100,14 @@ __device__ __forceinline__ void dma_lane_coords(int q, int lane, int& row, int& 
   else col = (((cs >> 2) ^ G::swz_m(row)) * 4 + ((cs & 3) ^ (((row >> 3) & 1) << 1))) * 8;
 }
 
+// A pointer that is the same in every lane, as one pair of scalar registers that the compiler does not look into.
+__device__ __forceinline__ void pin_scalar(const char*& p) {
+  const unsigned long long x = (unsigned long long)p;
+  int lo = __builtin_amdgcn_readfirstlane((int)(unsigned)x), hi = __builtin_amdgcn_readfirstlane((int)(unsigned)(x >> 32));
+  asm volatile("" : "+s"(lo), "+s"(hi));
+  p = (const char*)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
+}
+
 // Tensor-contraction index maps: walks the K index of a contraction tile by tile.  A tile covers the K modes below
 // `mode` whole and `step` indices of mode `mode` (see GemmArgs::gk_mode); the modes above are the digits of a counter.
 struct KWalker {
@@ -147,14 +155,20 @@ struct KWalker {
 };
 // element offset of k-value k (< BLOCK_K) of a tile from the tile's first k: digits of the modes the tile covers whole,
 // the rest along mode `mode`
-__device__ __forceinline__ long long gett_k_local(const GettDim& gk, int mode, int k, const long long* stride) {
-  long long o = 0;
-  for (int i = 0; i < mode; ++i) {
-    const int q = gett_div(k, gk.magic[i], gk.shift[i]);
-    o += (long long)(k - q * gk.extent[i]) * stride[i];
-    k = q;
+// (modulo 2^32 and written out over all modes like gett_offset_u32: a mode below `mode` gives a digit, mode `mode` takes
+// what is left of k, the modes above it nothing)
+__device__ __forceinline__ unsigned gett_k_local(const GettDim& gk, int mode, int k, const long long* stride) {
+  unsigned o = 0;
+#pragma unroll
+  for (int i = 0; i < kMaxModes; ++i) {
+    const bool whole = i < mode;
+    const unsigned magic = whole ? gk.magic[i] : 0u;
+    const int q = magic == 0 ? k : (int)((unsigned)(((unsigned long long)(unsigned)k * magic) >> 32) >> gk.shift[i]);
+    const int digit = k - q * (whole ? gk.extent[i] : 0);          // (mode `mode`: q = k, the digit is k itself)
+    k = whole ? q : 0;
+    o += (unsigned)digit * (unsigned)(unsigned long long)stride[i];
   }
-  return o + (long long)k * stride[mode];
+  return o;
 }
 
 // Makes every later use of x depend on the point where pin() stands (no instruction is emitted).
@@ -489,7 +503,10 @@ struct MfmaGemmConfig {
   // some sixty scalar instructions and a dozen branches, which a lone wave on a SIMD cannot hide.
   static constexpr int KTABLE_BYTES = (SOLO && GETT_) ? 16 * 1024 : 0;     // 1024 K tiles
   static constexpr int KTABLE_TILES = KTABLE_BYTES / 16;
-  static constexpr int LDS_BYTES = STAGE_BYTES * STAGES + KTABLE_BYTES;
+  // ... and, behind it, the walks over the M and N modes for every row and column of the tile, made once per row by one
+  // lane each: offsets in A and in B (4 bytes per row), of k inside a tile (4 bytes per k, A and B), and in C / D (8 bytes)
+  static constexpr int ROWTAB_BYTES = (SOLO && GETT_) ? (BM_ + BN_ + 2 * BK_) * 4 + (BM_ + BN_) * 8 : 0;
+  static constexpr int LDS_BYTES = STAGE_BYTES * STAGES + KTABLE_BYTES + ROWTAB_BYTES;
   static constexpr int DMA_A = (GA::NDMA + NWAVES - 1) / NWAVES;   // per wave, per tile
   static constexpr int DMA_B = (GB::NDMA + NWAVES - 1) / NWAVES;
   static constexpr int DMA_PER_TILE = DMA_A + DMA_B;
@@ -558,6 +575,19 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   const char* gb;
   long long a_step = 0, b_step = 0;
   unsigned offa[DMA_A], offb[DMA_B];
+  // Which 1 KiB chunk of a tile DMA instruction i of this wave fetches: chunk wave + i * NWAVES, or (GROUPED, the
+  // one-wave-per-SIMD instances) four consecutive chunks per group of four instructions, so that a group shares one LDS
+  // base in M0 and its instructions differ in their immediate offset, which the hardware adds to the LDS address and to
+  // the global address alike (the K loop then writes M0 four times per tile instead of sixteen).  The lane offsets are
+  // lowered by the immediate and raised by kDmaBias, which keeps them non-negative; the tile pointers ga / gb stand
+  // kDmaBias bytes in front of the tile.
+  constexpr bool GROUPED = Cfg::SOLO;
+  constexpr int kDmaBias = GROUPED ? 3072 : 0;
+  auto dma_group_chunk = [&](int i, int ndma) __attribute__((always_inline)) {      // first chunk of the group of instruction i
+    if constexpr (!GROUPED) return wave + i * NWAVES;
+    else { const int g4 = i & ~3, gs = (ndma - g4) < 4 ? (ndma - g4) : 4; return g4 * NWAVES + wave * gs; }
+  };
+  auto dma_chunk = [&](int i, int ndma) __attribute__((always_inline)) { return dma_group_chunk(i, ndma) + (GROUPED ? (i & 3) : 0); };
   [[maybe_unused]] KWalker walk;
   if constexpr (Cfg::GETT) walk.init(args.gk, args.gk_mode, args.gk_step);
   if constexpr (!Cfg::GETT) {
@@ -583,7 +613,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i) {
       int row, col;
-      dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
+      dma_lane_coords<GA, Cfg::A_KIND>(dma_chunk(i, DMA_A), lane, row, col);
       if constexpr (Cfg::PLANAR) {
         int& m = Cfg::A_KIND == OPK_KMAJOR ? row : col;
         bool imag;
@@ -603,7 +633,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i) {
       int row, col;
-      dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
+      dma_lane_coords<GB, Cfg::B_KIND>(dma_chunk(i, DMA_B), lane, row, col);
       if constexpr (RAGGED) {
         int& n = Cfg::B_KIND == OPK_KMAJOR ? row : col;
         const int last = Cfg::B_KIND == OPK_KMAJOR ? args.N - n0 - 1 : ((args.N - n0 - 1) >> 3) << 3;
@@ -621,24 +651,70 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // modes (done once per lane), the k part inside a tile is linear in the first K mode
     ga = (const char*)args.a;
     gb = (const char*)args.b;
+    if constexpr (Cfg::SOLO) {
+      // One walk over the M modes per row of the tile and one over the N modes per column, each by one lane of the
+      // workgroup, into tables in LDS; the lanes then look up the rows and columns of their DMA chunks (and, before the K
+      // loop, of their blocks of C / D).  Every lane walking the tables for its own sixteen chunks and sixteen block
+      // origins was thirty-two walks with integer divisions in front of the first DMA and the first MFMA.
+      static_assert(BM == Cfg::THREADS && BN == Cfg::THREADS && BK <= Cfg::THREADS, "one row, one column and at most one k per lane");
+      unsigned* tab_a = (unsigned*)(smem + Cfg::STAGE_BYTES * STAGES + Cfg::KTABLE_BYTES);
+      unsigned* tab_b = tab_a + BM;
+      unsigned* tab_ka = tab_b + BN;
+      unsigned* tab_kb = tab_ka + BK;
+      long long* tab_dm = (long long*)(tab_kb + BK);
+      long long* tab_dn = tab_dm + BM;
+      const int t = (int)threadIdx.x;
+      long long o0, o1;
+      gett_offsets32(args.gm, m0 + t, o0, o1);
+      tab_a[t] = (unsigned)(unsigned long long)o0;
+      tab_dm[t] = o1;
+      gett_offsets32(args.gn, n0 + t, o0, o1);
+      tab_b[t] = (unsigned)(unsigned long long)o0;
+      tab_dn[t] = o1;
+      if (t < BK) {
+        tab_ka[t] = gett_k_local(args.gk, args.gk_mode, t, args.gk.stride0);
+        tab_kb[t] = gett_k_local(args.gk, args.gk_mode, t, args.gk.stride1);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < DMA_A; ++i) {
+        int row, col;
+        dma_lane_coords<GA, Cfg::A_KIND>(dma_chunk(i, DMA_A), lane, row, col);
+        const int r = Cfg::A_KIND == OPK_KMAJOR ? row : col, k = Cfg::A_KIND == OPK_KMAJOR ? col : row;
+        offa[i] = (tab_a[r] + tab_ka[k]) * 2u;
+      }
+#pragma unroll
+      for (int i = 0; i < DMA_B; ++i) {
+        int row, col;
+        dma_lane_coords<GB, Cfg::B_KIND>(dma_chunk(i, DMA_B), lane, row, col);
+        const int r = Cfg::B_KIND == OPK_KMAJOR ? row : col, k = Cfg::B_KIND == OPK_KMAJOR ? col : row;
+        offb[i] = (tab_b[r] + tab_kb[k]) * 2u;
+      }
+    } else {
 #pragma unroll
     for (int i = 0; i < DMA_A; ++i) {
       int row, col;
-      dma_lane_coords<GA, Cfg::A_KIND>(wave + i * NWAVES, lane, row, col);
+      dma_lane_coords<GA, Cfg::A_KIND>(dma_chunk(i, DMA_A), lane, row, col);
       const int r = Cfg::A_KIND == OPK_KMAJOR ? row : col, k = Cfg::A_KIND == OPK_KMAJOR ? col : row;
-      long long o0, o1;
-      gett_offsets32(args.gm, m0 + r, o0, o1);
-      offa[i] = (unsigned)((o0 + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride0)) * 2);
+      offa[i] = (gett_offset_u32(args.gm, m0 + r, args.gm.stride0) + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride0)) * 2u;
     }
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i) {
       int row, col;
-      dma_lane_coords<GB, Cfg::B_KIND>(wave + i * NWAVES, lane, row, col);
+      dma_lane_coords<GB, Cfg::B_KIND>(dma_chunk(i, DMA_B), lane, row, col);
       const int r = Cfg::B_KIND == OPK_KMAJOR ? row : col, k = Cfg::B_KIND == OPK_KMAJOR ? col : row;
-      long long o0, o1;
-      gett_offsets32(args.gn, n0 + r, o0, o1);
-      offb[i] = (unsigned)((o0 + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride1)) * 2);
+      offb[i] = (gett_offset_u32(args.gn, n0 + r, args.gn.stride0) + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride1)) * 2u;
     }
+    }
+  }
+
+  if constexpr (GROUPED) {
+#pragma unroll
+    for (int i = 0; i < DMA_A; ++i) offa[i] += (unsigned)(kDmaBias - (i & 3) * 1024);
+#pragma unroll
+    for (int i = 0; i < DMA_B; ++i) offb[i] += (unsigned)(kDmaBias - (i & 3) * 1024);
+    ga -= kDmaBias;
+    gb -= kDmaBias;
   }
 
   auto issue_tile = [&](int stage) {
@@ -651,12 +727,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       pb = gb + walk.offset_b() * 2;
       walk.advance();
     }
-#pragma unroll
-    for (int i = 0; i < DMA_A; ++i)
-      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int i = 0; i < DMA_B; ++i)
-      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+    static_for<0, DMA_A>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + dma_group_chunk(i, DMA_A) * 1024), 16, GROUPED ? (i & 3) * 1024 : 0, 0);
+    });
+    static_for<0, DMA_B>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + dma_group_chunk(i, DMA_B) * 1024), 16, GROUPED ? (i & 3) * 1024 : 0, 0);
+    });
     if constexpr (!Cfg::GETT) {
       ga += a_step;
       gb += b_step;
@@ -681,18 +759,20 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // (the offsets pass through an empty assembly statement: their widening to 64 bits then stays next to the DMA
     // instruction, which takes the tile pointer from scalar registers and the 32-bit offset from the lane, instead of
     // being hoisted out of the loop as sixteen register pairs and a 64-bit addition per instruction)
-#pragma unroll
-    for (int i = 0; i < DMA_A; ++i)
-      if ((i % NP) == P) {
+    static_for<0, DMA_A>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      if constexpr ((i % NP) == P) {
         asm volatile("" : "+v"(offa[i]));
-        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + (wave + i * NWAVES) * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pa + offa[i]), GK_LDS_PTR(void, sa + dma_group_chunk(i, DMA_A) * 1024), 16, GROUPED ? (i & 3) * 1024 : 0, 0);
       }
-#pragma unroll
-    for (int i = 0; i < DMA_B; ++i)
-      if (((DMA_A + i) % NP) == P) {
+    });
+    static_for<0, DMA_B>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      if constexpr (((DMA_A + i) % NP) == P) {
         asm volatile("" : "+v"(offb[i]));
-        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + (wave + i * NWAVES) * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR(pb + offb[i]), GK_LDS_PTR(void, sb + dma_group_chunk(i, DMA_B) * 1024), 16, GROUPED ? (i & 3) * 1024 : 0, 0);
       }
+    });
     if constexpr (P == NP - 1 && !Cfg::GETT) {
       ga += a_step;
       gb += b_step;
@@ -720,8 +800,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   }
 
   // (SOLO: the loop leaves ga / gb at the last tile it fetched, so the tile behind the loop is kept here)
-  [[maybe_unused]] const char* ga_tail = ga;
-  [[maybe_unused]] const char* gb_tail = gb;
+  [[maybe_unused]] const char* ga_tail = ga + kDmaBias;
+  [[maybe_unused]] const char* gb_tail = gb + kDmaBias;
   if constexpr (Cfg::SOLO && RAGGED_K) {
     ga_tail += (long long)KT * a_step;
     gb_tail += (long long)KT * b_step;
@@ -732,13 +812,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   for (int s = 0; s < (Cfg::SOLO ? STAGES : STAGES - 1); ++s)
     if (s < KT) issue_tile(s);      // (SOLO: both stages are free and the loop issues tile kt + 2 from tile kt)
   if constexpr (Cfg::SOLO && Cfg::GETT) {
-    // element offsets of K tile t in A and in B (published by the barrier in front of the K loop)
+    // where K tile t starts in A and in B: the pointers that the DMA of the tile takes as its scalar base (published by the
+    // barrier in front of the K loop)
     long long* table = (long long*)(smem + Cfg::STAGE_BYTES * STAGES);
     for (int t = (int)threadIdx.x; t < KT; t += Cfg::THREADS) {
       long long oa, ob;
       gett_offsets32(args.gk, t * BK, oa, ob);
-      table[2 * t] = oa;
-      table[2 * t + 1] = ob;
+      table[2 * t] = (long long)(ga + oa * 2);
+      table[2 * t + 1] = (long long)(gb + ob * 2);
     }
   }
 
@@ -865,11 +946,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   [[maybe_unused]] long long solo_om[Cfg::GETT ? FM : 1], solo_on[Cfg::GETT ? FN : 1];
   [[maybe_unused]] auto solo_origins = [&](int row, int col) __attribute__((always_inline)) {
     if constexpr (Cfg::GETT) {
-      long long t0;
+      // (from the tables of the tile's rows and columns, see the DMA offsets)
+      const long long* tab_dm = (const long long*)(smem + Cfg::STAGE_BYTES * STAGES + Cfg::KTABLE_BYTES + (BM + BN + 2 * BK) * 4);
+      const long long* tab_dn = tab_dm + BM;
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi) gett_offsets32(args.gm, row + MI * fi, t0, solo_om[fi]);
+      for (int fi = 0; fi < FM; ++fi) solo_om[fi] = tab_dm[row - m0 + MI * fi];
 #pragma unroll
-      for (int fj = 0; fj < FN; ++fj) gett_offsets32(args.gn, col + MI * fj, t0, solo_on[fj]);
+      for (int fj = 0; fj < FN; ++fj) solo_on[fj] = tab_dn[col - n0 + MI * fj];
     }
   };
   [[maybe_unused]] auto solo_off = [&](int row, int col, int fi, int fj, long long ld, [[maybe_unused]] long long plane) -> long long {
@@ -879,7 +962,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   };
   if constexpr (Cfg::SOLO) {
     static_assert(!Cfg::GETT || CPATH != 0, "contractions run the four waves with 16-byte C / D accesses only");
-    if (load_c && !STREAM_C) solo_origins(solo_row, solo_col);
+    // (contractions: the walks over the modes -- integer divisions, sixteen per lane -- run here, while the first tiles are
+    // on their way, and their results stay in registers over the K loop; behind the loop they stood between the last MFMA
+    // and the first store)
+    if (Cfg::GETT || (load_c && !STREAM_C)) solo_origins(solo_row, solo_col);
     if constexpr (CPATH == 3) {
       // FP32 C with 16-byte accesses (at any 4-byte alignment), tiles over the edge included: rows and columns outside are
       // read from the last ones inside, and what is accumulated on them is never stored
@@ -1286,8 +1372,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       // instruction, which then takes the tile pointer from scalar registers and the 32-bit offset from the lane)
       unsigned& o = I < DMA_A ? offa[I < DMA_A ? I : 0] : offb[I < DMA_A ? 0 : I - DMA_A];
       asm volatile("" : "+v"(o));
-      if constexpr (I < DMA_A) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR((Cfg::GETT ? part_a : ga) + o), GK_LDS_PTR(void, sa + (wave + I * NWAVES) * 1024), 16, 0, 0);
-      else __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR((Cfg::GETT ? part_b : gb) + o), GK_LDS_PTR(void, sb + (wave + (I - DMA_A) * NWAVES) * 1024), 16, 0, 0);
+      if constexpr (I < DMA_A) __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR((Cfg::GETT ? part_a : ga) + o), GK_LDS_PTR(void, sa + dma_group_chunk(I, DMA_A) * 1024), 16, GROUPED ? (I & 3) * 1024 : 0, 0);
+      else __builtin_amdgcn_global_load_lds(GK_GLOBAL_PTR((Cfg::GETT ? part_b : gb) + o), GK_LDS_PTR(void, sb + dma_group_chunk(I - DMA_A, DMA_B) * 1024), 16, GROUPED ? ((I - DMA_A) & 3) * 1024 : 0, 0);
     };
     // LDS instruction R of the fragment reads of k-step KS2 (of the stage the readers stand at), into buffer KS2 & 1
     // (into buffer BUF)
@@ -1374,6 +1460,34 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
         asm volatile("v_accvgpr_write_b32 a[%2], %0\n\tv_accvgpr_write_b32 a[%3], %1" :: "v"(t0), "v"(t1), "n"(R + E), "n"(R + E + 1));
       }
     };
+    // Contractions: the table entry of K tile kt + 2 (where the tile starts in A and in B) is read from LDS in a slot of the
+    // last k-step of tile kt - 1, has arrived when the first k-step of tile kt starts, and becomes the tile pointers of the
+    // DMA in two MFMA slots of that k-step, behind the fragment reads (in front of the k-step that issues the DMA the two
+    // pairs of v_readfirstlane and the scalar additions behind them stood between two MFMAs: some hundred clocks per K tile
+    // in which the matrix core had nothing to do).
+    [[maybe_unused]] int4v ktab;                              // a table entry on its way from LDS
+    [[maybe_unused]] int gett_next_entry = 0;                 // which one the next DMA k-step asks for
+    [[maybe_unused]] auto gett_read_entry = [&](int t) __attribute__((always_inline)) {
+      const unsigned addr = lds_base + (unsigned)(Cfg::STAGE_BYTES * STAGES) + 16u * (unsigned)t;
+      asm volatile("ds_read_b128 %0, %1" : "=v"(ktab) : "v"(addr) : "memory");
+    };
+    [[maybe_unused]] auto gett_pointer_a = [&]() __attribute__((always_inline)) {
+      asm volatile("" : "+v"(ktab));
+      // (one pair of scalar registers, opaque to the compiler: the DMA instructions take it as their scalar base next to the
+      // lane's 32-bit offset)
+      part_a = (const char*)(((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane(ktab[1]) << 32) | (unsigned)__builtin_amdgcn_readfirstlane(ktab[0]));
+      pin_scalar(part_a);
+    };
+    [[maybe_unused]] auto gett_pointer_b = [&]() __attribute__((always_inline)) {
+      asm volatile("" : "+v"(ktab));
+      part_b = (const char*)(((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane(ktab[3]) << 32) | (unsigned)__builtin_amdgcn_readfirstlane(ktab[2]));
+      pin_scalar(part_b);
+    };
+    // What the read addresses move by when the readers go on to the next stage.  The additions (one per address register)
+    // stand in MFMA slots of the last k-step but one of a tile, behind its fragment reads, which are the last that use the
+    // old addresses; between the barrier and the first MFMA of the last k-step they were six to eight instructions with
+    // the matrix core idle (4096^3: 1.2-1.5 us).
+    [[maybe_unused]] unsigned stage_step = 0;
     // PAR: the fragment buffer that the MFMAs of this k-step read (the reads go into the other one)
     // RD: the k-step reads the fragments of the next one
     auto phase = [&](auto ks_c, auto dma_c, int dma_stage, auto lg_c, auto ag_c, auto first_c, auto par_c, auto rd_c) __attribute__((always_inline)) {
@@ -1417,6 +1531,27 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           read_op(std::integral_constant<int, i / RSP>{}, std::integral_constant<int, NKS>{}, std::integral_constant<int, (PAR ^ 1)>{});
           __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (!DMA && ks == KS - 2 && RD) {
+          // (odd distances from the last fragment read: the loads of C and the tile pointers of a contraction take even ones
+          // and the distances 1 and 5)
+          constexpr int NBA = RA::NBASE, NBB = RB::NBASE, S0 = NOPS * RSP + 7;
+          constexpr int SSTEP = (S0 + 2 * (NBA + NBB - 1) < NM) ? 2 : 1;
+          static_assert(S0 + SSTEP * (NBA + NBB - 1) < NM, "the address updates fit behind the fragment reads");
+          if constexpr (i >= S0 && (i - S0) % SSTEP == 0 && (i - S0) / SSTEP < NBA + NBB) {
+            constexpr int J = (i - S0) / SSTEP;
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (J < NBA) ra.cur[J] += stage_step; else rb.cur[J - NBA] += stage_step;
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        if constexpr (Cfg::GETT && DMA && RD) {
+          if constexpr (i == NOPS * RSP + 1) { __builtin_amdgcn_sched_barrier(0); gett_read_entry(gett_next_entry); __builtin_amdgcn_sched_barrier(0); }
+        }
+        if constexpr (Cfg::GETT && !DMA && ks == 0 && RD) {
+          static_assert(!Cfg::GETT || NOPS * RSP + 6 < NM, "the slots of the tile pointers lie behind the fragment reads");
+          if constexpr (i == NOPS * RSP + 1) { __builtin_amdgcn_sched_barrier(0); gett_pointer_a(); __builtin_amdgcn_sched_barrier(0); }
+          if constexpr (i == NOPS * RSP + 5) { __builtin_amdgcn_sched_barrier(0); gett_pointer_b(); __builtin_amdgcn_sched_barrier(0); }
+        }
         if constexpr (STREAM_C && !B_BOTH) {
           constexpr int LSLOT0 = NOPS * RSP + 2;                   // (behind the fragment reads)
           constexpr int LSTEP = (LSLOT0 + 4 * (CBLK - 1) < NM) ? 4 : (LSLOT0 + 3 * (CBLK - 1) < NM) ? 3 : 2;
@@ -1452,11 +1587,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // tile kt + 2 in step kt.  The last two tiles have nothing left to fetch and are written out behind the loop without
     // the DMA (a branch around every DMA instruction would cost more issue slots than the instruction; fetching the last
     // tile again into a stage nobody reads, as an earlier version did, costs the memory pipeline two tiles' worth of time).
-    [[maybe_unused]] int4v ktab;                              // contractions: a table entry on its way from LDS
     if (KT > 1) wait_vmcnt<DPT>(); else wait_vmcnt<0>();
     block_barrier();
     ra.set_stage(lds_base);
     rb.set_stage(lds_base + GA::BYTES);
+    if constexpr (Cfg::GETT) gett_read_entry(2 < KT ? 2 : KT - 1);      // (the table is published by the barrier above)
     static_for<0, NOPS>([&](auto r_c) { read_op(r_c, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
     // DMA: the tile fetches tile kt + 2; LAST: there is no tile kt + 1 (nothing to wait for, nothing to read ahead)
     // PEND: loads of C, younger than the DMA of tile kt + 1, that stay in flight over the wait for that tile
@@ -1473,30 +1608,18 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
             // (the loads of C that this tile has issued stay in flight: memory reads return in order, and they are younger than the DMA)
             wait_vmcnt<decltype(pend_c)::value>();
             block_barrier();
-            const unsigned stage_addr = lds_base + (unsigned)((kt + 1) & 1) * Cfg::STAGE_BYTES;
-            ra.set_stage(stage_addr);
-            rb.set_stage(stage_addr + GA::BYTES);
+            // (the readers' addresses moved on to the stage of tile kt + 1 in the k-step before, see stage_step)
           }
-          if constexpr (Cfg::GETT) {
-            // (read a k-step ago; the same value in every lane)
-            asm volatile("" : "+v"(ktab));
-            const unsigned long long oa = ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane(ktab[1]) << 32) | (unsigned)__builtin_amdgcn_readfirstlane(ktab[0]);
-            const unsigned long long ob = ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane(ktab[3]) << 32) | (unsigned)__builtin_amdgcn_readfirstlane(ktab[2]);
-            part_a = ga + (long long)oa * 2;
-            part_b = gb + (long long)ob * 2;
-          }
+          // contractions: the table entry of the tile that the DMA k-step of the next tile fetches (tile kt + 3, or the last
+          // tile once more) is read in a slot of this k-step and arrives with the fragments that it reads
+          if constexpr (Cfg::GETT) gett_next_entry = kt + 3 < KT ? kt + 3 : KT - 1;
           phase(ks_c, dma_c, kt & 1, NoGroup{}, ag_c, No{}, std::integral_constant<int, (ks & 1)>{}, std::integral_constant<bool, !LAST>{});
           if constexpr (decltype(dma_c)::value) { ga += a_step; gb += b_step; }
         } else {
-          if constexpr (Cfg::GETT && ks == 0) {
-            // the table entry of the tile that the next k-step fetches (tile kt + 2, or the last tile once more); it
-            // arrives with the fragments of that k-step
-            const int t = kt + 2 < KT ? kt + 2 : KT - 1;
-            const unsigned addr = lds_base + (unsigned)(Cfg::STAGE_BYTES * STAGES) + 16u * (unsigned)t;
-            asm volatile("ds_read_b128 %0, %1" : "=v"(ktab) : "v"(addr) : "memory");
-          }
+          if constexpr (ks == KS - 2) stage_step = ((kt + 1) & 1) ? (unsigned)Cfg::STAGE_BYTES : 0u - (unsigned)Cfg::STAGE_BYTES;
           if constexpr (ks == 0) phase(ks_c, No{}, 0, lg_c, NoGroup{}, first_c, std::integral_constant<int, 0>{}, Yes{});
           else phase(ks_c, No{}, 0, NoGroup{}, NoGroup{}, No{}, std::integral_constant<int, (ks & 1)>{}, Yes{});
+          if constexpr (ks == KS - 2) { ra.stage_addr += stage_step; rb.stage_addr += stage_step; }
         }
       });
     };
@@ -1528,6 +1651,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     if constexpr (RAGGED_K) {
       // the last, partial K tile, outside the schedule of the loop: the k-steps that hold valid values
       if (tail_k > 0) {
+        stage_step = 0;                                  // (the k-steps below read one stage)
         fetch_tail_tile(ga_tail, gb_tail);
         static_for<0, KS>([&](auto ks_c) {
           constexpr int ks = decltype(ks_c)::value;
@@ -1854,7 +1978,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     asm volatile("" : "+v"(lane_e));
     const int solo_row = (Cfg::PLANAR ? (m0 + wm * Cfg::WTM) / 2 : m0 + wm * Cfg::WTM) + 4 * (lane_e / MI);
     const int solo_col = (Cfg::COLS_FRAG ? (n0 + wn * Cfg::WTN) / 2 : n0 + wn * Cfg::WTN) + (lane_e % MI);      // (as before the K loop)
-    solo_origins(solo_row, solo_col);
+    if constexpr (!Cfg::GETT) solo_origins(solo_row, solo_col);
     if constexpr (Cfg::PLANAR) {
       // (row blocks of re A | im A) x (block columns of re B | im B): real part re*re - im*im into the upper left block,
       // imaginary part im*re + re*im into the lower left one; C came in through the same two

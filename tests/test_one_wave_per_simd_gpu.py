@@ -6,7 +6,7 @@ Comparisons with the eight-wave arrangement of the same tile come on top of that
 summation order is the same by construction -- C loaded before the K loop or absent, tiles over the edges, the fused,
 complex and contraction kernels: the k-steps and the products inside them run in the same order however a tile is dealt
 out to waves -- the two must agree bit for bit, which catches a wrong register, lane or address that a norm would let
-pass.  Where C is added during the first K tiles (plain products of at least eleven K tiles with FP32 C / D) the place of
+pass.  Where C is added during the first K tiles (plain products of at least eleven K tiles with FP32 or FP16 C / D) the place of
 that one addition differs, so the two agree to rounding only; there the tests pin what the order cannot change: linearity
 in C, D(C) - D(0) = C, and sums of small integers, which are exact in any order.
 
