@@ -77,10 +77,21 @@ __host__ __device__ inline int gett_div(int n, unsigned magic, int shift) {
   return (int)((unsigned)(((unsigned long long)(unsigned)n * magic) >> 32) >> shift);
 }
 // the two element offsets of index idx (< 2^31) of a GEMM dimension: a mixed-radix walk over its modes
-// (written out over all kMaxModes modes, a mode beyond nmodes as one of extent 1: on the device the table entries are then
-// read at constant places of the kernel arguments, once for all the walks of a kernel, where a loop over nmodes read them
-// again, and waited for them, in every iteration of every walk)
 __host__ __device__ inline void gett_offsets32(const GettDim& d, int idx, long long& off0, long long& off1) {
+  off0 = 0; off1 = 0;
+  for (int i = 0; i < d.nmodes; ++i) {
+    const int q = gett_div(idx, d.magic[i], d.shift[i]);
+    const int digit = idx - q * d.extent[i];
+    idx = q;
+    off0 += (long long)digit * d.stride0[i];
+    off1 += (long long)digit * d.stride1[i];
+  }
+}
+// The same walk written out over all kMaxModes modes, a mode beyond nmodes as one of extent 1: the table entries are then
+// read at constant places of the kernel arguments, once for all the walks of a kernel, where the loop over nmodes reads
+// them again, and waits for them, in every iteration of every walk.  It holds the tables in some sixty scalar registers
+// meanwhile: for kernels that make few walks and have the registers to spare (the one-wave-per-SIMD contraction kernel).
+__host__ __device__ inline void gett_offsets32_flat(const GettDim& d, int idx, long long& off0, long long& off1) {
   off0 = 0; off1 = 0;
 #pragma unroll
   for (int i = 0; i < kMaxModes; ++i) {
@@ -92,21 +103,6 @@ __host__ __device__ inline void gett_offsets32(const GettDim& d, int idx, long l
     off0 += (long long)digit * (on ? d.stride0[i] : 0ll);
     off1 += (long long)digit * (on ? d.stride1[i] : 0ll);
   }
-}
-// The same walk for one set of strides, modulo 2^32: the byte offset of a lane inside an operand tile (its DMA offset) is
-// below 2^32 and takes a third of the instructions this way.
-__host__ __device__ inline unsigned gett_offset_u32(const GettDim& d, int idx, const long long* stride) {
-  unsigned off = 0;
-#pragma unroll
-  for (int i = 0; i < kMaxModes; ++i) {
-    const bool on = i < d.nmodes;
-    const unsigned magic = on ? d.magic[i] : 0u;
-    const int q = magic == 0 ? idx : (int)((unsigned)(((unsigned long long)(unsigned)idx * magic) >> 32) >> d.shift[i]);
-    const int digit = idx - q * (on ? d.extent[i] : 1);
-    idx = q;
-    off += (unsigned)digit * (on ? (unsigned)(unsigned long long)stride[i] : 0u);
-  }
-  return off;
 }
 
 __host__ __device__ inline void gett_offsets(const GettDim& d, long long idx, long long& off0, long long& off1) {

@@ -155,9 +155,18 @@ struct KWalker {
 };
 // element offset of k-value k (< BLOCK_K) of a tile from the tile's first k: digits of the modes the tile covers whole,
 // the rest along mode `mode`
-// (modulo 2^32 and written out over all modes like gett_offset_u32: a mode below `mode` gives a digit, mode `mode` takes
-// what is left of k, the modes above it nothing)
-__device__ __forceinline__ unsigned gett_k_local(const GettDim& gk, int mode, int k, const long long* stride) {
+__device__ __forceinline__ long long gett_k_local(const GettDim& gk, int mode, int k, const long long* stride) {
+  long long o = 0;
+  for (int i = 0; i < mode; ++i) {
+    const int q = gett_div(k, gk.magic[i], gk.shift[i]);
+    o += (long long)(k - q * gk.extent[i]) * stride[i];
+    k = q;
+  }
+  return o + (long long)k * stride[mode];
+}
+// (the same modulo 2^32 and written out over all modes like gett_offsets32_flat: a mode below `mode` gives a digit, mode
+// `mode` takes what is left of k, the modes above it nothing)
+__device__ __forceinline__ unsigned gett_k_local_flat(const GettDim& gk, int mode, int k, const long long* stride) {
   unsigned o = 0;
 #pragma unroll
   for (int i = 0; i < kMaxModes; ++i) {
@@ -665,15 +674,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       long long* tab_dn = tab_dm + BM;
       const int t = (int)threadIdx.x;
       long long o0, o1;
-      gett_offsets32(args.gm, m0 + t, o0, o1);
+      gett_offsets32_flat(args.gm, m0 + t, o0, o1);
       tab_a[t] = (unsigned)(unsigned long long)o0;
       tab_dm[t] = o1;
-      gett_offsets32(args.gn, n0 + t, o0, o1);
+      gett_offsets32_flat(args.gn, n0 + t, o0, o1);
       tab_b[t] = (unsigned)(unsigned long long)o0;
       tab_dn[t] = o1;
       if (t < BK) {
-        tab_ka[t] = gett_k_local(args.gk, args.gk_mode, t, args.gk.stride0);
-        tab_kb[t] = gett_k_local(args.gk, args.gk_mode, t, args.gk.stride1);
+        tab_ka[t] = gett_k_local_flat(args.gk, args.gk_mode, t, args.gk.stride0);
+        tab_kb[t] = gett_k_local_flat(args.gk, args.gk_mode, t, args.gk.stride1);
       }
       __syncthreads();
 #pragma unroll
@@ -696,14 +705,18 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       int row, col;
       dma_lane_coords<GA, Cfg::A_KIND>(dma_chunk(i, DMA_A), lane, row, col);
       const int r = Cfg::A_KIND == OPK_KMAJOR ? row : col, k = Cfg::A_KIND == OPK_KMAJOR ? col : row;
-      offa[i] = (gett_offset_u32(args.gm, m0 + r, args.gm.stride0) + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride0)) * 2u;
+      long long o0, o1;
+      gett_offsets32(args.gm, m0 + r, o0, o1);
+      offa[i] = (unsigned)((o0 + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride0)) * 2);
     }
 #pragma unroll
     for (int i = 0; i < DMA_B; ++i) {
       int row, col;
       dma_lane_coords<GB, Cfg::B_KIND>(dma_chunk(i, DMA_B), lane, row, col);
       const int r = Cfg::B_KIND == OPK_KMAJOR ? row : col, k = Cfg::B_KIND == OPK_KMAJOR ? col : row;
-      offb[i] = (gett_offset_u32(args.gn, n0 + r, args.gn.stride0) + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride1)) * 2u;
+      long long o0, o1;
+      gett_offsets32(args.gn, n0 + r, o0, o1);
+      offb[i] = (unsigned)((o0 + gett_k_local(args.gk, args.gk_mode, k, args.gk.stride1)) * 2);
     }
     }
   }
