@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0
 HEADLINE_SETTLE_SECONDS = 0.4
 # HBM bytes per launch of the headline kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # summarised in profiles/ (None until measured)
-MEASURED_TRAFFIC_BYTES = 336_763_904   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131667.5 * 2.0 + 65536.0) KiB
+MEASURED_TRAFFIC_BYTES = 336_739_328   # profiles/mfma_gemm_config2_hbm_traffic.txt: (131655.5 * 2.0 + 65536.0) KiB
 TRAFFIC_SOURCE = "profiles/mfma_gemm_config2_hbm_traffic.txt (a constant from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE passes, not a reading of this run)"
 
 
