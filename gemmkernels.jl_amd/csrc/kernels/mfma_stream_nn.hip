@@ -2,5 +2,6 @@
 #define GK_A_KMAJOR false
 #define GK_B_KMAJOR true
 #define GK_FAMILY_FN family_mfma_stream_nn
+#define GK_FAMILY_FN_BF16 family_mfma_stream_nn_bf16
 #define GK_TAG "nn"
 #include "mfma_stream_instances.inc"

@@ -2,5 +2,6 @@
 #define GK_A_KMAJOR false
 #define GK_B_KMAJOR false
 #define GK_FAMILY_FN family_mfma_stream_nt
+#define GK_FAMILY_FN_BF16 family_mfma_stream_nt_bf16
 #define GK_TAG "nt"
 #include "mfma_stream_instances.inc"

@@ -2,5 +2,6 @@
 #define GK_A_KMAJOR true
 #define GK_B_KMAJOR true
 #define GK_FAMILY_FN family_mfma_stream_tn
+#define GK_FAMILY_FN_BF16 family_mfma_stream_tn_bf16
 #define GK_TAG "tn"
 #include "mfma_stream_instances.inc"

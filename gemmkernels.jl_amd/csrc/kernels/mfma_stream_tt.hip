@@ -2,5 +2,6 @@
 #define GK_A_KMAJOR true
 #define GK_B_KMAJOR false
 #define GK_FAMILY_FN family_mfma_stream_tt
+#define GK_FAMILY_FN_BF16 family_mfma_stream_tt_bf16
 #define GK_TAG "tt"
 #include "mfma_stream_instances.inc"
