@@ -957,6 +957,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
   // first row of every row block (the other three follow in the first M mode, whose stride in C / D is 1 and whose extent
   // is a multiple of 4: the host runs these instances on nothing else) and the N modes for its column of every block column.
   [[maybe_unused]] long long solo_om[Cfg::GETT ? FM : 1], solo_on[Cfg::GETT ? FN : 1];
+  [[maybe_unused]] float bcol_early[Cfg::FUSE == 4 ? FN : 1], brow_early[Cfg::FUSE == 4 ? FM * 4 : 1];      // the lane's bias values (see below)
   [[maybe_unused]] auto solo_origins = [&](int row, int col) __attribute__((always_inline)) {
     if constexpr (Cfg::GETT) {
       // (from the tables of the tile's rows and columns, see the DMA offsets)
@@ -979,6 +980,17 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
     // on their way, and their results stay in registers over the K loop; behind the loop they stood between the last MFMA
     // and the first store)
     if (Cfg::GETT || (load_c && !STREAM_C)) solo_origins(solo_row, solo_col);
+    // (hooks of D in closed form: the lane's bias values -- its column of every block column, or its rows of every row block --
+    // are fetched here, behind the DMA of the first tiles, and wait in registers; fetched behind the K loop their latency
+    // stood in front of the first store)
+    if constexpr (Cfg::FUSE == 4) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j) bcol_early[j] = args.epi_kind == 1 ? args.bias[solo_col + MI * j] : 0.0f;
+#pragma unroll
+      for (int fi = 0; fi < FM; ++fi)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) brow_early[4 * fi + v] = args.epi_kind == 2 ? args.bias[solo_row + MI * fi + v] : 0.0f;
+    }
     if constexpr (CPATH == 3) {
       // FP32 C with 16-byte accesses (at any 4-byte alignment), tiles over the edge included: rows and columns outside are
       // read from the last ones inside, and what is accumulated on them is never stored
@@ -2038,16 +2050,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
       const float p00 = args.t[H_RF2SH_D].p0[0], p01 = args.t[H_RF2SH_D].p1[0], p10 = args.t[H_SH2GL_D].p0[0], p11 = args.t[H_SH2GL_D].p1[0];
       const float post = args.acc_post_scale;
       const int epi = args.epi_kind;
-      const float* bias = args.bias;
       const bool d_wide = args.d_dtype == DT_F32 && ((((uintptr_t)args.d) | ((uintptr_t)args.ldd << 2)) & 15u) == 0;
-      // the lane's bias values, fetched once and together: its column of every block column, or its rows of every row block
+      [[maybe_unused]] const unsigned fused_voff = (unsigned)((4 * (lane_e / MI) + (long long)(lane_e % MI) * args.ldd) * 4);
+      [[maybe_unused]] const char* fused_tile = (const char*)args.d + ((long long)(m0 + wm * Cfg::WTM) + (long long)(n0 + wn * Cfg::WTN) * args.ldd) * 4;
+      [[maybe_unused]] const long long fused_col16 = (long long)args.ldd * (MI * 4);
+      // the lane's bias values: its column of every block column, or its rows of every row block
       float bcol[FN], brow[FM * 4];
 #pragma unroll
-      for (int j = 0; j < FN; ++j) bcol[j] = epi == 1 ? bias[solo_col + MI * j] : 0.0f;
+      for (int j = 0; j < FN; ++j) bcol[j] = bcol_early[j];        // (fetched in front of the K loop)
 #pragma unroll
-      for (int fi = 0; fi < FM; ++fi)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) brow[4 * fi + v] = epi == 2 ? bias[solo_row + MI * fi + v] : 0.0f;
+      for (int e = 0; e < FM * 4; ++e) brow[e] = brow_early[e];
       static_for<0, SFN>([&](auto fj_c) __attribute__((always_inline)) {
         constexpr int fj = decltype(fj_c)::value;
         float x[FM * 4];
@@ -2072,20 +2084,32 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
 #pragma unroll
           for (int e = 0; e < FM * 4; ++e) x[e] = f(x[e]);
         });
-#pragma unroll
-        for (int fi = 0; fi < FM; ++fi) {
+        static_for<0, FM>([&](auto fi_c) __attribute__((always_inline)) {
+          constexpr int fi = decltype(fi_c)::value;
           const long long off = solo_off(solo_row, solo_col, fi, fj, args.ldd, args.plane_d);
           if (d_wide) {
             float4v o;
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[v] = x[4 * fi + v];
-            float* dp = (float*)args.d + off;
-            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(dp), "v"(o) : "memory");       // (write-through, see path 4)
+            if constexpr (!Cfg::GETT && !Cfg::PLANAR && !Cfg::COLS_FRAG) {
+              // (the block column's origin in D from scalar registers, the lane's offset in it from a vector register, the row
+              // block as an immediate: no address arithmetic per store, as on path 4)
+              const unsigned vo = fused_voff;
+              const char* sb = fused_tile + fused_col16 * fj;
+              // (the wait states behind the store: a store of more than 8 bytes per lane reads its data registers over several
+              // clocks, and the vector ALU must not write one of them meanwhile; the compiler inserts these for its own
+              // stores and does not know that this statement is one -- without them the first value of a block came out
+              // wrong in a quarter of the lanes whenever the next instruction reused its register)
+              asm volatile("global_store_dwordx4 %0, %1, %2 offset:%3 sc0 sc1\n\ts_nop 1" :: "v"(vo), "v"(o), "s"(sb), "n"(fi * MI * 4) : "memory");
+            } else {
+              float* dp = (float*)args.d + off;
+              asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" :: "v"(dp), "v"(o) : "memory");       // (write-through, see path 4)
+            }
           } else {
 #pragma unroll
             for (int v = 0; v < 4; ++v) store_cd(args.d, args.d_dtype, off + v, x[4 * fi + v]);
           }
-        }
+        });
       });
       return;
     }
@@ -2138,6 +2162,24 @@ __global__ void __launch_bounds__(Cfg::THREADS) mfma_gemm_kernel(const GemmArgs 
           } else {
             asm volatile("global_store_dwordx4 %0, a[%2:%3], %1 offset:%4 sc0 sc1" :: "v"(vo), "s"(sb), "n"(R), "n"(R + 3), "n"(fi * MI * 4) : "memory");
           }
+        });
+      });
+    } else if constexpr (CPATH != 0 && !Cfg::GETT && !Cfg::PLANAR) {
+      // (as on path 4: the block column's origin in D from scalar registers, the lane's offset in it from a vector register,
+      // the row block as an immediate; write-through)
+      const unsigned d_voff = (unsigned)((4 * (lane_e / MI) + (long long)(lane_e % MI) * args.ldd) * 4);
+      const int col0 = Cfg::COLS_FRAG ? (n0 + wn * Cfg::WTN) / 2 : n0 + wn * Cfg::WTN;      // (as solo_col)
+      const char* d_tile = (const char*)args.d + ((long long)(m0 + wm * Cfg::WTM) + (long long)col0 * args.ldd) * 4;
+      const long long d_col16 = (long long)args.ldd * (MI * 4);
+      static_for<0, SFN>([&](auto fj_c) __attribute__((always_inline)) {
+        constexpr int fj = decltype(fj_c)::value;
+        const char* base = d_tile + d_col16 * fj;
+        static_for<0, FM>([&](auto fi_c) __attribute__((always_inline)) {
+          constexpr int fi = decltype(fi_c)::value;
+          const unsigned vo = d_voff;             // (named here: an operand of an assembly statement does not capture by itself)
+          const char* sb = base;
+          AccV& blk = acc[fi][fj];
+          asm volatile("global_store_dwordx4 %0, %1, %2 offset:%3 sc0 sc1" :: "v"(vo), "a"(blk), "s"(sb), "n"(fi * MI * 4) : "memory");
         });
       });
     } else if constexpr (CPATH != 0) {

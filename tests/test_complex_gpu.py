@@ -38,6 +38,27 @@ TRANSPOSES = [(False, False), (False, True), (True, False), (True, True)]
 CASES = [(ta, tb, block) for ta, tb in TRANSPOSES for block in _tiles(ta, tb)]
 
 
+def test_complex_d_as_a_window(gpu):
+    """D as a window of a larger complex matrix (leading dimension beyond M) on the four-wave kernel of 'N','N': same bits
+    as in a matrix of its own, nothing written outside the window."""
+    M, N, K = 256, 384, 320
+    conf = configs.complex_config(M, N, K, False, False, zero_c=True, block_shape=gk.NT(M=128, N=128, K=64))
+    assert "_w2x2" in gk.kernel_name(conf, Kernel.matmul_pipelined)
+    a = configs.complex_matrix(71, M, K)
+    b = configs.complex_matrix(72, K, N)
+    plain = run(conf, a, b, None, M, N)
+    want = to_c128(a) @ to_c128(b)
+    assert oracle.rel_frobenius(plain[0], want.real) <= TOL and oracle.rel_frobenius(plain[1], want.imag) <= TOL
+    ld = M + 24
+    big = gk.colmajor_empty((2, ld, N), torch.float32)
+    big.fill_(float("nan"))
+    D = big[:, :M, :]
+    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), None, D, kernel=Kernel.matmul_pipelined)
+    torch.cuda.synchronize()
+    assert np.array_equal(D.cpu().numpy(), plain)
+    assert bool(torch.isnan(big[:, M:, :]).all())
+
+
 @pytest.mark.parametrize("ta,tb,block", CASES)
 @pytest.mark.parametrize("zero_c", [True, False])
 def test_complex_all_transposes(gpu, ta, tb, block, zero_c):

@@ -156,6 +156,40 @@ def test_hooks_of_d_in_closed_form_and_a_bias_run_on_four_waves(gpu, epilogue_cl
     assert np.array_equal(d4, d8)
 
 
+@pytest.mark.parametrize("case", ["no C", "C before the loop", "bias per column", "bias per row"])
+def test_d_as_a_window_on_the_paths_that_store_from_a_scalar_base(gpu, case):
+    """D (and C) as windows of larger matrices, leading dimension beyond M, on the four-wave paths that take the block
+    column's origin from scalar registers: no C, C loaded before a short K loop, hooks of D in closed form with either bias.
+    Same bits as in a matrix of its own; nothing written outside the window."""
+    import torch
+    M, N, K = 512, 256, 192
+    a, b, c = operands(M, N, K, False, False, 7550)
+    E = Transform.Elementwise
+    with_c = case == "C before the loop"
+    hooks, epi_cls, bias = None, None, None
+    if case.startswith("bias"):
+        hooks = dict(transform_shared_to_global_d=E(Transform.relu))
+        epi_cls = Epilogue.Bias if case == "bias per column" else Epilogue.BiasRow
+        bias = rng.normal_f32(7554, N if epi_cls is Epilogue.Bias else M)
+    conf = config(M, N, K, False, False, (2, 2), zero_c=not with_c)
+    plain = helpers.run_gpu(conf, a, b, c if with_c else None, (M, N), transforms=hooks, epilogue_cls=epi_cls, bias=bias, kernel=Kernel.matmul_pipelined)
+    ref = helpers.run_oracle(conf, a, b, c if with_c else None, (M, N), transforms=hooks, epilogue=epi_cls(0) if epi_cls else None, bias=bias)
+    assert oracle.rel_frobenius(plain, ref) <= TOL
+    ld = M + 64
+    dbig = torch.full((N, ld), float("nan"), dtype=torch.float32, device="cuda")
+    D = dbig.t()[:M, :]
+    C = None
+    if with_c:
+        cbig = torch.full((N, ld), 7.0, dtype=torch.float32, device="cuda")
+        C = cbig.t()[:M, :]
+        C.copy_(torch.from_numpy(c).cuda())
+    keep = torch.from_numpy(np.ascontiguousarray(bias, dtype=np.float32)).cuda() if bias is not None else None
+    gk.matmul(conf, gk.colmajor(a), gk.colmajor(b), C, D, epilogue=epi_cls(keep) if epi_cls else None, kernel=Kernel.matmul_pipelined, **(hooks or {}))
+    torch.cuda.synchronize()
+    assert np.array_equal(D.cpu().numpy(), plain)
+    assert bool(torch.isnan(dbig.t()[M:, :]).all())
+
+
 def test_other_hooks_run_on_eight_waves(gpu):
     """Hooks on C, two ops in one hook of D, a scale folded next to a C, hooks on A that stay in the K loop."""
     M, N, K = 512, 256, 128
