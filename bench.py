@@ -61,6 +61,28 @@ def gk_name(conf):
     return kernel_name(conf, Kernel.matmul_pipelined)
 
 
+def matrix_core_ceiling():
+    """What a register-only loop of the kernels' MFMA instruction delivers on this device, under its power cap, on FP16
+    values spread over [-1, 1) and on zeros (gk_probe_matrix_rate: no memory access at all; a fifth of a second of launches
+    each after as much to settle).  Context for roofline.frac, whose denominator is the data-sheet peak."""
+    import ctypes
+    import torch
+    from gemmkernels import _lib
+    lib = _lib.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for key, rnd in (("random_fp16_tflops", 1), ("zeros_tflops", 0)):
+        t = ctypes.c_double(0.0)
+        for _ in range(2):       # (the first call settles clock and power)
+            rc = lib.gk_probe_matrix_rate(25, 2000, rnd, stream, ctypes.byref(t))
+            if rc != 0:
+                raise RuntimeError(_lib.last_error())
+        out[key] = round(t.value, 1)
+    out["frac_of_peak_on_random_fp16"] = round(out["random_fp16_tflops"] / PEAK_FP16_TFLOPS, 4)
+    out["what"] = "v_mfma_f32_16x16x32_f16 from registers only, one wave per SIMD, 64 accumulator blocks per wave; HIP events"
+    return out
+
+
 def observe_device(fn, bursts=100, launches_per_burst=100):
     """Shader clock, power and temperature the driver reports (sysfs of the first card) while `fn` runs
     back to back for a good second (the power reading is a moving average: the second half of the
@@ -291,6 +313,10 @@ def main():
             result["observed_device"] = observe_device(run)
         except Exception as e:      # readings are for orientation; never fail the benchmark over them
             result["observed_device"] = {"error": f"{type(e).__name__}: {e}"}
+        try:
+            result["matrix_core_ceiling"] = matrix_core_ceiling()
+        except Exception as e:
+            result["matrix_core_ceiling"] = {"error": f"{type(e).__name__}: {e}"}
         # ---------------- the other transposes and configs (outside the timed region) ----------------
         extras = {}
         for cfg, variant in [(2, "NT"), (2, "TN"), (2, "TT"), (1, None), (3, None), ("4a", None), ("4a-planar", None), ("4b", None), (5, None), ("skinny", None)]:

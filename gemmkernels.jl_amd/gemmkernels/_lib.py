@@ -114,6 +114,7 @@ _SIGNATURES = {
     "gk_split_k_noalloc_capacity": (ctypes.c_size_t, []),
     "gk_matmul_split_k_noalloc": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                  ctypes.POINTER(gk_transforms), ctypes.POINTER(gk_epilogue), ctypes.c_void_p]),
+    "gk_probe_matrix_rate": (ctypes.c_int, [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]),
     "gk_rtc_compile": (ctypes.c_int, [ctypes.POINTER(gk_config), ctypes.POINTER(ctypes.c_char_p), ctypes.c_int32,
                                       ctypes.POINTER(ctypes.c_void_p)]),
     "gk_rtc_matmul": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(gk_config), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

@@ -301,6 +301,14 @@ size_t gk_split_k_noalloc_capacity(void);
 int gk_matmul_split_k_noalloc(const gk_config* conf, const void* a, const void* b, const void* c, void* d,
                               const gk_transforms* transforms, const gk_epilogue* epilogue, void* stream);
 
+/* A measurement aid with no counterpart in the reference (its benchmarks quote fractions of a data-sheet peak): the
+ * rate, in TFLOP/s, of a register-only loop of the MFMA instruction the GEMM kernels use (v_mfma_f32_16x16x32_f16,
+ * one wave per SIMD, 64 accumulator blocks per wave, operands that change every 64 MFMAs), over `launches` launches
+ * of `iterations` loop passes each on `stream`, timed with events.  With random_operands != 0 the operands are FP16
+ * values spread over [-1, 1), otherwise zeros: under the power cap of the device the clock, and with it the rate,
+ * depends on the data.  bench.py reports both next to the rate of the headline kernel. */
+int gk_probe_matrix_rate(int32_t launches, int32_t iterations, int32_t random_operands, void* stream, double* tflops);
+
 /* Kernels specialised at run time (hipRTC).  The reference compiles one kernel per Config type and
  * inlines arbitrary Julia functors at the eight transform hooks (src/matmul.jl:38,
  * src/transform.jl:20-30); gk_matmul offers a closed op vocabulary and a table of tiles instead.

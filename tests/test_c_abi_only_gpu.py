@@ -51,3 +51,22 @@ def test_gemm_through_the_c_abi_without_torch(gpu):
     assert rc == _lib.GK_ERR_INVALID_ARGUMENT
     for buf in (A, B, C, D):
         buf.free()
+
+
+def test_matrix_rate_probe(gpu):
+    """The measurement aid of the benchmark: a register-only MFMA loop.  Its rate lies between what no MI355X could fall
+    below while it runs at all and the data-sheet peak of 2516.6 TFLOP/s; zeros draw less power than values spread over
+    [-1, 1) and are at least as fast; arguments out of range are refused."""
+    lib = _lib.lib()
+    rates = {}
+    for rnd in (1, 0):
+        t = ctypes.c_double(0.0)
+        for _ in range(2):
+            assert lib.gk_probe_matrix_rate(10, 1000, rnd, None, ctypes.byref(t)) == _lib.GK_OK, _lib.last_error()
+        rates[rnd] = t.value
+    print("matrix-core rate: %.0f TFLOP/s on random FP16 values, %.0f on zeros" % (rates[1], rates[0]), flush=True)
+    assert 500.0 < rates[1] <= 2516.6 * 1.01 and 500.0 < rates[0] <= 2516.6 * 1.01
+    assert rates[0] >= 0.97 * rates[1]
+    t = ctypes.c_double(0.0)
+    assert lib.gk_probe_matrix_rate(0, 1000, 1, None, ctypes.byref(t)) == _lib.GK_ERR_INVALID_ARGUMENT
+    assert lib.gk_probe_matrix_rate(10, 1000, 1, None, None) == _lib.GK_ERR_INVALID_ARGUMENT
