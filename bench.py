@@ -315,6 +315,7 @@ def main():
             result["observed_device"] = {"error": f"{type(e).__name__}: {e}"}
         try:
             result["matrix_core_ceiling"] = matrix_core_ceiling()
+            result["matrix_core_ceiling"]["headline_frac_of_random_fp16_ceiling"] = round(tflops / result["matrix_core_ceiling"]["random_fp16_tflops"], 4)
         except Exception as e:
             result["matrix_core_ceiling"] = {"error": f"{type(e).__name__}: {e}"}
         # ---------------- the other transposes and configs (outside the timed region) ----------------
